@@ -1,0 +1,15 @@
+"""moe355: MI355X (gfx950) fused MoE forward -- gate -> slot assignment -> expert FFN -> combine.
+
+The product is `libmoe355.so` (C ABI in `include/moe355.h`, HIP kernels in `csrc/`).  This package is the
+thin Python host side over that ABI: torch supplies device memory and the stream, nothing else.  There is no
+fallback path: if the library is not built, importing `cuplayground_amd.api` symbols that need it raises.
+"""
+from .api import (  # noqa: F401
+    MoEConfig,
+    MoELayer,
+    MoEError,
+    combine,
+    gemm_bias_act,
+    library_path,
+    load_library,
+)

@@ -1,0 +1,320 @@
+"""ctypes binding of include/moe355.h plus a small host-side mirror of the operator.
+
+`MoEConfig` carries exactly the keys of the reference's aristos_config.json (aristos_config.schema.json:5-58)
+and this build's extensions; `MoELayer` owns a handle and a workspace tensor and calls `moe_forward`.
+torch is used for device memory and the current HIP stream only.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import json
+import os
+from dataclasses import asdict, dataclass
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libmoe355.so")
+
+DTYPE_F32, DTYPE_TF32, DTYPE_BF16, DTYPE_FP16, DTYPE_FP8 = 0, 1, 2, 3, 4
+ACT_RELU, ACT_GELU, ACT_SWIGLU, ACT_NONE = 0, 1, 2, 3
+GATE_SOFTMAX, GATE_SIGMOID = 0, 1
+FFN_AUTO, FFN_TILED, FFN_PERSISTENT = 0, 1, 2
+STAGES = ("gate", "route", "ffn", "combine")
+
+EXPORTS = (
+    "moe_config_default", "moe_config_from_json_string", "moe_config_from_json_file", "moe_config_validate",
+    "moe_config_tokens", "moe_config_capacity", "moe_create", "moe_destroy", "moe_get_arch", "moe_workspace_bytes",
+    "moe_set_ffn_mode", "moe_forward", "moe_gate", "moe_route", "moe_gemm_bias_act", "moe_combine",
+    "moe_set_stage_timing", "moe_get_stage_ms", "moe_get_task_counts", "moe_last_hip_error", "moe_status_string",
+    "moe_version",
+)
+
+
+class MoEError(RuntimeError):
+    def __init__(self, status: int, what: str = ""):
+        self.status = status
+        msg = load_library().moe_status_string(status).decode()
+        super().__init__("moe355 status %d (%s)%s" % (status, msg, (": " + what) if what else ""))
+
+
+class _CConfig(C.Structure):
+    _fields_ = [("capacity_factor", C.c_double)] + [(n, C.c_int32) for n in (
+        "drop_tokens", "expert_top_k", "is_training", "hidden_act", "hidden_size", "intermediate_size", "micro_batch",
+        "num_experts", "sequence_len", "torch_dtype", "gate_fn", "norm_topk_prob")]
+
+
+class _CArch(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("device", "compute_units", "xcds", "wavefront_size", "lds_bytes_per_cu",
+                                         "max_clock_khz", "persistent_blocks")] + [("name", C.c_char * 64)]
+
+
+class _CWeights(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in ("gate_w", "gate_bias", "w_up", "w_gate", "w_down", "b_up", "b_gate",
+                                          "b_down", "s_up", "s_gate", "s_down")]
+
+
+class _CRouting(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in ("topk_idx", "topk_w", "slot", "expert_count", "expert_offset",
+                                          "token_indices")]
+
+
+_lib = None
+
+
+def library_path() -> str:
+    return _LIB_PATH
+
+
+def load_library():
+    """Loads libmoe355.so; raises if it has not been built (there is no other implementation to fall back to)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_LIB_PATH):
+        raise RuntimeError("libmoe355.so is not built: run `python -m cuplayground_amd.build` (needs hipcc)")
+    L = C.CDLL(_LIB_PATH)
+    vp, i32, i64 = C.c_void_p, C.c_int32, C.c_int64
+    cfgp = C.POINTER(_CConfig)
+    L.moe_config_default.argtypes = [cfgp]
+    L.moe_config_from_json_string.argtypes = [C.c_char_p, cfgp, C.c_char_p, C.c_size_t]
+    L.moe_config_from_json_file.argtypes = [C.c_char_p, cfgp, C.c_char_p, C.c_size_t]
+    L.moe_config_validate.argtypes = [cfgp, C.c_char_p, C.c_size_t]
+    L.moe_config_tokens.argtypes = [cfgp]; L.moe_config_tokens.restype = i64
+    L.moe_config_capacity.argtypes = [cfgp, C.POINTER(i64)]
+    L.moe_create.argtypes = [cfgp, C.POINTER(vp)]
+    L.moe_destroy.argtypes = [vp]
+    L.moe_get_arch.argtypes = [vp, C.POINTER(_CArch)]
+    L.moe_workspace_bytes.argtypes = [cfgp, C.POINTER(C.c_size_t)]
+    L.moe_set_ffn_mode.argtypes = [vp, C.c_int]
+    L.moe_forward.argtypes = [vp, vp, C.POINTER(_CWeights), vp, C.POINTER(_CRouting), vp, C.c_size_t, vp]
+    L.moe_gate.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, C.c_size_t, vp]
+    L.moe_route.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, C.c_size_t, vp]
+    L.moe_gemm_bias_act.argtypes = [vp, vp, vp, vp, i64, i64, i64, i32, i32, vp]
+    L.moe_combine.argtypes = [vp, vp, vp, i32, i32, i32, i32, vp, vp]
+    L.moe_set_stage_timing.argtypes = [vp, C.c_int]
+    L.moe_get_stage_ms.argtypes = [vp, C.c_int, C.POINTER(C.c_float)]
+    L.moe_get_task_counts.argtypes = [vp, vp, vp, C.POINTER(i64), C.POINTER(i64)]
+    L.moe_last_hip_error.argtypes = [vp]
+    L.moe_status_string.argtypes = [C.c_int]; L.moe_status_string.restype = C.c_char_p
+    L.moe_version.restype = C.c_int
+    _lib = L
+    return L
+
+
+def _check(rc: int, what: str = ""):
+    if rc != 0:
+        raise MoEError(rc, what)
+
+
+@dataclass
+class MoEConfig:
+    """The operator's knobs; names and meanings are those of aristos_config.json."""
+    capacity_factor: float = 1.0
+    drop_tokens: int = 0
+    expert_top_k: int = 1
+    is_training: int = 0
+    hidden_act: int = ACT_RELU
+    hidden_size: int = 1024
+    intermediate_size: int = 4096
+    micro_batch: int = 4
+    num_experts: int = 1
+    sequence_len: int = 2048
+    torch_dtype: int = DTYPE_F32
+    gate_fn: int = GATE_SOFTMAX
+    norm_topk_prob: int = 0
+
+    def to_c(self) -> _CConfig:
+        return _CConfig(float(self.capacity_factor), *[int(getattr(self, n)) for n, _ in _CConfig._fields_[1:]])
+
+    @classmethod
+    def _from_c(cls, c: _CConfig) -> "MoEConfig":
+        return cls(**{n: getattr(c, n) for n, _ in _CConfig._fields_})
+
+    @classmethod
+    def from_json(cls, text_or_path: str) -> "MoEConfig":
+        """Parses and validates with the library's own loader (the same one a C caller gets)."""
+        L = load_library()
+        c = _CConfig()
+        err = C.create_string_buffer(256)
+        if os.path.exists(text_or_path):
+            rc = L.moe_config_from_json_file(text_or_path.encode(), C.byref(c), err, len(err))
+        else:
+            rc = L.moe_config_from_json_string(text_or_path.encode(), C.byref(c), err, len(err))
+        _check(rc, err.value.decode())
+        return cls._from_c(c)
+
+    def to_json(self) -> str:
+        return json.dumps(asdict(self), indent=2)
+
+    def validate(self) -> None:
+        err = C.create_string_buffer(256)
+        c = self.to_c()
+        _check(load_library().moe_config_validate(C.byref(c), err, len(err)), err.value.decode())
+
+    @property
+    def tokens(self) -> int:
+        return self.micro_batch * self.sequence_len
+
+    @property
+    def capacity(self) -> int:
+        out = C.c_int64(0)
+        c = self.to_c()
+        _check(load_library().moe_config_capacity(C.byref(c), C.byref(out)))
+        return out.value
+
+    def workspace_bytes(self) -> int:
+        out = C.c_size_t(0)
+        c = self.to_c()
+        _check(load_library().moe_workspace_bytes(C.byref(c), C.byref(out)))
+        return out.value
+
+
+def _ptr(t):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _stream():
+    import torch
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _torch_act_dtype(torch_dtype: int):
+    import torch
+    return torch.float32 if torch_dtype == DTYPE_F32 else torch.bfloat16
+
+
+class MoELayer:
+    """One MoE layer shape bound to the current GPU: a `moe_handle` and its workspace."""
+
+    WEIGHT_KEYS = ("gate_w", "gate_bias", "w_up", "w_gate", "w_down", "b_up", "b_gate", "b_down", "s_up", "s_gate",
+                   "s_down")
+
+    def __init__(self, cfg: MoEConfig, ffn_mode: int = FFN_AUTO):
+        import torch
+        self.cfg = cfg
+        self.L = load_library()
+        self._h = C.c_void_p()
+        c = cfg.to_c()
+        _check(self.L.moe_create(C.byref(c), C.byref(self._h)), "moe_create")
+        self.workspace_bytes = cfg.workspace_bytes()
+        self.workspace = torch.empty(self.workspace_bytes, dtype=torch.uint8, device="cuda")
+        self.S, self.k, self.E, self.H = cfg.tokens, cfg.expert_top_k, cfg.num_experts, cfg.hidden_size
+        self.act_dtype = _torch_act_dtype(cfg.torch_dtype)
+        if ffn_mode != FFN_AUTO:
+            self.set_ffn_mode(ffn_mode)
+
+    def close(self):
+        if getattr(self, "_h", None) is not None and self._h:
+            self.L.moe_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @property
+    def arch(self) -> dict:
+        a = _CArch()
+        _check(self.L.moe_get_arch(self._h, C.byref(a)))
+        d = {n: getattr(a, n) for n, _ in _CArch._fields_}
+        d["name"] = a.name.decode()
+        return d
+
+    def set_ffn_mode(self, mode: int):
+        _check(self.L.moe_set_ffn_mode(self._h, mode))
+
+    def set_stage_timing(self, enable: bool):
+        _check(self.L.moe_set_stage_timing(self._h, int(enable)))
+
+    def stage_ms(self) -> dict:
+        out = {}
+        for i, n in enumerate(STAGES):
+            v = C.c_float(0)
+            _check(self.L.moe_get_stage_ms(self._h, i, C.byref(v)))
+            out[n] = v.value
+        return out
+
+    def task_counts(self):
+        a, b = C.c_int64(0), C.c_int64(0)
+        _check(self.L.moe_get_task_counts(self._h, _ptr(self.workspace), _stream(), C.byref(a), C.byref(b)))
+        return a.value, b.value
+
+    def _weights(self, weights: dict) -> _CWeights:
+        w = _CWeights()
+        for n in self.WEIGHT_KEYS:
+            t = weights.get(n)
+            setattr(w, n, None if t is None else t.data_ptr())
+        return w
+
+    def new_routing(self) -> dict:
+        import torch
+        dev = "cuda"
+        S, k, E = self.S, self.k, self.E
+        return dict(topk_idx=torch.empty(S, k, dtype=torch.int32, device=dev),
+                    topk_w=torch.empty(S, k, dtype=torch.float32, device=dev),
+                    slot=torch.empty(S, k, dtype=torch.int32, device=dev),
+                    expert_count=torch.empty(E, dtype=torch.int32, device=dev),
+                    expert_offset=torch.empty(E, dtype=torch.int32, device=dev),
+                    token_indices=torch.empty(S * k, dtype=torch.int32, device=dev))
+
+    def forward(self, x, weights: dict, out=None, routing: dict | None = None):
+        """out[S,H] = MoE(x).  `routing` (from new_routing()) receives the routing result when given."""
+        import torch
+        if out is None:
+            out = torch.empty(self.S, self.H, dtype=self.act_dtype, device=x.device)
+        w = self._weights(weights)
+        r = None
+        if routing is not None:
+            r = _CRouting(*[routing[n].data_ptr() for n, _ in _CRouting._fields_])
+        _check(self.L.moe_forward(self._h, _ptr(x), C.byref(w), _ptr(out), C.byref(r) if r is not None else None,
+                                  _ptr(self.workspace), self.workspace_bytes, _stream()), "moe_forward")
+        return out
+
+    def gate(self, x, gate_w, gate_bias=None, want_logits: bool = False):
+        import torch
+        idx = torch.empty(self.S, self.k, dtype=torch.int32, device=x.device)
+        wts = torch.empty(self.S, self.k, dtype=torch.float32, device=x.device)
+        logits = torch.empty(self.S, self.E, dtype=torch.float32, device=x.device) if want_logits else None
+        _check(self.L.moe_gate(self._h, _ptr(x), _ptr(gate_w), _ptr(gate_bias), _ptr(logits), _ptr(idx), _ptr(wts),
+                               _ptr(self.workspace), self.workspace_bytes, _stream()), "moe_gate")
+        return (idx, wts, logits) if want_logits else (idx, wts)
+
+    def route(self, topk_idx):
+        import torch
+        dev = topk_idx.device
+        S, k, E = self.S, self.k, self.E
+        r = dict(slot=torch.empty(S, k, dtype=torch.int32, device=dev),
+                 expert_count=torch.empty(E, dtype=torch.int32, device=dev),
+                 expert_offset=torch.empty(E, dtype=torch.int32, device=dev),
+                 token_indices=torch.empty(S * k, dtype=torch.int32, device=dev),
+                 pair_row=torch.empty(S, k, dtype=torch.int32, device=dev))
+        _check(self.L.moe_route(self._h, _ptr(topk_idx), _ptr(r["slot"]), _ptr(r["expert_count"]),
+                                _ptr(r["expert_offset"]), _ptr(r["token_indices"]), _ptr(r["pair_row"]),
+                                _ptr(self.workspace), self.workspace_bytes, _stream()), "moe_route")
+        return r
+
+
+def gemm_bias_act(A, B, bias, act: int):
+    """C = act(A.B^T + bias): the reference tile GEMM contract (mma.cuh:46-179) on dense operands."""
+    import torch
+    M, K = A.shape
+    N = B.shape[0]
+    dtype = DTYPE_F32 if A.dtype == torch.float32 else DTYPE_BF16
+    Cm = torch.empty(M, N, dtype=A.dtype, device=A.device)
+    _check(load_library().moe_gemm_bias_act(_ptr(A), _ptr(B), _ptr(bias), _ptr(Cm), M, N, K, dtype, act, _stream()),
+           "moe_gemm_bias_act")
+    return Cm
+
+
+def combine(y_rows, pair_row, topk_w, out=None):
+    """out[t,:] = sum_r w[t,r] * y_rows[pair_row[t,r],:] (combine.cuh:170-186 in gather form)."""
+    import torch
+    S, k = pair_row.shape
+    H = y_rows.shape[1]
+    dtype = DTYPE_F32 if y_rows.dtype == torch.float32 else DTYPE_BF16
+    if out is None:
+        out = torch.empty(S, H, dtype=y_rows.dtype, device=y_rows.device)
+    _check(load_library().moe_combine(_ptr(y_rows), _ptr(pair_row), _ptr(topk_w), S, k, H, dtype, _ptr(out),
+                                      _stream()), "moe_combine")
+    return out

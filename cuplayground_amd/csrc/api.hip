@@ -1,0 +1,484 @@
+// Host side of libmoe355: handle, workspace carving, stage sequencing.  No device memory is allocated here;
+// the caller owns every buffer (the reference carves one stream-ordered arena per driver, mma.cuh:385-391,
+// combine.cuh:214-224 -- the same idea, made the caller's).
+#include <cstdio>
+#include <cstring>
+#include <new>
+
+#include "moe_internal.hpp"
+
+namespace moe355 {
+
+// per-dtype pieces defined next to their kernels
+int bf16_block_m();
+int bf16_block_n();
+int f32_block_m();
+int f32_block_n();
+hipError_t launch_ffn_tiled_bf16(const FfnArgs&, int max_mtiles, int nnt0, int nnt1, hipStream_t);
+hipError_t launch_ffn_persistent_bf16(const FfnArgs&, int blocks, hipStream_t);
+int ffn_persistent_occupancy_bf16();
+hipError_t launch_gemm_dense_bf16(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t, int,
+                                  hipStream_t);
+hipError_t launch_ffn_tiled_f32(const FfnArgs&, int max_mtiles, int nnt0, int nnt1, hipStream_t);
+hipError_t launch_ffn_persistent_f32(const FfnArgs&, int blocks, hipStream_t);
+hipError_t launch_gemm_dense_f32(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t, int,
+                                 hipStream_t);
+hipError_t launch_ffn_fp8(const FfnArgs&, int max_mtiles, int nnt0, int nnt1, int blocks, hipStream_t);
+int fp8_block_m();
+int fp8_block_n0();
+int fp8_block_n1();
+
+namespace {
+
+constexpr size_t kAlign = 256;
+size_t align_up(size_t v) { return (v + kAlign - 1) / kAlign * kAlign; }
+int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
+
+struct Derived {
+    int S, H, I, E, k, A;
+    int act_dtype;     // MOE_DTYPE_F32 or MOE_DTYPE_BF16
+    size_t act_bytes;
+    int64_t capacity;
+    FfnPlan plan;
+    int nblk;          // workgroups of the slot-assignment kernels
+    int max_mtiles;
+};
+
+struct WsLayout {
+    size_t logits, topk_idx, topk_w, slot, pair_row, token_indices, expert_count, expert_offset, rank_local,
+        block_hist, mtiles, seg0, seg1, segq, qstate, done0, h, y, total;
+};
+
+int check_supported(const moe_config& c) {
+    if (c.torch_dtype == MOE_DTYPE_TF32 || c.torch_dtype == MOE_DTYPE_FP16) return MOE_ERR_UNSUPPORTED;
+    if (c.num_experts > kMaxExperts || c.expert_top_k > kMaxTopK) return MOE_ERR_UNSUPPORTED;
+    if (c.torch_dtype == MOE_DTYPE_FP8_E4M3_B128 &&
+        (c.hidden_size % 128 || c.intermediate_size % 128 || c.hidden_act != MOE_ACT_SWIGLU))
+        return MOE_ERR_UNSUPPORTED;
+    const size_t gate_lds = (size_t)4 * c.hidden_size * (c.torch_dtype == MOE_DTYPE_F32 ? 4 : 2);
+    if (gate_lds > 160 * 1024) return MOE_ERR_UNSUPPORTED;
+    return MOE_OK;
+}
+
+int derive(const moe_config& c, Derived* d) {
+    int rc = moe_config_validate(&c, nullptr, 0);
+    if (rc) return rc;
+    rc = check_supported(c);
+    if (rc) return rc;
+    d->S = (int)moe_config_tokens(&c);
+    d->H = c.hidden_size;
+    d->I = c.intermediate_size;
+    d->E = c.num_experts;
+    d->k = c.expert_top_k;
+    d->A = d->S * d->k;
+    d->act_dtype = c.torch_dtype == MOE_DTYPE_F32 ? MOE_DTYPE_F32 : MOE_DTYPE_BF16;
+    d->act_bytes = d->act_dtype == MOE_DTYPE_F32 ? 4 : 2;
+    moe_config_capacity(&c, &d->capacity);
+    if (d->capacity > d->A) d->capacity = d->A;
+    d->plan = ffn_plan(c.torch_dtype, c.hidden_act, d->H, d->I, d->A, d->E);
+    d->nblk = ceil_div(d->A, kRouteBlock);
+    d->max_mtiles = ceil_div(d->A, d->plan.block_m) + d->E;
+    return MOE_OK;
+}
+
+WsLayout layout(const Derived& d) {
+    WsLayout w;
+    size_t off = 0;
+    auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes); return o; };
+    w.logits = take((size_t)d.S * d.E * 4);
+    w.topk_idx = take((size_t)d.A * 4);
+    w.topk_w = take((size_t)d.A * 4);
+    w.slot = take((size_t)d.A * 4);
+    w.pair_row = take((size_t)d.A * 4);
+    w.token_indices = take((size_t)d.A * 4);
+    w.expert_count = take((size_t)d.E * 4);
+    w.expert_offset = take((size_t)(d.E + 1) * 4);
+    w.rank_local = take((size_t)d.A * 4);
+    w.block_hist = take((size_t)d.nblk * d.E * 4);
+    w.mtiles = take((size_t)d.max_mtiles * sizeof(MTile));
+    w.seg0 = take((size_t)d.E * sizeof(Segment));
+    w.seg1 = take((size_t)d.E * sizeof(Segment));
+    w.segq = take((size_t)2 * d.E * sizeof(Segment));
+    w.qstate = take(sizeof(QueueState));
+    w.done0 = take((size_t)d.max_mtiles * 4);
+    w.h = take((size_t)d.A * d.I * d.act_bytes);
+    w.y = take((size_t)d.A * d.H * d.act_bytes);
+    w.total = off;
+    return w;
+}
+
+}  // namespace
+
+FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t, int) {
+    FfnPlan p;
+    const bool sw = act == MOE_ACT_SWIGLU;
+    if (dtype == MOE_DTYPE_F32) {
+        p.block_m = f32_block_m();
+        p.nnt0 = sw ? ceil_div(I, f32_block_n() / 2) : ceil_div(I, f32_block_n());
+        p.nnt1 = ceil_div(H, f32_block_n());
+    } else if (dtype == MOE_DTYPE_FP8_E4M3_B128) {
+        p.block_m = fp8_block_m();
+        p.nnt0 = ceil_div(I, fp8_block_n0());
+        p.nnt1 = ceil_div(H, fp8_block_n1());
+    } else {
+        p.block_m = bf16_block_m();
+        p.nnt0 = sw ? ceil_div(I, bf16_block_n() / 2) : ceil_div(I, bf16_block_n());
+        p.nnt1 = ceil_div(H, bf16_block_n());
+    }
+    return p;
+}
+
+}  // namespace moe355
+
+using namespace moe355;
+
+struct moe_handle {
+    moe_config cfg;
+    Derived d;
+    WsLayout ws;
+    moe_arch arch;
+    int ffn_mode;
+    int timing;
+    hipEvent_t ev[MOE_STAGE_COUNT + 1];
+    bool ev_valid;
+    bool ev_recorded;
+    int last_hip;
+};
+
+namespace {
+
+int hip_fail(moe_handle* h, hipError_t e) {
+    if (h) h->last_hip = (int)e;
+    return MOE_ERR_HIP;
+}
+
+int check_ws(const moe_handle* h, const void* ws, size_t bytes) {
+    if (!ws || ((uintptr_t)ws % kAlign) || bytes < h->ws.total) return MOE_ERR_WORKSPACE;
+    return MOE_OK;
+}
+
+template <typename T>
+T* at(void* ws, size_t off) { return reinterpret_cast<T*>(static_cast<char*>(ws) + off); }
+
+RouteArgs route_args(const moe_handle* h, void* ws) {
+    const Derived& d = h->d;
+    const WsLayout& w = h->ws;
+    RouteArgs a;
+    a.topk_idx = at<int32_t>(ws, w.topk_idx);
+    a.rank_local = at<int32_t>(ws, w.rank_local);
+    a.block_hist = at<int32_t>(ws, w.block_hist);
+    a.slot = at<int32_t>(ws, w.slot);
+    a.pair_row = at<int32_t>(ws, w.pair_row);
+    a.token_indices = at<int32_t>(ws, w.token_indices);
+    a.expert_count = at<int32_t>(ws, w.expert_count);
+    a.expert_offset = at<int32_t>(ws, w.expert_offset);
+    a.mtiles = at<MTile>(ws, w.mtiles);
+    a.seg_phase0 = at<Segment>(ws, w.seg0);
+    a.seg_phase1 = at<Segment>(ws, w.seg1);
+    a.seg_queue = at<Segment>(ws, w.segq);
+    a.q = at<QueueState>(ws, w.qstate);
+    a.done0 = at<int32_t>(ws, w.done0);
+    a.S = d.S; a.k = d.k; a.E = d.E; a.A = d.A; a.nblk = d.nblk;
+    a.drop = h->cfg.drop_tokens;
+    a.capacity = (int)d.capacity;
+    a.block_m = d.plan.block_m;
+    a.nnt0 = d.plan.nnt0;
+    a.nnt1 = d.plan.nnt1;
+    a.max_mtiles = d.max_mtiles;
+    return a;
+}
+
+}  // namespace
+
+extern "C" {
+
+int moe_workspace_bytes(const moe_config* cfg, size_t* bytes) {
+    if (!cfg || !bytes) return MOE_ERR_BAD_ARGUMENT;
+    Derived d;
+    const int rc = derive(*cfg, &d);
+    if (rc) return rc;
+    *bytes = layout(d).total;
+    return MOE_OK;
+}
+
+int moe_create(const moe_config* cfg, moe_handle** out) {
+    if (!cfg || !out) return MOE_ERR_BAD_ARGUMENT;
+    *out = nullptr;
+    Derived d;
+    int rc = derive(*cfg, &d);
+    if (rc) return rc;
+    int ndev = 0;
+    if (hipGetDeviceCount(&ndev) != hipSuccess || ndev < 1) return MOE_ERR_NO_DEVICE;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return MOE_ERR_NO_DEVICE;
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return MOE_ERR_NO_DEVICE;
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) return MOE_ERR_NO_DEVICE;   // the only code object we carry
+    moe_handle* h = new (std::nothrow) moe_handle();
+    if (!h) return MOE_ERR_BAD_ARGUMENT;
+    h->cfg = *cfg;
+    h->d = d;
+    h->ws = layout(d);
+    h->ffn_mode = MOE_FFN_AUTO;
+    h->timing = 0;
+    h->ev_valid = false;
+    h->ev_recorded = false;
+    h->last_hip = 0;
+    memset(&h->arch, 0, sizeof h->arch);
+    h->arch.device = dev;
+    h->arch.compute_units = prop.multiProcessorCount;
+    h->arch.xcds = 8;   // MI355X: 8 accelerator complex dies of 32 CUs
+    h->arch.wavefront_size = prop.warpSize;
+    h->arch.lds_bytes_per_cu = (int)prop.maxSharedMemoryPerMultiProcessor;
+    h->arch.max_clock_khz = prop.clockRate;
+    snprintf(h->arch.name, sizeof h->arch.name, "%s", prop.gcnArchName);
+    h->arch.persistent_blocks = prop.multiProcessorCount * ffn_persistent_blocks(cfg->torch_dtype, cfg->hidden_act, 1);
+    *out = h;
+    return MOE_OK;
+}
+
+int moe_destroy(moe_handle* h) {
+    if (!h) return MOE_OK;
+    if (h->ev_valid)
+        for (auto& e : h->ev) (void)hipEventDestroy(e);
+    delete h;
+    return MOE_OK;
+}
+
+int moe_get_arch(const moe_handle* h, moe_arch* out) {
+    if (!h || !out) return MOE_ERR_BAD_ARGUMENT;
+    *out = h->arch;
+    return MOE_OK;
+}
+
+int moe_set_ffn_mode(moe_handle* h, int mode) {
+    if (!h || mode < MOE_FFN_AUTO || mode > MOE_FFN_PERSISTENT) return MOE_ERR_BAD_ARGUMENT;
+    h->ffn_mode = mode;
+    return MOE_OK;
+}
+
+int moe_set_stage_timing(moe_handle* h, int enable) {
+    if (!h) return MOE_ERR_BAD_ARGUMENT;
+    if (enable && !h->ev_valid) {
+        for (auto& e : h->ev) {
+            hipError_t rc = hipEventCreate(&e);
+            if (rc != hipSuccess) return hip_fail(h, rc);
+        }
+        h->ev_valid = true;
+    }
+    h->timing = enable ? 1 : 0;
+    return MOE_OK;
+}
+
+int moe_get_stage_ms(moe_handle* h, int stage, float* ms) {
+    if (!h || !ms || stage < 0 || stage >= MOE_STAGE_COUNT) return MOE_ERR_BAD_ARGUMENT;
+    if (!h->ev_valid || !h->ev_recorded) return MOE_ERR_BAD_ARGUMENT;
+    hipError_t rc = hipEventSynchronize(h->ev[MOE_STAGE_COUNT]);
+    if (rc != hipSuccess) return hip_fail(h, rc);
+    rc = hipEventElapsedTime(ms, h->ev[stage], h->ev[stage + 1]);
+    if (rc != hipSuccess) return hip_fail(h, rc);
+    return MOE_OK;
+}
+
+int moe_last_hip_error(const moe_handle* h) { return h ? h->last_hip : 0; }
+
+int moe_gate(moe_handle* h, const void* x, const void* gate_w, const float* gate_bias, float* logits,
+             int32_t* topk_idx, float* topk_w, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!h || !x || !gate_w || !topk_idx || !topk_w) return MOE_ERR_BAD_ARGUMENT;
+    int rc = check_ws(h, workspace, workspace_bytes);
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    const Derived& d = h->d;
+    float* lg = logits ? logits : at<float>(workspace, h->ws.logits);
+    hipError_t e = launch_gate_logits(x, gate_w, gate_bias, lg, d.S, d.H, d.E, d.act_dtype, st);
+    if (e != hipSuccess) return hip_fail(h, e);
+    e = launch_topk(lg, d.S, d.E, d.k, h->cfg.gate_fn, h->cfg.norm_topk_prob, topk_idx, topk_w, st);
+    if (e != hipSuccess) return hip_fail(h, e);
+    return MOE_OK;
+}
+
+int moe_route(moe_handle* h, const int32_t* topk_idx, int32_t* slot, int32_t* expert_count, int32_t* expert_offset,
+              int32_t* token_indices, int32_t* pair_row, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!h || !topk_idx || !slot || !expert_count || !expert_offset || !token_indices) return MOE_ERR_BAD_ARGUMENT;
+    int rc = check_ws(h, workspace, workspace_bytes);
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    RouteArgs a = route_args(h, workspace);
+    a.topk_idx = topk_idx;
+    hipError_t e = launch_route(a, st);
+    if (e != hipSuccess) return hip_fail(h, e);
+    const Derived& d = h->d;
+    struct Copy { void* dst; const void* src; size_t n; };
+    const Copy copies[] = {
+        {slot, a.slot, (size_t)d.A * 4},
+        {expert_count, a.expert_count, (size_t)d.E * 4},
+        {expert_offset, a.expert_offset, (size_t)d.E * 4},
+        {token_indices, a.token_indices, (size_t)d.A * 4},
+        {pair_row, a.pair_row, (size_t)d.A * 4},
+    };
+    for (const Copy& c : copies) {
+        if (!c.dst) continue;
+        e = hipMemcpyAsync(c.dst, c.src, c.n, hipMemcpyDeviceToDevice, st);
+        if (e != hipSuccess) return hip_fail(h, e);
+    }
+    return MOE_OK;
+}
+
+int moe_forward(moe_handle* h, const void* x, const moe_weights* w, void* out, const moe_routing_out* routing,
+                void* workspace, size_t workspace_bytes, void* stream) {
+    if (!h || !x || !w || !out) return MOE_ERR_BAD_ARGUMENT;
+    const moe_config& c = h->cfg;
+    const bool sw = c.hidden_act == MOE_ACT_SWIGLU;
+    const bool fp8 = c.torch_dtype == MOE_DTYPE_FP8_E4M3_B128;
+    if (!w->gate_w || !w->w_up || !w->w_down) return MOE_ERR_BAD_ARGUMENT;
+    if (sw != (w->w_gate != nullptr)) return MOE_ERR_BAD_ARGUMENT;
+    if (!sw && w->b_gate) return MOE_ERR_BAD_ARGUMENT;
+    if (fp8 && (!w->s_up || !w->s_down || !w->s_gate)) return MOE_ERR_BAD_ARGUMENT;
+    if (!fp8 && (w->s_up || w->s_down || w->s_gate)) return MOE_ERR_BAD_ARGUMENT;
+    int rc = check_ws(h, workspace, workspace_bytes);
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    const Derived& d = h->d;
+    const WsLayout& L = h->ws;
+    hipError_t e;
+    const bool timing = h->timing && h->ev_valid;
+    auto mark = [&](int i) -> hipError_t { return timing ? hipEventRecord(h->ev[i], st) : hipSuccess; };
+
+    if ((e = mark(0)) != hipSuccess) return hip_fail(h, e);
+    // ---- gate ----
+    float* logits = at<float>(workspace, L.logits);
+    int32_t* topk_idx = at<int32_t>(workspace, L.topk_idx);
+    float* topk_w = at<float>(workspace, L.topk_w);
+    e = launch_gate_logits(x, w->gate_w, w->gate_bias, logits, d.S, d.H, d.E, d.act_dtype, st);
+    if (e != hipSuccess) return hip_fail(h, e);
+    e = launch_topk(logits, d.S, d.E, d.k, c.gate_fn, c.norm_topk_prob, topk_idx, topk_w, st);
+    if (e != hipSuccess) return hip_fail(h, e);
+    if ((e = mark(1)) != hipSuccess) return hip_fail(h, e);
+    // ---- slots, capacity, task tables ----
+    const RouteArgs ra = route_args(h, workspace);
+    e = launch_route(ra, st);
+    if (e != hipSuccess) return hip_fail(h, e);
+    if ((e = mark(2)) != hipSuccess) return hip_fail(h, e);
+    // ---- expert FFN ----
+    FfnArgs fa;
+    fa.x = x;
+    fa.token_indices = ra.token_indices;
+    fa.w_up = w->w_up; fa.w_gate = w->w_gate; fa.w_down = w->w_down;
+    fa.b_up = w->b_up; fa.b_gate = w->b_gate; fa.b_down = w->b_down;
+    fa.s_up = w->s_up; fa.s_gate = w->s_gate; fa.s_down = w->s_down;
+    fa.h = at<char>(workspace, L.h);
+    fa.y = at<char>(workspace, L.y);
+    fa.mtiles = ra.mtiles;
+    fa.seg_phase0 = ra.seg_phase0; fa.seg_phase1 = ra.seg_phase1; fa.seg_queue = ra.seg_queue;
+    fa.q = ra.q;
+    fa.done0 = ra.done0;
+    fa.H = d.H; fa.I = d.I; fa.E = d.E;
+    fa.act = c.hidden_act;
+    fa.spin_limit = 1 << 24;
+    int mode = h->ffn_mode;
+    if (mode == MOE_FFN_AUTO) mode = MOE_FFN_PERSISTENT;
+    if (fp8) {
+        e = launch_ffn_fp8(fa, d.max_mtiles, d.plan.nnt0, d.plan.nnt1,
+                           mode == MOE_FFN_PERSISTENT ? h->arch.persistent_blocks : 0, st);
+    } else if (mode == MOE_FFN_PERSISTENT) {
+        e = launch_ffn_persistent(fa, c.torch_dtype, h->arch.persistent_blocks, st);
+    } else {
+        e = launch_ffn_tiled(fa, c.torch_dtype, d.max_mtiles, st);
+    }
+    if (e != hipSuccess) return hip_fail(h, e);
+    if ((e = mark(3)) != hipSuccess) return hip_fail(h, e);
+    // ---- combine ----
+    e = launch_combine(fa.y, ra.pair_row, topk_w, d.S, d.k, d.H, d.act_dtype, out, st);
+    if (e != hipSuccess) return hip_fail(h, e);
+    if ((e = mark(4)) != hipSuccess) return hip_fail(h, e);
+    if (timing) h->ev_recorded = true;
+
+    if (routing) {
+        struct Copy { void* dst; const void* src; size_t n; };
+        const Copy copies[] = {
+            {routing->topk_idx, topk_idx, (size_t)d.A * 4},
+            {routing->topk_w, topk_w, (size_t)d.A * 4},
+            {routing->slot, ra.slot, (size_t)d.A * 4},
+            {routing->expert_count, ra.expert_count, (size_t)d.E * 4},
+            {routing->expert_offset, ra.expert_offset, (size_t)d.E * 4},
+            {routing->token_indices, ra.token_indices, (size_t)d.A * 4},
+        };
+        for (const Copy& cp : copies) {
+            if (!cp.dst) continue;
+            e = hipMemcpyAsync(cp.dst, cp.src, cp.n, hipMemcpyDeviceToDevice, st);
+            if (e != hipSuccess) return hip_fail(h, e);
+        }
+    }
+    return MOE_OK;
+}
+
+int moe_get_task_counts(moe_handle* h, const void* workspace, void* stream, int64_t* gemm0_tasks,
+                        int64_t* gemm1_tasks) {
+    if (!h || !workspace) return MOE_ERR_BAD_ARGUMENT;
+    QueueState q;
+    hipStream_t st = (hipStream_t)stream;
+    hipError_t e = hipMemcpyAsync(&q, static_cast<const char*>(workspace) + h->ws.qstate, sizeof q,
+                                  hipMemcpyDeviceToHost, st);
+    if (e != hipSuccess) return hip_fail(h, e);
+    e = hipStreamSynchronize(st);
+    if (e != hipSuccess) return hip_fail(h, e);
+    if (gemm0_tasks) *gemm0_tasks = q.tasks_phase0;
+    if (gemm1_tasks) *gemm1_tasks = q.tasks_phase1;
+    return q.stall ? MOE_ERR_QUEUE_STALL : MOE_OK;
+}
+
+int moe_gemm_bias_act(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N, int64_t K,
+                      int32_t dtype, int32_t act, void* stream) {
+    if (!A || !B || !C || M < 1 || N < 1 || K < 1) return MOE_ERR_BAD_ARGUMENT;
+    if (act != MOE_ACT_RELU && act != MOE_ACT_GELU && act != MOE_ACT_NONE) return MOE_ERR_BAD_ARGUMENT;
+    if (M > INT32_MAX / 2 || N > INT32_MAX / 2 || K > INT32_MAX / 2) return MOE_ERR_UNSUPPORTED;
+    hipError_t e;
+    if (dtype == MOE_DTYPE_F32) {
+        if (K % 16 || N % 2) return MOE_ERR_UNSUPPORTED;
+        e = launch_gemm_dense_f32(A, B, bias, C, M, N, K, act, (hipStream_t)stream);
+    } else if (dtype == MOE_DTYPE_BF16) {
+        if (K % 64 || N % 4) return MOE_ERR_UNSUPPORTED;
+        e = launch_gemm_dense_bf16(A, B, bias, C, M, N, K, act, (hipStream_t)stream);
+    } else {
+        return MOE_ERR_UNSUPPORTED;
+    }
+    return e == hipSuccess ? MOE_OK : MOE_ERR_HIP;
+}
+
+int moe_combine(const void* y_rows, const int32_t* pair_row, const float* topk_w, int32_t S, int32_t k, int32_t H,
+                int32_t act_dtype, void* out, void* stream) {
+    if (!y_rows || !pair_row || !topk_w || !out || S < 0 || k < 1 || H < 1) return MOE_ERR_BAD_ARGUMENT;
+    if (act_dtype != MOE_DTYPE_F32 && act_dtype != MOE_DTYPE_BF16) return MOE_ERR_UNSUPPORTED;
+    if (H % (act_dtype == MOE_DTYPE_F32 ? 4 : 8)) return MOE_ERR_UNSUPPORTED;
+    const hipError_t e = launch_combine(y_rows, pair_row, topk_w, S, k, H, act_dtype, out, (hipStream_t)stream);
+    return e == hipSuccess ? MOE_OK : MOE_ERR_HIP;
+}
+
+}  // extern "C"
+
+namespace moe355 {
+
+hipError_t launch_ffn_tiled(const FfnArgs& a, int dtype, int max_mtiles, hipStream_t st) {
+    const FfnPlan p = ffn_plan(dtype, a.act, a.H, a.I, 0, a.E);
+    if (dtype == MOE_DTYPE_F32) return launch_ffn_tiled_f32(a, max_mtiles, p.nnt0, p.nnt1, st);
+    return launch_ffn_tiled_bf16(a, max_mtiles, p.nnt0, p.nnt1, st);
+}
+
+hipError_t launch_ffn_persistent(const FfnArgs& a, int dtype, int blocks, hipStream_t st) {
+    if (dtype == MOE_DTYPE_F32) return launch_ffn_persistent_f32(a, blocks, st);
+    return launch_ffn_persistent_bf16(a, blocks, st);
+}
+
+int ffn_persistent_blocks(int dtype, int, int compute_units) {
+    if (dtype == MOE_DTYPE_F32) return compute_units * 4;
+    if (dtype == MOE_DTYPE_FP8_E4M3_B128) return compute_units * 4;
+    return compute_units * ffn_persistent_occupancy_bf16();
+}
+
+hipError_t launch_gemm_bias_act(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N,
+                                int64_t K, int dtype, int act, hipStream_t st) {
+    if (dtype == MOE_DTYPE_F32) return launch_gemm_dense_f32(A, B, bias, C, M, N, K, act, st);
+    return launch_gemm_dense_bf16(A, B, bias, C, M, N, K, act, st);
+}
+
+}  // namespace moe355

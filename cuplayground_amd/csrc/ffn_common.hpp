@@ -1,0 +1,92 @@
+// Task decoding and the phase-0 -> phase-1 dependency protocol shared by the FFN kernels.
+//
+// The reference distributes tilesM*tilesNx first-GEMM tasks and tilesM*tilesN second-GEMM tasks
+// (scheduling.cuh:212-222): a scheduler thread (scheduling.cuh:170-200) or warp (warpScheduler.cuh:167-265)
+// pops ready processors and rings their doorbells, and the second-GEMM tasks of a row block become
+// schedulable when that block's first-GEMM row is complete (gtQHeads[m] = tilesN, scheduling.cuh:233-236).
+// On gfx950 the doorbells are replaced by one global atomic counter that every persistent workgroup pops
+// (no scheduler workgroup), and gtQHeads by done0[m]: each finished phase-0 tile adds one with release
+// semantics, and a phase-1 task acquires done0[m] == nnt0 before it reads the intermediate rows.  Because task
+// ids are popped in increasing order and every phase-0 task of a row block precedes its phase-1 tasks in
+// the queue, a waiting workgroup only ever waits for tasks that are already running: the wait cannot
+// deadlock whatever the number of resident workgroups.
+#pragma once
+
+#include "moe_internal.hpp"
+
+namespace moe355 {
+
+struct Task {
+    int phase;
+    int expert;
+    int mtile;     // index into the MTile table
+    int ntile;     // column tile of this phase
+    int row0;      // first packed row
+    int rows;      // valid rows in the block
+    int nnt0;      // phase-0 column tiles per row block (the dependency target)
+};
+
+// Finds the segment holding task id `id` (segments are sorted by begin, possibly empty) and decodes it.
+// All arguments are wavefront-uniform, so the loads are scalar.
+__device__ __forceinline__ Task decode_task(const Segment* __restrict__ segs, int nseg, const MTile* __restrict__ mtiles,
+                                            int id, int nnt0) {
+    int lo = 0, hi = nseg - 1;
+    while (lo < hi) {   // last segment with begin <= id
+        const int mid = (lo + hi + 1) >> 1;
+        if (segs[mid].begin <= id) lo = mid; else hi = mid - 1;
+    }
+    const Segment s = segs[lo];
+    const int local = id - s.begin;
+    Task t;
+    t.phase = s.phase;
+    t.expert = s.expert;
+    t.ntile = local / s.nmt;
+    t.mtile = s.mt0 + (local - t.ntile * s.nmt);
+    const MTile m = mtiles[t.mtile];
+    t.row0 = m.row0;
+    t.rows = m.rows;
+    t.nnt0 = nnt0;
+    return t;
+}
+
+// Called by every thread of the workgroup after its phase-0 stores.
+__device__ __forceinline__ void signal_phase0_done(int32_t* done0, int mtile) {
+    __threadfence();   // agent-scope release of this thread's stores (L2 write-back across XCDs included)
+    __syncthreads();
+    if (threadIdx.x == 0) __hip_atomic_fetch_add(done0 + mtile, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Called by every thread of the workgroup before a phase-1 task reads the intermediate rows.
+__device__ __forceinline__ void wait_phase0_done(const int32_t* done0, int mtile, int target, int spin_limit,
+                                                 QueueState* q) {
+    if (threadIdx.x == 0) {
+        int spins = 0;
+        while (__hip_atomic_load(done0 + mtile, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) < target) {
+            __builtin_amdgcn_s_sleep(8);
+            if (++spins > spin_limit) {   // never hang the device: record the stall and carry on
+                __hip_atomic_store(&q->stall, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                break;
+            }
+        }
+    }
+    __syncthreads();
+    __threadfence();   // agent-scope acquire for every thread's subsequent loads
+}
+
+__device__ __forceinline__ uint32_t pack2_bf16(float lo, float hi) {
+    uint32_t a = __float_as_uint(lo), b = __float_as_uint(hi);
+    a += 0x7FFFu + ((a >> 16) & 1u);
+    b += 0x7FFFu + ((b >> 16) & 1u);
+    return (a >> 16) | (b & 0xFFFF0000u);
+}
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t v) { return __uint_as_float((uint32_t)v << 16); }
+
+__device__ __forceinline__ float act_apply(float v, int act) {
+    if (act == MOE_ACT_RELU) return v > 0.0f ? v : 0.0f;
+    if (act == MOE_ACT_GELU) return 0.5f * v * (1.0f + erff(v * 0.70710678118654752440f));
+    return v;
+}
+__device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }
+
+}  // namespace moe355

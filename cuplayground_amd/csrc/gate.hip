@@ -1,0 +1,188 @@
+// Router stage: gate logits, top-k selection and gate weights.
+//
+// The reference has no router (its config macros E_TOP_K / NUM_EXPERTS are defined at
+// CMakeLists.txt:207,213 and never read), so the semantics are this library's:
+//   logits[t,e] = sum_k x[t,k] * gate_w[e,k] (+ gate_bias[e]) with gate_w [E,H] row-major, the (N,K)
+//   operand convention of the reference GEMM (mma.cuh:417-419).
+// The fp32 summation order is fixed so that the integer routing results are reproducible bit for bit:
+// lane l of a wavefront owns partial sum l and takes, in ascending k, every k with (k/8) % 64 == l using
+// one fmaf per element; the 64 partials are folded by an xor butterfly (32,16,8,4,2,1); the bias is added
+// last.  Top-k is taken on the logits (softmax and sigmoid are monotone), ties to the lower expert index.
+#include "moe_internal.hpp"
+
+namespace moe355 {
+namespace {
+
+__device__ __forceinline__ void load8(const float* p, float (&v)[8]) {
+    const float4 a = reinterpret_cast<const float4*>(p)[0];
+    const float4 b = reinterpret_cast<const float4*>(p)[1];
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+    v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+__device__ __forceinline__ void load8(const uint16_t* p, float (&v)[8]) {
+    const uint4 a = reinterpret_cast<const uint4*>(p)[0];
+    v[0] = __uint_as_float(a.x << 16); v[1] = __uint_as_float(a.x & 0xFFFF0000u);
+    v[2] = __uint_as_float(a.y << 16); v[3] = __uint_as_float(a.y & 0xFFFF0000u);
+    v[4] = __uint_as_float(a.z << 16); v[5] = __uint_as_float(a.z & 0xFFFF0000u);
+    v[6] = __uint_as_float(a.w << 16); v[7] = __uint_as_float(a.w & 0xFFFF0000u);
+}
+
+constexpr int kGateTokens = 4;   // one wavefront per token, four tokens per workgroup
+
+// grid = (ceil(S/4), expert chunks); dynamic LDS = 4 * H * sizeof(T)
+template <typename T>
+__global__ __launch_bounds__(256) void gate_logits_kernel(const T* __restrict__ x, const T* __restrict__ gate_w,
+                                                          const float* __restrict__ gate_bias,
+                                                          float* __restrict__ logits, int S, int H, int E,
+                                                          int experts_per_block) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    T* sx = reinterpret_cast<T*>(smem);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int t0 = blockIdx.x * kGateTokens;
+    constexpr int kVec = 16 / (int)sizeof(T);
+    const int vec_per_row = H / kVec;
+    for (int i = threadIdx.x; i < kGateTokens * vec_per_row; i += 256) {
+        const int r = i / vec_per_row, c = i - r * vec_per_row;
+        const int t = t0 + r;
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (t < S) v = reinterpret_cast<const uint4*>(x + (size_t)t * H)[c];
+        reinterpret_cast<uint4*>(sx)[i] = v;
+    }
+    __syncthreads();
+    const int t = t0 + wave;
+    if (t >= S) return;
+    const T* xr = sx + (size_t)wave * H;
+    const int e0 = blockIdx.y * experts_per_block;
+    const int e1 = min(E, e0 + experts_per_block);
+    const int nchunk = H >> 3;
+    for (int e = e0; e < e1; ++e) {
+        const T* wr = gate_w + (size_t)e * H;
+        float acc = 0.0f;
+        for (int c = lane; c < nchunk; c += kWave) {
+            float xv[8], wv[8];
+            load8(xr + c * 8, xv);
+            load8(wr + c * 8, wv);
+#pragma unroll
+            for (int v = 0; v < 8; ++v) acc = __builtin_fmaf(xv[v], wv[v], acc);
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) acc = acc + __shfl_xor(acc, off, kWave);
+        if (lane == 0) logits[(size_t)t * E + e] = gate_bias ? acc + gate_bias[e] : acc;
+    }
+}
+
+struct Cand {
+    float v;
+    int i;
+};
+__device__ __forceinline__ bool better(const Cand& a, const Cand& b) {
+    return a.v > b.v || (a.v == b.v && a.i < b.i);
+}
+
+// One wavefront per token; lane l keeps logits of experts l, l+64, ... (at most 8) in registers.
+__global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ logits, int S, int E, int k, int gate_fn,
+                                                   int norm, int32_t* __restrict__ topk_idx,
+                                                   float* __restrict__ topk_w) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int t = blockIdx.x * 4 + wave;
+    if (t >= S) return;
+    constexpr int J = kMaxExperts / kWave;
+    float v[J];
+    unsigned avail = 0;
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+        const int e = j * kWave + lane;
+        v[j] = 0.0f;
+        if (e < E) {
+            v[j] = logits[(size_t)t * E + e];
+            avail |= 1u << j;
+        }
+    }
+    const unsigned valid = avail;
+    float my_l = 0.0f;
+    int my_i = 0;
+    float top_l = 0.0f;
+    for (int r = 0; r < k; ++r) {
+        Cand c{-INFINITY, 0x7FFFFFFF};
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            if ((avail >> j) & 1u) {
+                Cand d{v[j], j * kWave + lane};
+                if (better(d, c)) c = d;
+            }
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            Cand o{__shfl_xor(c.v, off, kWave), __shfl_xor(c.i, off, kWave)};
+            if (better(o, c)) c = o;
+        }
+        if ((c.i & (kWave - 1)) == lane) avail &= ~(1u << (c.i >> 6));
+        if (lane == r) { my_l = c.v; my_i = c.i; }
+        if (r == 0) top_l = c.v;
+    }
+    float p = 0.0f;
+    if (gate_fn == MOE_GATE_SOFTMAX) {
+        float part = 0.0f;
+#pragma unroll
+        for (int j = 0; j < J; ++j)
+            if ((valid >> j) & 1u) part = part + expf(v[j] - top_l);
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) part = part + __shfl_xor(part, off, kWave);
+        if (lane < k) p = expf(my_l - top_l) / part;
+    } else {
+        if (lane < k) p = 1.0f / (1.0f + expf(-my_l));
+    }
+    if (norm) {
+        float sum = p;
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) sum = sum + __shfl_xor(sum, off, kWave);
+        p = p / sum;
+    }
+    if (lane < k) {
+        topk_idx[(size_t)t * k + lane] = my_i;
+        topk_w[(size_t)t * k + lane] = p;
+    }
+}
+
+}  // namespace
+
+hipError_t launch_gate_logits(const void* x, const void* gate_w, const float* gate_bias, float* logits, int S, int H,
+                              int E, int act_dtype, hipStream_t st) {
+    const int token_blocks = (S + kGateTokens - 1) / kGateTokens;
+    // enough workgroups to occupy the chip even when S is small (decode shapes)
+    int chunks = 1;
+    while (token_blocks * chunks < 1024 && chunks < E) chunks *= 2;
+    const int per = (E + chunks - 1) / chunks;
+    chunks = (E + per - 1) / per;
+    const dim3 grid(token_blocks, chunks);
+    if (act_dtype == MOE_DTYPE_F32) {
+        const size_t lds = (size_t)kGateTokens * H * 4;
+        if (lds > 160 * 1024) return hipErrorInvalidValue;
+        if (lds > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gate_logits_kernel<float>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return e;
+        }
+        gate_logits_kernel<float><<<grid, 256, lds, st>>>((const float*)x, (const float*)gate_w, gate_bias, logits, S,
+                                                          H, E, per);
+    } else {
+        const size_t lds = (size_t)kGateTokens * H * 2;
+        if (lds > 160 * 1024) return hipErrorInvalidValue;
+        if (lds > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gate_logits_kernel<uint16_t>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return e;
+        }
+        gate_logits_kernel<uint16_t><<<grid, 256, lds, st>>>((const uint16_t*)x, (const uint16_t*)gate_w, gate_bias,
+                                                             logits, S, H, E, per);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_topk(const float* logits, int S, int E, int k, int gate_fn, int norm, int32_t* topk_idx,
+                       float* topk_w, hipStream_t st) {
+    topk_kernel<<<(S + 3) / 4, 256, 0, st>>>(logits, S, E, k, gate_fn, norm, topk_idx, topk_w);
+    return hipGetLastError();
+}
+
+}  // namespace moe355

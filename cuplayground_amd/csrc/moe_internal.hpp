@@ -1,0 +1,120 @@
+// Internal declarations shared by the host side of libmoe355 and its gfx950 kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/moe355.h"
+
+namespace moe355 {
+
+constexpr int kWave = 64;          // gfx950 wavefront
+constexpr int kMaxExperts = 512;   // top-k keeps E/64 logits per lane in registers, 8 at most
+constexpr int kMaxTopK = 16;
+constexpr int kRouteBlock = 256;   // pairs per workgroup in the slot-assignment kernels
+
+// One row block of an expert: rows [row0, row0 + rows) of the packed (expert-major) row space.
+struct MTile {
+    int32_t expert;
+    int32_t row0;
+    int32_t rows;
+    int32_t pad;
+};
+
+// A run of consecutive task ids that share (phase, expert).  Task id - begin = ntile * nmt + mtile_local.
+struct Segment {
+    int32_t begin;    // first task id
+    int32_t phase;    // 0 = up(/gate) projection + activation, 1 = down projection
+    int32_t expert;
+    int32_t mt0;      // index of the expert's first MTile
+    int32_t nmt;      // row blocks of the expert
+    int32_t nnt;      // column tiles of this phase
+    int32_t pad0, pad1;
+};
+
+// Words at the start of the queue-state block of the workspace (see QueueState offsets in api.cpp).
+struct QueueState {
+    int32_t head;          // next task id to pop (persistent mode)
+    int32_t total_tasks;   // tasks in the merged queue
+    int32_t tasks_phase0;
+    int32_t tasks_phase1;
+    int32_t num_mtiles;
+    int32_t kept_rows;
+    int32_t stall;         // set when a bounded dependency wait expired
+    int32_t nseg;          // segments in the merged queue
+    int32_t pad[8];
+};
+
+// Everything the FFN kernels need; passed by value.
+struct FfnArgs {
+    const void* x;              // [S,H]
+    const int32_t* token_indices;
+    const void* w_up;           // [E,I,H]
+    const void* w_gate;         // [E,I,H] or null
+    const void* w_down;         // [E,H,I]
+    const void* b_up;
+    const void* b_gate;
+    const void* b_down;
+    const float* s_up;
+    const float* s_gate;
+    const float* s_down;
+    void* h;                    // [A,I] intermediate, activation dtype
+    void* y;                    // [A,H] expert outputs, activation dtype
+    const MTile* mtiles;
+    const Segment* seg_phase0;  // E segments, task ids local to phase 0
+    const Segment* seg_phase1;  // E segments, task ids local to phase 1
+    const Segment* seg_queue;   // 2E segments in queue order
+    QueueState* q;
+    int32_t* done0;             // per MTile: finished phase-0 column tiles
+    int32_t H, I, E;
+    int32_t act;
+    int32_t spin_limit;
+};
+
+struct RouteArgs {
+    const int32_t* topk_idx;    // [A]
+    int32_t* rank_local;        // [A]
+    int32_t* block_hist;        // [nblk, E] counts, then exclusive prefix over blocks
+    int32_t* slot;              // [A]
+    int32_t* pair_row;          // [A]
+    int32_t* token_indices;     // [A]
+    int32_t* expert_count;      // [E]
+    int32_t* expert_offset;     // [E+1]
+    MTile* mtiles;
+    Segment* seg_phase0;
+    Segment* seg_phase1;
+    Segment* seg_queue;
+    QueueState* q;
+    int32_t* done0;
+    int32_t S, k, E, A, nblk;
+    int32_t drop;
+    int32_t capacity;
+    int32_t block_m;            // rows per MTile
+    int32_t nnt0, nnt1;         // column tiles of phase 0 / phase 1
+    int32_t max_mtiles;
+};
+
+// ---- launchers (defined next to their kernels) ----
+hipError_t launch_gate_logits(const void* x, const void* gate_w, const float* gate_bias, float* logits, int S, int H,
+                              int E, int act_dtype, hipStream_t st);
+hipError_t launch_topk(const float* logits, int S, int E, int k, int gate_fn, int norm, int32_t* topk_idx,
+                       float* topk_w, hipStream_t st);
+hipError_t launch_route(const RouteArgs& a, hipStream_t st);
+hipError_t launch_combine(const void* y_rows, const int32_t* pair_row, const float* topk_w, int S, int k, int H,
+                          int act_dtype, void* out, hipStream_t st);
+
+// FFN stage.  block_m / block_n are the tile sizes the routing stage must be told about.
+struct FfnPlan {
+    int block_m;
+    int nnt0;        // column tiles of phase 0
+    int nnt1;        // column tiles of phase 1
+};
+FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E);
+hipError_t launch_ffn_tiled(const FfnArgs& a, int dtype, int max_mtiles, hipStream_t st);
+hipError_t launch_ffn_persistent(const FfnArgs& a, int dtype, int blocks, hipStream_t st);
+int ffn_persistent_blocks(int dtype, int act, int compute_units);
+
+hipError_t launch_gemm_bias_act(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N,
+                                int64_t K, int dtype, int act, hipStream_t st);
+
+}  // namespace moe355

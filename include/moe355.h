@@ -1,0 +1,180 @@
+/*
+ * moe355 -- C ABI of the MI355X (gfx950) fused MoE forward: gate -> slot assignment -> expert FFN -> combine,
+ * all experts resident on one GPU.
+ *
+ * The reference (osayamenja/cuPlayground) has no FFI: its operator surface is the JSON knob file
+ * (aristos_config.json, aristos_config.schema.json:5-71) turned into compile definitions
+ * (CMakeLists.txt:167-216) and the data contracts of its kernels.  Each entry point below names the
+ * reference interface it stands in for.  All pointers are plain host or device addresses; `stream` is a
+ * hipStream_t passed as void* (NULL = the null stream).  Every function returns a moe_status and never
+ * exits the process (the reference prints and calls exit(1), util.cuh:24-36).
+ *
+ * Tensor conventions (row-major everywhere, K contiguous -- the (M,K) x (N,K) -> (M,N) convention of the
+ * reference GEMM, mma.cuh:415-427):
+ *   x        [S, H]        activations      f32 | bf16
+ *   gate_w   [E, H]        router weights   activation dtype
+ *   w_up     [E, I, H]     expert up proj   f32 | bf16 | e4m3 bytes
+ *   w_gate   [E, I, H]     SwiGLU gate proj (hidden_act = 2 only)
+ *   w_down   [E, H, I]     expert down proj
+ *   b_*      [E, I] / [E, H]  optional biases, activation dtype
+ *   s_*      [E, N/128, K/128] fp32 block scales (torch_dtype = 4 only)
+ *   out      [S, H]        activation dtype
+ */
+#ifndef MOE355_H
+#define MOE355_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MOE355_VERSION 1
+
+typedef enum moe_status {
+    MOE_OK = 0,
+    MOE_ERR_BAD_CONFIG = 1,       /* a knob is outside its domain, or JSON is malformed / missing a key     */
+    MOE_ERR_UNSUPPORTED = 2,      /* valid knob values this build has no kernel for (tf32, fp16, E > 512 ...) */
+    MOE_ERR_WORKSPACE = 3,        /* workspace pointer NULL, misaligned or smaller than moe_workspace_bytes    */
+    MOE_ERR_BAD_ARGUMENT = 4,     /* NULL where a tensor is required, or an extra tensor the config excludes   */
+    MOE_ERR_HIP = 5,              /* a HIP call failed; moe_last_hip_error() returns its hipError_t            */
+    MOE_ERR_NO_DEVICE = 6,        /* no gfx950 device is visible                                               */
+    MOE_ERR_QUEUE_STALL = 7       /* the persistent kernel's bounded dependency wait expired                   */
+} moe_status;
+
+/* torch_dtype: the reference enum (aristos_config.schema.json:54-58) plus 4 */
+enum { MOE_DTYPE_F32 = 0, MOE_DTYPE_TF32 = 1, MOE_DTYPE_BF16 = 2, MOE_DTYPE_FP16 = 3, MOE_DTYPE_FP8_E4M3_B128 = 4 };
+/* hidden_act: the reference enum (aristos_config.schema.json:24-28) plus 2 */
+enum { MOE_ACT_RELU = 0, MOE_ACT_GELU = 1, MOE_ACT_SWIGLU = 2, MOE_ACT_NONE = 3 /* moe_gemm_bias_act only */ };
+enum { MOE_GATE_SOFTMAX = 0, MOE_GATE_SIGMOID = 1 };
+
+/*
+ * One field per key of aristos_config.schema.json:5-58, in the schema's order, then this build's extensions.
+ * Relaxations of the schema (a file valid under the reference schema loads unchanged):
+ *   capacity_factor  number > 0 (schema: integer >= 1)        hidden_act   adds 2 = SwiGLU
+ *   torch_dtype      adds 4 = e4m3 weights + 128x128 scales   sequence_len any integer >= 1 (schema: x128)
+ *   micro_batch      any integer >= 1 (schema: x2)            hidden_size / intermediate_size stay x64
+ * Tokens per call: S = micro_batch * sequence_len.
+ */
+typedef struct moe_config {
+    double capacity_factor;
+    int32_t drop_tokens;
+    int32_t expert_top_k;
+    int32_t is_training;        /* parsed and kept; the forward path ignores it, as the reference does */
+    int32_t hidden_act;
+    int32_t hidden_size;
+    int32_t intermediate_size;
+    int32_t micro_batch;
+    int32_t num_experts;
+    int32_t sequence_len;
+    int32_t torch_dtype;
+    /* extensions */
+    int32_t gate_fn;            /* MOE_GATE_*; default softmax */
+    int32_t norm_topk_prob;     /* default: 1 when expert_top_k > 1, else 0 */
+} moe_config;
+
+/* Replaces the CMake JSON reader (CMakeLists.txt:167-203).  `err` (may be NULL) receives a message. */
+int moe_config_default(moe_config* cfg);
+int moe_config_from_json_string(const char* json, moe_config* cfg, char* err, size_t err_len);
+int moe_config_from_json_file(const char* path, moe_config* cfg, char* err, size_t err_len);
+int moe_config_validate(const moe_config* cfg, char* err, size_t err_len);
+int64_t moe_config_tokens(const moe_config* cfg);                  /* S */
+int moe_config_capacity(const moe_config* cfg, int64_t* capacity); /* ceil(capacity_factor * S * k / E) */
+
+/* Replaces Hardware<Arch,maxRegs,Board>::blocks (arch.cuh:16-69): the resident-workgroup budget of the
+ * device the handle was created on, queried at run time. */
+typedef struct moe_arch {
+    int32_t device;
+    int32_t compute_units;
+    int32_t xcds;
+    int32_t wavefront_size;
+    int32_t lds_bytes_per_cu;
+    int32_t max_clock_khz;
+    int32_t persistent_blocks;   /* workgroups the persistent FFN kernel is launched with */
+    char name[64];
+} moe_arch;
+
+typedef struct moe_handle moe_handle;
+
+int moe_create(const moe_config* cfg, moe_handle** out);
+int moe_destroy(moe_handle* h);
+int moe_get_arch(const moe_handle* h, moe_arch* out);
+int moe_workspace_bytes(const moe_config* cfg, size_t* bytes);
+
+typedef struct moe_weights {
+    const void* gate_w;
+    const float* gate_bias;   /* [E] fp32 or NULL */
+    const void* w_up;
+    const void* w_gate;       /* SwiGLU only, else NULL */
+    const void* w_down;
+    const void* b_up;         /* NULL = no bias */
+    const void* b_gate;
+    const void* b_down;
+    const float* s_up;        /* fp8 only */
+    const float* s_gate;
+    const float* s_down;
+} moe_weights;
+
+/* Optional device buffers receiving the routing result (any member may be NULL). */
+typedef struct moe_routing_out {
+    int32_t* topk_idx;        /* [S,k] expert of pair (t,r), ranks in descending score          */
+    float*   topk_w;          /* [S,k] gate weight of the pair                                  */
+    int32_t* slot;            /* [S,k] position inside the expert's row block, -1 = dropped     */
+    int32_t* expert_count;    /* [E]   kept rows per expert                                     */
+    int32_t* expert_offset;   /* [E]   exclusive scan of expert_count                           */
+    int32_t* token_indices;   /* [S*k] token of each packed row, -1 past the last kept row      */
+} moe_routing_out;
+
+/* Variants of the FFN stage; MOE_FFN_AUTO lets the library choose. */
+enum { MOE_FFN_AUTO = 0, MOE_FFN_TILED = 1 /* one launch per GEMM */, MOE_FFN_PERSISTENT = 2 /* task queue */ };
+int moe_set_ffn_mode(moe_handle* h, int mode);
+
+/*
+ * The whole layer, asynchronous on `stream`, no host synchronisation, no allocation.  This is the path the
+ * reference assembles from fGET (mma.cuh:46-179), its schedulers (scheduling.cuh:170-200,
+ * warpScheduler.cuh:167-265) and Combine (combine.cuh:100-188).
+ */
+int moe_forward(moe_handle* h, const void* x, const moe_weights* w, void* out, const moe_routing_out* routing,
+                void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- single stages, same kernels, for parity tests and callers that own the pipeline ---- */
+
+/* Router: logits = x.gate_w^T (+bias), top-k on logits, softmax|sigmoid weights.  logits may be NULL. */
+int moe_gate(moe_handle* h, const void* x, const void* gate_w, const float* gate_bias,
+             float* logits, int32_t* topk_idx, float* topk_w, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Slot assignment + capacity drop from topk_idx; the producer of the tokenIndices[] that the reference's
+ * combine consumes (combine.cuh:115,134).  pair_row may be NULL. */
+int moe_route(moe_handle* h, const int32_t* topk_idx, int32_t* slot, int32_t* expert_count, int32_t* expert_offset,
+              int32_t* token_indices, int32_t* pair_row, void* workspace, size_t workspace_bytes, void* stream);
+
+/* The reference tile GEMM contract, C = act(A.B^T + bias) (mma.cuh:46-179, processor/tiling.cuh:29-38).
+ * dtype is MOE_DTYPE_F32 or MOE_DTYPE_BF16; act is RELU, GELU or NONE; bias [N] may be NULL. */
+int moe_gemm_bias_act(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N, int64_t K,
+                      int32_t dtype, int32_t act, void* stream);
+
+/* out[t,:] = sum_r w[t,r] * y[pair_row[t,r],:]  (fp32, ascending r, one rounding); pair_row < 0 skipped.
+ * With k = 1 and unit weights this is the reference's CombineMode::single row scatter
+ * (combine.cuh:170-186). */
+int moe_combine(const void* y_rows, const int32_t* pair_row, const float* topk_w, int32_t S, int32_t k, int32_t H,
+                int32_t act_dtype, void* out, void* stream);
+
+/* ---- measurement hooks ---- */
+enum { MOE_STAGE_GATE = 0, MOE_STAGE_ROUTE = 1, MOE_STAGE_FFN = 2, MOE_STAGE_COMBINE = 3, MOE_STAGE_COUNT = 4 };
+/* When enabled, moe_forward brackets each stage with hipEvents on the caller's stream. */
+int moe_set_stage_timing(moe_handle* h, int enable);
+/* Milliseconds of stage `stage` in the last moe_forward; synchronises on that call's last event. */
+int moe_get_stage_ms(moe_handle* h, int stage, float* ms);
+/* Tile tasks the FFN stage of the last moe_forward issued to its queue (GEMM0 tasks, GEMM1 tasks); reads
+ * back a few words from the workspace, so it synchronises the stream. */
+int moe_get_task_counts(moe_handle* h, const void* workspace, void* stream, int64_t* gemm0_tasks, int64_t* gemm1_tasks);
+
+int moe_last_hip_error(const moe_handle* h);
+const char* moe_status_string(int status);
+int moe_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOE355_H */

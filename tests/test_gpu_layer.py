@@ -1,0 +1,134 @@
+"""GPU parity of the whole layer (moe_forward through the C ABI) against the CPU oracle."""
+import os
+
+import numpy as np
+import pytest
+
+from oracle import binding as ob
+from helpers import OUT_TOL, from_device, max_rel_err, product_config, upload_inputs
+from test_oracle_layer import CASES, dense_mixture
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+FFN_TILED, FFN_PERSISTENT = 1, 2
+ROUTING_KEYS = ("topk_idx", "slot", "expert_count", "expert_offset", "token_indices")
+
+
+@pytest.fixture(scope="module")
+def moe():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    import cuplayground_amd
+    cuplayground_amd.load_library()
+    return cuplayground_amd
+
+
+def run_layer(moe, cfg, inp, mode):
+    import torch
+    layer = moe.MoELayer(product_config(cfg), ffn_mode=mode)
+    dev = upload_inputs(cfg, inp)
+    routing = layer.new_routing()
+    out = layer.forward(dev["x"], dev, routing=routing)
+    torch.cuda.synchronize()
+    layer.task_counts()            # raises if the persistent queue recorded a stalled dependency wait
+    res = {k: from_device(v) for k, v in routing.items()}
+    res["out"] = from_device(out)
+    layer.close()
+    return res
+
+
+def check_routing(got, want):
+    for key in ROUTING_KEYS:
+        assert np.array_equal(got[key], want[key]), key
+    assert np.abs(got["topk_w"] - want["topk_w"]).max() <= 2e-6
+
+
+@pytest.mark.parametrize("mode", [FFN_TILED, FFN_PERSISTENT], ids=["tiled", "persistent"])
+def test_c1_against_golden_fixture(moe, mode):
+    cfg = ob.BASELINE["C1"]
+    g = np.load(os.path.join(GOLDEN, "c1_layer.npz"))
+    got = run_layer(moe, cfg, ob.make_inputs(cfg, 42), mode)
+    check_routing(got, g)
+    assert max_rel_err(got["out"], g["out"]) <= OUT_TOL[ob.F32]
+    assert (got["out"][(g["slot"] < 0).all(axis=1)] == 0).all()
+
+
+@pytest.mark.parametrize("mode", [FFN_TILED, FFN_PERSISTENT], ids=["tiled", "persistent"])
+@pytest.mark.parametrize("name", sorted(CASES))
+def test_small_layers_vs_oracle(moe, name, mode):
+    cfg = CASES[name]
+    inp = ob.make_inputs(cfg, seed=11, with_bias="bias" in name)
+    want = ob.forward(cfg, inp)
+    got = run_layer(moe, cfg, inp, mode)
+    check_routing(got, want)
+    err = max_rel_err(ob.to_f32(got["out"], cfg.act_dtype), ob.to_f32(want["out"], cfg.act_dtype))
+    assert err <= OUT_TOL[cfg.dtype], err
+    # and against float64 math that shares nothing with the oracle's loops
+    ref = dense_mixture(cfg, inp, want)
+    assert max_rel_err(ob.to_f32(got["out"], cfg.act_dtype), ref) <= max(OUT_TOL[cfg.dtype], 2e-5)
+
+
+RAGGED = {
+    # rows per expert straddle tile boundaries, some experts get nothing, biases on
+    "bf16_gelu_ragged": ob.Cfg(S=700, H=192, I=320, E=5, k=2, act=ob.ACT_GELU, dtype=ob.BF16, drop=1,
+                               capacity_factor=1.1),
+    "bf16_relu_bias": ob.Cfg(S=300, H=128, I=192, E=3, k=1, act=ob.ACT_RELU, dtype=ob.BF16, norm_topk=0, drop=0),
+    "bf16_swiglu_skew": ob.Cfg(S=1500, H=256, I=192, E=64, k=6, act=ob.ACT_SWIGLU, dtype=ob.BF16, drop=1,
+                               capacity_factor=1.0, zipf_bias=True),
+    "bf16_swiglu_bias_dropless": ob.Cfg(S=513, H=320, I=448, E=8, k=2, act=ob.ACT_SWIGLU, dtype=ob.BF16, drop=0),
+    "f32_swiglu_ragged": ob.Cfg(S=333, H=192, I=320, E=7, k=3, act=ob.ACT_SWIGLU, dtype=ob.F32, drop=1,
+                                capacity_factor=0.75),
+    "fp8_decode_small": ob.Cfg(S=64, H=512, I=256, E=32, k=8, act=ob.ACT_SWIGLU, dtype=ob.FP8,
+                               gate_fn=ob.GATE_SIGMOID, drop=0),
+    "fp8_many_rows_bias": ob.Cfg(S=200, H=384, I=384, E=4, k=2, act=ob.ACT_SWIGLU, dtype=ob.FP8,
+                                 gate_fn=ob.GATE_SIGMOID, drop=1, capacity_factor=1.0),
+    "one_token": ob.Cfg(S=1, H=64, I=64, E=2, k=1, act=ob.ACT_GELU, dtype=ob.BF16, norm_topk=0, drop=0),
+}
+
+
+@pytest.mark.parametrize("mode", [FFN_TILED, FFN_PERSISTENT], ids=["tiled", "persistent"])
+@pytest.mark.parametrize("name", sorted(RAGGED))
+def test_ragged_layers_vs_oracle(moe, name, mode):
+    cfg = RAGGED[name]
+    inp = ob.make_inputs(cfg, seed=3, with_bias="bias" in name)
+    want = ob.forward(cfg, inp)
+    got = run_layer(moe, cfg, inp, mode)
+    check_routing(got, want)
+    err = max_rel_err(ob.to_f32(got["out"], cfg.act_dtype), ob.to_f32(want["out"], cfg.act_dtype))
+    assert err <= OUT_TOL[cfg.dtype], err
+    dead = (want["slot"] < 0).all(axis=1)
+    assert (ob.to_f32(got["out"], cfg.act_dtype)[dead] == 0).all()
+
+
+def test_repeat_calls_are_deterministic_and_workspace_is_reusable(moe):
+    import torch
+    cfg = RAGGED["bf16_swiglu_skew"]
+    inp = ob.make_inputs(cfg, seed=3)
+    layer = moe.MoELayer(product_config(cfg))
+    dev = upload_inputs(cfg, inp)
+    a = layer.forward(dev["x"], dev).clone()
+    for mode in (FFN_TILED, FFN_PERSISTENT, FFN_PERSISTENT):
+        layer.set_ffn_mode(mode)
+        b = layer.forward(dev["x"], dev)
+        assert torch.equal(a, b)
+    layer.close()
+
+
+def test_argument_errors(moe):
+    import torch
+    cfg = CASES["bf16_gelu_top2"]
+    layer = moe.MoELayer(product_config(cfg))
+    dev = upload_inputs(cfg, ob.make_inputs(cfg, seed=11))
+    with pytest.raises(moe.MoEError) as e:      # w_gate given for a non-SwiGLU layer
+        layer.forward(dev["x"], {**dev, "w_gate": dev["w_up"]})
+    assert e.value.status == 4
+    with pytest.raises(moe.MoEError) as e:      # scales given for a bf16 layer
+        layer.forward(dev["x"], {**dev, "s_up": dev["gate_w"], "s_down": dev["gate_w"], "s_gate": dev["gate_w"]})
+    assert e.value.status == 4
+    ws = layer.workspace
+    layer.workspace = ws[: ws.numel() // 2]
+    layer.workspace_bytes = layer.workspace.numel()
+    with pytest.raises(moe.MoEError) as e:
+        layer.forward(dev["x"], dev)
+    assert e.value.status == 3
+    layer.close()

@@ -1,0 +1,125 @@
+"""Host-side checks that need no GPU: the C-ABI library loads, exports what the header declares, and its
+config loader implements the reference schema (aristos_config.schema.json) plus the documented relaxations."""
+import ctypes as C
+import json
+import os
+import re
+
+import pytest
+
+import cuplayground_amd as moe
+from cuplayground_amd import api
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+REFERENCE_JSON = {  # the values of the reference's own aristos_config.json:1-13
+    "capacity_factor": 1, "drop_tokens": 0, "expert_top_k": 1, "is_training": 0, "hidden_act": 0, "hidden_size": 1024,
+    "intermediate_size": 4096, "micro_batch": 4, "num_experts": 1, "sequence_len": 2048, "torch_dtype": 0}
+
+
+def test_library_exports_every_declared_symbol():
+    L = moe.load_library()
+    header = open(os.path.join(ROOT, "include", "moe355.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(moe_[a-z0-9_]+)\s*\(", header))
+    assert declared == set(api.EXPORTS)
+    for name in declared:
+        assert hasattr(L, name), name
+    assert L.moe_version() == 1
+    assert L.moe_status_string(0) == b"ok" and L.moe_status_string(3).startswith(b"workspace")
+
+
+def test_reference_config_file_loads_unchanged(tmp_path):
+    p = tmp_path / "aristos_config.json"
+    p.write_text(json.dumps(REFERENCE_JSON, indent=2))
+    cfg = moe.MoEConfig.from_json(str(p))
+    for k, v in REFERENCE_JSON.items():
+        assert getattr(cfg, k) == v
+    assert cfg.gate_fn == 0 and cfg.norm_topk_prob == 0
+    assert cfg.tokens == 4 * 2048
+    assert moe.MoEConfig.from_json(json.dumps(REFERENCE_JSON)) == cfg
+
+
+def test_defaults_are_the_reference_file():
+    c = api._CConfig()
+    assert moe.load_library().moe_config_default(C.byref(c)) == 0
+    assert moe.MoEConfig._from_c(c) == moe.MoEConfig(**REFERENCE_JSON)
+
+
+@pytest.mark.parametrize("key", ["hidden_act", "hidden_size", "intermediate_size", "expert_top_k", "capacity_factor",
+                                 "drop_tokens", "num_experts", "sequence_len", "micro_batch", "torch_dtype"])
+def test_required_keys(key):   # aristos_config.schema.json:60-71
+    d = dict(REFERENCE_JSON); del d[key]
+    with pytest.raises(moe.MoEError) as e:
+        moe.MoEConfig.from_json(json.dumps(d))
+    assert e.value.status == 1 and key in str(e.value)
+
+
+def test_is_training_is_optional_and_extra_keys_are_ignored():
+    d = dict(REFERENCE_JSON); del d["is_training"]
+    d["$schema"] = "x"; d["note"] = {"nested": [1, 2, {"a": "}"}]}
+    assert moe.MoEConfig.from_json(json.dumps(d)).is_training == 0
+
+
+@pytest.mark.parametrize("patch", [
+    {"capacity_factor": 0}, {"capacity_factor": -1.5}, {"drop_tokens": 2}, {"expert_top_k": 0}, {"expert_top_k": 1.5},
+    {"is_training": 3}, {"hidden_act": 3}, {"hidden_act": -1}, {"hidden_size": 1000}, {"hidden_size": 0},
+    {"intermediate_size": 4100}, {"micro_batch": 0}, {"num_experts": 0}, {"sequence_len": 0}, {"torch_dtype": 5},
+    {"gate_fn": 2}, {"norm_topk_prob": 2}, {"expert_top_k": 2, "num_experts": 1}, {"hidden_size": 64.5},
+])
+def test_domain_violations_are_rejected(patch):
+    d = dict(REFERENCE_JSON); d.update(patch)
+    with pytest.raises(moe.MoEError) as e:
+        moe.MoEConfig.from_json(json.dumps(d))
+    assert e.value.status == 1
+
+
+@pytest.mark.parametrize("text", ["", "[]", "{", '{"a" 1}', '{"hidden_size": }', '{"hidden_size": 64,}', "{} x"])
+def test_malformed_json(text):
+    with pytest.raises(moe.MoEError) as e:
+        moe.MoEConfig.from_json(text)
+    assert e.value.status == 1
+
+
+def test_extensions_and_relaxations():
+    d = dict(REFERENCE_JSON)
+    d.update(capacity_factor=1.25, hidden_act=2, torch_dtype=4, sequence_len=64, micro_batch=1, num_experts=256,
+             expert_top_k=8, gate_fn=1, hidden_size=7168, intermediate_size=2048)
+    cfg = moe.MoEConfig.from_json(json.dumps(d))
+    assert cfg.capacity_factor == 1.25 and cfg.tokens == 64 and cfg.norm_topk_prob == 1   # default on for k > 1
+    d["norm_topk_prob"] = 0
+    assert moe.MoEConfig.from_json(json.dumps(d)).norm_topk_prob == 0
+    assert moe.MoEConfig.from_json(moe.MoEConfig(**REFERENCE_JSON).to_json()) == moe.MoEConfig(**REFERENCE_JSON)
+
+
+def test_capacity_matches_oracle(oracle):
+    for name, c in oracle.BASELINE.items():
+        pc = moe.MoEConfig(capacity_factor=c.capacity_factor, expert_top_k=c.k, num_experts=c.E, micro_batch=1,
+                           sequence_len=c.S)
+        assert pc.capacity == c.capacity, name
+
+
+def test_workspace_and_unsupported_shapes():
+    base = dict(capacity_factor=1.0, drop_tokens=1, expert_top_k=2, hidden_act=1, hidden_size=256, intermediate_size=512,
+                micro_batch=1, num_experts=8, sequence_len=128, torch_dtype=2)
+    small = moe.MoEConfig(**base).workspace_bytes()
+    big = moe.MoEConfig(**{**base, "sequence_len": 256}).workspace_bytes()
+    assert 0 < small < big and small % 256 == 0
+    # at least the two intermediates: h [A,I] and y [A,H] in bf16
+    assert small >= 128 * 2 * (512 + 256) * 2
+    for patch in ({"torch_dtype": 1}, {"torch_dtype": 3}, {"num_experts": 1024}, {"expert_top_k": 17, "num_experts": 64}):
+        with pytest.raises(moe.MoEError) as e:
+            moe.MoEConfig(**{**base, **patch}).workspace_bytes()
+        assert e.value.status == 2
+    with pytest.raises(moe.MoEError) as e:
+        moe.MoEConfig(**{**base, "hidden_size": 100}).workspace_bytes()
+    assert e.value.status == 1
+
+
+def test_null_arguments_are_errors_not_crashes():
+    L = moe.load_library()
+    assert L.moe_config_default(None) == 4
+    assert L.moe_workspace_bytes(None, None) == 4
+    assert L.moe_create(None, None) == 4
+    assert L.moe_destroy(None) == 0
+    assert L.moe_forward(None, None, None, None, None, None, 0, None) == 4
+    assert L.moe_gemm_bias_act(None, None, None, None, 1, 1, 1, 0, 0, None) == 4

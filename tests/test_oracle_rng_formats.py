@@ -1,0 +1,104 @@
+"""Pins the oracle's generator and storage-format conversions against published vectors and torch CPU casts."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import binding as ob
+
+# Random123 known-answer vectors for philox4x32-10 (kat_vectors in the Random123 distribution)
+KAT = [
+    ([0, 0, 0, 0], [0, 0], [0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8]),
+    ([0xffffffff] * 4, [0xffffffff] * 2, [0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd]),
+    ([0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344], [0xa4093822, 0x299f31d0],
+     [0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1]),
+]
+
+
+@pytest.mark.parametrize("ctr,key,want", KAT)
+def test_philox_known_answers(ctr, key, want):
+    assert [int(v) for v in ob.philox(ctr, key)] == want
+
+
+def test_normal_is_counter_based_and_standard():
+    a = ob.normal(100_003, 42, 7)
+    b = ob.normal(50_000, 42, 7)
+    assert np.array_equal(a[:50_000], b)            # element i does not depend on n
+    assert not np.array_equal(a[:1000], ob.normal(1000, 42, 8))
+    assert not np.array_equal(a[:1000], ob.normal(1000, 43, 7))
+    z = ob.normal(2_000_000, 1, 1)
+    assert abs(z.mean()) < 3e-3 and abs(z.std() - 1) < 3e-3
+    assert abs((z ** 3).mean()) < 1e-2 and abs((z ** 4).mean() - 3) < 3e-2
+    w = ob.normal(1_000_000, 1, 2, 0.0, 0.02)
+    assert abs(w.std() - 0.02) < 1e-4
+
+
+def test_bf16_every_code_point_round_trips():
+    codes = np.arange(65536, dtype=np.uint16)
+    f = ob.bf16_to_f32(codes)
+    back = ob.f32_to_bf16(f)
+    nan = np.isnan(f)
+    assert np.array_equal(back[~nan], codes[~nan])
+    assert np.isnan(ob.bf16_to_f32(back[nan])).all()
+
+
+def test_bf16_rounding_matches_torch():
+    rng = np.random.default_rng(0)
+    x = np.concatenate([rng.standard_normal(200_000).astype(np.float32) * 10.0 ** rng.integers(-20, 20, 200_000),
+                        np.array([0.0, -0.0, 1.0, 1.00390625, 1.01171875, 3.3895e38, 1e-40], np.float32)])
+    want = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(ob.f32_to_bf16(x), want)
+
+
+def test_e4m3_decode_matches_torch_for_all_codes():
+    codes = np.arange(256, dtype=np.uint8)
+    want = torch.from_numpy(codes).view(torch.float8_e4m3fn).float().numpy()
+    got = np.array([ob.lib().orc_e4m3_to_f32(int(c)) for c in codes], np.float32)
+    nan = np.isnan(want)
+    assert set(codes[nan]) == {0x7F, 0xFF}
+    assert np.array_equal(got[~nan], want[~nan]) and np.isnan(got[nan]).all()
+    assert got[0x7E] == 448.0 and got[0x01] == 2.0 ** -9 and got[0x08] == 2.0 ** -6
+
+
+def test_e4m3_encode_round_trips_and_matches_torch():
+    L = ob.lib()
+    for c in range(256):
+        if c & 0x7F == 0x7F:
+            continue
+        assert L.orc_f32_to_e4m3(L.orc_e4m3_to_f32(c)) == c
+    rng = np.random.default_rng(1)
+    x = (rng.standard_normal(100_000) * 10.0 ** rng.uniform(-4, 2.5, 100_000)).astype(np.float32)
+    x = x[np.abs(x) <= 448.0]
+    want = torch.from_numpy(x).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    got = np.array([L.orc_f32_to_e4m3(float(v)) for v in x], np.uint8)
+    assert np.array_equal(got, want)
+    # ties go to even, values beyond the largest finite saturate
+    assert L.orc_f32_to_e4m3(17.0) == L.orc_f32_to_e4m3(16.0)      # 17 is halfway between 16 and 18
+    assert L.orc_f32_to_e4m3(19.0) == L.orc_f32_to_e4m3(20.0)
+    assert L.orc_f32_to_e4m3(1e6) == 0x7E and L.orc_f32_to_e4m3(-1e6) == 0xFE
+
+
+def test_block128_quantisation():
+    rng = np.random.default_rng(2)
+    w = (rng.standard_normal((2, 256, 384)) * 0.02).astype(np.float32)
+    w[1, 128:, :128] = 0.0
+    q, s = ob.quant_block128(w)
+    assert q.shape == w.shape and s.shape == (2, 2, 3)
+    for e in range(2):
+        for i in range(2):
+            for j in range(3):
+                blk = w[e, i * 128:(i + 1) * 128, j * 128:(j + 1) * 128]
+                amax = np.abs(blk).max()
+                assert s[e, i, j] == (np.float32(amax) / np.float32(448.0) if amax > 0 else 1.0)
+    d = ob.dequant_block128(q, s)
+    scale = np.repeat(np.repeat(s, 128, axis=1), 128, axis=2)
+    # normal range: half an ulp of a 3-bit mantissa = 2^-4 relative; subnormal range: half a step of scale*2^-9
+    assert (np.abs(d - w) <= np.maximum(np.abs(w) * 2.0 ** -4, scale * 2.0 ** -10) * (1 + 1e-6)).all()
+    assert np.array_equal(np.abs(d).reshape(2, 2, 128, 3, 128).max(axis=(2, 4)) > 0, s != 1.0)
+
+
+def test_capacity_formula():
+    assert ob.BASELINE["C1"].capacity == 16
+    assert ob.BASELINE["C2"].capacity == 640
+    assert ob.BASELINE["C3"].capacity == 4096
+    assert ob.BASELINE["C4"].capacity == 1536
+    assert ob.Cfg(S=10, H=64, I=64, E=3, k=1, capacity_factor=1.0).capacity == 4   # ceil(10/3)

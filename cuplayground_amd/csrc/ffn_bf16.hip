@@ -270,10 +270,7 @@ __global__ __launch_bounds__(T::THREADS) void ffn_persistent_kernel(FfnArgs a) {
     const int nseg = a.q->nseg;
     const int nnt0 = a.seg_phase0[0].nnt;
     for (;;) {
-        if (threadIdx.x == 0) s_task = atomicAdd(&a.q->head, 1);
-        __syncthreads();
-        const int id = s_task;
-        __syncthreads();                    // s_task may be overwritten only after everyone has read it
+        const int id = __builtin_amdgcn_readfirstlane(pop_task(&a.q->head, &s_task));
         if (id >= total) break;             // uniform exit: every wavefront leaves here
         const Task t = decode_task(a.seg_queue, nseg, a.mtiles, id, nnt0);
         if (t.phase == 1) wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q);

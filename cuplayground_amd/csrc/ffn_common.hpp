@@ -49,16 +49,31 @@ __device__ __forceinline__ Task decode_task(const Segment* __restrict__ segs, in
     return t;
 }
 
+// The three queue primitives below are deliberately NOT inlined.  Each contains a branch taken by thread 0
+// only; inlined into the persistent loop, the compiler's control-flow structuriser merged the thread-0
+// region at the end of one iteration with the one at the start of the next and let the other lanes run ahead
+// through the next iteration's barriers with a stale task id.  As separate functions every divergent region
+// reconverges before the function returns, and the loop itself only has wavefront-uniform branches.
+
+// Pops the next task id for the whole workgroup (s_task is one int of LDS).
+__device__ __noinline__ int pop_task(int32_t* head, int* s_task) {
+    if (threadIdx.x == 0) *s_task = atomicAdd(head, 1);
+    __syncthreads();
+    const int id = __builtin_amdgcn_readfirstlane(*s_task);
+    __syncthreads();   // s_task may be overwritten only after everyone has read it
+    return id;
+}
+
 // Called by every thread of the workgroup after its phase-0 stores.
-__device__ __forceinline__ void signal_phase0_done(int32_t* done0, int mtile) {
+__device__ __noinline__ void signal_phase0_done(int32_t* done0, int mtile) {
     __threadfence();   // agent-scope release of this thread's stores (L2 write-back across XCDs included)
     __syncthreads();
     if (threadIdx.x == 0) __hip_atomic_fetch_add(done0 + mtile, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Called by every thread of the workgroup before a phase-1 task reads the intermediate rows.
-__device__ __forceinline__ void wait_phase0_done(const int32_t* done0, int mtile, int target, int spin_limit,
-                                                 QueueState* q) {
+__device__ __noinline__ void wait_phase0_done(const int32_t* done0, int mtile, int target, int spin_limit,
+                                              QueueState* q) {
     if (threadIdx.x == 0) {
         int spins = 0;
         while (__hip_atomic_load(done0 + mtile, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) < target) {

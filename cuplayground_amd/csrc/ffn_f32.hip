@@ -158,10 +158,7 @@ __global__ __launch_bounds__(256) void ffn_persistent_f32_kernel(FfnArgs a) {
     const int nseg = a.q->nseg;
     const int nnt0 = a.seg_phase0[0].nnt;
     for (;;) {
-        if (threadIdx.x == 0) s_task = atomicAdd(&a.q->head, 1);
-        __syncthreads();
-        const int id = s_task;
-        __syncthreads();
+        const int id = __builtin_amdgcn_readfirstlane(pop_task(&a.q->head, &s_task));
         if (id >= total) break;
         const Task t = decode_task(a.seg_queue, nseg, a.mtiles, id, nnt0);
         if (t.phase == 1) wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q);

@@ -91,7 +91,7 @@ def load_library():
     L.moe_gemm_bias_act.argtypes = [vp, vp, vp, vp, i64, i64, i64, i32, i32, vp]
     L.moe_combine.argtypes = [vp, vp, vp, i32, i32, i32, i32, vp, vp]
     L.moe_set_stage_timing.argtypes = [vp, C.c_int]
-    L.moe_get_stage_ms.argtypes = [vp, C.c_int, C.POINTER(C.c_float)]
+    L.moe_get_stage_ms.argtypes = [vp, C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_int32)]
     L.moe_get_task_counts.argtypes = [vp, vp, vp, C.POINTER(i64), C.POINTER(i64)]
     L.moe_last_hip_error.argtypes = [vp]
     L.moe_status_string.argtypes = [C.c_int]; L.moe_status_string.restype = C.c_char_p
@@ -228,11 +228,14 @@ class MoELayer:
         _check(self.L.moe_set_stage_timing(self._h, int(enable)))
 
     def stage_ms(self) -> dict:
+        """Mean milliseconds per stage over the forward calls recorded since set_stage_timing(True)."""
         out = {}
+        calls = C.c_int32(0)
         for i, n in enumerate(STAGES):
             v = C.c_float(0)
-            _check(self.L.moe_get_stage_ms(self._h, i, C.byref(v)))
+            _check(self.L.moe_get_stage_ms(self._h, i, C.byref(v), C.byref(calls)))
             out[n] = v.value
+        out["calls"] = calls.value
         return out
 
     def task_counts(self):

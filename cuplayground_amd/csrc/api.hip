@@ -132,6 +132,8 @@ FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t, int) {
 
 using namespace moe355;
 
+constexpr int kTimedCalls = 64;
+
 struct moe_handle {
     moe_config cfg;
     Derived d;
@@ -139,9 +141,10 @@ struct moe_handle {
     moe_arch arch;
     int ffn_mode;
     int timing;
-    hipEvent_t ev[MOE_STAGE_COUNT + 1];
+    // stage timing: a ring of kTimedCalls x (MOE_STAGE_COUNT + 1) events, one row per moe_forward call
+    hipEvent_t ev[kTimedCalls][MOE_STAGE_COUNT + 1];
     bool ev_valid;
-    bool ev_recorded;
+    int64_t ev_calls;      // calls recorded since timing was enabled
     int last_hip;
 };
 
@@ -222,7 +225,7 @@ int moe_create(const moe_config* cfg, moe_handle** out) {
     h->ffn_mode = MOE_FFN_AUTO;
     h->timing = 0;
     h->ev_valid = false;
-    h->ev_recorded = false;
+    h->ev_calls = 0;
     h->last_hip = 0;
     memset(&h->arch, 0, sizeof h->arch);
     h->arch.device = dev;
@@ -240,7 +243,8 @@ int moe_create(const moe_config* cfg, moe_handle** out) {
 int moe_destroy(moe_handle* h) {
     if (!h) return MOE_OK;
     if (h->ev_valid)
-        for (auto& e : h->ev) (void)hipEventDestroy(e);
+        for (auto& row : h->ev)
+            for (auto& e : row) (void)hipEventDestroy(e);
     delete h;
     return MOE_OK;
 }
@@ -260,23 +264,34 @@ int moe_set_ffn_mode(moe_handle* h, int mode) {
 int moe_set_stage_timing(moe_handle* h, int enable) {
     if (!h) return MOE_ERR_BAD_ARGUMENT;
     if (enable && !h->ev_valid) {
-        for (auto& e : h->ev) {
-            hipError_t rc = hipEventCreate(&e);
-            if (rc != hipSuccess) return hip_fail(h, rc);
-        }
+        for (auto& row : h->ev)
+            for (auto& e : row) {
+                hipError_t rc = hipEventCreate(&e);
+                if (rc != hipSuccess) return hip_fail(h, rc);
+            }
         h->ev_valid = true;
     }
     h->timing = enable ? 1 : 0;
+    h->ev_calls = 0;
     return MOE_OK;
 }
 
-int moe_get_stage_ms(moe_handle* h, int stage, float* ms) {
+int moe_get_stage_ms(moe_handle* h, int stage, float* ms, int32_t* calls) {
     if (!h || !ms || stage < 0 || stage >= MOE_STAGE_COUNT) return MOE_ERR_BAD_ARGUMENT;
-    if (!h->ev_valid || !h->ev_recorded) return MOE_ERR_BAD_ARGUMENT;
-    hipError_t rc = hipEventSynchronize(h->ev[MOE_STAGE_COUNT]);
-    if (rc != hipSuccess) return hip_fail(h, rc);
-    rc = hipEventElapsedTime(ms, h->ev[stage], h->ev[stage + 1]);
-    if (rc != hipSuccess) return hip_fail(h, rc);
+    if (!h->ev_valid || h->ev_calls < 1) return MOE_ERR_BAD_ARGUMENT;
+    const int n = (int)(h->ev_calls < kTimedCalls ? h->ev_calls : kTimedCalls);
+    double sum = 0.0;
+    for (int i = 0; i < n; ++i) {
+        const int row = (int)((h->ev_calls - 1 - i) % kTimedCalls);
+        hipError_t rc = hipEventSynchronize(h->ev[row][MOE_STAGE_COUNT]);
+        if (rc != hipSuccess) return hip_fail(h, rc);
+        float t = 0.0f;
+        rc = hipEventElapsedTime(&t, h->ev[row][stage], h->ev[row][stage + 1]);
+        if (rc != hipSuccess) return hip_fail(h, rc);
+        sum += t;
+    }
+    *ms = (float)(sum / n);
+    if (calls) *calls = n;
     return MOE_OK;
 }
 
@@ -342,7 +357,8 @@ int moe_forward(moe_handle* h, const void* x, const moe_weights* w, void* out, c
     const WsLayout& L = h->ws;
     hipError_t e;
     const bool timing = h->timing && h->ev_valid;
-    auto mark = [&](int i) -> hipError_t { return timing ? hipEventRecord(h->ev[i], st) : hipSuccess; };
+    const int ev_row = (int)(h->ev_calls % kTimedCalls);
+    auto mark = [&](int i) -> hipError_t { return timing ? hipEventRecord(h->ev[ev_row][i], st) : hipSuccess; };
 
     if ((e = mark(0)) != hipSuccess) return hip_fail(h, e);
     // ---- gate ----
@@ -391,7 +407,7 @@ int moe_forward(moe_handle* h, const void* x, const moe_weights* w, void* out, c
     e = launch_combine(fa.y, ra.pair_row, topk_w, d.S, d.k, d.H, d.act_dtype, out, st);
     if (e != hipSuccess) return hip_fail(h, e);
     if ((e = mark(4)) != hipSuccess) return hip_fail(h, e);
-    if (timing) h->ev_recorded = true;
+    if (timing) h->ev_calls += 1;
 
     if (routing) {
         struct Copy { void* dst; const void* src; size_t n; };

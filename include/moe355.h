@@ -162,10 +162,12 @@ int moe_combine(const void* y_rows, const int32_t* pair_row, const float* topk_w
 
 /* ---- measurement hooks ---- */
 enum { MOE_STAGE_GATE = 0, MOE_STAGE_ROUTE = 1, MOE_STAGE_FFN = 2, MOE_STAGE_COMBINE = 3, MOE_STAGE_COUNT = 4 };
-/* When enabled, moe_forward brackets each stage with hipEvents on the caller's stream. */
+/* When enabled, moe_forward brackets each stage with hipEvents on the caller's stream (no synchronisation
+ * is added).  Enabling or disabling restarts the count of recorded calls. */
 int moe_set_stage_timing(moe_handle* h, int enable);
-/* Milliseconds of stage `stage` in the last moe_forward; synchronises on that call's last event. */
-int moe_get_stage_ms(moe_handle* h, int stage, float* ms);
+/* Mean milliseconds of stage `stage` over the moe_forward calls recorded since timing was enabled (the most
+ * recent 64 at most); *calls (may be NULL) receives how many were averaged.  Synchronises on their events. */
+int moe_get_stage_ms(moe_handle* h, int stage, float* ms, int32_t* calls);
 /* Tile tasks the FFN stage of the last moe_forward issued to its queue (GEMM0 tasks, GEMM1 tasks); reads
  * back a few words from the workspace, so it synchronises the stream. */
 int moe_get_task_counts(moe_handle* h, const void* workspace, void* stream, int64_t* gemm0_tasks, int64_t* gemm1_tasks);

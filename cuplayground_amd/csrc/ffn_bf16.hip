@@ -19,6 +19,8 @@ namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __attribute__((address_space(3))) void lds_void;
+typedef const __attribute__((address_space(1))) void gbl_void;
 
 constexpr int kBK = 64;               // bf16 elements of K per slab = one 128-byte LDS row
 constexpr int kRowBytes = kBK * 2;
@@ -32,7 +34,8 @@ struct Tile {
     static constexpr int ROWS_PER_PASS = THREADS / 8;
     static constexpr int RA = BM / ROWS_PER_PASS; // 16-byte loads per thread per slab, token tile
     static constexpr int RB = BN / ROWS_PER_PASS; // ... weight tile
-    static constexpr int LDS_BYTES = 2 * (BM + BN) * kRowBytes;
+    static constexpr int STAGE_BYTES = (BM + BN) * kRowBytes;
+    static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
     static_assert(TM >= 1 && TN >= 1 && RA >= 1 && RB >= 1, "tile too small for the wave grid");
     static_assert(TN % 2 == 0, "SwiGLU pairs column tiles inside a wavefront");
 };
@@ -63,7 +66,8 @@ __device__ __forceinline__ void gemm_tile(const TaskPtrs& p, unsigned char* smem
     constexpr int BM = T::BM, BN = T::BN, TM = T::TM, TN = T::TN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / T::WN, wn = wave % T::WN;
-    const int chunk = tid & 7, prow = tid >> 3;
+    const int prow = tid >> 3;
+    const int chunk = (tid & 7) ^ (prow & 7);   // LDS slot (row, c) holds global chunk c ^ (row & 7)
 
     // ---- per-thread source rows ----
     const uint16_t* a_src[T::RA];
@@ -93,9 +97,6 @@ __device__ __forceinline__ void gemm_tile(const TaskPtrs& p, unsigned char* smem
         b_src[i] = base + (int64_t)col * p.K + chunk * 8;
     }
 
-    unsigned char* sA[2] = {smem, smem + (BM + BN) * kRowBytes};
-    unsigned char* sB[2] = {smem + BM * kRowBytes, smem + (BM + BN) * kRowBytes + BM * kRowBytes};
-
     f32x16 acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -104,55 +105,49 @@ __device__ __forceinline__ void gemm_tile(const TaskPtrs& p, unsigned char* smem
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    uint4 ra[T::RA], rb[T::RB];
+    // Slab kt of both tiles goes from global memory straight into LDS stage kt % 2 (no VGPR staging): one
+    // global_load_lds_dwordx4 per 8 rows and wavefront writes 1 KiB of consecutive LDS, lane l landing in
+    // row (l >> 3), chunk slot (l & 7); the xor swizzle is applied on the global side (see a_src / b_src).
+    const int wrow = __builtin_amdgcn_readfirstlane(prow & ~7);
     const int KT = p.K / kBK;
+    auto issue = [&](int kt, int stage) {
+        unsigned char* sa = smem + stage * T::STAGE_BYTES;
+        unsigned char* sb = sa + BM * kRowBytes;
+        const int koff = kt * kBK;
 #pragma unroll
-    for (int i = 0; i < T::RA; ++i) ra[i] = *reinterpret_cast<const uint4*>(a_src[i]);
+        for (int i = 0; i < T::RA; ++i)
+            __builtin_amdgcn_global_load_lds((gbl_void*)(a_src[i] + koff),
+                                             (lds_void*)(sa + (wrow + i * T::ROWS_PER_PASS) * kRowBytes), 16, 0, 0);
 #pragma unroll
-    for (int i = 0; i < T::RB; ++i) rb[i] = *reinterpret_cast<const uint4*>(b_src[i]);
-#pragma unroll
-    for (int i = 0; i < T::RA; ++i)
-        *reinterpret_cast<uint4*>(sA[0] + swz(prow + i * T::ROWS_PER_PASS, chunk)) = ra[i];
-#pragma unroll
-    for (int i = 0; i < T::RB; ++i)
-        *reinterpret_cast<uint4*>(sB[0] + swz(prow + i * T::ROWS_PER_PASS, chunk)) = rb[i];
-    __syncthreads();
-
+        for (int i = 0; i < T::RB; ++i)
+            __builtin_amdgcn_global_load_lds((gbl_void*)(b_src[i] + koff),
+                                             (lds_void*)(sb + (wrow + i * T::ROWS_PER_PASS) * kRowBytes), 16, 0, 0);
+    };
+    __syncthreads();                        // the previous task's last slab may still be being read
+    issue(0, 0);
     const int frow = lane & 31, fk = lane >> 5;
     for (int kt = 0; kt < KT; ++kt) {
         const int cur = kt & 1;
-        const bool more = kt + 1 < KT;
-        if (more) {
-            const int koff = (kt + 1) * kBK;
-#pragma unroll
-            for (int i = 0; i < T::RA; ++i) ra[i] = *reinterpret_cast<const uint4*>(a_src[i] + koff);
-#pragma unroll
-            for (int i = 0; i < T::RB; ++i) rb[i] = *reinterpret_cast<const uint4*>(b_src[i] + koff);
-        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wavefront's share of slab kt has landed
+        __syncthreads();                                    // ... and everyone else's; stage cur^1 is free again
+        if (kt + 1 < KT) issue(kt + 1, cur ^ 1);
+        const unsigned char* sa = smem + cur * T::STAGE_BYTES;
+        const unsigned char* sb = sa + BM * kRowBytes;
 #pragma unroll
         for (int ks = 0; ks < kBK / 16; ++ks) {
             bf16x8 af[TM], bfr[TN];
 #pragma unroll
             for (int i = 0; i < TM; ++i)
-                af[i] = *reinterpret_cast<const bf16x8*>(sA[cur] + swz(wm * 32 * TM + i * 32 + frow, ks * 2 + fk));
+                af[i] = *reinterpret_cast<const bf16x8*>(sa + swz(wm * 32 * TM + i * 32 + frow, ks * 2 + fk));
 #pragma unroll
             for (int j = 0; j < TN; ++j)
-                bfr[j] = *reinterpret_cast<const bf16x8*>(sB[cur] + swz(wn * 32 * TN + j * 32 + frow, ks * 2 + fk));
+                bfr[j] = *reinterpret_cast<const bf16x8*>(sb + swz(wn * 32 * TN + j * 32 + frow, ks * 2 + fk));
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[j], af[i], acc[i][j], 0, 0, 0);
         }
-        if (more) {
-#pragma unroll
-            for (int i = 0; i < T::RA; ++i)
-                *reinterpret_cast<uint4*>(sA[cur ^ 1] + swz(prow + i * T::ROWS_PER_PASS, chunk)) = ra[i];
-#pragma unroll
-            for (int i = 0; i < T::RB; ++i)
-                *reinterpret_cast<uint4*>(sB[cur ^ 1] + swz(prow + i * T::ROWS_PER_PASS, chunk)) = rb[i];
-        }
-        __syncthreads();
     }
 
     // ---- epilogue ----

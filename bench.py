@@ -187,7 +187,7 @@ def main():
         "config": {"workload": "%s: S=%d H=%d I=%d E=%d top%d %s %s" % (
             tag, cfg.S, cfg.H, cfg.I, cfg.E, cfg.k, {0: "relu", 1: "gelu", 2: "swiglu"}[cfg.act],
             "drop cf=%g" % cfg.capacity_factor if cfg.drop else "dropless"),
-            "ffn_mode": args.ffn_mode, "kept_assignments": kept, "tile_tasks": [tasks0, tasks1]},
+            "ffn_mode": args.ffn_mode, "persistent_blocks": layer.arch["persistent_blocks"], "kept_assignments": kept, "tile_tasks": [tasks0, tasks1]},
         "tflops": layer_flops / (ms_per_step * 1e-3) / 1e12,
         "stage_ms": {k: round(v, 4) for k, v in stage.items()},
         "roofline": roofline, "cpu_baseline": cpu,

@@ -2,6 +2,7 @@
 // the caller owns every buffer (the reference carves one stream-ordered arena per driver, mma.cuh:385-391,
 // combine.cuh:214-224 -- the same idea, made the caller's).
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 
@@ -10,13 +11,14 @@
 namespace moe355 {
 
 // per-dtype pieces defined next to their kernels
-int bf16_block_m();
-int bf16_block_n();
+int bf16_block_m(int64_t pairs, int experts);
+int bf16_block_n0(int block_m);
+int bf16_block_n1(int block_m);
 int f32_block_m();
 int f32_block_n();
-hipError_t launch_ffn_tiled_bf16(const FfnArgs&, int max_mtiles, int nnt0, int nnt1, hipStream_t);
-hipError_t launch_ffn_persistent_bf16(const FfnArgs&, int blocks, hipStream_t);
-int ffn_persistent_occupancy_bf16();
+hipError_t launch_ffn_tiled_bf16(const FfnArgs&, int block_m, int max_mtiles, int nnt0, int nnt1, hipStream_t);
+hipError_t launch_ffn_persistent_bf16(const FfnArgs&, int block_m, int blocks, hipStream_t);
+int ffn_persistent_occupancy_bf16(int block_m);
 hipError_t launch_gemm_dense_bf16(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t, int,
                                   hipStream_t);
 hipError_t launch_ffn_tiled_f32(const FfnArgs&, int max_mtiles, int nnt0, int nnt1, hipStream_t);
@@ -109,7 +111,7 @@ WsLayout layout(const Derived& d) {
 
 }  // namespace
 
-FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t, int) {
+FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E) {
     FfnPlan p;
     const bool sw = act == MOE_ACT_SWIGLU;
     if (dtype == MOE_DTYPE_F32) {
@@ -121,9 +123,9 @@ FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t, int) {
         p.nnt0 = ceil_div(I, fp8_block_n0());
         p.nnt1 = ceil_div(H, fp8_block_n1());
     } else {
-        p.block_m = bf16_block_m();
-        p.nnt0 = sw ? ceil_div(I, bf16_block_n() / 2) : ceil_div(I, bf16_block_n());
-        p.nnt1 = ceil_div(H, bf16_block_n());
+        p.block_m = bf16_block_m(A, E);
+        p.nnt0 = sw ? ceil_div(I, bf16_block_n0(p.block_m) / 2) : ceil_div(I, bf16_block_n0(p.block_m));
+        p.nnt1 = ceil_div(H, bf16_block_n1(p.block_m));
     }
     return p;
 }
@@ -235,7 +237,12 @@ int moe_create(const moe_config* cfg, moe_handle** out) {
     h->arch.lds_bytes_per_cu = (int)prop.maxSharedMemoryPerMultiProcessor;
     h->arch.max_clock_khz = prop.clockRate;
     snprintf(h->arch.name, sizeof h->arch.name, "%s", prop.gcnArchName);
-    h->arch.persistent_blocks = prop.multiProcessorCount * ffn_persistent_blocks(cfg->torch_dtype, cfg->hidden_act, 1);
+    int per_cu = ffn_persistent_blocks(cfg->torch_dtype, d.plan.block_m, 1);
+    if (const char* env = getenv("MOE355_BLOCKS_PER_CU")) {   // tuning knob: resident workgroups per CU
+        const int v = atoi(env);
+        if (v >= 1 && v <= 16) per_cu = v;
+    }
+    h->arch.persistent_blocks = prop.multiProcessorCount * per_cu;
     *out = h;
     return MOE_OK;
 }
@@ -397,9 +404,9 @@ int moe_forward(moe_handle* h, const void* x, const moe_weights* w, void* out, c
         e = launch_ffn_fp8(fa, d.max_mtiles, d.plan.nnt0, d.plan.nnt1,
                            mode == MOE_FFN_PERSISTENT ? h->arch.persistent_blocks : 0, st);
     } else if (mode == MOE_FFN_PERSISTENT) {
-        e = launch_ffn_persistent(fa, c.torch_dtype, h->arch.persistent_blocks, st);
+        e = launch_ffn_persistent(fa, c.torch_dtype, d.plan, h->arch.persistent_blocks, st);
     } else {
-        e = launch_ffn_tiled(fa, c.torch_dtype, d.max_mtiles, st);
+        e = launch_ffn_tiled(fa, c.torch_dtype, d.plan, d.max_mtiles, st);
     }
     if (e != hipSuccess) return hip_fail(h, e);
     if ((e = mark(3)) != hipSuccess) return hip_fail(h, e);
@@ -474,21 +481,20 @@ int moe_combine(const void* y_rows, const int32_t* pair_row, const float* topk_w
 
 namespace moe355 {
 
-hipError_t launch_ffn_tiled(const FfnArgs& a, int dtype, int max_mtiles, hipStream_t st) {
-    const FfnPlan p = ffn_plan(dtype, a.act, a.H, a.I, 0, a.E);
+hipError_t launch_ffn_tiled(const FfnArgs& a, int dtype, const FfnPlan& p, int max_mtiles, hipStream_t st) {
     if (dtype == MOE_DTYPE_F32) return launch_ffn_tiled_f32(a, max_mtiles, p.nnt0, p.nnt1, st);
-    return launch_ffn_tiled_bf16(a, max_mtiles, p.nnt0, p.nnt1, st);
+    return launch_ffn_tiled_bf16(a, p.block_m, max_mtiles, p.nnt0, p.nnt1, st);
 }
 
-hipError_t launch_ffn_persistent(const FfnArgs& a, int dtype, int blocks, hipStream_t st) {
+hipError_t launch_ffn_persistent(const FfnArgs& a, int dtype, const FfnPlan& p, int blocks, hipStream_t st) {
     if (dtype == MOE_DTYPE_F32) return launch_ffn_persistent_f32(a, blocks, st);
-    return launch_ffn_persistent_bf16(a, blocks, st);
+    return launch_ffn_persistent_bf16(a, p.block_m, blocks, st);
 }
 
-int ffn_persistent_blocks(int dtype, int, int compute_units) {
+int ffn_persistent_blocks(int dtype, int block_m, int compute_units) {
     if (dtype == MOE_DTYPE_F32) return compute_units * 4;
     if (dtype == MOE_DTYPE_FP8_E4M3_B128) return compute_units * 4;
-    return compute_units * ffn_persistent_occupancy_bf16();
+    return compute_units * ffn_persistent_occupancy_bf16(block_m);
 }
 
 hipError_t launch_gemm_bias_act(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N,

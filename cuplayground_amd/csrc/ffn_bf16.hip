@@ -5,13 +5,18 @@
 // order add-then-activate (processor/tiling.cuh:29-38).  Everything else is designed for CDNA4:
 //   * v_mfma_f32_32x32x16_bf16; the weight tile is the MFMA "A" operand and the token tile the "B" operand,
 //     so each lane ends up with 4 consecutive output columns of one token row and stores 8 bytes at a time;
-//   * tiles are staged through LDS in 128-byte rows (64 bf16 of K) whose 16-byte chunks are xor-swizzled
-//     with the row number, which makes both the ds_write_b128 and the ds_read_b128 patterns conflict free;
-//   * LDS is double buffered and the next K slab is fetched into registers while the current one feeds the
-//     matrix cores: one barrier per slab;
+//   * K slabs of 64 bf16 go from global memory straight into LDS (global_load_lds_dwordx4, no VGPR staging)
+//     as 128-byte rows whose 16-byte chunks are xor-swizzled with (row >> 1) & 7: the LDS has 64 banks, a
+//     ds_read_b128 is served 16 lanes at a time, and with this swizzle 16 consecutive rows of one logical
+//     chunk fall into 16 distinct bank groups (measured: SQ_LDS_BANK_CONFLICT = 0);
+//   * 2 (or 3) LDS stages; the loads of the next slab are issued a quarter at a time between the MFMAs of the
+//     current one so they never queue up behind each other, and MFMA operand fragments are double buffered
+//     in registers across the four 16-wide k sub-steps of a slab;
 //   * dispatch is fused into the A-tile load: phase 0 gathers token rows through token_indices[];
-//   * SwiGLU pairs gate and up columns inside one wavefront (first half of its columns from w_gate, second
+//   * SwiGLU pairs gate and up columns inside one wavefront (first half of its tile rows from w_gate, second
 //     half from w_up), so silu(g)*u happens in registers.
+// Two plans: "large" (256-row blocks, 512 threads: 256x256 tiles for the up projection, 256x128 for the
+// down projection) when experts see many rows, "small" (128x128 tiles, 256 threads) otherwise.
 #include "ffn_common.hpp"
 
 namespace moe355 {
@@ -19,15 +24,16 @@ namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) void lds_void;
 typedef const __attribute__((address_space(1))) void gbl_void;
 
 constexpr int kBK = 64;               // bf16 elements of K per slab = one 128-byte LDS row
 constexpr int kRowBytes = kBK * 2;
 
-template <int BM_, int BN_, int WM_, int WN_>
+template <int BM_, int BN_, int WM_, int WN_, int NS_>
 struct Tile {
-    static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_;
+    static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_, NS = NS_;
     static constexpr int THREADS = WM * WN * kWave;
     static constexpr int TM = BM / WM / 32;       // 32x32 MFMA tiles per wavefront along tokens
     static constexpr int TN = BN / WN / 32;       // ... along weight rows
@@ -35,12 +41,11 @@ struct Tile {
     static constexpr int RA = BM / ROWS_PER_PASS; // 16-byte loads per thread per slab, token tile
     static constexpr int RB = BN / ROWS_PER_PASS; // ... weight tile
     static constexpr int STAGE_BYTES = (BM + BN) * kRowBytes;
-    static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
+    static constexpr int LDS_BYTES = NS * STAGE_BYTES;
     static_assert(TM >= 1 && TN >= 1 && RA >= 1 && RB >= 1, "tile too small for the wave grid");
-    static_assert(TN % 2 == 0, "SwiGLU pairs column tiles inside a wavefront");
+    static_assert(NS == 2 || NS == 3, "two or three LDS stages");
+    static_assert(RA <= 4 && RB <= 4, "a slab's loads are spread over the four k sub-steps");
 };
-
-__device__ __forceinline__ int swz(int row, int chunk) { return row * kRowBytes + ((chunk ^ (row & 7)) << 4); }
 
 // What one task needs, resolved to pointers.
 struct TaskPtrs {
@@ -59,15 +64,26 @@ struct TaskPtrs {
     int n0;                      // first output column of this tile
     int act;                     // epilogue
     bool swiglu;
+    bool publish;                // the rows will be read by other workgroups of the same launch
 };
+
+// 8 bytes of output; rows that another workgroup of the same launch will read are published (ffn_common.hpp).
+__device__ __forceinline__ void store8(uint16_t* p, uint32_t lo, uint32_t hi, bool publish) {
+    if (publish) {
+        publish8(p, lo, hi);
+    } else {
+        u32x2 o = {lo, hi};
+        *reinterpret_cast<u32x2*>(p) = o;
+    }
+}
 
 template <class T>
 __device__ __forceinline__ void gemm_tile(const TaskPtrs& p, unsigned char* smem) {
-    constexpr int BM = T::BM, BN = T::BN, TM = T::TM, TN = T::TN;
+    constexpr int BM = T::BM, BN = T::BN, TM = T::TM, TN = T::TN, NS = T::NS;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / T::WN, wn = wave % T::WN;
     const int prow = tid >> 3;
-    const int chunk = (tid & 7) ^ (prow & 7);   // LDS slot (row, c) holds global chunk c ^ (row & 7)
+    const int chunk = (tid & 7) ^ ((prow >> 1) & 7);   // LDS slot (row, c) holds global chunk c ^ ((row >> 1) & 7)
 
     // ---- per-thread source rows ----
     const uint16_t* a_src[T::RA];
@@ -105,48 +121,84 @@ __device__ __forceinline__ void gemm_tile(const TaskPtrs& p, unsigned char* smem
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    // Slab kt of both tiles goes from global memory straight into LDS stage kt % 2 (no VGPR staging): one
-    // global_load_lds_dwordx4 per 8 rows and wavefront writes 1 KiB of consecutive LDS, lane l landing in
-    // row (l >> 3), chunk slot (l & 7); the xor swizzle is applied on the global side (see a_src / b_src).
+    // One global_load_lds_dwordx4 per 8 rows and wavefront writes 1 KiB of consecutive LDS: lane l lands in
+    // row (l >> 3), chunk slot (l & 7); the swizzle is applied on the global side (see `chunk`).
     const int wrow = __builtin_amdgcn_readfirstlane(prow & ~7);
     const int KT = p.K / kBK;
-    auto issue = [&](int kt, int stage) {
-        unsigned char* sa = smem + stage * T::STAGE_BYTES;
+    auto issue_part = [&](int kt, int part) {   // the loads of slab kt that belong to k sub-step `part`
+        unsigned char* sa = smem + (kt % NS) * T::STAGE_BYTES;
         unsigned char* sb = sa + BM * kRowBytes;
         const int koff = kt * kBK;
 #pragma unroll
         for (int i = 0; i < T::RA; ++i)
-            __builtin_amdgcn_global_load_lds((gbl_void*)(a_src[i] + koff),
-                                             (lds_void*)(sa + (wrow + i * T::ROWS_PER_PASS) * kRowBytes), 16, 0, 0);
+            if (i == part)
+                __builtin_amdgcn_global_load_lds((gbl_void*)(a_src[i] + koff),
+                                                 (lds_void*)(sa + (wrow + i * T::ROWS_PER_PASS) * kRowBytes), 16, 0, 0);
 #pragma unroll
         for (int i = 0; i < T::RB; ++i)
-            __builtin_amdgcn_global_load_lds((gbl_void*)(b_src[i] + koff),
-                                             (lds_void*)(sb + (wrow + i * T::ROWS_PER_PASS) * kRowBytes), 16, 0, 0);
+            if (i == part)
+                __builtin_amdgcn_global_load_lds((gbl_void*)(b_src[i] + koff),
+                                                 (lds_void*)(sb + (wrow + i * T::ROWS_PER_PASS) * kRowBytes), 16, 0, 0);
     };
     __syncthreads();                        // the previous task's last slab may still be being read
-    issue(0, 0);
+#pragma unroll
+    for (int s = 0; s < NS - 1; ++s)
+        if (s < KT) {
+#pragma unroll
+            for (int part = 0; part < 4; ++part) issue_part(s, part);
+        }
+
     const int frow = lane & 31, fk = lane >> 5;
+    const int sw = (frow >> 1) & 7;
+    int a_off[TM], b_off[TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) a_off[i] = (wm * 32 * TM + i * 32 + frow) * kRowBytes;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) b_off[j] = BM * kRowBytes + (wn * 32 * TN + j * 32 + frow) * kRowBytes;
+
+    bf16x8 af[2][TM], bfr[2][TN];
     for (int kt = 0; kt < KT; ++kt) {
-        const int cur = kt & 1;
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wavefront's share of slab kt has landed
-        __syncthreads();                                    // ... and everyone else's; stage cur^1 is free again
-        if (kt + 1 < KT) issue(kt + 1, cur ^ 1);
-        const unsigned char* sa = smem + cur * T::STAGE_BYTES;
-        const unsigned char* sb = sa + BM * kRowBytes;
+        // this wavefront's share of slab kt has landed (with three stages one younger slab may be in flight)
+        if (NS == 2 || kt + 1 >= KT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(T::RA + T::RB) : "memory");
+        __syncthreads();                    // ... and everyone else's; the stage about to be refilled is free
+        const bool pre = kt + NS - 1 < KT;
+        const unsigned char* st = smem + (kt % NS) * T::STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) af[0][i] = *reinterpret_cast<const bf16x8*>(st + a_off[i] + ((fk ^ sw) << 4));
+#pragma unroll
+        for (int j = 0; j < TN; ++j) bfr[0][j] = *reinterpret_cast<const bf16x8*>(st + b_off[j] + ((fk ^ sw) << 4));
 #pragma unroll
         for (int ks = 0; ks < kBK / 16; ++ks) {
-            bf16x8 af[TM], bfr[TN];
+            const int cb = ks & 1, nb = cb ^ 1;
+            if (pre) issue_part(kt + NS - 1, ks);
+            if (ks < 3) {
+                const int c = (((ks + 1) * 2 + fk) ^ sw) << 4;
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
-                af[i] = *reinterpret_cast<const bf16x8*>(sa + swz(wm * 32 * TM + i * 32 + frow, ks * 2 + fk));
+                for (int i = 0; i < TM; ++i) af[nb][i] = *reinterpret_cast<const bf16x8*>(st + a_off[i] + c);
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
-                bfr[j] = *reinterpret_cast<const bf16x8*>(sb + swz(wn * 32 * TN + j * 32 + frow, ks * 2 + fk));
+                for (int j = 0; j < TN; ++j) bfr[nb][j] = *reinterpret_cast<const bf16x8*>(st + b_off[j] + c);
+            }
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[j], af[i], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cb][j], af[cb][i], acc[i][j], 0, 0, 0);
+            // instruction order inside the sub-step: one LDS read behind each of the first MFMAs, then the
+            // global loads one MFMA apart, then the remaining MFMAs
+            if (ks < 3) {
+#pragma unroll
+                for (int n = 0; n < TM + TN; ++n) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                }
+            }
+#pragma unroll
+            for (int n = 0; n < 2; ++n) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
         }
     }
 
@@ -159,24 +211,23 @@ __device__ __forceinline__ void gemm_tile(const TaskPtrs& p, unsigned char* smem
         if (m >= p.rows) continue;
         uint16_t* crow = p.c_base + (int64_t)m * p.N;
         if (p.swiglu) {
+            if constexpr (TN % 2 == 0) {
 #pragma unroll
-            for (int j = 0; j < TN / 2; ++j) {
+                for (int j = 0; j < TN / 2; ++j) {
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int col = p.n0 + wn * 16 * TN + j * 32 + 8 * q + 4 * fk;
-                    if (col >= p.N) continue;
-                    float v[4];
+                    for (int q = 0; q < 4; ++q) {
+                        const int col = p.n0 + wn * 16 * TN + j * 32 + 8 * q + 4 * fk;
+                        if (col >= p.N) continue;
+                        float v[4];
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        float g = acc[i][j][4 * q + r], u = acc[i][j + TN / 2][4 * q + r];
-                        if (p.bias1) g = g + bf16_bits_to_f32(p.bias1[col + r]);
-                        if (p.bias0) u = u + bf16_bits_to_f32(p.bias0[col + r]);
-                        v[r] = silu(g) * u;
+                        for (int r = 0; r < 4; ++r) {
+                            float g = acc[i][j][4 * q + r], u = acc[i][j + TN / 2][4 * q + r];
+                            if (p.bias1) g = g + bf16_bits_to_f32(p.bias1[col + r]);
+                            if (p.bias0) u = u + bf16_bits_to_f32(p.bias0[col + r]);
+                            v[r] = silu(g) * u;
+                        }
+                        store8(crow + col, pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]), p.publish);
                     }
-                    uint2 o;
-                    o.x = pack2_bf16(v[0], v[1]);
-                    o.y = pack2_bf16(v[2], v[3]);
-                    *reinterpret_cast<uint2*>(crow + col) = o;
                 }
             }
         } else {
@@ -193,10 +244,7 @@ __device__ __forceinline__ void gemm_tile(const TaskPtrs& p, unsigned char* smem
                         if (p.bias0) u = u + bf16_bits_to_f32(p.bias0[col + r]);
                         v[r] = act_apply(u, p.act);
                     }
-                    uint2 o;
-                    o.x = pack2_bf16(v[0], v[1]);
-                    o.y = pack2_bf16(v[2], v[3]);
-                    *reinterpret_cast<uint2*>(crow + col) = o;
+                    store8(crow + col, pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]), p.publish);
                 }
             }
         }
@@ -204,7 +252,7 @@ __device__ __forceinline__ void gemm_tile(const TaskPtrs& p, unsigned char* smem
 }
 
 template <class T>
-__device__ __forceinline__ TaskPtrs resolve(const FfnArgs& a, const Task& t) {
+__device__ __forceinline__ TaskPtrs resolve(const FfnArgs& a, const Task& t, bool publish) {
     TaskPtrs p;
     const int64_t HI = (int64_t)a.H * a.I;
     const bool sw = a.act == MOE_ACT_SWIGLU;
@@ -223,6 +271,7 @@ __device__ __forceinline__ TaskPtrs resolve(const FfnArgs& a, const Task& t) {
         p.n0 = t.ntile * (sw ? T::BN / 2 : T::BN);
         p.act = a.act;
         p.swiglu = sw;
+        p.publish = publish;
     } else {
         p.a_base = (const uint16_t*)a.h;
         p.gather = nullptr;
@@ -238,29 +287,45 @@ __device__ __forceinline__ TaskPtrs resolve(const FfnArgs& a, const Task& t) {
         p.n0 = t.ntile * T::BN;
         p.act = MOE_ACT_NONE;
         p.swiglu = false;
+        p.publish = false;
     }
     p.rows = t.rows;
     return p;
 }
 
+// A plan pairs the tile of the up(/gate) projection with the tile of the down projection; both use the
+// same row-block height and the same workgroup size.
+template <class T0_, class T1_>
+struct Plan {
+    using T0 = T0_;
+    using T1 = T1_;
+    static_assert(T0::BM == T1::BM && T0::THREADS == T1::THREADS, "phases share row blocks and workgroup size");
+    static_assert(T0::TN % 2 == 0, "SwiGLU pairs column tiles inside a wavefront");
+    static constexpr int THREADS = T0::THREADS;
+    static constexpr int LDS_BYTES = T0::LDS_BYTES > T1::LDS_BYTES ? T0::LDS_BYTES : T1::LDS_BYTES;
+};
+using LargePlan = Plan<Tile<256, 256, 2, 4, 2>, Tile<256, 128, 2, 4, 3>>;
+using SmallPlan = Plan<Tile<128, 128, 2, 2, 2>, Tile<128, 128, 2, 2, 2>>;
+
 // One launch per phase; workgroup b runs task b of that phase.
-template <class T>
-__global__ __launch_bounds__(T::THREADS) void ffn_tiled_kernel(FfnArgs a, int phase) {
+template <class P>
+__global__ __launch_bounds__(P::THREADS) void ffn_tiled_kernel(FfnArgs a, int phase) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int ntasks = phase ? a.q->tasks_phase1 : a.q->tasks_phase0;
     const int id = blockIdx.x;
     if (id >= ntasks) return;
     const int nnt0 = a.seg_phase0[0].nnt;
     const Task t = decode_task(phase ? a.seg_phase1 : a.seg_phase0, a.E, a.mtiles, id, nnt0);
-    const TaskPtrs p = resolve<T>(a, t);
-    gemm_tile<T>(p, smem);
+    if (phase == 0) gemm_tile<typename P::T0>(resolve<typename P::T0>(a, t, false), smem);
+    else gemm_tile<typename P::T1>(resolve<typename P::T1>(a, t, false), smem);
 }
 
-// Persistent workgroups popping (expert, tile) tasks from one global atomic counter.
-template <class T>
-__global__ __launch_bounds__(T::THREADS) void ffn_persistent_kernel(FfnArgs a) {
+// Persistent workgroups popping (expert, tile) tasks from one global atomic counter (protocol: ffn_common.hpp).
+template <class P>
+__global__ __launch_bounds__(P::THREADS) void ffn_persistent_kernel(FfnArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ int s_task;
+    queue_kernel_entry();
     const int total = a.q->total_tasks;
     const int nseg = a.q->nseg;
     const int nnt0 = a.seg_phase0[0].nnt;
@@ -268,10 +333,13 @@ __global__ __launch_bounds__(T::THREADS) void ffn_persistent_kernel(FfnArgs a) {
         const int id = __builtin_amdgcn_readfirstlane(pop_task(&a.q->head, &s_task));
         if (id >= total) break;             // uniform exit: every wavefront leaves here
         const Task t = decode_task(a.seg_queue, nseg, a.mtiles, id, nnt0);
-        if (t.phase == 1) wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q);
-        const TaskPtrs p = resolve<T>(a, t);
-        gemm_tile<T>(p, smem);
-        if (t.phase == 0) signal_phase0_done(a.done0, t.mtile);
+        if (t.phase == 0) {
+            gemm_tile<typename P::T0>(resolve<typename P::T0>(a, t, true), smem);
+            signal_phase0_done(a.done0, t.mtile);
+        } else {
+            wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q);
+            gemm_tile<typename P::T1>(resolve<typename P::T1>(a, t, false), smem);
+        }
     }
 }
 
@@ -298,10 +366,9 @@ __global__ __launch_bounds__(T::THREADS) void gemm_dense_kernel(const uint16_t* 
     p.n0 = blockIdx.x * T::BN;
     p.act = act;
     p.swiglu = false;
+    p.publish = false;
     gemm_tile<T>(p, smem);
 }
-
-using TileA = Tile<128, 128, 2, 2>;   // 256 threads, 64x64 per wavefront, 64 KiB LDS
 
 template <class K>
 hipError_t allow_lds(K kernel, int bytes) {
@@ -309,47 +376,72 @@ hipError_t allow_lds(K kernel, int bytes) {
                                bytes);
 }
 
-}  // namespace
-
-int bf16_block_m() { return TileA::BM; }
-int bf16_block_n() { return TileA::BN; }
-
-hipError_t launch_ffn_tiled_bf16(const FfnArgs& a, int max_mtiles, int nnt0, int nnt1, hipStream_t st) {
-    using T = TileA;
-    hipError_t e = allow_lds(&ffn_tiled_kernel<T>, T::LDS_BYTES);
+template <class P>
+hipError_t launch_tiled(const FfnArgs& a, int max_mtiles, int nnt0, int nnt1, hipStream_t st) {
+    hipError_t e = allow_lds(&ffn_tiled_kernel<P>, P::LDS_BYTES);
     if (e != hipSuccess) return e;
-    ffn_tiled_kernel<T><<<max_mtiles * nnt0, T::THREADS, T::LDS_BYTES, st>>>(a, 0);
-    ffn_tiled_kernel<T><<<max_mtiles * nnt1, T::THREADS, T::LDS_BYTES, st>>>(a, 1);
+    ffn_tiled_kernel<P><<<max_mtiles * nnt0, P::THREADS, P::LDS_BYTES, st>>>(a, 0);
+    ffn_tiled_kernel<P><<<max_mtiles * nnt1, P::THREADS, P::LDS_BYTES, st>>>(a, 1);
     return hipGetLastError();
 }
 
-hipError_t launch_ffn_persistent_bf16(const FfnArgs& a, int blocks, hipStream_t st) {
-    using T = TileA;
-    hipError_t e = allow_lds(&ffn_persistent_kernel<T>, T::LDS_BYTES);
+template <class P>
+hipError_t launch_persistent(const FfnArgs& a, int blocks, hipStream_t st) {
+    hipError_t e = allow_lds(&ffn_persistent_kernel<P>, P::LDS_BYTES);
     if (e != hipSuccess) return e;
-    ffn_persistent_kernel<T><<<blocks, T::THREADS, T::LDS_BYTES, st>>>(a);
+    ffn_persistent_kernel<P><<<blocks, P::THREADS, P::LDS_BYTES, st>>>(a);
     return hipGetLastError();
 }
 
-int ffn_persistent_occupancy_bf16() {
-    using T = TileA;
+template <class P>
+int occupancy() {
     int n = 0;
-    if (allow_lds(&ffn_persistent_kernel<T>, T::LDS_BYTES) != hipSuccess) return 1;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, reinterpret_cast<const void*>(&ffn_persistent_kernel<T>),
-                                                     T::THREADS, T::LDS_BYTES) != hipSuccess || n < 1)
+    if (allow_lds(&ffn_persistent_kernel<P>, P::LDS_BYTES) != hipSuccess) return 1;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, reinterpret_cast<const void*>(&ffn_persistent_kernel<P>),
+                                                     P::THREADS, P::LDS_BYTES) != hipSuccess || n < 1)
         n = 1;
     return n;
 }
 
+}  // namespace
+
+// Row-block height chosen for a layer: 256 when the average expert sees at least 256 rows.
+int bf16_block_m(int64_t pairs, int experts) { return pairs / (experts > 0 ? experts : 1) >= 256 ? 256 : 128; }
+int bf16_block_n0(int block_m) { return block_m == 256 ? LargePlan::T0::BN : SmallPlan::T0::BN; }
+int bf16_block_n1(int block_m) { return block_m == 256 ? LargePlan::T1::BN : SmallPlan::T1::BN; }
+
+hipError_t launch_ffn_tiled_bf16(const FfnArgs& a, int block_m, int max_mtiles, int nnt0, int nnt1, hipStream_t st) {
+    return block_m == 256 ? launch_tiled<LargePlan>(a, max_mtiles, nnt0, nnt1, st)
+                          : launch_tiled<SmallPlan>(a, max_mtiles, nnt0, nnt1, st);
+}
+
+hipError_t launch_ffn_persistent_bf16(const FfnArgs& a, int block_m, int blocks, hipStream_t st) {
+    return block_m == 256 ? launch_persistent<LargePlan>(a, blocks, st) : launch_persistent<SmallPlan>(a, blocks, st);
+}
+
+int ffn_persistent_occupancy_bf16(int block_m) {
+    return block_m == 256 ? occupancy<LargePlan>() : occupancy<SmallPlan>();
+}
+
 hipError_t launch_gemm_dense_bf16(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N,
                                   int64_t K, int act, hipStream_t st) {
-    using T = TileA;
-    hipError_t e = allow_lds(&gemm_dense_kernel<T>, T::LDS_BYTES);
-    if (e != hipSuccess) return e;
-    const dim3 grid((unsigned)((N + T::BN - 1) / T::BN), (unsigned)((M + T::BM - 1) / T::BM));
-    gemm_dense_kernel<T><<<grid, T::THREADS, T::LDS_BYTES, st>>>((const uint16_t*)A, (const uint16_t*)B,
-                                                                 (const uint16_t*)bias, (uint16_t*)C, (int)M, (int)N,
-                                                                 (int)K, act);
+    if (M >= 1024 && N >= 1024) {
+        using T = LargePlan::T0;
+        hipError_t e = allow_lds(&gemm_dense_kernel<T>, T::LDS_BYTES);
+        if (e != hipSuccess) return e;
+        const dim3 grid((unsigned)((N + T::BN - 1) / T::BN), (unsigned)((M + T::BM - 1) / T::BM));
+        gemm_dense_kernel<T><<<grid, T::THREADS, T::LDS_BYTES, st>>>((const uint16_t*)A, (const uint16_t*)B,
+                                                                     (const uint16_t*)bias, (uint16_t*)C, (int)M,
+                                                                     (int)N, (int)K, act);
+    } else {
+        using T = SmallPlan::T0;
+        hipError_t e = allow_lds(&gemm_dense_kernel<T>, T::LDS_BYTES);
+        if (e != hipSuccess) return e;
+        const dim3 grid((unsigned)((N + T::BN - 1) / T::BN), (unsigned)((M + T::BM - 1) / T::BM));
+        gemm_dense_kernel<T><<<grid, T::THREADS, T::LDS_BYTES, st>>>((const uint16_t*)A, (const uint16_t*)B,
+                                                                     (const uint16_t*)bias, (uint16_t*)C, (int)M,
+                                                                     (int)N, (int)K, act);
+    }
     return hipGetLastError();
 }
 

@@ -64,11 +64,32 @@ __device__ __noinline__ int pop_task(int32_t* head, int* s_task) {
     return id;
 }
 
+// Visibility of the intermediate rows between workgroups that may sit on different XCDs (one L2 each):
+//   producer: every intermediate store is an agent-scope store (publish8 / publish4: written through to
+//             memory); each wavefront waits for its own stores (workgroup-scope release = s_waitcnt vmcnt(0)),
+//             the workgroup meets at a barrier, one lane adds to done0[m] with an agent-scope atomic;
+//   consumer: one lane polls done0[m] with agent-scope atomic loads, the workgroup meets at a barrier, and
+//             only then issues its first load of the block's rows.  Those lines cannot already sit in the
+//             consumer's L1 or L2: within a launch every intermediate row is written once, before it is ever
+//             read, and the agent-scope acquire at kernel entry (queue_kernel_entry) drops what an earlier
+//             launch left behind.
+// No cache-wide write-back or invalidate happens per task: with agent-scope release/acquire fences around
+// every task those two operations cost more than the GEMMs they protected (4.3 ms of a 13 ms layer).
+__device__ __forceinline__ void queue_kernel_entry() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent"); }
+
+__device__ __forceinline__ void publish8(void* p, uint32_t lo, uint32_t hi) {
+    __hip_atomic_store(reinterpret_cast<uint64_t*>(p), ((uint64_t)hi << 32) | lo, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void publish4(void* p, uint32_t v) {
+    __hip_atomic_store(reinterpret_cast<uint32_t*>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // Called by every thread of the workgroup after its phase-0 stores.
 __device__ __noinline__ void signal_phase0_done(int32_t* done0, int mtile) {
-    __threadfence();   // agent-scope release of this thread's stores (L2 write-back across XCDs included)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");   // this wavefront's published stores have completed
     __syncthreads();
-    if (threadIdx.x == 0) __hip_atomic_fetch_add(done0 + mtile, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    if (threadIdx.x == 0) __hip_atomic_fetch_add(done0 + mtile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Called by every thread of the workgroup before a phase-1 task reads the intermediate rows.
@@ -76,7 +97,7 @@ __device__ __noinline__ void wait_phase0_done(const int32_t* done0, int mtile, i
                                               QueueState* q) {
     if (threadIdx.x == 0) {
         int spins = 0;
-        while (__hip_atomic_load(done0 + mtile, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) < target) {
+        while (__hip_atomic_load(done0 + mtile, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
             __builtin_amdgcn_s_sleep(8);
             if (++spins > spin_limit) {   // never hang the device: record the stall and carry on
                 __hip_atomic_store(&q->stall, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -85,7 +106,7 @@ __device__ __noinline__ void wait_phase0_done(const int32_t* done0, int mtile, i
         }
     }
     __syncthreads();
-    __threadfence();   // agent-scope acquire for every thread's subsequent loads
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");   // keeps the block's loads behind the barrier
 }
 
 __device__ __forceinline__ uint32_t pack2_bf16(float lo, float hi) {

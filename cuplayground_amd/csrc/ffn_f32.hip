@@ -22,6 +22,7 @@ struct TaskPtrsF {
     float* c_base;
     int N, K, rows, n0, act;
     bool swiglu;
+    bool publish;   // rows are read by other workgroups of the same launch
 };
 
 __device__ __forceinline__ void gemm_tile_f32(const TaskPtrsF& p, float (*As)[FBM + FPAD], float (*Bs)[FBN + FPAD]) {
@@ -84,7 +85,8 @@ __device__ __forceinline__ void gemm_tile_f32(const TaskPtrsF& p, float (*As)[FB
                 float g = acc[i][q], u = acc[i][q + 2];
                 if (p.bias1) g = g + p.bias1[c];
                 if (p.bias0) u = u + p.bias0[c];
-                crow[c] = silu(g) * u;
+                const float v = silu(g) * u;
+                if (p.publish) publish4(crow + c, __float_as_uint(v)); else crow[c] = v;
             }
         } else {
 #pragma unroll
@@ -93,13 +95,14 @@ __device__ __forceinline__ void gemm_tile_f32(const TaskPtrsF& p, float (*As)[FB
                 if (c >= p.N) continue;
                 float u = acc[i][q];
                 if (p.bias0) u = u + p.bias0[c];
-                crow[c] = act_apply(u, p.act);
+                const float v = act_apply(u, p.act);
+                if (p.publish) publish4(crow + c, __float_as_uint(v)); else crow[c] = v;
             }
         }
     }
 }
 
-__device__ __forceinline__ TaskPtrsF resolve_f32(const FfnArgs& a, const Task& t) {
+__device__ __forceinline__ TaskPtrsF resolve_f32(const FfnArgs& a, const Task& t, bool publish) {
     TaskPtrsF p;
     const int64_t HI = (int64_t)a.H * a.I;
     const bool sw = a.act == MOE_ACT_SWIGLU;
@@ -118,6 +121,7 @@ __device__ __forceinline__ TaskPtrsF resolve_f32(const FfnArgs& a, const Task& t
         p.n0 = t.ntile * (sw ? FBN / 2 : FBN);
         p.act = a.act;
         p.swiglu = sw;
+        p.publish = publish;
     } else {
         p.a_base = (const float*)a.h;
         p.gather = nullptr;
@@ -133,6 +137,7 @@ __device__ __forceinline__ TaskPtrsF resolve_f32(const FfnArgs& a, const Task& t
         p.n0 = t.ntile * FBN;
         p.act = MOE_ACT_NONE;
         p.swiglu = false;
+        p.publish = false;
     }
     p.rows = t.rows;
     return p;
@@ -146,7 +151,7 @@ __global__ __launch_bounds__(256) void ffn_tiled_f32_kernel(FfnArgs a, int phase
     if (id >= ntasks) return;
     const int nnt0 = a.seg_phase0[0].nnt;
     const Task t = decode_task(phase ? a.seg_phase1 : a.seg_phase0, a.E, a.mtiles, id, nnt0);
-    const TaskPtrsF p = resolve_f32(a, t);
+    const TaskPtrsF p = resolve_f32(a, t, false);
     gemm_tile_f32(p, As, Bs);
 }
 
@@ -154,6 +159,7 @@ __global__ __launch_bounds__(256) void ffn_persistent_f32_kernel(FfnArgs a) {
     __shared__ __align__(16) float As[FBK][FBM + FPAD];
     __shared__ __align__(16) float Bs[FBK][FBN + FPAD];
     __shared__ int s_task;
+    queue_kernel_entry();
     const int total = a.q->total_tasks;
     const int nseg = a.q->nseg;
     const int nnt0 = a.seg_phase0[0].nnt;
@@ -162,7 +168,7 @@ __global__ __launch_bounds__(256) void ffn_persistent_f32_kernel(FfnArgs a) {
         if (id >= total) break;
         const Task t = decode_task(a.seg_queue, nseg, a.mtiles, id, nnt0);
         if (t.phase == 1) wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q);
-        const TaskPtrsF p = resolve_f32(a, t);
+        const TaskPtrsF p = resolve_f32(a, t, true);
         gemm_tile_f32(p, As, Bs);
         if (t.phase == 0) signal_phase0_done(a.done0, t.mtile);
     }
@@ -177,7 +183,7 @@ __global__ __launch_bounds__(256) void gemm_dense_f32_kernel(const float* A, con
     p.a_base = A; p.gather = nullptr; p.a_row0 = row0; p.a_ld = K;
     p.b0 = B; p.b1 = nullptr; p.bias0 = bias; p.bias1 = nullptr;
     p.c_base = C + (int64_t)row0 * N;
-    p.N = N; p.K = K; p.rows = min(FBM, M - row0); p.n0 = blockIdx.x * FBN; p.act = act; p.swiglu = false;
+    p.N = N; p.K = K; p.rows = min(FBM, M - row0); p.n0 = blockIdx.x * FBN; p.act = act; p.swiglu = false; p.publish = false;
     gemm_tile_f32(p, As, Bs);
 }
 

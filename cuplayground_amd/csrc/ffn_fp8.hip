@@ -60,6 +60,7 @@ struct Fp8Task {
     int64_t a_row0;
     uint16_t* c_base;           // h or y at the first row of the block
     int K, N, rows, c0, phase;
+    bool publish;   // rows are read by other workgroups of the same launch
 };
 
 __device__ __forceinline__ void fp8_tile(const Fp8Task& t, float* red) {
@@ -154,7 +155,8 @@ __device__ __forceinline__ void fp8_tile(const Fp8Task& t, float* red) {
         uint2 st;
         st.x = pack2_bf16(o[0], o[1]);
         st.y = pack2_bf16(o[2], o[3]);
-        *reinterpret_cast<uint2*>(crow + col) = st;
+        if (t.publish) publish8(crow + col, st.x, st.y);
+        else *reinterpret_cast<uint2*>(crow + col) = st;
     } else {
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
@@ -173,8 +175,9 @@ __device__ __forceinline__ void fp8_tile(const Fp8Task& t, float* red) {
     }
 }
 
-__device__ __forceinline__ Fp8Task resolve_fp8(const FfnArgs& a, const Task& t) {
+__device__ __forceinline__ Fp8Task resolve_fp8(const FfnArgs& a, const Task& t, bool publish) {
     Fp8Task p;
+    p.publish = publish && t.phase == 0;
     const int64_t HI = (int64_t)a.H * a.I;
     const int kbH = a.H >> 7, kbI = a.I >> 7;
     p.phase = t.phase;
@@ -218,13 +221,14 @@ __global__ __launch_bounds__(256) void ffn_tiled_fp8_kernel(FfnArgs a, int phase
     if (id >= ntasks) return;
     const int nnt0 = a.seg_phase0[0].nnt;
     const Task t = decode_task(phase ? a.seg_phase1 : a.seg_phase0, a.E, a.mtiles, id, nnt0);
-    const Fp8Task p = resolve_fp8(a, t);
+    const Fp8Task p = resolve_fp8(a, t, false);
     fp8_tile(p, red);
 }
 
 __global__ __launch_bounds__(256) void ffn_persistent_fp8_kernel(FfnArgs a) {
     __shared__ float red[QWAVES * QGROUPS * 4 * 64];
     __shared__ int s_task;
+    queue_kernel_entry();
     const int total = a.q->total_tasks;
     const int nseg = a.q->nseg;
     const int nnt0 = a.seg_phase0[0].nnt;
@@ -233,7 +237,7 @@ __global__ __launch_bounds__(256) void ffn_persistent_fp8_kernel(FfnArgs a) {
         if (id >= total) break;
         const Task t = decode_task(a.seg_queue, nseg, a.mtiles, id, nnt0);
         if (t.phase == 1) wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q);
-        const Fp8Task p = resolve_fp8(a, t);
+        const Fp8Task p = resolve_fp8(a, t, true);
         fp8_tile(p, red);
         if (t.phase == 0) signal_phase0_done(a.done0, t.mtile);
     }

@@ -110,9 +110,9 @@ struct FfnPlan {
     int nnt1;        // column tiles of phase 1
 };
 FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E);
-hipError_t launch_ffn_tiled(const FfnArgs& a, int dtype, int max_mtiles, hipStream_t st);
-hipError_t launch_ffn_persistent(const FfnArgs& a, int dtype, int blocks, hipStream_t st);
-int ffn_persistent_blocks(int dtype, int act, int compute_units);
+hipError_t launch_ffn_tiled(const FfnArgs& a, int dtype, const FfnPlan& p, int max_mtiles, hipStream_t st);
+hipError_t launch_ffn_persistent(const FfnArgs& a, int dtype, const FfnPlan& p, int blocks, hipStream_t st);
+int ffn_persistent_blocks(int dtype, int block_m, int compute_units);
 
 hipError_t launch_gemm_bias_act(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N,
                                 int64_t K, int dtype, int act, hipStream_t st);

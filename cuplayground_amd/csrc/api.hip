@@ -11,7 +11,7 @@
 namespace moe355 {
 
 // per-dtype pieces defined next to their kernels
-int bf16_block_m(int64_t pairs, int experts);
+int bf16_block_m(int64_t pairs, int experts, int up_columns);
 int bf16_block_n0(int block_m);
 int bf16_block_n1(int block_m);
 int f32_block_m();
@@ -57,8 +57,7 @@ int check_supported(const moe_config& c) {
     if (c.torch_dtype == MOE_DTYPE_FP8_E4M3_B128 &&
         (c.hidden_size % 128 || c.intermediate_size % 128 || c.hidden_act != MOE_ACT_SWIGLU))
         return MOE_ERR_UNSUPPORTED;
-    const size_t gate_lds = (size_t)4 * c.hidden_size * (c.torch_dtype == MOE_DTYPE_F32 ? 4 : 2);
-    if (gate_lds > 160 * 1024) return MOE_ERR_UNSUPPORTED;
+    if (c.hidden_size > 16384) return MOE_ERR_UNSUPPORTED;   // the router keeps a token row in registers
     return MOE_OK;
 }
 
@@ -123,7 +122,7 @@ FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E) {
         p.nnt0 = ceil_div(I, fp8_block_n0());
         p.nnt1 = ceil_div(H, fp8_block_n1());
     } else {
-        p.block_m = bf16_block_m(A, E);
+        p.block_m = bf16_block_m(A, E, sw ? 2 * I : I);
         p.nnt0 = sw ? ceil_div(I, bf16_block_n0(p.block_m) / 2) : ceil_div(I, bf16_block_n0(p.block_m));
         p.nnt1 = ceil_div(H, bf16_block_n1(p.block_m));
     }
@@ -190,6 +189,13 @@ RouteArgs route_args(const moe_handle* h, void* ws) {
     a.nnt0 = d.plan.nnt0;
     a.nnt1 = d.plan.nnt1;
     a.max_mtiles = d.max_mtiles;
+    // phase-0 tasks an average expert contributes; enough experts of them to cover two tasks per workgroup
+    const int64_t avg_mt = d.A / ((int64_t)d.E * d.plan.block_m) > 0 ? d.A / ((int64_t)d.E * d.plan.block_m) : 1;
+    const int64_t per_expert = avg_mt * d.plan.nnt0;
+    int64_t lag = (2 * (int64_t)h->arch.persistent_blocks + per_expert - 1) / per_expert;
+    if (lag < 1) lag = 1;
+    if (lag > d.E) lag = d.E;
+    a.lag = (int)lag;
     return a;
 }
 
@@ -399,7 +405,11 @@ int moe_forward(moe_handle* h, const void* x, const moe_weights* w, void* out, c
     fa.act = c.hidden_act;
     fa.spin_limit = 1 << 24;
     int mode = h->ffn_mode;
-    if (mode == MOE_FFN_AUTO) mode = MOE_FFN_PERSISTENT;
+    if (mode == MOE_FFN_AUTO) {
+        // the queue pays off once there are more tasks than resident workgroups; tiny layers launch per phase
+        const int64_t est_tasks = ((int64_t)d.A / d.plan.block_m + 1) * (d.plan.nnt0 + d.plan.nnt1);
+        mode = est_tasks >= 2 * (int64_t)h->arch.persistent_blocks ? MOE_FFN_PERSISTENT : MOE_FFN_TILED;
+    }
     if (fp8) {
         e = launch_ffn_fp8(fa, d.max_mtiles, d.plan.nnt0, d.plan.nnt1,
                            mode == MOE_FFN_PERSISTENT ? h->arch.persistent_blocks : 0, st);

@@ -405,8 +405,13 @@ int occupancy() {
 
 }  // namespace
 
-// Row-block height chosen for a layer: 256 when the average expert sees at least 256 rows.
-int bf16_block_m(int64_t pairs, int experts) { return pairs / (experts > 0 ? experts : 1) >= 256 ? 256 : 128; }
+// Row-block height chosen for a layer: 256 when the average expert sees at least 256 rows and the up
+// projection still splits into a few tasks per compute unit at that size.
+int bf16_block_m(int64_t pairs, int experts, int up_columns) {
+    if (pairs / (experts > 0 ? experts : 1) < 256) return 128;
+    const int64_t tasks = (pairs / 256) * ((up_columns + LargePlan::T0::BN - 1) / LargePlan::T0::BN);
+    return tasks >= 3 * 256 ? 256 : 128;
+}
 int bf16_block_n0(int block_m) { return block_m == 256 ? LargePlan::T0::BN : SmallPlan::T0::BN; }
 int bf16_block_n1(int block_m) { return block_m == 256 ? LargePlan::T1::BN : SmallPlan::T1::BN; }
 

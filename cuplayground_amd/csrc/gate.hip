@@ -27,48 +27,112 @@ __device__ __forceinline__ void load8(const uint16_t* p, float (&v)[8]) {
     v[6] = __uint_as_float(a.w << 16); v[7] = __uint_as_float(a.w & 0xFFFF0000u);
 }
 
-constexpr int kGateTokens = 4;   // one wavefront per token, four tokens per workgroup
-
-// grid = (ceil(S/4), expert chunks); dynamic LDS = 4 * H * sizeof(T)
-template <typename T>
+// A wavefront keeps TPW token rows in registers (lane l owns the 8-element chunks l, l+64, ... of each row, as
+// fp32) and walks over its share of the experts: one 16-byte load of the expert's row per chunk feeds 8*TPW
+// fmafs.  grid = (token groups of 4*TPW, expert chunks); NCH = chunks per lane = ceil(H / 512).
+template <typename T, int NCH, int TPW>
 __global__ __launch_bounds__(256) void gate_logits_kernel(const T* __restrict__ x, const T* __restrict__ gate_w,
                                                           const float* __restrict__ gate_bias,
                                                           float* __restrict__ logits, int S, int H, int E,
                                                           int experts_per_block) {
-    extern __shared__ __align__(16) unsigned char smem[];
-    T* sx = reinterpret_cast<T*>(smem);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int t0 = blockIdx.x * kGateTokens;
-    constexpr int kVec = 16 / (int)sizeof(T);
-    const int vec_per_row = H / kVec;
-    for (int i = threadIdx.x; i < kGateTokens * vec_per_row; i += 256) {
-        const int r = i / vec_per_row, c = i - r * vec_per_row;
-        const int t = t0 + r;
-        uint4 v = make_uint4(0, 0, 0, 0);
-        if (t < S) v = reinterpret_cast<const uint4*>(x + (size_t)t * H)[c];
-        reinterpret_cast<uint4*>(sx)[i] = v;
+    const int t0 = (blockIdx.x * 4 + wave) * TPW;
+    if (t0 >= S) return;
+    const int nchunk = H >> 3;
+    float xr[TPW][NCH][8];
+#pragma unroll
+    for (int q = 0; q < TPW; ++q) {
+        const int t = min(t0 + q, S - 1);          // a ragged last group recomputes the last token; not stored
+#pragma unroll
+        for (int j = 0; j < NCH; ++j) {
+            const int c = lane + j * kWave;
+            if (c < nchunk) load8(x + (size_t)t * H + c * 8, xr[q][j]);
+            else {
+#pragma unroll
+                for (int v = 0; v < 8; ++v) xr[q][j][v] = 0.0f;
+            }
+        }
     }
-    __syncthreads();
-    const int t = t0 + wave;
-    if (t >= S) return;
-    const T* xr = sx + (size_t)wave * H;
     const int e0 = blockIdx.y * experts_per_block;
     const int e1 = min(E, e0 + experts_per_block);
-    const int nchunk = H >> 3;
-    for (int e = e0; e < e1; ++e) {
+    // raw 16-byte chunks of the next expert's row are fetched while the current expert is being summed
+    typedef unsigned int raw_t __attribute__((ext_vector_type(sizeof(T) == 4 ? 8 : 4)));
+    raw_t wn[NCH];
+    auto fetch = [&](int e) {
         const T* wr = gate_w + (size_t)e * H;
-        float acc = 0.0f;
-        for (int c = lane; c < nchunk; c += kWave) {
-            float xv[8], wv[8];
-            load8(xr + c * 8, xv);
-            load8(wr + c * 8, wv);
 #pragma unroll
-            for (int v = 0; v < 8; ++v) acc = __builtin_fmaf(xv[v], wv[v], acc);
+        for (int j = 0; j < NCH; ++j) {
+            const int c = lane + j * kWave;
+            if (c < nchunk) wn[j] = *reinterpret_cast<const raw_t*>(wr + c * 8);
+        }
+    };
+    fetch(e0);
+    for (int e = e0; e < e1; ++e) {
+        raw_t wc[NCH];
+#pragma unroll
+        for (int j = 0; j < NCH; ++j) wc[j] = wn[j];
+        if (e + 1 < e1) fetch(e + 1);
+        float acc[TPW];
+#pragma unroll
+        for (int q = 0; q < TPW; ++q) acc[q] = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NCH; ++j) {
+            const int c = lane + j * kWave;
+            if (c < nchunk) {
+                float wv[8];
+                if constexpr (sizeof(T) == 4) {
+#pragma unroll
+                    for (int v = 0; v < 8; ++v) wv[v] = __uint_as_float(wc[j][v]);
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        wv[2 * v] = __uint_as_float(wc[j][v] << 16);
+                        wv[2 * v + 1] = __uint_as_float(wc[j][v] & 0xFFFF0000u);
+                    }
+                }
+#pragma unroll
+                for (int q = 0; q < TPW; ++q)
+#pragma unroll
+                    for (int v = 0; v < 8; ++v) acc[q] = __builtin_fmaf(xr[q][j][v], wv[v], acc[q]);
+            }
         }
 #pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) acc = acc + __shfl_xor(acc, off, kWave);
-        if (lane == 0) logits[(size_t)t * E + e] = gate_bias ? acc + gate_bias[e] : acc;
+        for (int q = 0; q < TPW; ++q) {
+            float r = acc[q];
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) r = r + __shfl_xor(r, off, kWave);
+            if (lane == 0 && t0 + q < S) logits[(size_t)(t0 + q) * E + e] = gate_bias ? r + gate_bias[e] : r;
+        }
     }
+}
+
+template <typename T, int NCH, int TPW>
+hipError_t launch_gate_variant(const void* x, const void* gate_w, const float* gate_bias, float* logits, int S, int H,
+                               int E, hipStream_t st) {
+    const int token_blocks = (S + 4 * TPW - 1) / (4 * TPW);
+    // enough workgroups to occupy the chip even when S is small (decode shapes)
+    int chunks = 1;
+    while (token_blocks * chunks < 1024 && chunks < E) chunks *= 2;
+    const int per = (E + chunks - 1) / chunks;
+    chunks = (E + per - 1) / per;
+    gate_logits_kernel<T, NCH, TPW><<<dim3(token_blocks, chunks), 256, 0, st>>>((const T*)x, (const T*)gate_w,
+                                                                                gate_bias, logits, S, H, E, per);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t launch_gate_typed(const void* x, const void* gate_w, const float* gate_bias, float* logits, int S, int H,
+                             int E, hipStream_t st) {
+    const bool many = (int64_t)S * E >= 4 * 4096;   // enough (token, expert) work to give each wavefront 4 tokens
+    if (H <= 1024) return many ? launch_gate_variant<T, 2, 4>(x, gate_w, gate_bias, logits, S, H, E, st)
+                               : launch_gate_variant<T, 2, 1>(x, gate_w, gate_bias, logits, S, H, E, st);
+    if (H <= 2048) return many ? launch_gate_variant<T, 4, 4>(x, gate_w, gate_bias, logits, S, H, E, st)
+                               : launch_gate_variant<T, 4, 1>(x, gate_w, gate_bias, logits, S, H, E, st);
+    if (H <= 4096) return many ? launch_gate_variant<T, 8, 2>(x, gate_w, gate_bias, logits, S, H, E, st)
+                               : launch_gate_variant<T, 8, 1>(x, gate_w, gate_bias, logits, S, H, E, st);
+    if (H <= 8192) return launch_gate_variant<T, 16, 1>(x, gate_w, gate_bias, logits, S, H, E, st);
+    if (H <= 16384) return launch_gate_variant<T, 32, 1>(x, gate_w, gate_bias, logits, S, H, E, st);
+    return hipErrorInvalidValue;
 }
 
 struct Cand {
@@ -148,35 +212,8 @@ __global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ log
 
 hipError_t launch_gate_logits(const void* x, const void* gate_w, const float* gate_bias, float* logits, int S, int H,
                               int E, int act_dtype, hipStream_t st) {
-    const int token_blocks = (S + kGateTokens - 1) / kGateTokens;
-    // enough workgroups to occupy the chip even when S is small (decode shapes)
-    int chunks = 1;
-    while (token_blocks * chunks < 1024 && chunks < E) chunks *= 2;
-    const int per = (E + chunks - 1) / chunks;
-    chunks = (E + per - 1) / per;
-    const dim3 grid(token_blocks, chunks);
-    if (act_dtype == MOE_DTYPE_F32) {
-        const size_t lds = (size_t)kGateTokens * H * 4;
-        if (lds > 160 * 1024) return hipErrorInvalidValue;
-        if (lds > 48 * 1024) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gate_logits_kernel<float>),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            if (e != hipSuccess) return e;
-        }
-        gate_logits_kernel<float><<<grid, 256, lds, st>>>((const float*)x, (const float*)gate_w, gate_bias, logits, S,
-                                                          H, E, per);
-    } else {
-        const size_t lds = (size_t)kGateTokens * H * 2;
-        if (lds > 160 * 1024) return hipErrorInvalidValue;
-        if (lds > 48 * 1024) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gate_logits_kernel<uint16_t>),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            if (e != hipSuccess) return e;
-        }
-        gate_logits_kernel<uint16_t><<<grid, 256, lds, st>>>((const uint16_t*)x, (const uint16_t*)gate_w, gate_bias,
-                                                             logits, S, H, E, per);
-    }
-    return hipGetLastError();
+    if (act_dtype == MOE_DTYPE_F32) return launch_gate_typed<float>(x, gate_w, gate_bias, logits, S, H, E, st);
+    return launch_gate_typed<uint16_t>(x, gate_w, gate_bias, logits, S, H, E, st);
 }
 
 hipError_t launch_topk(const float* logits, int S, int E, int k, int gate_fn, int norm, int32_t* topk_idx,

@@ -92,6 +92,7 @@ struct RouteArgs {
     int32_t block_m;            // rows per MTile
     int32_t nnt0, nnt1;         // column tiles of phase 0 / phase 1
     int32_t max_mtiles;
+    int32_t lag;                // experts of phase-0 work queued between an expert's two phases
 };
 
 // ---- launchers (defined next to their kernels) ----

@@ -56,11 +56,43 @@ __device__ __forceinline__ void write_segment(Segment* s, int begin, int phase, 
     s->pad0 = 0; s->pad1 = 0;
 }
 
+// Exclusive prefix sum of one int per thread over a workgroup of kMaxExperts threads (wave shuffles, then the
+// eight wave totals through LDS).  *total receives the sum.  Every thread must call it.
+__device__ __forceinline__ int block_exclusive_scan(int v, int* s_wave, int* total) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int inc = v;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        const int o = __shfl_up(inc, off, kWave);
+        if (lane >= off) inc += o;
+    }
+    __syncthreads();                      // s_wave may still be read by a previous call
+    if (lane == kWave - 1) s_wave[wave] = inc;
+    __syncthreads();
+    int base = 0, sum = 0;
+#pragma unroll
+    for (int w = 0; w < kMaxExperts / kWave; ++w) {
+        const int t = s_wave[w];
+        if (w < wave) base += t;
+        sum += t;
+    }
+    *total = sum;
+    return base + inc - v;
+}
+
+// Queue order with lag L: phase-0 segments of experts 0..L-1, then (phase-0 of e, phase-1 of e-L) for
+// e = L..E-1, then the phase-1 segments of the last L experts.
+__device__ __forceinline__ void queue_slot(int s, int E, int L, int* phase, int* ex) {
+    if (s < L) { *phase = 0; *ex = s; }
+    else if (s < 2 * E - L) { const int r = s - L; *phase = r & 1; *ex = (r & 1) ? (r >> 1) : L + (r >> 1); }
+    else { *phase = 1; *ex = E - L + (s - (2 * E - L)); }
+}
+
 // One workgroup of kMaxExperts threads: thread e owns expert e.
 __global__ __launch_bounds__(kMaxExperts) void route_scan_kernel(RouteArgs a) {
-    __shared__ int s_kept[kMaxExperts];
-    __shared__ int s_off[kMaxExperts + 1];
-    __shared__ int s_mt0[kMaxExperts + 1];
+    __shared__ int s_wave[kMaxExperts / kWave];
+    __shared__ int s_nmt[kMaxExperts];
+    __shared__ int s_mt0[kMaxExperts];
     const int e = threadIdx.x;
     int kept = 0;
     if (e < a.E) {
@@ -73,59 +105,59 @@ __global__ __launch_bounds__(kMaxExperts) void route_scan_kernel(RouteArgs a) {
         }
         kept = (a.drop && run > a.capacity) ? a.capacity : run;
     }
-    s_kept[e] = kept;
+    const int nmt = (kept + a.block_m - 1) / a.block_m;
+    int total_rows, total_mt, total_tasks;
+    const int off = block_exclusive_scan(kept, s_wave, &total_rows);
+    const int mt0 = block_exclusive_scan(nmt, s_wave, &total_mt);
+    s_nmt[e] = nmt;
+    s_mt0[e] = mt0;
     __syncthreads();
+    // the merged queue: thread t owns segments 2t and 2t+1.  A phase-1 task must not be popped while the
+    // phase-0 tasks it depends on are still running, or its workgroup idles: `lag` experts of phase-0 work
+    // (at least a couple of tasks per resident workgroup) sit between the two.
+    const int nseg = 2 * a.E;
+    int ph[2] = {0, 0}, ex[2] = {0, 0}, size[2] = {0, 0};
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int sidx = 2 * e + j;
+        if (sidx < nseg) {
+            queue_slot(sidx, a.E, a.lag, &ph[j], &ex[j]);
+            size[j] = s_nmt[ex[j]] * (ph[j] ? a.nnt1 : a.nnt0);
+        }
+    }
+    const int begin = block_exclusive_scan(size[0] + size[1], s_wave, &total_tasks);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int sidx = 2 * e + j;
+        if (sidx < nseg)
+            write_segment(a.seg_queue + sidx, begin + (j ? size[0] : 0), ph[j], ex[j], s_mt0[ex[j]], s_nmt[ex[j]],
+                          ph[j] ? a.nnt1 : a.nnt0);
+    }
     if (e == 0) {
-        int off = 0, mt = 0;
-        for (int i = 0; i < a.E; ++i) {
-            s_off[i] = off;
-            s_mt0[i] = mt;
-            off += s_kept[i];
-            mt += (s_kept[i] + a.block_m - 1) / a.block_m;
-        }
-        s_off[a.E] = off;
-        s_mt0[a.E] = mt;
-        // queue order: phase-0 tasks of expert e are followed by phase-1 tasks of expert e-1, so a phase-1
-        // task never has to wait long for the phase-0 tasks it depends on
-        int begin = 0;
-        const int nseg = 2 * a.E;
-        for (int s = 0; s < nseg; ++s) {
-            int phase, ex;
-            if (s == 0) { phase = 0; ex = 0; }
-            else if (s == nseg - 1) { phase = 1; ex = a.E - 1; }
-            else if (s & 1) { phase = 0; ex = (s + 1) >> 1; }
-            else { phase = 1; ex = (s - 2) >> 1; }
-            const int nmt = s_mt0[ex + 1] - s_mt0[ex];
-            const int nnt = phase ? a.nnt1 : a.nnt0;
-            write_segment(a.seg_queue + s, begin, phase, ex, s_mt0[ex], nmt, nnt);
-            begin += nmt * nnt;
-        }
         a.q->head = 0;
-        a.q->total_tasks = begin;
-        a.q->tasks_phase0 = mt * a.nnt0;
-        a.q->tasks_phase1 = mt * a.nnt1;
-        a.q->num_mtiles = mt;
-        a.q->kept_rows = off;
+        a.q->total_tasks = total_tasks;
+        a.q->tasks_phase0 = total_mt * a.nnt0;
+        a.q->tasks_phase1 = total_mt * a.nnt1;
+        a.q->num_mtiles = total_mt;
+        a.q->kept_rows = total_rows;
         a.q->stall = 0;
         a.q->nseg = nseg;
+        a.expert_offset[a.E] = total_rows;
     }
-    __syncthreads();
     if (e < a.E) {
         a.expert_count[e] = kept;
-        a.expert_offset[e] = s_off[e];
-        const int mt0 = s_mt0[e], nmt = s_mt0[e + 1] - s_mt0[e];
+        a.expert_offset[e] = off;
         write_segment(a.seg_phase0 + e, mt0 * a.nnt0, 0, e, mt0, nmt, a.nnt0);
         write_segment(a.seg_phase1 + e, mt0 * a.nnt1, 1, e, mt0, nmt, a.nnt1);
         for (int i = 0; i < nmt; ++i) {
             MTile t;
             t.expert = e;
-            t.row0 = s_off[e] + i * a.block_m;
+            t.row0 = off + i * a.block_m;
             t.rows = min(a.block_m, kept - i * a.block_m);
             t.pad = 0;
             a.mtiles[mt0 + i] = t;
         }
     }
-    if (e == 0) a.expert_offset[a.E] = s_off[a.E];
     for (int i = threadIdx.x; i < a.max_mtiles; i += blockDim.x) a.done0[i] = 0;
 }
 

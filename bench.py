@@ -21,6 +21,10 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
+# Bytes per FFN-kernel launch that crossed the L2 <-> memory-fabric boundary, from two rocprofv3 --pmc runs of this
+# script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter showed for a 1 GiB
+# device copy in the same run (--calibrate-copy): read x2.000, write x1.000.  Summaries are kept under profiles/.
+MEASURED_TRAFFIC_BYTES = {"mixtral": 32.797e9 + 1.074e9, "decode_fp8": 9.837e9 + 0.010e9}
 
 
 def workloads():
@@ -89,6 +93,8 @@ def main():
     ap.add_argument("--ffn-mode", type=int, default=0, help="0 auto, 1 tiled (two launches), 2 persistent queue")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample (0 = skip)")
     ap.add_argument("--seed", type=int, default=42)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 1 GiB device-to-device copy (a known-size reference for HBM byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the MoE layer with all experts resident on ONE GPU; --gpus %d is not "
@@ -112,6 +118,13 @@ def main():
     routing = layer.new_routing()
     out = torch.empty(cfg.S, cfg.H, dtype=layer.act_dtype, device="cuda")
 
+    if args.calibrate_copy:
+        src = torch.zeros(1 << 30, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)              # reads 1 GiB and writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         layer.forward(dev["x"], dev, out=out, routing=routing)
     torch.cuda.synchronize()
@@ -146,6 +159,7 @@ def main():
         if cfg.dtype == ob.F32:
             roofline["peak"] = 157.3
     roofline["frac"] = roofline["achieved"] / roofline["peak"]
+    roofline["traffic"] = MEASURED_TRAFFIC_BYTES.get(args.workload)
 
     # ---- CPU baseline + parity spot check on the same sample ----
     cpu = None

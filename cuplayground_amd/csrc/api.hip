@@ -29,6 +29,7 @@ hipError_t launch_ffn_fp8(const FfnArgs&, int max_mtiles, int nnt0, int nnt1, in
 int fp8_block_m();
 int fp8_block_n0();
 int fp8_block_n1();
+int ffn_persistent_occupancy_fp8();
 
 namespace {
 
@@ -503,7 +504,7 @@ hipError_t launch_ffn_persistent(const FfnArgs& a, int dtype, const FfnPlan& p, 
 
 int ffn_persistent_blocks(int dtype, int block_m, int compute_units) {
     if (dtype == MOE_DTYPE_F32) return compute_units * 4;
-    if (dtype == MOE_DTYPE_FP8_E4M3_B128) return compute_units * 4;
+    if (dtype == MOE_DTYPE_FP8_E4M3_B128) return compute_units * ffn_persistent_occupancy_fp8();
     return compute_units * ffn_persistent_occupancy_bf16(block_m);
 }
 

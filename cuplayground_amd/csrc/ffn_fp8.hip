@@ -25,8 +25,9 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int QBM = 16;      // token rows per task
-constexpr int QN0 = 64;      // intermediate columns per phase-0 task (64 gate rows + 64 up rows)
-constexpr int QN1 = 128;     // output columns per phase-1 task
+constexpr int QN0 = 64;      // intermediate columns per phase-0 sub-tile (64 gate rows + 64 up rows)
+constexpr int QN1 = 128;     // output columns per phase-1 sub-tile
+constexpr int QSUB = 2;      // sub-tiles per task: halves the pops, decodes and dependency traffic per byte streamed
 constexpr int QGROUPS = 8;   // 16-row weight groups per task
 constexpr int QWAVES = 4;
 
@@ -175,7 +176,7 @@ __device__ __forceinline__ void fp8_tile(const Fp8Task& t, float* red) {
     }
 }
 
-__device__ __forceinline__ Fp8Task resolve_fp8(const FfnArgs& a, const Task& t, bool publish) {
+__device__ __forceinline__ Fp8Task resolve_fp8(const FfnArgs& a, const Task& t, int sub, bool publish) {
     Fp8Task p;
     p.publish = publish && t.phase == 0;
     const int64_t HI = (int64_t)a.H * a.I;
@@ -183,7 +184,7 @@ __device__ __forceinline__ Fp8Task resolve_fp8(const FfnArgs& a, const Task& t, 
     p.phase = t.phase;
     p.rows = t.rows;
     if (t.phase == 0) {
-        p.c0 = t.ntile * QN0;
+        p.c0 = (t.ntile * QSUB + sub) * QN0;
         p.K = a.H;
         p.N = a.I;
         p.w[0] = (const uint8_t*)a.w_gate + t.expert * HI;
@@ -198,7 +199,7 @@ __device__ __forceinline__ Fp8Task resolve_fp8(const FfnArgs& a, const Task& t, 
         p.a_row0 = 0;
         p.c_base = (uint16_t*)a.h + (int64_t)t.row0 * a.I;
     } else {
-        p.c0 = t.ntile * QN1;
+        p.c0 = (t.ntile * QSUB + sub) * QN1;
         p.K = a.I;
         p.N = a.H;
         p.w[0] = p.w[1] = (const uint8_t*)a.w_down + t.expert * HI;
@@ -221,11 +222,13 @@ __global__ __launch_bounds__(256) void ffn_tiled_fp8_kernel(FfnArgs a, int phase
     if (id >= ntasks) return;
     const int nnt0 = a.seg_phase0[0].nnt;
     const Task t = decode_task(phase ? a.seg_phase1 : a.seg_phase0, a.E, a.mtiles, id, nnt0);
-    const Fp8Task p = resolve_fp8(a, t, false);
-    fp8_tile(p, red);
+    for (int sub = 0; sub < QSUB; ++sub) {
+        const Fp8Task p = resolve_fp8(a, t, sub, false);
+        if (p.c0 < p.N) fp8_tile(p, red);
+    }
 }
 
-__global__ __launch_bounds__(256) void ffn_persistent_fp8_kernel(FfnArgs a) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void ffn_persistent_fp8_kernel(FfnArgs a) {
     __shared__ float red[QWAVES * QGROUPS * 4 * 64];
     __shared__ int s_task;
     queue_kernel_entry();
@@ -237,8 +240,10 @@ __global__ __launch_bounds__(256) void ffn_persistent_fp8_kernel(FfnArgs a) {
         if (id >= total) break;
         const Task t = decode_task(a.seg_queue, nseg, a.mtiles, id, nnt0);
         if (t.phase == 1) wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q);
-        const Fp8Task p = resolve_fp8(a, t, true);
-        fp8_tile(p, red);
+        for (int sub = 0; sub < QSUB; ++sub) {
+            const Fp8Task p = resolve_fp8(a, t, sub, true);
+            if (p.c0 < p.N) fp8_tile(p, red);
+        }
         if (t.phase == 0) signal_phase0_done(a.done0, t.mtile);
     }
 }
@@ -246,8 +251,16 @@ __global__ __launch_bounds__(256) void ffn_persistent_fp8_kernel(FfnArgs a) {
 }  // namespace
 
 int fp8_block_m() { return QBM; }
-int fp8_block_n0() { return QN0; }
-int fp8_block_n1() { return QN1; }
+int fp8_block_n0() { return QN0 * QSUB; }
+int fp8_block_n1() { return QN1 * QSUB; }
+
+int ffn_persistent_occupancy_fp8() {
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, reinterpret_cast<const void*>(&ffn_persistent_fp8_kernel), 256,
+                                                     0) != hipSuccess || n < 1)
+        n = 1;
+    return n;
+}
 
 hipError_t launch_ffn_fp8(const FfnArgs& a, int max_mtiles, int nnt0, int nnt1, int blocks, hipStream_t st) {
     if (blocks > 0) {

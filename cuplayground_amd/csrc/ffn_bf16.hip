@@ -9,8 +9,8 @@
 //     as 128-byte rows whose 16-byte chunks are xor-swizzled with (row >> 1) & 7: the LDS has 64 banks, a
 //     ds_read_b128 is served 16 lanes at a time, and with this swizzle 16 consecutive rows of one logical
 //     chunk fall into 16 distinct bank groups (measured: SQ_LDS_BANK_CONFLICT = 0);
-//   * 2 (or 3) LDS stages; the loads of the next slab are issued a quarter at a time between the MFMAs of the
-//     current one so they never queue up behind each other, and MFMA operand fragments are double buffered
+//   * 2 (or 3) LDS stages; the loads of the next slab are issued one MFMA apart during the first two of the
+//     current slab's four sub-steps (early enough to land, spread enough not to queue up behind each other), and MFMA operand fragments are double buffered
 //     in registers across the four 16-wide k sub-steps of a slab;
 //   * dispatch is fused into the A-tile load: phase 0 gathers token rows through token_indices[];
 //   * SwiGLU pairs gate and up columns inside one wavefront (first half of its tile rows from w_gate, second
@@ -171,7 +171,10 @@ __device__ __forceinline__ void gemm_tile(const TaskPtrs& p, unsigned char* smem
 #pragma unroll
         for (int ks = 0; ks < kBK / 16; ++ks) {
             const int cb = ks & 1, nb = cb ^ 1;
-            if (pre) issue_part(kt + NS - 1, ks);
+            if (pre && ks < 2) {   // half of the next slab's loads in each of the first two sub-steps
+                issue_part(kt + NS - 1, 2 * ks);
+                issue_part(kt + NS - 1, 2 * ks + 1);
+            }
             if (ks < 3) {
                 const int c = (((ks + 1) * 2 + fk) ^ sw) << 4;
 #pragma unroll
@@ -184,8 +187,8 @@ __device__ __forceinline__ void gemm_tile(const TaskPtrs& p, unsigned char* smem
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cb][j], af[cb][i], acc[i][j], 0, 0, 0);
-            // instruction order inside the sub-step: one LDS read behind each of the first MFMAs, then the
-            // global loads one MFMA apart, then the remaining MFMAs
+            // instruction order inside the sub-step: one LDS read behind each of the first MFMAs, then (first two
+            // sub-steps) the global loads one MFMA apart, then the remaining MFMAs
             if (ks < 3) {
 #pragma unroll
                 for (int n = 0; n < TM + TN; ++n) {
@@ -193,10 +196,12 @@ __device__ __forceinline__ void gemm_tile(const TaskPtrs& p, unsigned char* smem
                     __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
                 }
             }
+            if (ks < 2) {
 #pragma unroll
-            for (int n = 0; n < 2; ++n) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                for (int n = 0; n < (T::RA + T::RB + 1) / 2; ++n) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                }
             }
             __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
         }

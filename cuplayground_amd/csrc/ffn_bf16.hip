@@ -309,7 +309,7 @@ struct Plan {
     static constexpr int THREADS = T0::THREADS;
     static constexpr int LDS_BYTES = T0::LDS_BYTES > T1::LDS_BYTES ? T0::LDS_BYTES : T1::LDS_BYTES;
 };
-using LargePlan = Plan<Tile<256, 256, 2, 4, 2>, Tile<256, 128, 2, 4, 3>>;
+using LargePlan = Plan<Tile<256, 256, 2, 4, 2>, Tile<256, 256, 2, 4, 2>>;
 using SmallPlan = Plan<Tile<128, 128, 2, 2, 2>, Tile<128, 128, 2, 2, 2>>;
 
 // One launch per phase; workgroup b runs task b of that phase.

@@ -190,11 +190,15 @@ RouteArgs route_args(const moe_handle* h, void* ws) {
     a.nnt0 = d.plan.nnt0;
     a.nnt1 = d.plan.nnt1;
     a.max_mtiles = d.max_mtiles;
-    // phase-0 tasks an average expert contributes; enough experts of them to cover two tasks per workgroup
+    // phase-0 tasks an average expert contributes; enough experts of them to cover four tasks per workgroup
     const int64_t avg_mt = d.A / ((int64_t)d.E * d.plan.block_m) > 0 ? d.A / ((int64_t)d.E * d.plan.block_m) : 1;
     const int64_t per_expert = avg_mt * d.plan.nnt0;
-    int64_t lag = (2 * (int64_t)h->arch.persistent_blocks + per_expert - 1) / per_expert;
+    int64_t lag = (4 * (int64_t)h->arch.persistent_blocks + per_expert - 1) / per_expert;
     if (lag < 1) lag = 1;
+    if (const char* env = getenv("MOE355_QUEUE_LAG")) {   // tuning knob: experts of phase-0 work between phases
+        const int v = atoi(env);
+        if (v >= 1) lag = v;
+    }
     if (lag > d.E) lag = d.E;
     a.lag = (int)lag;
     return a;

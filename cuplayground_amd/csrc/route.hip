@@ -94,15 +94,43 @@ __global__ __launch_bounds__(kMaxExperts) void route_scan_kernel(RouteArgs a) {
     __shared__ int s_nmt[kMaxExperts];
     __shared__ int s_mt0[kMaxExperts];
     const int e = threadIdx.x;
-    int kept = 0;
-    if (e < a.E) {
-        int run = 0;
-        for (int b = 0; b < a.nblk; ++b) {
-            const size_t i = (size_t)b * a.E + e;
+    // per-expert exclusive prefix over the workgroups' histograms: the kMaxExperts threads split into
+    // `parts` groups that each take a contiguous run of workgroups (two passes over block_hist)
+    __shared__ int s_part[kMaxExperts];
+    __shared__ int s_total[kMaxExperts];
+    int epad = 1;
+    while (epad < a.E) epad <<= 1;
+    const int parts = kMaxExperts / epad;
+    const int pe = threadIdx.x % epad, part = threadIdx.x / epad;
+    const int chunk = (a.nblk + parts - 1) / parts;
+    const int b0 = min(a.nblk, part * chunk), b1 = min(a.nblk, b0 + chunk);
+    int sum = 0;
+    if (pe < a.E) {
+#pragma unroll 4
+        for (int b = b0; b < b1; ++b) sum += a.block_hist[(size_t)b * a.E + pe];
+    }
+    s_part[threadIdx.x] = sum;
+    __syncthreads();
+    if (pe < a.E) {
+        int run = 0, total = 0;
+        for (int q = 0; q < parts; ++q) {
+            const int v = s_part[q * epad + pe];
+            if (q < part) run += v;
+            total += v;
+        }
+        if (part == 0) s_total[pe] = total;
+#pragma unroll 4
+        for (int b = b0; b < b1; ++b) {
+            const size_t i = (size_t)b * a.E + pe;
             const int v = a.block_hist[i];
             a.block_hist[i] = run;
             run += v;
         }
+    }
+    __syncthreads();
+    int kept = 0;
+    if (e < a.E) {
+        const int run = s_total[e];
         kept = (a.drop && run > a.capacity) ? a.capacity : run;
     }
     const int nmt = (kept + a.block_m - 1) / a.block_m;

@@ -77,8 +77,10 @@ __device__ __forceinline__ void store8(uint16_t* p, uint32_t lo, uint32_t hi, bo
     }
 }
 
-template <class T>
-__device__ __forceinline__ void gemm_tile(const TaskPtrs& p, unsigned char* smem) {
+// PARTIAL: the row block holds fewer than BM rows; 32-row MFMA sub-tiles that lie entirely in the padding are
+// skipped (their LDS reads too).  A separate instantiation keeps the full-tile loop free of branches.
+template <class T, bool PARTIAL>
+__device__ __forceinline__ void gemm_tile_impl(const TaskPtrs& p, unsigned char* smem) {
     constexpr int BM = T::BM, BN = T::BN, TM = T::TM, TN = T::TN, NS = T::NS;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / T::WN, wn = wave % T::WN;
@@ -150,6 +152,8 @@ __device__ __forceinline__ void gemm_tile(const TaskPtrs& p, unsigned char* smem
 
     const int frow = lane & 31, fk = lane >> 5;
     const int sw = (frow >> 1) & 7;
+    // 32-row sub-tiles of this wavefront that contain at least one real row (wavefront-uniform)
+    const int tm_active = PARTIAL ? min(TM, max(0, (p.rows - wm * 32 * TM + 31) >> 5)) : TM;
     int a_off[TM], b_off[TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i) a_off[i] = (wm * 32 * TM + i * 32 + frow) * kRowBytes;
@@ -165,7 +169,8 @@ __device__ __forceinline__ void gemm_tile(const TaskPtrs& p, unsigned char* smem
         const bool pre = kt + NS - 1 < KT;
         const unsigned char* st = smem + (kt % NS) * T::STAGE_BYTES;
 #pragma unroll
-        for (int i = 0; i < TM; ++i) af[0][i] = *reinterpret_cast<const bf16x8*>(st + a_off[i] + ((fk ^ sw) << 4));
+        for (int i = 0; i < TM; ++i)
+            if (!PARTIAL || i < tm_active) af[0][i] = *reinterpret_cast<const bf16x8*>(st + a_off[i] + ((fk ^ sw) << 4));
 #pragma unroll
         for (int j = 0; j < TN; ++j) bfr[0][j] = *reinterpret_cast<const bf16x8*>(st + b_off[j] + ((fk ^ sw) << 4));
 #pragma unroll
@@ -178,32 +183,35 @@ __device__ __forceinline__ void gemm_tile(const TaskPtrs& p, unsigned char* smem
             if (ks < 3) {
                 const int c = (((ks + 1) * 2 + fk) ^ sw) << 4;
 #pragma unroll
-                for (int i = 0; i < TM; ++i) af[nb][i] = *reinterpret_cast<const bf16x8*>(st + a_off[i] + c);
+                for (int i = 0; i < TM; ++i)
+                    if (!PARTIAL || i < tm_active) af[nb][i] = *reinterpret_cast<const bf16x8*>(st + a_off[i] + c);
 #pragma unroll
                 for (int j = 0; j < TN; ++j) bfr[nb][j] = *reinterpret_cast<const bf16x8*>(st + b_off[j] + c);
             }
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
+            for (int i = 0; i < TM; ++i) {
+                if (PARTIAL && i >= tm_active) continue;
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cb][j], af[cb][i], acc[i][j], 0, 0, 0);
+            }
             // instruction order inside the sub-step: one LDS read behind each of the first MFMAs, then (first two
             // sub-steps) the global loads one MFMA apart, then the remaining MFMAs
-            if (ks < 3) {
+            if (!PARTIAL && ks < 3) {
 #pragma unroll
                 for (int n = 0; n < TM + TN; ++n) {
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                     __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
                 }
             }
-            if (ks < 2) {
+            if (!PARTIAL && ks < 2) {
 #pragma unroll
                 for (int n = 0; n < (T::RA + T::RB + 1) / 2; ++n) {
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                     __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
                 }
             }
-            __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
+            if (!PARTIAL) __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
         }
     }
 
@@ -254,6 +262,12 @@ __device__ __forceinline__ void gemm_tile(const TaskPtrs& p, unsigned char* smem
             }
         }
     }
+}
+
+template <class T>
+__device__ __forceinline__ void gemm_tile(const TaskPtrs& p, unsigned char* smem) {
+    if (p.rows >= T::BM) gemm_tile_impl<T, false>(p, smem);
+    else gemm_tile_impl<T, true>(p, smem);
 }
 
 template <class T>

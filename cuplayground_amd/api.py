@@ -22,7 +22,8 @@ STAGES = ("gate", "route", "ffn", "combine")
 
 EXPORTS = (
     "moe_config_default", "moe_config_from_json_string", "moe_config_from_json_file", "moe_config_validate",
-    "moe_config_tokens", "moe_config_capacity", "moe_create", "moe_destroy", "moe_get_arch", "moe_workspace_bytes",
+    "moe_config_tokens", "moe_config_capacity", "moe_create", "moe_destroy", "moe_get_arch", "moe_get_plan",
+    "moe_workspace_bytes",
     "moe_set_ffn_mode", "moe_forward", "moe_gate", "moe_route", "moe_gemm_bias_act", "moe_combine",
     "moe_set_stage_timing", "moe_get_stage_ms", "moe_get_task_counts", "moe_last_hip_error", "moe_status_string",
     "moe_version",
@@ -83,6 +84,7 @@ def load_library():
     L.moe_create.argtypes = [cfgp, C.POINTER(vp)]
     L.moe_destroy.argtypes = [vp]
     L.moe_get_arch.argtypes = [vp, C.POINTER(_CArch)]
+    L.moe_get_plan.argtypes = [vp, C.POINTER(i32), C.POINTER(i32), C.POINTER(i32)]
     L.moe_workspace_bytes.argtypes = [cfgp, C.POINTER(C.c_size_t)]
     L.moe_set_ffn_mode.argtypes = [vp, C.c_int]
     L.moe_forward.argtypes = [vp, vp, C.POINTER(_CWeights), vp, C.POINTER(_CRouting), vp, C.c_size_t, vp]
@@ -220,6 +222,12 @@ class MoELayer:
         d = {n: getattr(a, n) for n, _ in _CArch._fields_}
         d["name"] = a.name.decode()
         return d
+
+    @property
+    def plan(self) -> dict:
+        a, b, c = C.c_int32(0), C.c_int32(0), C.c_int32(0)
+        _check(self.L.moe_get_plan(self._h, C.byref(a), C.byref(b), C.byref(c)))
+        return dict(block_rows=a.value, col_tiles_up=b.value, col_tiles_down=c.value)
 
     def set_ffn_mode(self, mode: int):
         _check(self.L.moe_set_ffn_mode(self._h, mode))

@@ -273,6 +273,14 @@ int moe_get_arch(const moe_handle* h, moe_arch* out) {
     return MOE_OK;
 }
 
+int moe_get_plan(const moe_handle* h, int32_t* block_rows, int32_t* col_tiles_up, int32_t* col_tiles_down) {
+    if (!h) return MOE_ERR_BAD_ARGUMENT;
+    if (block_rows) *block_rows = h->d.plan.block_m;
+    if (col_tiles_up) *col_tiles_up = h->d.plan.nnt0;
+    if (col_tiles_down) *col_tiles_down = h->d.plan.nnt1;
+    return MOE_OK;
+}
+
 int moe_set_ffn_mode(moe_handle* h, int mode) {
     if (!h || mode < MOE_FFN_AUTO || mode > MOE_FFN_PERSISTENT) return MOE_ERR_BAD_ARGUMENT;
     h->ffn_mode = mode;

@@ -100,6 +100,9 @@ typedef struct moe_handle moe_handle;
 int moe_create(const moe_config* cfg, moe_handle** out);
 int moe_destroy(moe_handle* h);
 int moe_get_arch(const moe_handle* h, moe_arch* out);
+/* The tiling the handle chose: rows per row block, and column tiles of the up(/gate) and of the down projection.
+ * Task totals follow the reference's bound tilesM*tilesNx + tilesM*tilesN (scheduling.cuh:212-222) per expert. */
+int moe_get_plan(const moe_handle* h, int32_t* block_rows, int32_t* col_tiles_up, int32_t* col_tiles_down);
 int moe_workspace_bytes(const moe_config* cfg, size_t* bytes);
 
 typedef struct moe_weights {

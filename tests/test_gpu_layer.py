@@ -83,6 +83,12 @@ RAGGED = {
     "fp8_many_rows_bias": ob.Cfg(S=200, H=384, I=384, E=4, k=2, act=ob.ACT_SWIGLU, dtype=ob.FP8,
                                  gate_fn=ob.GATE_SIGMOID, drop=1, capacity_factor=1.0),
     "one_token": ob.Cfg(S=1, H=64, I=64, E=2, k=1, act=ob.ACT_GELU, dtype=ob.BF16, norm_topk=0, drop=0),
+    # every expert selected by every token; a single expert; the widest router the kernels take; capacity of one row
+    "all_experts_selected": ob.Cfg(S=100, H=64, I=64, E=4, k=4, act=ob.ACT_SWIGLU, dtype=ob.BF16, drop=0),
+    "single_expert": ob.Cfg(S=300, H=128, I=64, E=1, k=1, act=ob.ACT_GELU, dtype=ob.BF16, norm_topk=0, drop=0),
+    "many_experts_bias": ob.Cfg(S=128, H=128, I=128, E=512, k=16, act=ob.ACT_SWIGLU, dtype=ob.BF16, drop=0),
+    "capacity_one": ob.Cfg(S=64, H=64, I=128, E=8, k=2, act=ob.ACT_RELU, dtype=ob.BF16, drop=1, capacity_factor=0.05),
+    "f32_single_expert_top1": ob.Cfg(S=70, H=64, I=64, E=1, k=1, act=ob.ACT_RELU, dtype=ob.F32, norm_topk=0, drop=0),
 }
 
 
@@ -98,6 +104,28 @@ def test_ragged_layers_vs_oracle(moe, name, mode):
     assert err <= OUT_TOL[cfg.dtype], err
     dead = (want["slot"] < 0).all(axis=1)
     assert (ob.to_f32(got["out"], cfg.act_dtype)[dead] == 0).all()
+
+
+@pytest.mark.parametrize("name", ["bf16_swiglu_skew", "bf16_gelu_ragged", "fp8_decode_small", "f32_swiglu_ragged"])
+def test_task_totals_match_the_reference_bound(moe, name):
+    """tasks = sum over experts of tilesM * tilesNx (first GEMM) and tilesM * tilesN (second GEMM)
+    (scheduling.cuh:212-222), with tilesM from the routed row counts; the hardware description is sane."""
+    import torch
+    cfg = RAGGED[name]
+    inp = ob.make_inputs(cfg, seed=3)
+    want = ob.forward(cfg, inp)
+    layer = moe.MoELayer(product_config(cfg), ffn_mode=FFN_PERSISTENT)
+    dev = upload_inputs(cfg, inp)
+    layer.forward(dev["x"], dev)
+    torch.cuda.synchronize()
+    t0, t1 = layer.task_counts()
+    plan = layer.plan
+    tiles_m = sum(-(-int(c) // plan["block_rows"]) for c in want["expert_count"])
+    assert t0 == tiles_m * plan["col_tiles_up"] and t1 == tiles_m * plan["col_tiles_down"]
+    arch = layer.arch
+    assert arch["name"].startswith("gfx950") and arch["wavefront_size"] == 64 and arch["compute_units"] >= 1
+    assert arch["persistent_blocks"] >= arch["compute_units"]
+    layer.close()
 
 
 def test_repeat_calls_are_deterministic_and_workspace_is_reusable(moe):

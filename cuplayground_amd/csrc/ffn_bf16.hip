@@ -17,6 +17,8 @@
 //     half from w_up), so silu(g)*u happens in registers.
 // Two plans: "large" (256-row blocks, 512 threads: 256x256 tiles for the up projection, 256x128 for the
 // down projection) when experts see many rows, "small" (128x128 tiles, 256 threads) otherwise.
+#include <cstdlib>
+
 #include "ffn_common.hpp"
 
 namespace moe355 {
@@ -431,11 +433,15 @@ int occupancy() {
 }  // namespace
 
 // Row-block height chosen for a layer: 256 when the average expert sees at least 256 rows and the up
-// projection still splits into a few tasks per compute unit at that size.
+// projection still gives every compute unit a task at that size.
 int bf16_block_m(int64_t pairs, int experts, int up_columns) {
+    if (const char* env = getenv("MOE355_BLOCK_ROWS")) {   // tuning knob: force the row-block height
+        const int v = atoi(env);
+        if (v == 128 || v == 256) return v;
+    }
     if (pairs / (experts > 0 ? experts : 1) < 256) return 128;
     const int64_t tasks = (pairs / 256) * ((up_columns + LargePlan::T0::BN - 1) / LargePlan::T0::BN);
-    return tasks >= 3 * 256 ? 256 : 128;
+    return tasks >= 256 ? 256 : 128;
 }
 int bf16_block_n0(int block_m) { return block_m == 256 ? LargePlan::T0::BN : SmallPlan::T0::BN; }
 int bf16_block_n1(int block_m) { return block_m == 256 ? LargePlan::T1::BN : SmallPlan::T1::BN; }

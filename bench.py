@@ -160,6 +160,11 @@ def main():
             roofline["peak"] = 157.3
     roofline["frac"] = roofline["achieved"] / roofline["peak"]
     roofline["traffic"] = MEASURED_TRAFFIC_BYTES.get(args.workload)
+    # ceilings measured on this box in this run (the published peaks assume the maximum clock)
+    peaks = moe.measured_peaks()
+    arch = layer.arch
+    roofline["measured_peak"] = peaks["hbm_read_gbs"] if cfg.dtype == ob.FP8 else peaks["mfma_bf16_tflops"]
+    roofline["frac_of_measured_peak"] = roofline["achieved"] / roofline["measured_peak"]
 
     # ---- CPU baseline + parity spot check on the same sample ----
     cpu = None
@@ -204,6 +209,9 @@ def main():
             "ffn_mode": args.ffn_mode, "persistent_blocks": layer.arch["persistent_blocks"], "kept_assignments": kept, "tile_tasks": [tasks0, tasks1]},
         "tflops": layer_flops / (ms_per_step * 1e-3) / 1e12,
         "stage_ms": {k: round(v, 4) for k, v in stage.items()},
+        "device": {"name": arch["name"], "compute_units": arch["compute_units"], "max_clock_khz": arch["max_clock_khz"],
+                   "measured_mfma_bf16_tflops": round(peaks["mfma_bf16_tflops"], 1),
+                   "measured_hbm_read_gbs": round(peaks["hbm_read_gbs"], 1)},
         "roofline": roofline, "cpu_baseline": cpu,
         "parity": {"routing_bit_exact": routing_exact, "max_rel_err_sample": parity},
     }

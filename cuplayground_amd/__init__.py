@@ -12,4 +12,5 @@ from .api import (  # noqa: F401
     gemm_bias_act,
     library_path,
     load_library,
+    measured_peaks,
 )

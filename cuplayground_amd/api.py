@@ -25,7 +25,8 @@ EXPORTS = (
     "moe_config_tokens", "moe_config_capacity", "moe_create", "moe_destroy", "moe_get_arch", "moe_get_plan",
     "moe_workspace_bytes",
     "moe_set_ffn_mode", "moe_forward", "moe_gate", "moe_route", "moe_gemm_bias_act", "moe_combine",
-    "moe_set_stage_timing", "moe_get_stage_ms", "moe_get_task_counts", "moe_last_hip_error", "moe_status_string",
+    "moe_set_stage_timing", "moe_get_stage_ms", "moe_get_task_counts", "moe_measure_mfma_tflops",
+    "moe_measure_hbm_read_gbs", "moe_last_hip_error", "moe_status_string",
     "moe_version",
 )
 
@@ -95,6 +96,8 @@ def load_library():
     L.moe_set_stage_timing.argtypes = [vp, C.c_int]
     L.moe_get_stage_ms.argtypes = [vp, C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_int32)]
     L.moe_get_task_counts.argtypes = [vp, vp, vp, C.POINTER(i64), C.POINTER(i64)]
+    L.moe_measure_mfma_tflops.argtypes = [vp, C.c_size_t, vp, C.POINTER(C.c_float)]
+    L.moe_measure_hbm_read_gbs.argtypes = [vp, C.c_size_t, vp, vp, C.POINTER(C.c_float)]
     L.moe_last_hip_error.argtypes = [vp]
     L.moe_status_string.argtypes = [C.c_int]; L.moe_status_string.restype = C.c_char_p
     L.moe_version.restype = C.c_int
@@ -304,6 +307,20 @@ class MoELayer:
                                 _ptr(r["expert_offset"]), _ptr(r["token_indices"]), _ptr(r["pair_row"]),
                                 _ptr(self.workspace), self.workspace_bytes, _stream()), "moe_route")
         return r
+
+
+def measured_peaks() -> dict:
+    """bf16 MFMA issue rate (TFLOP/s) and streaming read bandwidth (GB/s) measured on the current device."""
+    import torch
+    L = load_library()
+    buf = torch.zeros(2 << 30, dtype=torch.uint8, device="cuda")
+    scratch = torch.zeros(4 << 20, dtype=torch.uint8, device="cuda")
+    tf, gb = C.c_float(0), C.c_float(0)
+    _check(L.moe_measure_mfma_tflops(_ptr(scratch), scratch.numel(), _stream(), C.byref(tf)), "moe_measure_mfma_tflops")
+    _check(L.moe_measure_hbm_read_gbs(_ptr(buf), buf.numel(), _ptr(scratch), _stream(), C.byref(gb)),
+           "moe_measure_hbm_read_gbs")
+    del buf
+    return {"mfma_bf16_tflops": tf.value, "hbm_read_gbs": gb.value}
 
 
 def gemm_bias_act(A, B, bias, act: int):

@@ -24,7 +24,7 @@ PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
 # Bytes per FFN-kernel launch that crossed the L2 <-> memory-fabric boundary, from two rocprofv3 --pmc runs of this
 # script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter showed for a 1 GiB
 # device copy in the same run (--calibrate-copy): read x2.000, write x1.000.  Summaries are kept under profiles/.
-MEASURED_TRAFFIC_BYTES = {"mixtral": 32.797e9 + 1.074e9, "decode_fp8": 9.837e9 + 0.010e9}
+MEASURED_TRAFFIC_BYTES = {"mixtral": 28.224e9 + 1.089e9, "decode_fp8": 9.905e9 + 0.012e9}
 
 
 def workloads():
@@ -145,21 +145,22 @@ def main():
     ffn_flops = 2.0 * g * kept * cfg.H * cfg.I
     layer_flops = ffn_flops + 2.0 * cfg.S * cfg.H * cfg.E
     ffn_s = stage["ffn"] * 1e-3
+    queue = layer.ffn_mode == 2   # one launch of the task-queue kernel; otherwise one launch per projection
     if cfg.dtype == ob.FP8:
         active = int((cnt > 0).sum())
         scale_bytes = 3 * (cfg.H // 128) * (cfg.I // 128) * 4
         ffn_bytes = active * (3.0 * cfg.H * cfg.I + scale_bytes) + 2.0 * kept * cfg.H * 2
         roofline = {"bound": "hbm", "achieved": ffn_bytes / ffn_s / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                    "traffic": None, "kernel": "ffn_persistent_fp8_kernel", "kernel_ms": stage["ffn"],
+                    "traffic": None, "kernel": "ffn_persistent_fp8_kernel" if queue else "ffn_tiled_fp8_kernel x2", "kernel_ms": stage["ffn"],
                     "algorithmic_bytes": ffn_bytes, "active_experts": active}
     else:
         roofline = {"bound": "mfma", "achieved": ffn_flops / ffn_s / 1e12, "peak": PEAK_BF16_TFLOPS,
-                    "unit": "TFLOP/s", "traffic": None, "kernel": "ffn_persistent_kernel", "kernel_ms": stage["ffn"],
+                    "unit": "TFLOP/s", "traffic": None, "kernel": "ffn_persistent_kernel" if queue else "ffn_tiled_kernel x2", "kernel_ms": stage["ffn"],
                     "algorithmic_flops": ffn_flops}
         if cfg.dtype == ob.F32:
             roofline["peak"] = 157.3
     roofline["frac"] = roofline["achieved"] / roofline["peak"]
-    roofline["traffic"] = MEASURED_TRAFFIC_BYTES.get(args.workload)
+    roofline["traffic"] = MEASURED_TRAFFIC_BYTES.get(args.workload) if queue else None
     # ceilings measured on this box in this run (the published peaks assume the maximum clock)
     peaks = moe.measured_peaks()
     arch = layer.arch
@@ -206,7 +207,7 @@ def main():
         "config": {"workload": "%s: S=%d H=%d I=%d E=%d top%d %s %s" % (
             tag, cfg.S, cfg.H, cfg.I, cfg.E, cfg.k, {0: "relu", 1: "gelu", 2: "swiglu"}[cfg.act],
             "drop cf=%g" % cfg.capacity_factor if cfg.drop else "dropless"),
-            "ffn_mode": args.ffn_mode, "persistent_blocks": layer.arch["persistent_blocks"], "kept_assignments": kept, "tile_tasks": [tasks0, tasks1]},
+            "ffn_mode": layer.ffn_mode, "persistent_blocks": layer.arch["persistent_blocks"], "kept_assignments": kept, "tile_tasks": [tasks0, tasks1]},
         "tflops": layer_flops / (ms_per_step * 1e-3) / 1e12,
         "stage_ms": {k: round(v, 4) for k, v in stage.items()},
         "device": {"name": arch["name"], "compute_units": arch["compute_units"], "max_clock_khz": arch["max_clock_khz"],

@@ -24,7 +24,7 @@ EXPORTS = (
     "moe_config_default", "moe_config_from_json_string", "moe_config_from_json_file", "moe_config_validate",
     "moe_config_tokens", "moe_config_capacity", "moe_create", "moe_destroy", "moe_get_arch", "moe_get_plan",
     "moe_workspace_bytes",
-    "moe_set_ffn_mode", "moe_forward", "moe_gate", "moe_route", "moe_gemm_bias_act", "moe_combine",
+    "moe_set_ffn_mode", "moe_get_ffn_mode", "moe_forward", "moe_gate", "moe_route", "moe_gemm_bias_act", "moe_combine",
     "moe_set_stage_timing", "moe_get_stage_ms", "moe_get_task_counts", "moe_measure_mfma_tflops",
     "moe_measure_hbm_read_gbs", "moe_last_hip_error", "moe_status_string",
     "moe_version",
@@ -88,6 +88,7 @@ def load_library():
     L.moe_get_plan.argtypes = [vp, C.POINTER(i32), C.POINTER(i32), C.POINTER(i32)]
     L.moe_workspace_bytes.argtypes = [cfgp, C.POINTER(C.c_size_t)]
     L.moe_set_ffn_mode.argtypes = [vp, C.c_int]
+    L.moe_get_ffn_mode.argtypes = [vp, C.POINTER(C.c_int32)]
     L.moe_forward.argtypes = [vp, vp, C.POINTER(_CWeights), vp, C.POINTER(_CRouting), vp, C.c_size_t, vp]
     L.moe_gate.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, C.c_size_t, vp]
     L.moe_route.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, C.c_size_t, vp]
@@ -234,6 +235,13 @@ class MoELayer:
 
     def set_ffn_mode(self, mode: int):
         _check(self.L.moe_set_ffn_mode(self._h, mode))
+
+    @property
+    def ffn_mode(self) -> int:
+        """The FFN variant forward() runs: 1 = one launch per projection, 2 = task queue."""
+        m = C.c_int32(0)
+        _check(self.L.moe_get_ffn_mode(self._h, C.byref(m)))
+        return m.value
 
     def set_stage_timing(self, enable: bool):
         _check(self.L.moe_set_stage_timing(self._h, int(enable)))

@@ -204,6 +204,19 @@ RouteArgs route_args(const moe_handle* h, void* ws) {
     return a;
 }
 
+// The mode a forward call runs in.  The queue pays off once there are more tasks than resident workgroups; tiny
+// layers launch once per projection.  Row blocks are estimated on the host as the larger of kept rows / block rows
+// and the experts that can be hit at all (every hit expert owns at least one row block).
+int resolved_ffn_mode(const moe_handle* h) {
+    if (h->ffn_mode != MOE_FFN_AUTO) return h->ffn_mode;
+    const Derived& d = h->d;
+    int64_t row_blocks = d.A / d.plan.block_m + 1;
+    const int64_t hit = d.A < d.E ? d.A : d.E;
+    if (row_blocks < hit) row_blocks = hit;
+    const int64_t est_tasks = row_blocks * (d.plan.nnt0 + d.plan.nnt1);
+    return est_tasks >= 2 * (int64_t)h->arch.persistent_blocks ? MOE_FFN_PERSISTENT : MOE_FFN_TILED;
+}
+
 }  // namespace
 
 extern "C" {
@@ -284,6 +297,12 @@ int moe_get_plan(const moe_handle* h, int32_t* block_rows, int32_t* col_tiles_up
 int moe_set_ffn_mode(moe_handle* h, int mode) {
     if (!h || mode < MOE_FFN_AUTO || mode > MOE_FFN_PERSISTENT) return MOE_ERR_BAD_ARGUMENT;
     h->ffn_mode = mode;
+    return MOE_OK;
+}
+
+int moe_get_ffn_mode(const moe_handle* h, int32_t* mode) {
+    if (!h || !mode) return MOE_ERR_BAD_ARGUMENT;
+    *mode = resolved_ffn_mode(h);
     return MOE_OK;
 }
 
@@ -417,12 +436,7 @@ int moe_forward(moe_handle* h, const void* x, const moe_weights* w, void* out, c
     fa.H = d.H; fa.I = d.I; fa.E = d.E;
     fa.act = c.hidden_act;
     fa.spin_limit = 1 << 24;
-    int mode = h->ffn_mode;
-    if (mode == MOE_FFN_AUTO) {
-        // the queue pays off once there are more tasks than resident workgroups; tiny layers launch per phase
-        const int64_t est_tasks = ((int64_t)d.A / d.plan.block_m + 1) * (d.plan.nnt0 + d.plan.nnt1);
-        mode = est_tasks >= 2 * (int64_t)h->arch.persistent_blocks ? MOE_FFN_PERSISTENT : MOE_FFN_TILED;
-    }
+    const int mode = resolved_ffn_mode(h);
     if (fp8) {
         e = launch_ffn_fp8(fa, d.max_mtiles, d.plan.nnt0, d.plan.nnt1,
                            mode == MOE_FFN_PERSISTENT ? h->arch.persistent_blocks : 0, st);

@@ -132,6 +132,8 @@ typedef struct moe_routing_out {
 /* Variants of the FFN stage; MOE_FFN_AUTO lets the library choose. */
 enum { MOE_FFN_AUTO = 0, MOE_FFN_TILED = 1 /* one launch per GEMM */, MOE_FFN_PERSISTENT = 2 /* task queue */ };
 int moe_set_ffn_mode(moe_handle* h, int mode);
+/* The variant a forward call on this handle runs (MOE_FFN_TILED or MOE_FFN_PERSISTENT), with AUTO resolved. */
+int moe_get_ffn_mode(const moe_handle* h, int32_t* mode);
 
 /*
  * The whole layer, asynchronous on `stream`, no host synchronisation, no allocation.  This is the path the

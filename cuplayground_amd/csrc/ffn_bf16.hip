@@ -18,6 +18,7 @@
 // Two plans: "large" (256-row blocks, 512 threads: 256x256 tiles for the up projection, 256x128 for the
 // down projection) when experts see many rows, "small" (128x128 tiles, 256 threads) otherwise.
 #include <cstdlib>
+#include <type_traits>
 
 #include "ffn_common.hpp"
 
@@ -25,7 +26,7 @@ namespace moe355 {
 namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) void lds_void;
 typedef const __attribute__((address_space(1))) void gbl_void;
@@ -37,16 +38,16 @@ template <int BM_, int BN_, int WM_, int WN_, int NS_>
 struct Tile {
     static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_, NS = NS_;
     static constexpr int THREADS = WM * WN * kWave;
-    static constexpr int TM = BM / WM / 32;       // 32x32 MFMA tiles per wavefront along tokens
-    static constexpr int TN = BN / WN / 32;       // ... along weight rows
+    static constexpr int TM = BM / WM / 16;       // 16x16 MFMA tiles per wavefront along tokens
+    static constexpr int TN = BN / WN / 16;       // ... along weight rows
     static constexpr int ROWS_PER_PASS = THREADS / 8;
     static constexpr int RA = BM / ROWS_PER_PASS; // 16-byte loads per thread per slab, token tile
     static constexpr int RB = BN / ROWS_PER_PASS; // ... weight tile
     static constexpr int STAGE_BYTES = (BM + BN) * kRowBytes;
     static constexpr int LDS_BYTES = NS * STAGE_BYTES;
-    static_assert(TM >= 1 && TN >= 1 && RA >= 1 && RB >= 1, "tile too small for the wave grid");
-    static_assert(NS == 2 || NS == 3, "two or three LDS stages");
-    static_assert(RA <= 4 && RB <= 4, "a slab's loads are spread over the four k sub-steps");
+    static_assert(TM >= 2 && TM % 2 == 0 && TN >= 2 && TN % 2 == 0, "a wavefront's tile is split in token halves; SwiGLU pairs weight-row halves");
+    static_assert(RA >= 1 && RB >= 1, "tile too small for the workgroup");
+    static_assert(NS == 2, "two LDS stages");
 };
 
 // What one task needs, resolved to pointers.
@@ -85,11 +86,18 @@ __device__ __forceinline__ void store8(uint16_t* p, uint32_t lo, uint32_t hi, bo
     }
 }
 
-// PARTIAL: the row block holds fewer than BM rows; 32-row MFMA sub-tiles that lie entirely in the padding are
+// PARTIAL: the row block holds fewer than BM rows; 16-row MFMA sub-tiles that lie entirely in the padding are
 // skipped (their LDS reads too).  A separate instantiation keeps the full-tile loop free of branches.
+//
+// Loop structure.  A 64-wide slab is consumed in four units (k half s, token half h) of HM x TN MFMAs; the
+// fragments of the next unit are read from LDS under the MFMAs of the current one.  The one barrier per slab sits
+// before the last unit: by then every wavefront has read all of the slab's fragments, so the barrier both frees
+// this stage for the loads of slab kt+2 (issued right behind it) and publishes slab kt+1, whose first fragments
+// are read under the last unit's MFMAs.  The first and the last two slabs are peeled off so that the steady-state
+// loop is one basic block, which is what lets the scheduling hints hold.
 template <class T, bool PARTIAL>
 __device__ __forceinline__ void gemm_tile_impl(const TaskPtrs& p, unsigned char* smem) {
-    constexpr int BM = T::BM, BN = T::BN, TM = T::TM, TN = T::TN, NS = T::NS;
+    constexpr int BM = T::BM, BN = T::BN, TM = T::TM, TN = T::TN, HM = TM / 2;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / T::WN, wn = wave % T::WN;
     const int prow = tid >> 3;
@@ -123,150 +131,156 @@ __device__ __forceinline__ void gemm_tile_impl(const TaskPtrs& p, unsigned char*
         b_src[i] = base + (int64_t)col * p.K + chunk * 8;
     }
 
-    f32x16 acc[TM][TN];
+    f32x4 acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+            for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
 
     // One global_load_lds_dwordx4 per 8 rows and wavefront writes 1 KiB of consecutive LDS: lane l lands in
     // row (l >> 3), chunk slot (l & 7); the swizzle is applied on the global side (see `chunk`).
     const int wrow = __builtin_amdgcn_readfirstlane(prow & ~7);
     const int KT = p.K / kBK;
-    auto issue_part = [&](int kt, int part) {   // the loads of slab kt that belong to k sub-step `part`
-        unsigned char* sa = smem + (kt % NS) * T::STAGE_BYTES;
+    auto issue = [&](int kt) {
+        unsigned char* sa = smem + (kt & 1) * T::STAGE_BYTES;
         unsigned char* sb = sa + BM * kRowBytes;
         const int koff = kt * kBK;
 #pragma unroll
         for (int i = 0; i < T::RA; ++i)
-            if (i == part)
-                __builtin_amdgcn_global_load_lds((gbl_void*)(a_src[i] + koff),
-                                                 (lds_void*)(sa + (wrow + i * T::ROWS_PER_PASS) * kRowBytes), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gbl_void*)(a_src[i] + koff),
+                                             (lds_void*)(sa + (wrow + i * T::ROWS_PER_PASS) * kRowBytes), 16, 0, 0);
 #pragma unroll
         for (int i = 0; i < T::RB; ++i)
-            if (i == part)
-                __builtin_amdgcn_global_load_lds((gbl_void*)(b_src[i] + koff),
-                                                 (lds_void*)(sb + (wrow + i * T::ROWS_PER_PASS) * kRowBytes), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gbl_void*)(b_src[i] + koff),
+                                             (lds_void*)(sb + (wrow + i * T::ROWS_PER_PASS) * kRowBytes), 16, 0, 0);
     };
-    __syncthreads();                        // the previous task's last slab may still be being read
-#pragma unroll
-    for (int s = 0; s < NS - 1; ++s)
-        if (s < KT) {
-#pragma unroll
-            for (int part = 0; part < 4; ++part) issue_part(s, part);
-        }
+    __syncthreads();                        // the previous task may still be reading the stages
+    issue(0);
+    if (KT > 1) issue(1);
 
-    const int frow = lane & 31, fk = lane >> 5;
+    const int frow = lane & 15, fk = lane >> 4;
     const int sw = (frow >> 1) & 7;
-    // 32-row sub-tiles of this wavefront that contain at least one real row (wavefront-uniform)
-    const int tm_active = PARTIAL ? min(TM, max(0, (p.rows - wm * 32 * TM + 31) >> 5)) : TM;
-    int a_off[TM], b_off[TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i) a_off[i] = (wm * 32 * TM + i * 32 + frow) * kRowBytes;
-#pragma unroll
-    for (int j = 0; j < TN; ++j) b_off[j] = BM * kRowBytes + (wn * 32 * TN + j * 32 + frow) * kRowBytes;
+    // 16-row sub-tiles of this wavefront that contain at least one real row (wavefront-uniform)
+    const int ta = PARTIAL ? min(TM, max(0, (p.rows - wm * 16 * TM + 15) >> 4)) : TM;
+    const int a_base = (wm * 16 * TM + frow) * kRowBytes;
+    const int b_base = BM * kRowBytes + (wn * 16 * TN + frow) * kRowBytes;
 
-    bf16x8 af[2][TM], bfr[2][TN];
-    for (int kt = 0; kt < KT; ++kt) {
-        // this wavefront's share of slab kt has landed (with three stages one younger slab may be in flight)
-        if (NS == 2 || kt + 1 >= KT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(T::RA + T::RB) : "memory");
-        __syncthreads();                    // ... and everyone else's; the stage about to be refilled is free
-        const bool pre = kt + NS - 1 < KT;
-        const unsigned char* st = smem + (kt % NS) * T::STAGE_BYTES;
+    bf16x8 af[2][HM], bfr[2][TN];
+    auto read_a = [&](const unsigned char* st, int s, int h, int buf) {
+        const int c = ((s * 4 + fk) ^ sw) << 4;
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
-            if (!PARTIAL || i < tm_active) af[0][i] = *reinterpret_cast<const bf16x8*>(st + a_off[i] + ((fk ^ sw) << 4));
+        for (int i = 0; i < HM; ++i)
+            if (!PARTIAL || h * HM + i < ta)
+                af[buf][i] = *reinterpret_cast<const bf16x8*>(st + a_base + (h * HM + i) * 16 * kRowBytes + c);
+    };
+    auto read_b = [&](const unsigned char* st, int s, int buf) {
+        const int c = ((s * 4 + fk) ^ sw) << 4;
 #pragma unroll
-        for (int j = 0; j < TN; ++j) bfr[0][j] = *reinterpret_cast<const bf16x8*>(st + b_off[j] + ((fk ^ sw) << 4));
+        for (int j = 0; j < TN; ++j) bfr[buf][j] = *reinterpret_cast<const bf16x8*>(st + b_base + j * 16 * kRowBytes + c);
+    };
+    auto mfmas = [&](int h, int abuf, int bbuf) {
 #pragma unroll
-        for (int ks = 0; ks < kBK / 16; ++ks) {
-            const int cb = ks & 1, nb = cb ^ 1;
-            if (pre && ks < 2) {   // half of the next slab's loads in each of the first two sub-steps
-                issue_part(kt + NS - 1, 2 * ks);
-                issue_part(kt + NS - 1, 2 * ks + 1);
-            }
-            if (ks < 3) {
-                const int c = (((ks + 1) * 2 + fk) ^ sw) << 4;
+        for (int i = 0; i < HM; ++i) {
+            if (PARTIAL && h * HM + i >= ta) continue;
 #pragma unroll
-                for (int i = 0; i < TM; ++i)
-                    if (!PARTIAL || i < tm_active) af[nb][i] = *reinterpret_cast<const bf16x8*>(st + a_off[i] + c);
-#pragma unroll
-                for (int j = 0; j < TN; ++j) bfr[nb][j] = *reinterpret_cast<const bf16x8*>(st + b_off[j] + c);
-            }
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                if (PARTIAL && i >= tm_active) continue;
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cb][j], af[cb][i], acc[i][j], 0, 0, 0);
-            }
-            // instruction order inside the sub-step: one LDS read behind each of the first MFMAs, then (first two
-            // sub-steps) the global loads one MFMA apart, then the remaining MFMAs
-            if (!PARTIAL && ks < 3) {
-#pragma unroll
-                for (int n = 0; n < TM + TN; ++n) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                }
-            }
-            if (!PARTIAL && ks < 2) {
-#pragma unroll
-                for (int n = 0; n < (T::RA + T::RB + 1) / 2; ++n) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-                }
-            }
-            if (!PARTIAL) __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
+            for (int j = 0; j < TN; ++j)
+                acc[h * HM + i][j] =
+                    __builtin_amdgcn_mfma_f32_16x16x32_bf16(bfr[bbuf][j], af[abuf][i], acc[h * HM + i][j], 0, 0, 0);
         }
+    };
+    // instruction order inside a unit: behind every second MFMA one LDS read and (last unit) one global load
+    auto hints = [&](auto nds_c, auto nvm_c) {
+        constexpr int nds = decltype(nds_c)::value, nvm = decltype(nvm_c)::value;
+        if (PARTIAL) return;
+        constexpr int npair = nds > nvm ? nds : nvm;
+        constexpr int NM = HM * TN;
+#pragma unroll
+        for (int n = 0; n < npair; ++n) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            if (n < nds) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            if (n < nvm) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
+        if (NM > 2 * npair) __builtin_amdgcn_sched_group_barrier(0x008, NM - 2 * npair, 0);
+    };
+    constexpr int NLOADS = T::RA + T::RB;
+    typedef std::integral_constant<int, 0> Zero;
+
+    // slab 0 has landed when at most the loads of slab 1 are outstanding (loads return in issue order)
+    if (KT > 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NLOADS) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    read_a(smem, 0, 0, 0);
+    read_b(smem, 0, 0);
+    auto slab = [&](auto more_c, auto pre2_c, int kt) {
+        constexpr bool MORE = decltype(more_c)::value, PRE2 = decltype(pre2_c)::value;
+        const unsigned char* st = smem + (kt & 1) * T::STAGE_BYTES;
+        const unsigned char* sn = smem + ((kt + 1) & 1) * T::STAGE_BYTES;
+        read_a(st, 0, 1, 1);
+        mfmas(0, 0, 0);
+        hints(std::integral_constant<int, HM>{}, Zero{});
+        read_a(st, 1, 0, 0);
+        read_b(st, 1, 1);
+        mfmas(1, 1, 0);
+        hints(std::integral_constant<int, HM + TN>{}, Zero{});
+        read_a(st, 1, 1, 1);
+        mfmas(0, 0, 1);
+        hints(std::integral_constant<int, HM>{}, Zero{});
+        // every fragment of slab kt is in registers; this wavefront's share of slab kt+1 has landed
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (MORE) {
+            read_a(sn, 0, 0, 0);
+            read_b(sn, 0, 0);
+        }
+        if (PRE2) issue(kt + 2);
+        mfmas(1, 1, 1);
+        hints(std::integral_constant<int, MORE ? HM + TN : 0>{}, std::integral_constant<int, PRE2 ? NLOADS : 0>{});
+    };
+    int kt = 0;
+    for (; kt < KT - 2; ++kt) slab(std::true_type{}, std::true_type{}, kt);
+    if (KT > 1) {
+        slab(std::true_type{}, std::false_type{}, kt);
+        ++kt;
     }
+    slab(std::false_type{}, std::false_type{}, kt);
 
     // ---- epilogue ----
-    // acc[i][j][r]: token row = wm*32*TM + i*32 + (lane & 31);
-    //               weight row inside the 32-wide MFMA tile = 8*(r/4) + 4*(lane >> 5) + (r % 4)
+    // acc[i][j][r]: token row = wm*16*TM + i*16 + (lane & 15); weight row inside the 16-wide MFMA tile = 4*(lane >> 4) + r
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-        const int m = wm * 32 * TM + i * 32 + frow;
+        const int m = wm * 16 * TM + i * 16 + frow;
         if (m >= p.rows) continue;
         uint16_t* crow = p.c_base + (int64_t)m * p.N;
         if (p.swiglu) {
-            if constexpr (TN % 2 == 0) {
 #pragma unroll
-                for (int j = 0; j < TN / 2; ++j) {
+            for (int j = 0; j < TN / 2; ++j) {
+                const int col = p.n0 + wn * 8 * TN + j * 16 + 4 * fk;
+                if (col >= p.N) continue;
+                float v[4];
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const int col = p.n0 + wn * 16 * TN + j * 32 + 8 * q + 4 * fk;
-                        if (col >= p.N) continue;
-                        float v[4];
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) {
-                            float g = acc[i][j][4 * q + r], u = acc[i][j + TN / 2][4 * q + r];
-                            if (p.bias1) g = g + bf16_bits_to_f32(p.bias1[col + r]);
-                            if (p.bias0) u = u + bf16_bits_to_f32(p.bias0[col + r]);
-                            v[r] = silu_fast(g) * u;
-                        }
-                        store8(crow + col, pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]), p.publish);
-                    }
+                for (int r = 0; r < 4; ++r) {
+                    float g = acc[i][j][r], u = acc[i][j + TN / 2][r];
+                    if (p.bias1) g = g + bf16_bits_to_f32(p.bias1[col + r]);
+                    if (p.bias0) u = u + bf16_bits_to_f32(p.bias0[col + r]);
+                    v[r] = silu_fast(g) * u;
                 }
+                store8(crow + col, pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]), p.publish);
             }
         } else {
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
+                const int col = p.n0 + wn * 16 * TN + j * 16 + 4 * fk;
+                if (col >= p.N) continue;
+                float v[4];
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int col = p.n0 + wn * 32 * TN + j * 32 + 8 * q + 4 * fk;
-                    if (col >= p.N) continue;
-                    float v[4];
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        float u = acc[i][j][4 * q + r];
-                        if (p.bias0) u = u + bf16_bits_to_f32(p.bias0[col + r]);
-                        v[r] = act_apply(u, p.act);
-                    }
-                    store8(crow + col, pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]), p.publish);
+                for (int r = 0; r < 4; ++r) {
+                    float u = acc[i][j][r];
+                    if (p.bias0) u = u + bf16_bits_to_f32(p.bias0[col + r]);
+                    v[r] = act_apply(u, p.act);
                 }
+                store8(crow + col, pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]), p.publish);
             }
         }
     }
@@ -327,7 +341,6 @@ struct Plan {
     using T0 = T0_;
     using T1 = T1_;
     static_assert(T0::BM == T1::BM && T0::THREADS == T1::THREADS, "phases share row blocks and workgroup size");
-    static_assert(T0::TN % 2 == 0, "SwiGLU pairs column tiles inside a wavefront");
     static constexpr int THREADS = T0::THREADS;
     static constexpr int LDS_BYTES = T0::LDS_BYTES > T1::LDS_BYTES ? T0::LDS_BYTES : T1::LDS_BYTES;
 };

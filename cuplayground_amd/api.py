@@ -97,7 +97,7 @@ def load_library():
     L.moe_set_stage_timing.argtypes = [vp, C.c_int]
     L.moe_get_stage_ms.argtypes = [vp, C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_int32)]
     L.moe_get_task_counts.argtypes = [vp, vp, vp, C.POINTER(i64), C.POINTER(i64)]
-    L.moe_measure_mfma_tflops.argtypes = [vp, C.c_size_t, vp, C.POINTER(C.c_float)]
+    L.moe_measure_mfma_tflops.argtypes = [vp, C.c_size_t, vp, C.c_int, C.POINTER(C.c_float)]
     L.moe_measure_hbm_read_gbs.argtypes = [vp, C.c_size_t, vp, vp, C.POINTER(C.c_float)]
     L.moe_last_hip_error.argtypes = [vp]
     L.moe_status_string.argtypes = [C.c_int]; L.moe_status_string.restype = C.c_char_p
@@ -318,17 +318,18 @@ class MoELayer:
 
 
 def measured_peaks() -> dict:
-    """bf16 MFMA issue rate (TFLOP/s) and streaming read bandwidth (GB/s) measured on the current device."""
+    """bf16 MFMA issue rate (TFLOP/s; zero and random operands) and streaming read bandwidth (GB/s) of this device."""
     import torch
     L = load_library()
     buf = torch.zeros(2 << 30, dtype=torch.uint8, device="cuda")
     scratch = torch.zeros(4 << 20, dtype=torch.uint8, device="cuda")
-    tf, gb = C.c_float(0), C.c_float(0)
-    _check(L.moe_measure_mfma_tflops(_ptr(scratch), scratch.numel(), _stream(), C.byref(tf)), "moe_measure_mfma_tflops")
+    tf, tfr, gb = C.c_float(0), C.c_float(0), C.c_float(0)
+    _check(L.moe_measure_mfma_tflops(_ptr(scratch), scratch.numel(), _stream(), 0, C.byref(tf)), "moe_measure_mfma_tflops")
+    _check(L.moe_measure_mfma_tflops(_ptr(scratch), scratch.numel(), _stream(), 1, C.byref(tfr)), "moe_measure_mfma_tflops")
     _check(L.moe_measure_hbm_read_gbs(_ptr(buf), buf.numel(), _ptr(scratch), _stream(), C.byref(gb)),
            "moe_measure_hbm_read_gbs")
     del buf
-    return {"mfma_bf16_tflops": tf.value, "hbm_read_gbs": gb.value}
+    return {"mfma_bf16_tflops": tf.value, "mfma_bf16_tflops_random_operands": tfr.value, "hbm_read_gbs": gb.value}
 
 
 def gemm_bias_act(A, B, bias, act: int):

@@ -1,5 +1,5 @@
 // Measured ceilings of the device the library runs on, reported next to the published peaks: an MFMA
-// issue-only kernel (no memory traffic) and a streaming read.  The reference sizes its launches from a
+// issue-only kernel (no memory traffic; on zero and on random operands) and a streaming read.  The reference sizes its launches from a
 // hard-coded occupancy table (arch.cuh:22-69) and times kernels with %globaltimer (mma.cuh:51-57); here the
 // ceilings are measured with hipEvents on the caller's stream.
 #include "moe_internal.hpp"
@@ -8,24 +8,49 @@ namespace moe355 {
 namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-__global__ __launch_bounds__(256) void peak_mfma_kernel(float* out, int iters) {
-    bf16x8 a, b;
+__device__ __forceinline__ uint32_t mix32(uint32_t h) {
+    h ^= h >> 16; h *= 0x7feb352du; h ^= h >> 15; h *= 0x846ca68bu; h ^= h >> 16;
+    return h;
+}
+// two bf16 values with random sign, mantissa and an exponent in 2^-7 .. 2^-1
+__device__ __forceinline__ uint32_t random_bf16x2(uint32_t seed) {
+    const uint32_t h = mix32(seed), g = mix32(h);
+    const uint32_t lo = (h & 0x8000u) | ((120 + ((h >> 7) % 7)) << 7) | (h & 0x7F);
+    const uint32_t hi = (g & 0x8000u) | ((120 + ((g >> 7) % 7)) << 7) | (g & 0x7F);
+    return lo | (hi << 16);
+}
+
+// The FFN kernels' MFMA (v_mfma_f32_16x16x32_bf16) back to back on register operands, 16 independent accumulators.
+// random = 0: every operand register holds zero; random = 1: random bf16 operands.  The two differ by a quarter on
+// MI355X: with operands that toggle the datapaths the board runs into its power limit and lowers the clock.
+__global__ __launch_bounds__(512) void peak_mfma_kernel(float* out, int iters, int random) {
+    bf16x8 a[4], b[4];
 #pragma unroll
-    for (int v = 0; v < 8; ++v) { a[v] = (__bf16)(threadIdx.x * 0.001f + v); b[v] = (__bf16)(v * 0.5f); }
-    f32x16 c0 = {0}, c1 = {0}, c2 = {0}, c3 = {0};
-    for (int i = 0; i < iters; ++i) {
-        c0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c0, 0, 0, 0);
-        c1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c1, 0, 0, 0);
-        c2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c2, 0, 0, 0);
-        c3 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c3, 0, 0, 0);
+    for (int i = 0; i < 4; ++i) {
+        u32x4 v, w;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            v[q] = random ? random_bf16x2(threadIdx.x * 131 + i * 17 + q) : 0u;
+            w[q] = random ? random_bf16x2(threadIdx.x * 257 + i * 19 + q + 7777) : 0u;
+        }
+        a[i] = __builtin_bit_cast(bf16x8, v);
+        b[i] = __builtin_bit_cast(bf16x8, w);
+    }
+    f32x4 acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+            acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i & 3], b[(i >> 2) & 3], acc[i], 0, 0, 0);
     }
     float s = 0.0f;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) s += c0[r] + c1[r] + c2[r] + c3[r];
-    out[blockIdx.x * 256 + threadIdx.x] = s;
+    for (int i = 0; i < 16; ++i) s += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+    out[blockIdx.x * 512 + threadIdx.x] = s;
 }
 
 __global__ __launch_bounds__(256) void peak_read_kernel(const u32x4* __restrict__ src, size_t n, unsigned* out) {
@@ -50,19 +75,19 @@ using namespace moe355;
 extern "C" {
 
 // scratch: device buffer of at least 2 MiB (outputs of the MFMA kernel; only written).
-int moe_measure_mfma_tflops(void* scratch, size_t scratch_bytes, void* stream, float* tflops) {
+int moe_measure_mfma_tflops(void* scratch, size_t scratch_bytes, void* stream, int random_operands, float* tflops) {
     if (!scratch || !tflops || scratch_bytes < (size_t)2 << 20) return MOE_ERR_BAD_ARGUMENT;
     hipStream_t st = (hipStream_t)stream;
     int dev = 0;
     hipDeviceProp_t prop;
     if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return MOE_ERR_NO_DEVICE;
-    const int blocks = prop.multiProcessorCount * 2;   // two wavefronts per SIMD
-    const int iters = 8192;
+    const int blocks = prop.multiProcessorCount;       // 512 threads each: two wavefronts per SIMD
+    const int iters = 20000;                            // ~10 ms: long enough for the clock to settle
     hipEvent_t e0, e1;
     if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) return MOE_ERR_HIP;
-    peak_mfma_kernel<<<blocks, 256, 0, st>>>((float*)scratch, 64);
+    peak_mfma_kernel<<<blocks, 512, 0, st>>>((float*)scratch, iters, random_operands);
     (void)hipEventRecord(e0, st);
-    peak_mfma_kernel<<<blocks, 256, 0, st>>>((float*)scratch, iters);
+    peak_mfma_kernel<<<blocks, 512, 0, st>>>((float*)scratch, iters, random_operands);
     (void)hipEventRecord(e1, st);
     hipError_t rc = hipEventSynchronize(e1);
     float ms = 0.0f;
@@ -70,7 +95,7 @@ int moe_measure_mfma_tflops(void* scratch, size_t scratch_bytes, void* stream, f
     (void)hipEventDestroy(e0);
     (void)hipEventDestroy(e1);
     if (rc != hipSuccess || ms <= 0.0f) return MOE_ERR_HIP;
-    *tflops = (float)((double)blocks * 4 * iters * 4 * 32768.0 / (ms * 1e-3) / 1e12);
+    *tflops = (float)((double)blocks * 8 * iters * 16 * 16384.0 / (ms * 1e-3) / 1e12);
     return MOE_OK;
 }
 

@@ -178,10 +178,12 @@ int moe_get_stage_ms(moe_handle* h, int stage, float* ms, int32_t* calls);
 int moe_get_task_counts(moe_handle* h, const void* workspace, void* stream, int64_t* gemm0_tasks, int64_t* gemm1_tasks);
 
 /* Ceilings measured on the current device, to be quoted beside the published peaks: bf16 MFMA issue rate with no
- * memory traffic (scratch: >= 2 MiB of device memory, overwritten), and streaming read bandwidth over `bytes` bytes
+ * memory traffic (scratch: >= 2 MiB of device memory, overwritten; random_operands = 0: all-zero operands, the
+ * clock stays at its maximum; 1: random bf16 operands, the board's power limit lowers the clock -- this is the
+ * ceiling a GEMM on real data can approach), and streaming read bandwidth over `bytes` bytes
  * of `src` (>= 1 GiB, so the caches cannot serve it).  Both synchronise the stream.  No counterpart in the reference,
  * whose launch sizing is a hard-coded table (arch.cuh:22-69). */
-int moe_measure_mfma_tflops(void* scratch, size_t scratch_bytes, void* stream, float* tflops);
+int moe_measure_mfma_tflops(void* scratch, size_t scratch_bytes, void* stream, int random_operands, float* tflops);
 int moe_measure_hbm_read_gbs(const void* src, size_t bytes, void* scratch, void* stream, float* gbs);
 
 int moe_last_hip_error(const moe_handle* h);

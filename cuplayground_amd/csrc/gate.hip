@@ -29,7 +29,7 @@ __device__ __forceinline__ void load8(const uint16_t* p, float (&v)[8]) {
 
 // A wavefront keeps TPW token rows in registers (lane l owns the 8-element chunks l, l+64, ... of each row, as
 // fp32) and walks over its share of the experts: one 16-byte load of the expert's row per chunk feeds 8*TPW
-// fmafs.  grid = (token groups of 4*TPW, expert chunks); NCH = chunks per lane = ceil(H / 512).
+// fmafs; the 64 partial sums of 16 (token, expert) pairs are folded together (see the loop).  grid = (token groups of 4*TPW, expert chunks); NCH = chunks per lane = ceil(H / 512).
 template <typename T, int NCH, int TPW>
 __global__ __launch_bounds__(256) void gate_logits_kernel(const T* __restrict__ x, const T* __restrict__ gate_w,
                                                           const float* __restrict__ gate_bias,
@@ -67,42 +67,64 @@ __global__ __launch_bounds__(256) void gate_logits_kernel(const T* __restrict__ 
         }
     };
     fetch(e0);
-    for (int e = e0; e < e1; ++e) {
-        raw_t wc[NCH];
+    // Experts are taken EG at a time so that EG * TPW = 16 partial-sum registers are folded together: at xor
+    // distance 32, 16, 8, 4 a lane keeps one register of each pair and hands the other to its partner, which
+    // halves the registers per step instead of running six shuffles per sum.  Every sum still adds lane l to
+    // lane l ^ d for d = 32, 16, 8, 4, 2, 1 in that order, so the result is bit-identical to the plain butterfly.
+    constexpr int EG = 16 / TPW;
+    for (int eb = e0; eb < e1; eb += EG) {
+        float red[16];
 #pragma unroll
-        for (int j = 0; j < NCH; ++j) wc[j] = wn[j];
-        if (e + 1 < e1) fetch(e + 1);
-        float acc[TPW];
+        for (int r = 0; r < 16; ++r) red[r] = 0.0f;
 #pragma unroll
-        for (int q = 0; q < TPW; ++q) acc[q] = 0.0f;
+        for (int g = 0; g < EG; ++g) {
+            const int e = eb + g;
+            if (e >= e1) break;
+            raw_t wc[NCH];
 #pragma unroll
-        for (int j = 0; j < NCH; ++j) {
-            const int c = lane + j * kWave;
-            if (c < nchunk) {
-                float wv[8];
-                if constexpr (sizeof(T) == 4) {
+            for (int j = 0; j < NCH; ++j) wc[j] = wn[j];
+            if (e + 1 < e1) fetch(e + 1);
 #pragma unroll
-                    for (int v = 0; v < 8; ++v) wv[v] = __uint_as_float(wc[j][v]);
-                } else {
+            for (int j = 0; j < NCH; ++j) {
+                const int c = lane + j * kWave;
+                if (c < nchunk) {
+                    float wv[8];
+                    if constexpr (sizeof(T) == 4) {
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) {
-                        wv[2 * v] = __uint_as_float(wc[j][v] << 16);
-                        wv[2 * v + 1] = __uint_as_float(wc[j][v] & 0xFFFF0000u);
+                        for (int v = 0; v < 8; ++v) wv[v] = __uint_as_float(wc[j][v]);
+                    } else {
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) {
+                            wv[2 * v] = __uint_as_float(wc[j][v] << 16);
+                            wv[2 * v + 1] = __uint_as_float(wc[j][v] & 0xFFFF0000u);
+                        }
                     }
+#pragma unroll
+                    for (int q = 0; q < TPW; ++q)
+#pragma unroll
+                        for (int v = 0; v < 8; ++v)
+                            red[g * TPW + q] = __builtin_fmaf(xr[q][j][v], wv[v], red[g * TPW + q]);
                 }
-#pragma unroll
-                for (int q = 0; q < TPW; ++q)
-#pragma unroll
-                    for (int v = 0; v < 8; ++v) acc[q] = __builtin_fmaf(xr[q][j][v], wv[v], acc[q]);
             }
         }
 #pragma unroll
-        for (int q = 0; q < TPW; ++q) {
-            float r = acc[q];
+        for (int step = 0; step < 4; ++step) {
+            const int off = 32 >> step, n = 16 >> step;
+            const bool hi = (lane & off) != 0;
 #pragma unroll
-            for (int off = 32; off >= 1; off >>= 1) r = r + __shfl_xor(r, off, kWave);
-            if (lane == 0 && t0 + q < S) logits[(size_t)(t0 + q) * E + e] = gate_bias ? r + gate_bias[e] : r;
+            for (int i = 0; i < n / 2; ++i) {
+                const float keep = hi ? red[2 * i + 1] : red[2 * i];
+                const float send = hi ? red[2 * i] : red[2 * i + 1];
+                red[i] = keep + __shfl_xor(send, off, kWave);
+            }
         }
+        float sum = red[0];
+        sum = sum + __shfl_xor(sum, 2, kWave);
+        sum = sum + __shfl_xor(sum, 1, kWave);
+        // the lane's register index: bit 0 came from lane bit 5, bit 1 from bit 4, bit 2 from bit 3, bit 3 from bit 2
+        const int r = ((lane >> 5) & 1) | (((lane >> 4) & 1) << 1) | (((lane >> 3) & 1) << 2) | (((lane >> 2) & 1) << 3);
+        const int e = eb + r / TPW, t = t0 + r % TPW;
+        if ((lane & 3) == 0 && e < e1 && t < S) logits[(size_t)t * E + e] = gate_bias ? sum + gate_bias[e] : sum;
     }
 }
 

@@ -123,3 +123,17 @@ def test_null_arguments_are_errors_not_crashes():
     assert L.moe_destroy(None) == 0
     assert L.moe_forward(None, None, None, None, None, None, 0, None) == 4
     assert L.moe_gemm_bias_act(None, None, None, None, 1, 1, 1, 0, 0, None) == 4
+
+
+def test_torch_operator_has_no_cpu_path():
+    """The operator is declared for CUDA (and meta) only: CPU tensors must be refused by the dispatcher."""
+    import torch
+    import cuplayground_amd.torch_op  # noqa: F401  (registers torch.ops.moe355.forward)
+    x = torch.zeros(128, 64)
+    w = torch.zeros(2, 64)
+    e = torch.zeros(2, 64, 64)
+    cfg = '{"hidden_size": 64, "intermediate_size": 64, "num_experts": 2, "sequence_len": 128, "micro_batch": 1}'
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        torch.ops.moe355.forward(x, w, e, None, e, cfg)
+    m = torch.ops.moe355.forward(x.to("meta"), w.to("meta"), e.to("meta"), None, e.to("meta"), cfg)
+    assert m.shape == x.shape

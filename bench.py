@@ -37,6 +37,7 @@ def workloads():
 def make_device_inputs(cfg, seed):
     """Synthetic operands generated on the GPU: tokens N(0,1), weights N(0,0.02), rounded to storage."""
     import torch
+    import cuplayground_amd as moe
     from oracle import binding as ob
     g = torch.Generator(device="cuda").manual_seed(seed)
     adt = torch.float32 if cfg.dtype == ob.F32 else torch.bfloat16
@@ -58,14 +59,8 @@ def make_device_inputs(cfg, seed):
         shape = (E, H, I) if n == "w_down" else (E, I, H)
         if cfg.dtype == ob.FP8:
             w = normal(shape, 0.02, torch.float32)
-            N, K = shape[1], shape[2]
-            blocks = w.view(E, N // 128, 128, K // 128, 128)
-            s = blocks.abs().amax(dim=(2, 4)) / 448.0
-            s = torch.where(s > 0, s, torch.ones_like(s))
-            q = (blocks / s[:, :, None, :, None]).reshape(shape).to(torch.float8_e4m3fn)
-            d[n] = q.view(torch.uint8)
-            d["s_" + n[2:]] = s.contiguous()
-            del w, blocks, q
+            d[n], d["s_" + n[2:]] = moe.quantize_block128(w)   # e4m3 codes + one scale per 128x128 block
+            del w
         else:
             d[n] = normal(shape, 0.02, adt)
     return d

@@ -13,4 +13,5 @@ from .api import (  # noqa: F401
     library_path,
     load_library,
     measured_peaks,
+    quantize_block128,
 )

@@ -26,7 +26,7 @@ EXPORTS = (
     "moe_workspace_bytes",
     "moe_set_ffn_mode", "moe_get_ffn_mode", "moe_forward", "moe_gate", "moe_route", "moe_gemm_bias_act", "moe_combine",
     "moe_set_stage_timing", "moe_get_stage_ms", "moe_get_task_counts", "moe_measure_mfma_tflops",
-    "moe_measure_hbm_read_gbs", "moe_last_hip_error", "moe_status_string",
+    "moe_measure_hbm_read_gbs", "moe_quant_block128", "moe_last_hip_error", "moe_status_string",
     "moe_version",
 )
 
@@ -97,6 +97,7 @@ def load_library():
     L.moe_set_stage_timing.argtypes = [vp, C.c_int]
     L.moe_get_stage_ms.argtypes = [vp, C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_int32)]
     L.moe_get_task_counts.argtypes = [vp, vp, vp, C.POINTER(i64), C.POINTER(i64)]
+    L.moe_quant_block128.argtypes = [vp, C.c_int32, C.c_int64, C.c_int64, C.c_int64, vp, vp, vp]
     L.moe_measure_mfma_tflops.argtypes = [vp, C.c_size_t, vp, C.c_int, C.POINTER(C.c_float)]
     L.moe_measure_hbm_read_gbs.argtypes = [vp, C.c_size_t, vp, vp, C.POINTER(C.c_float)]
     L.moe_last_hip_error.argtypes = [vp]
@@ -330,6 +331,22 @@ def measured_peaks() -> dict:
            "moe_measure_hbm_read_gbs")
     del buf
     return {"mfma_bf16_tflops": tf.value, "mfma_bf16_tflops_random_operands": tfr.value, "hbm_read_gbs": gb.value}
+
+
+def quantize_block128(w):
+    """[.., N, K] fp32/bf16 weights on the GPU -> (uint8 e4m3 codes of the same shape, fp32 scales [.., N/128, K/128])."""
+    import torch
+    N, K = w.shape[-2], w.shape[-1]
+    mats = w.numel() // (N * K)
+    w = w.contiguous()
+    q = torch.empty(w.shape, dtype=torch.uint8, device=w.device)
+    s = torch.empty(*w.shape[:-2], N // 128, K // 128, dtype=torch.float32, device=w.device)
+    dtype = DTYPE_F32 if w.dtype == torch.float32 else DTYPE_BF16
+    if w.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("quantize_block128 takes fp32 or bf16 weights")
+    _check(load_library().moe_quant_block128(_ptr(w), dtype, mats, N, K, _ptr(q), _ptr(s), _stream()),
+           "moe_quant_block128")
+    return q, s
 
 
 def gemm_bias_act(A, B, bias, act: int):

@@ -186,6 +186,13 @@ int moe_get_task_counts(moe_handle* h, const void* workspace, void* stream, int6
 int moe_measure_mfma_tflops(void* scratch, size_t scratch_bytes, void* stream, int random_operands, float* tflops);
 int moe_measure_hbm_read_gbs(const void* src, size_t bytes, void* scratch, void* stream, float* gbs);
 
+/* Weight preparation for torch_dtype = 4: `matrices` row-major [N,K] matrices (fp32 or bf16; N and K multiples of
+ * 128) become OCP e4m3 bytes q[matrices,N,K] plus one fp32 scale per 128x128 block, scales[matrices,N/128,K/128]:
+ * scale = amax/448 (1 for an all-zero block), q = e4m3(w/scale) rounded to nearest even, saturating.  Asynchronous on
+ * `stream`.  No counterpart in the reference, whose dtypes stop at fp16 (aristos_config.schema.json:49-53). */
+int moe_quant_block128(const void* w, int32_t src_dtype, int64_t matrices, int64_t N, int64_t K, void* q,
+                       float* scales, void* stream);
+
 int moe_last_hip_error(const moe_handle* h);
 const char* moe_status_string(int status);
 int moe_version(void);

@@ -190,3 +190,30 @@ def test_full_size_routing_matches_golden_digests(moe, name):
     assert np.array_equal(from_device(r["token_indices"]), want["token_indices"])
     assert np.abs(from_device(w) - want["topk_w"]).max() <= 2e-6
     layer.close()
+
+
+@pytest.mark.parametrize("src", ["f32", "bf16"])
+def test_quant_block128_bit_exact(moe, src):
+    """The GPU quantiser against the oracle's, codes and scales bit for bit, including the awkward values."""
+    import torch
+    rng = np.random.default_rng(17)
+    w = (rng.standard_normal((3, 256, 384)) * 0.02).astype(np.float32)
+    w[0, :128, :128] = 0.0                                   # an all-zero block: scale 1, codes 0
+    w[1, 5, 7] = 3.0                                         # one dominant value: the rest lands in the subnormals
+    w[1, 130, 200] = -np.float32(1e-30)
+    w[2, :128, 128:256] *= np.float32(1e-20)                 # tiny magnitudes, still scaled to the full range
+    # exact ties of the 3-bit mantissa after scaling by 1/448 * 448 = 1: block maximum 448 keeps scale 1
+    w[2, 128:, 256:] = 0.0
+    w[2, 128, 256] = 448.0
+    w[2, 129, 256:264] = np.array([1.0625, 1.1875, 17.0, 19.0, 0.0009765625, 0.0029296875, 447.9, 464.0], np.float32)
+    if src == "bf16":
+        bits = ob.f32_to_bf16(w)
+        w = ob.bf16_to_f32(bits)
+        dev = to_device(bits, "bf16")
+    else:
+        dev = to_device(w, "f32")
+    want_q, want_s = ob.quant_block128(w)
+    q, s = moe.quantize_block128(dev)
+    torch.cuda.synchronize()
+    assert np.array_equal(s.cpu().numpy().view(np.uint32), want_s.view(np.uint32))
+    assert np.array_equal(q.cpu().numpy(), want_q)

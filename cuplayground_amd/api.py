@@ -24,7 +24,7 @@ EXPORTS = (
     "moe_config_default", "moe_config_from_json_string", "moe_config_from_json_file", "moe_config_validate",
     "moe_config_tokens", "moe_config_capacity", "moe_create", "moe_destroy", "moe_get_arch", "moe_get_plan",
     "moe_workspace_bytes",
-    "moe_set_ffn_mode", "moe_get_ffn_mode", "moe_forward", "moe_gate", "moe_route", "moe_gemm_bias_act", "moe_combine",
+    "moe_set_ffn_mode", "moe_get_ffn_mode", "moe_forward", "moe_gate", "moe_router_stats", "moe_route", "moe_gemm_bias_act", "moe_combine",
     "moe_set_stage_timing", "moe_get_stage_ms", "moe_get_task_counts", "moe_measure_mfma_tflops",
     "moe_measure_hbm_read_gbs", "moe_quant_block128", "moe_last_hip_error", "moe_status_string",
     "moe_version",
@@ -90,6 +90,7 @@ def load_library():
     L.moe_set_ffn_mode.argtypes = [vp, C.c_int]
     L.moe_get_ffn_mode.argtypes = [vp, C.POINTER(C.c_int32)]
     L.moe_forward.argtypes = [vp, vp, C.POINTER(_CWeights), vp, C.POINTER(_CRouting), vp, C.c_size_t, vp]
+    L.moe_router_stats.argtypes = [vp, vp, vp, vp, vp, vp, vp, C.c_size_t, vp]
     L.moe_gate.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, C.c_size_t, vp]
     L.moe_route.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, C.c_size_t, vp]
     L.moe_gemm_bias_act.argtypes = [vp, vp, vp, vp, i64, i64, i64, i32, i32, vp]
@@ -302,6 +303,18 @@ class MoELayer:
         _check(self.L.moe_gate(self._h, _ptr(x), _ptr(gate_w), _ptr(gate_bias), _ptr(logits), _ptr(idx), _ptr(wts),
                                _ptr(self.workspace), self.workspace_bytes, _stream()), "moe_gate")
         return (idx, wts, logits) if want_logits else (idx, wts)
+
+    def router_stats(self, logits, topk_idx) -> dict:
+        """load[E], mean_prob[E] and aux_loss (a 1-element tensor) from the router's logits and choices."""
+        import torch
+        dev = logits.device
+        out = dict(load=torch.empty(self.E, dtype=torch.float32, device=dev),
+                   mean_prob=torch.empty(self.E, dtype=torch.float32, device=dev),
+                   aux_loss=torch.empty(1, dtype=torch.float32, device=dev))
+        _check(self.L.moe_router_stats(self._h, _ptr(logits), _ptr(topk_idx), _ptr(out["load"]), _ptr(out["mean_prob"]),
+                                       _ptr(out["aux_loss"]), _ptr(self.workspace), self.workspace_bytes, _stream()),
+               "moe_router_stats")
+        return out
 
     def route(self, topk_idx):
         import torch

@@ -49,7 +49,7 @@ struct Derived {
 
 struct WsLayout {
     size_t logits, topk_idx, topk_w, slot, pair_row, token_indices, expert_count, expert_offset, rank_local,
-        block_hist, mtiles, seg0, seg1, segq, qstate, done0, h, y, total;
+        block_hist, mtiles, seg0, seg1, segq, qstate, done0, stats_prob, stats_cnt, h, y, total;
 };
 
 int check_supported(const moe_config& c) {
@@ -103,6 +103,8 @@ WsLayout layout(const Derived& d) {
     w.segq = take((size_t)2 * d.E * sizeof(Segment));
     w.qstate = take(sizeof(QueueState));
     w.done0 = take((size_t)d.max_mtiles * 4);
+    w.stats_prob = take((size_t)kStatsBlocks * d.E * 8);
+    w.stats_cnt = take((size_t)kStatsBlocks * d.E * 4);
     w.h = take((size_t)d.A * d.I * d.act_bytes);
     w.y = take((size_t)d.A * d.H * d.act_bytes);
     w.total = off;
@@ -355,6 +357,19 @@ int moe_gate(moe_handle* h, const void* x, const void* gate_w, const float* gate
     e = launch_topk(lg, d.S, d.E, d.k, h->cfg.gate_fn, h->cfg.norm_topk_prob, topk_idx, topk_w, st);
     if (e != hipSuccess) return hip_fail(h, e);
     return MOE_OK;
+}
+
+int moe_router_stats(moe_handle* h, const float* logits, const int32_t* topk_idx, float* load, float* mean_prob,
+                     float* aux_loss, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!h || !logits || !topk_idx || (!load && !mean_prob && !aux_loss)) return MOE_ERR_BAD_ARGUMENT;
+    int rc = check_ws(h, workspace, workspace_bytes);
+    if (rc) return rc;
+    const Derived& d = h->d;
+    const hipError_t e = launch_router_stats(logits, topk_idx, d.S, d.E, d.k, h->cfg.gate_fn,
+                                             at<double>(workspace, h->ws.stats_prob),
+                                             at<int32_t>(workspace, h->ws.stats_cnt), load, mean_prob, aux_loss,
+                                             (hipStream_t)stream);
+    return e == hipSuccess ? MOE_OK : hip_fail(h, e);
 }
 
 int moe_route(moe_handle* h, const int32_t* topk_idx, int32_t* slot, int32_t* expert_count, int32_t* expert_offset,

@@ -230,7 +230,98 @@ __global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ log
     }
 }
 
+// Router statistics for a load-balancing loss.  Block b, wavefront w takes tokens (4b + w) + 4*gridDim.x*i; a lane
+// keeps fp64 sums of the gate scores of its experts; wavefront sums meet in LDS in wavefront order and are written as
+// per-block partials, so the result does not depend on scheduling.
+__global__ __launch_bounds__(256) void router_stats_partial_kernel(const float* __restrict__ logits,
+                                                                   const int32_t* __restrict__ topk_idx, int S, int E,
+                                                                   int k, int gate_fn, double* __restrict__ part_prob,
+                                                                   int32_t* __restrict__ part_cnt) {
+    __shared__ double s_sum[4][kMaxExperts];
+    __shared__ int s_cnt[kMaxExperts];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    constexpr int J = kMaxExperts / kWave;
+    for (int e = threadIdx.x; e < E; e += 256) s_cnt[e] = 0;
+    __syncthreads();
+    double acc[J];
+#pragma unroll
+    for (int j = 0; j < J; ++j) acc[j] = 0.0;
+    for (int t = blockIdx.x * 4 + wave; t < S; t += 4 * gridDim.x) {
+        float v[J];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            const int e = j * kWave + lane;
+            v[j] = e < E ? logits[(size_t)t * E + e] : -INFINITY;
+            mx = fmaxf(mx, v[j]);
+        }
+        if (gate_fn == MOE_GATE_SOFTMAX) {
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, kWave));
+            float part = 0.0f;
+#pragma unroll
+            for (int j = 0; j < J; ++j) {
+                v[j] = j * kWave + lane < E ? expf(v[j] - mx) : 0.0f;
+                part = part + v[j];
+            }
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) part = part + __shfl_xor(part, off, kWave);
+#pragma unroll
+            for (int j = 0; j < J; ++j) acc[j] += (double)(v[j] / part);
+        } else {
+#pragma unroll
+            for (int j = 0; j < J; ++j)
+                if (j * kWave + lane < E) acc[j] += (double)(1.0f / (1.0f + expf(-v[j])));
+        }
+        if (lane < k) atomicAdd(&s_cnt[topk_idx[(size_t)t * k + lane]], 1);
+    }
+#pragma unroll
+    for (int j = 0; j < J; ++j)
+        if (j * kWave + lane < E) s_sum[wave][j * kWave + lane] = acc[j];
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += 256) {
+        part_prob[(size_t)blockIdx.x * E + e] = ((s_sum[0][e] + s_sum[1][e]) + s_sum[2][e]) + s_sum[3][e];
+        part_cnt[(size_t)blockIdx.x * E + e] = s_cnt[e];
+    }
+}
+
+__global__ __launch_bounds__(512) void router_stats_final_kernel(const double* __restrict__ part_prob,
+                                                                 const int32_t* __restrict__ part_cnt, int blocks,
+                                                                 int S, int E, int k, float* __restrict__ load,
+                                                                 float* __restrict__ mean_prob,
+                                                                 float* __restrict__ aux_loss) {
+    __shared__ double s_prod[kMaxExperts];
+    const int e = threadIdx.x;
+    if (e < E) {
+        double sum = 0.0;
+        long long cnt = 0;
+        for (int b = 0; b < blocks; ++b) {
+            sum += part_prob[(size_t)b * E + e];
+            cnt += part_cnt[(size_t)b * E + e];
+        }
+        const double mp = sum / (double)S, ld = (double)cnt / ((double)S * (double)k);
+        if (mean_prob) mean_prob[e] = (float)mp;
+        if (load) load[e] = (float)ld;
+        s_prod[e] = mp * ld;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0 && aux_loss) {
+        double a = 0.0;
+        for (int i = 0; i < E; ++i) a += s_prod[i];
+        *aux_loss = (float)((double)E * a);
+    }
+}
+
 }  // namespace
+
+hipError_t launch_router_stats(const float* logits, const int32_t* topk_idx, int S, int E, int k, int gate_fn,
+                               double* part_prob, int32_t* part_cnt, float* load, float* mean_prob, float* aux_loss,
+                               hipStream_t st) {
+    const int blocks = min(kStatsBlocks, (S + 3) / 4);
+    router_stats_partial_kernel<<<blocks, 256, 0, st>>>(logits, topk_idx, S, E, k, gate_fn, part_prob, part_cnt);
+    router_stats_final_kernel<<<1, 512, 0, st>>>(part_prob, part_cnt, blocks, S, E, k, load, mean_prob, aux_loss);
+    return hipGetLastError();
+}
 
 hipError_t launch_gate_logits(const void* x, const void* gate_w, const float* gate_bias, float* logits, int S, int H,
                               int E, int act_dtype, hipStream_t st) {

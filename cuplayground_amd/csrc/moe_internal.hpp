@@ -100,6 +100,10 @@ hipError_t launch_gate_logits(const void* x, const void* gate_w, const float* ga
                               int E, int act_dtype, hipStream_t st);
 hipError_t launch_topk(const float* logits, int S, int E, int k, int gate_fn, int norm, int32_t* topk_idx,
                        float* topk_w, hipStream_t st);
+constexpr int kStatsBlocks = 64;   // per-block partials of the router statistics kept in the workspace
+hipError_t launch_router_stats(const float* logits, const int32_t* topk_idx, int S, int E, int k, int gate_fn,
+                               double* part_prob, int32_t* part_cnt, float* load, float* mean_prob, float* aux_loss,
+                               hipStream_t st);
 hipError_t launch_route(const RouteArgs& a, hipStream_t st);
 hipError_t launch_combine(const void* y_rows, const int32_t* pair_row, const float* topk_w, int S, int k, int H,
                           int act_dtype, void* out, hipStream_t st);

@@ -149,6 +149,15 @@ int moe_forward(moe_handle* h, const void* x, const moe_weights* w, void* out, c
 int moe_gate(moe_handle* h, const void* x, const void* gate_w, const float* gate_bias,
              float* logits, int32_t* topk_idx, float* topk_w, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Router statistics for a load-balancing loss (the training knob is_training, aristos_config.schema.json:20-23, has no
+ * consumer in the reference).  From the fp32 logits [S,E] and topk_idx [S,k] that moe_gate returned:
+ *   load[e]      = share of the S*k assignments the router gave expert e, before any capacity drop;
+ *   mean_prob[e] = mean over tokens of expert e's gate score (softmax probability over all E, or sigmoid);
+ *   aux_loss     = E * sum_e load[e] * mean_prob[e]   (1 for a uniform router).
+ * Sums run in fp64 in a fixed order (reproducible); any of the three outputs may be NULL. */
+int moe_router_stats(moe_handle* h, const float* logits, const int32_t* topk_idx, float* load, float* mean_prob,
+                     float* aux_loss, void* workspace, size_t workspace_bytes, void* stream);
+
 /* Slot assignment + capacity drop from topk_idx; the producer of the tokenIndices[] that the reference's
  * combine consumes (combine.cuh:115,134).  pair_row may be NULL. */
 int moe_route(moe_handle* h, const int32_t* topk_idx, int32_t* slot, int32_t* expert_count, int32_t* expert_offset,

@@ -67,6 +67,7 @@ def lib():
         L.orc_capacity.argtypes = [C.c_double, i64, i64, i64, C.POINTER(i64)]
         L.orc_gate_logits.argtypes = [vp, vp, vp, i32, i32, i32, i32, vp]
         L.orc_topk.argtypes = [vp, i32, i32, i32, i32, i32, vp, vp]
+        L.orc_router_stats.argtypes = [vp, vp, i32, i32, i32, i32, vp, vp, vp]
         L.orc_route.argtypes = [vp, i32, i32, i32, i32, i64, vp, vp, vp, vp, vp]
         L.orc_gemm_bias_act.argtypes = [vp, vp, vp, vp, i64, i64, i64, i32, i32]
         L.orc_ffn_rows.argtypes = [C.POINTER(_Cfg), vp, C.POINTER(_Weights), vp, vp, i64, vp]
@@ -259,6 +260,15 @@ def topk(logits, k, gate_fn, norm_topk):
     idx = np.empty((S, k), np.int32); w = np.empty((S, k), np.float32)
     lib().orc_topk(_p(logits), S, E, k, gate_fn, norm_topk, _p(idx), _p(w))
     return idx, w
+
+
+def router_stats(logits, topk_idx, gate_fn):
+    logits = _c(logits, np.float32); topk_idx = _c(topk_idx, np.int32)
+    S, E = logits.shape
+    k = topk_idx.shape[1]
+    load = np.empty(E, np.float32); mp = np.empty(E, np.float32); aux = np.empty(1, np.float32)
+    lib().orc_router_stats(_p(logits), _p(topk_idx), S, E, k, gate_fn, _p(load), _p(mp), _p(aux))
+    return dict(load=load, mean_prob=mp, aux_loss=float(aux[0]))
 
 
 def route_slots(topk_idx, E, drop, capacity):

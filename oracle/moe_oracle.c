@@ -286,6 +286,41 @@ void orc_topk(const float* logits, int32_t S, int32_t E, int32_t k, int32_t gate
 }
 
 /* ------------------------------------------------------------------------------------------------
+ * Router statistics for a load-balancing loss.  Build-defined: the reference parses is_training
+ * (aristos_config.schema.json:20-23) and never reads it.  load[e] = assignments to expert e / (S*k) before
+ * any drop; mean_prob[e] = mean over tokens of expert e's gate score (fp32 softmax over all E, or sigmoid),
+ * summed in fp64 in ascending token order; aux_loss = E * sum_e load[e]*mean_prob[e].
+ * ---------------------------------------------------------------------------------------------- */
+void orc_router_stats(const float* logits, const int32_t* topk_idx, int32_t S, int32_t E, int32_t k, int32_t gate_fn,
+                      float* load, float* mean_prob, float* aux_loss) {
+    double* sum = (double*)calloc((size_t)E, sizeof(double));
+    int64_t* cnt = (int64_t*)calloc((size_t)E, sizeof(int64_t));
+    for (int32_t t = 0; t < S; ++t) {
+        const float* l = logits + (int64_t)t * E;
+        if (gate_fn == ORC_GATE_SOFTMAX) {
+            float m = l[0];
+            for (int32_t e = 1; e < E; ++e) if (l[e] > m) m = l[e];
+            float denom = 0.0f;
+            for (int32_t e = 0; e < E; ++e) denom = denom + expf(l[e] - m);
+            for (int32_t e = 0; e < E; ++e) sum[e] += (double)(expf(l[e] - m) / denom);
+        } else {
+            for (int32_t e = 0; e < E; ++e) sum[e] += (double)(1.0f / (1.0f + expf(-l[e])));
+        }
+        for (int32_t r = 0; r < k; ++r) cnt[topk_idx[(int64_t)t * k + r]] += 1;
+    }
+    double aux = 0.0;
+    for (int32_t e = 0; e < E; ++e) {
+        const double mp = sum[e] / (double)S, ld = (double)cnt[e] / ((double)S * (double)k);
+        if (mean_prob) mean_prob[e] = (float)mp;
+        if (load) load[e] = (float)ld;
+        aux += mp * ld;
+    }
+    if (aux_loss) *aux_loss = (float)((double)E * aux);
+    free(sum);
+    free(cnt);
+}
+
+/* ------------------------------------------------------------------------------------------------
  * Slot assignment and capacity drop.  The reference only shows the consumer side: a tile of expert rows
  * carries tokenIndices[] and a valid-row count (combine.cuh:115,121-122,134,170).  Build-defined producer:
  * pairs are numbered p = t*k + r; slot[p] = number of earlier pairs routed to the same expert (a stable

@@ -13,6 +13,8 @@
  *   - orc_gate_logits          pinned against float64 dot products (value) and against a pure-Python
  *                              restatement of the summation order (bit pattern)
  *   - orc_topk                 pinned by brute-force full sorts with key (score desc, index asc)
+ *   - orc_router_stats         pinned by closed forms (uniform router: 1/E, 1/E, loss 1; one-hot router) and
+ *                              a float64 numpy restatement
  *   - orc_route                pinned by a stable sort of the flattened expert ids and by its invariants
  *   - orc_combine              pinned by the reference driver's identity case (combine.cuh:220-231),
  *                              permutation and linearity properties
@@ -81,6 +83,8 @@ void orc_gate_logits(const void* x, const void* gate_w, const float* gate_bias,
                      int32_t S, int32_t H, int32_t E, int32_t act_dtype, float* logits);
 void orc_topk(const float* logits, int32_t S, int32_t E, int32_t k, int32_t gate_fn, int32_t norm_topk,
               int32_t* topk_idx, float* topk_w);
+void orc_router_stats(const float* logits, const int32_t* topk_idx, int32_t S, int32_t E, int32_t k, int32_t gate_fn,
+                      float* load, float* mean_prob, float* aux_loss);
 void orc_route(const int32_t* topk_idx, int32_t S, int32_t k, int32_t E, int32_t drop, int64_t capacity,
                int32_t* slot, int32_t* expert_count, int32_t* expert_offset, int32_t* token_indices,
                int32_t* pair_row);

@@ -217,3 +217,26 @@ def test_quant_block128_bit_exact(moe, src):
     torch.cuda.synchronize()
     assert np.array_equal(s.cpu().numpy().view(np.uint32), want_s.view(np.uint32))
     assert np.array_equal(q.cpu().numpy(), want_q)
+
+
+@pytest.mark.parametrize("name", ["C1", "C4", "C5"])
+def test_router_stats_vs_oracle(moe, name):
+    """moe_router_stats on the GPU's own logits and choices against the oracle's fp64 sums (fp32 results, 1e-6)."""
+    import torch
+    cfg = ob.BASELINE[name]
+    small = ob.Cfg(S=min(cfg.S, 2048), H=min(cfg.H, 512), I=256, E=cfg.E, k=cfg.k, act=cfg.act, dtype=ob.BF16,
+                   gate_fn=cfg.gate_fn, norm_topk=cfg.norm_topk, drop=0, zipf_bias=cfg.zipf_bias)
+    inp = ob.make_inputs(small, seed=13, router_only=True)
+    dev = upload_inputs(small, inp)
+    layer = moe.MoELayer(product_config(small))
+    idx, _, logits = layer.gate(dev["x"], dev["gate_w"], dev.get("gate_bias"), want_logits=True)
+    got = layer.router_stats(logits, idx)
+    torch.cuda.synchronize()
+    want = ob.router_stats(logits.cpu().numpy(), idx.cpu().numpy(), small.gate_fn)
+    assert np.allclose(got["mean_prob"].cpu().numpy(), want["mean_prob"], rtol=1e-6, atol=1e-9)
+    assert np.array_equal(got["load"].cpu().numpy(), want["load"])
+    assert abs(float(got["aux_loss"].cpu()[0]) - want["aux_loss"]) <= 1e-6 * max(1.0, abs(want["aux_loss"]))
+    again = layer.router_stats(logits, idx)
+    torch.cuda.synchronize()
+    assert torch.equal(again["mean_prob"], got["mean_prob"]) and torch.equal(again["aux_loss"], got["aux_loss"])
+    layer.close()

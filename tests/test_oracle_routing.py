@@ -138,3 +138,46 @@ def test_route_skew_all_tokens_one_expert():
     assert list(r["expert_count"]) == [25, 0, 0, 0]
     r = ob.route_slots(idx, 4, 0, 25)
     assert np.array_equal(r["slot"][:, 0], np.arange(100)) and list(r["expert_count"]) == [100, 0, 0, 0]
+
+
+# ---- router statistics (load-balancing loss) ----
+
+def test_router_stats_closed_forms():
+    S, E, k = 64, 8, 2
+    # a uniform router: every score 1/E, assignments spread evenly -> loss exactly 1
+    logits = np.zeros((S, E), np.float32)
+    idx = np.stack([(np.arange(S) * k + r) % E for r in range(k)], axis=1).astype(np.int32)
+    st = ob.router_stats(logits, idx, ob.GATE_SOFTMAX)
+    assert np.allclose(st["mean_prob"], 1.0 / E, rtol=0, atol=1e-7)
+    assert np.array_equal(st["load"], np.full(E, 1.0 / E, np.float32))
+    assert abs(st["aux_loss"] - 1.0) <= 1e-6
+    # a router that always picks expert 3 with probability ~1: load one-hot, loss ~E
+    logits = np.full((S, E), -40.0, np.float32); logits[:, 3] = 40.0
+    idx = np.full((S, 1), 3, np.int32)
+    st = ob.router_stats(logits, idx, ob.GATE_SOFTMAX)
+    assert st["load"][3] == 1.0 and st["load"].sum() == 1.0
+    assert abs(st["mean_prob"][3] - 1.0) <= 1e-6 and abs(st["aux_loss"] - E) <= 1e-5
+    # sigmoid scores at logit 0 are 1/2 each
+    st = ob.router_stats(np.zeros((S, E), np.float32), idx, ob.GATE_SIGMOID)
+    assert np.array_equal(st["mean_prob"], np.full(E, 0.5, np.float32))
+
+
+@pytest.mark.parametrize("gate_fn", [ob.GATE_SOFTMAX, ob.GATE_SIGMOID])
+def test_router_stats_vs_float64(gate_fn):
+    rng = np.random.default_rng(5)
+    S, E, k = 300, 24, 3
+    logits = rng.standard_normal((S, E)).astype(np.float32) * 3
+    idx, _ = ob.topk(logits, k, gate_fn, 0)
+    st = ob.router_stats(logits, idx, gate_fn)
+    l64 = logits.astype(np.float64)
+    if gate_fn == ob.GATE_SOFTMAX:
+        p = np.exp(l64 - l64.max(1, keepdims=True)); p /= p.sum(1, keepdims=True)
+    else:
+        p = 1.0 / (1.0 + np.exp(-l64))
+    load = np.bincount(idx.reshape(-1), minlength=E) / (S * k)
+    assert np.allclose(st["mean_prob"], p.mean(0), rtol=2e-6, atol=0)
+    assert np.allclose(st["load"], load, rtol=1e-7, atol=0)
+    assert abs(st["aux_loss"] - E * float((load * p.mean(0)).sum())) <= 2e-6 * E
+    assert abs(st["load"].sum() - 1.0) <= 1e-6
+    if gate_fn == ob.GATE_SOFTMAX:
+        assert abs(st["mean_prob"].sum() - 1.0) <= 1e-6

@@ -13,7 +13,10 @@ SOURCES = ["config.cpp", "api.hip", "gate.hip", "route.hip", "combine.hip", "ffn
            "ffn_fp8.hip", "peaks.hip", "quant.hip"]
 # packed-fp32 VALU forms are disabled for every device code object of this library
 FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-x", "hip", "-Wall", "-Wno-unused-function",
-         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         # the epilogues index the accumulator registers in fully unrolled loops; without this the 8 x 8 x 4 loop of
+         # the large bf16 tile exceeds the default limit, stays rolled and sends the accumulators through memory
+         "-mllvm", "-pragma-unroll-threshold=1000000"]
 
 
 def _compile(src: str, extra) -> str:

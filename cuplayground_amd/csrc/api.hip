@@ -144,6 +144,7 @@ struct moe_handle {
     WsLayout ws;
     moe_arch arch;
     int ffn_mode;
+    int queue_groups;      // task queues of the FFN stage: one per XCD, or 1
     int timing;
     // stage timing: a ring of kTimedCalls x (MOE_STAGE_COUNT + 1) events, one row per moe_forward call
     hipEvent_t ev[kTimedCalls][MOE_STAGE_COUNT + 1];
@@ -203,6 +204,7 @@ RouteArgs route_args(const moe_handle* h, void* ws) {
     }
     if (lag > d.E) lag = d.E;
     a.lag = (int)lag;
+    a.groups = h->queue_groups;
     return a;
 }
 
@@ -269,6 +271,13 @@ int moe_create(const moe_config* cfg, moe_handle** out) {
         if (v >= 1 && v <= 16) per_cu = v;
     }
     h->arch.persistent_blocks = prop.multiProcessorCount * per_cu;
+    // One task queue per XCD for the MFMA-bound bf16 tiles, whose operand tiles are then shared in that XCD's L2;
+    // the f32 and fp8 paths keep a single queue.
+    h->queue_groups = cfg->torch_dtype == MOE_DTYPE_BF16 ? h->arch.xcds : 1;
+    if (const char* env = getenv("MOE355_QUEUE_GROUPS")) {   // tuning knob
+        const int v = atoi(env);
+        if (v == 1 || v == 2 || v == 4 || v == 8) h->queue_groups = v;
+    }
     *out = h;
     return MOE_OK;
 }
@@ -445,12 +454,20 @@ int moe_forward(moe_handle* h, const void* x, const moe_weights* w, void* out, c
     fa.h = at<char>(workspace, L.h);
     fa.y = at<char>(workspace, L.y);
     fa.mtiles = ra.mtiles;
+    fa.groups = ra.groups;
     fa.seg_phase0 = ra.seg_phase0; fa.seg_phase1 = ra.seg_phase1; fa.seg_queue = ra.seg_queue;
     fa.q = ra.q;
     fa.done0 = ra.done0;
     fa.H = d.H; fa.I = d.I; fa.E = d.E;
     fa.act = c.hidden_act;
     fa.spin_limit = 1 << 24;
+    {
+        const int64_t lim = (int64_t)1 << 32, es = d.act_bytes;
+        fa.ring_ok = (int64_t)d.S * d.H * es < lim && (int64_t)d.A * d.I * es < lim && (int64_t)d.I * d.H * es < lim;
+        fa.x_bytes = (uint32_t)((int64_t)d.S * d.H * es);
+        fa.h_bytes = (uint32_t)((int64_t)d.A * d.I * es);
+        fa.w_bytes = (uint32_t)((int64_t)d.I * d.H * es);
+    }
     const int mode = resolved_ffn_mode(h);
     if (fp8) {
         e = launch_ffn_fp8(fa, d.max_mtiles, d.plan.nnt0, d.plan.nnt1,

@@ -28,6 +28,7 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void lds_void;
 typedef const __attribute__((address_space(1))) void gbl_void;
 
@@ -44,6 +45,8 @@ struct Tile {
     static constexpr int RA = BM / ROWS_PER_PASS; // 16-byte loads per thread per slab, token tile
     static constexpr int RB = BN / ROWS_PER_PASS; // ... weight tile
     static constexpr int STAGE_BYTES = (BM + BN) * kRowBytes;
+    // four wavefronts of 128 x 128 outputs: full row blocks take the hand-ordered slab loop (mainloop_ring)
+    static constexpr bool RING = BM == 256 && BN == 256 && WM == 2 && WN == 2;
     static constexpr int LDS_BYTES = NS * STAGE_BYTES;
     static_assert(TM >= 2 && TM % 2 == 0 && TN >= 2 && TN % 2 == 0, "a wavefront's tile is split in token halves; SwiGLU pairs weight-row halves");
     static_assert(RA >= 1 && RB >= 1, "tile too small for the workgroup");
@@ -68,6 +71,8 @@ struct TaskPtrs {
     int act;                     // epilogue
     bool swiglu;
     bool publish;                // the rows will be read by other workgroups of the same launch
+    bool ring_ok;                // every operand offset of this launch fits 32 bits (buffer addressing)
+    uint32_t a_extent, b_extent; // bytes of the token operand (from a_base) and of one weight matrix (from b0 / b1)
 };
 
 // silu for a bf16 result: hardware exp2 and reciprocal (about 1 ulp each in fp32, far below the bf16 rounding of
@@ -96,7 +101,7 @@ __device__ __forceinline__ void store8(uint16_t* p, uint32_t lo, uint32_t hi, bo
 // are read under the last unit's MFMAs.  The first and the last two slabs are peeled off so that the steady-state
 // loop is one basic block, which is what lets the scheduling hints hold.
 template <class T, bool PARTIAL>
-__device__ __forceinline__ void gemm_tile_impl(const TaskPtrs& p, unsigned char* smem) {
+__device__ __forceinline__ void mainloop_generic(const TaskPtrs& p, unsigned char* smem, f32x4 (&acc)[T::TM][T::TN]) {
     constexpr int BM = T::BM, BN = T::BN, TM = T::TM, TN = T::TN, HM = TM / 2;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / T::WN, wn = wave % T::WN;
@@ -131,7 +136,6 @@ __device__ __forceinline__ void gemm_tile_impl(const TaskPtrs& p, unsigned char*
         b_src[i] = base + (int64_t)col * p.K + chunk * 8;
     }
 
-    f32x4 acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -245,15 +249,24 @@ __device__ __forceinline__ void gemm_tile_impl(const TaskPtrs& p, unsigned char*
         ++kt;
     }
     slab(std::false_type{}, std::false_type{}, kt);
+}
 
-    // ---- epilogue ----
-    // acc[i][j][r]: token row = wm*16*TM + i*16 + (lane & 15); weight row inside the 16-wide MFMA tile = 4*(lane >> 4) + r
+// acc[i][j][r]: token row = wm*16*TM + i*16 + (lane & 15); weight row inside the 16-wide MFMA tile = 4*(lane >> 4) + r.
+// MODE: 0 none / ReLU, 2 exact-erf GELU, 3 SwiGLU.  The choice is made once per tile so that the unrolled store loop
+// does not branch around the (large) GELU code for every element.
+template <class T, int MODE>
+__device__ __forceinline__ void epilogue_impl(const TaskPtrs& p, f32x4 (&acc)[T::TM][T::TN]) {
+    constexpr int TM = T::TM, TN = T::TN;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wm = wave / T::WN, wn = wave % T::WN;
+    const int frow = lane & 15, fk = lane >> 4;
+    const float relu_floor = p.act == MOE_ACT_RELU ? 0.0f : -INFINITY;   // MODE 0: max(u, floor)
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const int m = wm * 16 * TM + i * 16 + frow;
         if (m >= p.rows) continue;
         uint16_t* crow = p.c_base + (int64_t)m * p.N;
-        if (p.swiglu) {
+        if constexpr (MODE == 3) {
 #pragma unroll
             for (int j = 0; j < TN / 2; ++j) {
                 const int col = p.n0 + wn * 8 * TN + j * 16 + 4 * fk;
@@ -278,7 +291,7 @@ __device__ __forceinline__ void gemm_tile_impl(const TaskPtrs& p, unsigned char*
                 for (int r = 0; r < 4; ++r) {
                     float u = acc[i][j][r];
                     if (p.bias0) u = u + bf16_bits_to_f32(p.bias0[col + r]);
-                    v[r] = act_apply(u, p.act);
+                    v[r] = MODE == 2 ? 0.5f * u * (1.0f + erff(u * 0.70710678118654752440f)) : fmaxf(u, relu_floor);
                 }
                 store8(crow + col, pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]), p.publish);
             }
@@ -287,9 +300,270 @@ __device__ __forceinline__ void gemm_tile_impl(const TaskPtrs& p, unsigned char*
 }
 
 template <class T>
+__device__ __forceinline__ void epilogue(const TaskPtrs& p, f32x4 (&acc)[T::TM][T::TN]) {
+    if (p.swiglu) epilogue_impl<T, 3>(p, acc);
+    else if (p.act == MOE_ACT_GELU) epilogue_impl<T, 2>(p, acc);
+    else epilogue_impl<T, 0>(p, acc);
+}
+
+// The epilogue of a tile that is not ragged in N (rows may be), staged through LDS.
+//
+// In the accumulator layout the 16 lanes that are neighbours in the wavefront hold 16 different rows, so a store
+// straight from the registers writes 64 separate 8-byte pieces per instruction and the tile's stores take longer than
+// its arithmetic (14 us of a 100 us tile).  Each wavefront therefore writes its bf16 results into its own piece of
+// the (now idle) slab stages, 64 rows at a time, and reads them back row-major: 16 bytes per lane, a whole row of the
+// wavefront's columns per 16 (8 for SwiGLU) neighbouring lanes, four (eight) rows per store instruction.  No barrier
+// is needed between the two steps (same wavefront, LDS operations complete in order); the one barrier before the
+// first write waits for the other wavefronts' last fragment reads.  The row pitch is padded by 16 bytes, which puts
+// the 8-byte writes of 32 neighbouring lanes on distinct banks.  The bias values of this lane's columns are loaded
+// once (or are -0.0f, the neutral element of the addition), so the element loop has no branch.
+__device__ __forceinline__ void store16(uint16_t* p, u32x4 v, bool publish) {
+    if (publish) asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");   // agent scope, as publish8
+    else *reinterpret_cast<u32x4*>(p) = v;
+}
+
+template <class T, int MODE>
+__device__ __forceinline__ void epilogue_full_n_impl(const TaskPtrs& p, unsigned char* smem, f32x4 (&acc)[8][8]) {
+
+    static_assert(T::TM == 8 && T::TN == 8 && T::WN == 2, "four wavefronts of 128 x 128");
+    constexpr int NJ = MODE == 3 ? 4 : 8;        // groups of 16 output columns per wavefront
+    constexpr int ROW_BYTES = NJ * 32, PITCH = ROW_BYTES + 16;
+    constexpr int LANES_PER_ROW = ROW_BYTES / 16, ROWS_PER_PASS = 64 / LANES_PER_ROW;
+    static_assert(4 * 64 * PITCH <= T::LDS_BYTES, "the staging pieces of the four wavefronts fit the slab stages");
+    // Everything below is derived from a thread id the compiler cannot see through: otherwise it computes these
+    // addresses before the slab loop, finds no register to keep them in, and reloads them from scratch memory
+    // between the stores (each reload then waits for the store before it).
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int frow = lane & 15, fk = lane >> 4;
+    const int col0 = p.n0 + wn * 16 * NJ;        // first output column of this wavefront
+    float b0[NJ][4], b1[NJ][4];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) b0[j][r] = b1[j][r] = -0.0f;
+    if (p.bias0) {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) b0[j][r] = bf16_bits_to_f32(p.bias0[col0 + 16 * j + 4 * fk + r]);
+    }
+    if (MODE == 3 && p.bias1) {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) b1[j][r] = bf16_bits_to_f32(p.bias1[col0 + 16 * j + 4 * fk + r]);
+    }
+    const float relu_floor = p.act == MOE_ACT_RELU ? 0.0f : -INFINITY;   // MODE 0: max(u, floor)
+    unsigned char* stage = smem + wave * (64 * PITCH);
+    unsigned char* wr = stage + frow * PITCH + fk * 8;
+    const int rd_row = lane / LANES_PER_ROW, rd_chunk = lane % LANES_PER_ROW;
+    const unsigned char* rd = stage + rd_row * PITCH + rd_chunk * 16;
+    const int rows_left = p.rows - wm * 128 - rd_row;                 // this lane stores row r0 + rd_row when r0 < rows_left
+    const uint32_t lane_off = (uint32_t)(rd_row * p.N + col0 + rd_chunk * 8);   // elements from the uniform row pointer
+    const bool publish = p.publish;
+    __syncthreads();                             // every wavefront has read its last fragments from the stages
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+#pragma unroll
+        for (int ii = 0; ii < 4; ++ii) {
+            const int i = half * 4 + ii;
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                float v[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if constexpr (MODE == 3) {
+                        const float g = acc[i][j][r] + b1[j][r], u = acc[i][j + 4][r] + b0[j][r];
+                        v[r] = silu_fast(g) * u;
+                    } else {
+                        const float u = acc[i][j][r] + b0[j][r];
+                        v[r] = MODE == 2 ? 0.5f * u * (1.0f + erff(u * 0.70710678118654752440f)) : fmaxf(u, relu_floor);
+                    }
+                }
+                u32x2 o = {pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3])};
+                *reinterpret_cast<u32x2*>(wr + ii * 16 * PITCH + j * 32) = o;
+            }
+        }
+        constexpr int NQ = 64 / ROWS_PER_PASS;
+        u32x4 v[NQ];
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) v[q] = *reinterpret_cast<const u32x4*>(rd + q * ROWS_PER_PASS * PITCH);
+        uint16_t* rows0 = p.c_base + (int64_t)(wm * 128 + half * 64) * p.N;   // uniform
+        if (publish) {
+#pragma unroll
+            for (int q = 0; q < NQ; ++q)
+                if (half * 64 + q * ROWS_PER_PASS < rows_left)
+                    store16(rows0 + (int64_t)(q * ROWS_PER_PASS) * p.N + lane_off, v[q], true);
+        } else {
+#pragma unroll
+            for (int q = 0; q < NQ; ++q)
+                if (half * 64 + q * ROWS_PER_PASS < rows_left)
+                    store16(rows0 + (int64_t)(q * ROWS_PER_PASS) * p.N + lane_off, v[q], false);
+        }
+    }
+}
+
+template <class T>
+__device__ __forceinline__ void epilogue_full_n(const TaskPtrs& p, unsigned char* smem, f32x4 (&acc)[8][8]) {
+    if (p.swiglu) epilogue_full_n_impl<T, 3>(p, smem, acc);
+    else if (p.act == MOE_ACT_GELU) epilogue_full_n_impl<T, 2>(p, smem, acc);
+    else epilogue_full_n_impl<T, 0>(p, smem, acc);
+}
+
+// The slab loop of a full 256 x 256 tile on four wavefronts of 128 x 128, with the instruction order fixed by hand.
+//
+// Why not the compiler's order: with one wavefront per SIMD nothing else hides a stall, and the global->LDS loads of
+// a slab (64 KB per compute unit) need more than one slab of flight time to stream in at the rate the L2 delivers.
+// So (a) both k halves of a slab's fragments are double buffered in registers, which frees the slab's LDS stage at
+// mid-slab, (b) the loads of slab kt+2 are issued into that stage right away, two per MFMA row, and stay in flight
+// across the barriers (bare s_barrier: a __syncthreads() would wait for them), (c) MFMAs, LDS reads and their
+// s_waitcnt are inline asm in the order written by gen_slab_schedule.py (ffn_bf16_slab_*.inc); the compiler places
+// nothing between them but the scalar address updates of the loads.  The accumulators are tied asm operands in
+// AGPRs, so they stay put for the whole loop.  Loads use buffer addressing: a 32-bit byte offset per row, computed
+// once per task, plus a scalar k offset -- no vector ALU instruction is left in the loop.
+// Takes partial row blocks too (the whole tile is computed, rows past the end are not stored).
+// Needs: K a multiple of 128, a tile that is not ragged in N, operand extents below 4 GiB.
+template <class T>
+__device__ __forceinline__ void gemm_tile_ring(const TaskPtrs& p, unsigned char* smem) {
+    static_assert(T::RING && T::TM == 8 && T::TN == 8 && T::RA == 8 && T::RB == 8, "four wavefronts of 128 x 128");
+    constexpr int BM = T::BM, STAGE = T::STAGE_BYTES;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int prow = tid >> 3;
+    const int chunk = (tid & 7) ^ ((prow >> 1) & 7);
+    const int wrow = __builtin_amdgcn_readfirstlane(prow & ~7);
+
+    const int KT = p.K / kBK;                  // even, >= 2
+
+    unsigned voff_a[8], voff_b[8];
+#pragma unroll
+    for (int n = 0; n < 8; ++n) {
+        const int r = min(prow + n * T::ROWS_PER_PASS, p.rows - 1);   // padding rows re-read the last row; never stored
+        const int64_t src_row = p.gather ? (int64_t)p.gather[r] : p.a_row0 + r;
+        voff_a[n] = (unsigned)((src_row * p.a_ld + chunk * 8) * 2);
+        const int j = prow + n * T::ROWS_PER_PASS;
+        const int col = p.swiglu ? p.n0 + (j >> 7) * 64 + (j & 63) : p.n0 + j;
+        voff_b[n] = (unsigned)(((int64_t)col * p.K + chunk * 8) * 2);
+    }
+    auto uniform = [](const void* q) {          // the bases are the same in every lane; say so, or each load loops over lanes
+        const uint64_t v = (uint64_t)q;
+        // readfirstlane returns int: go through uint32_t, or a low half with bit 31 set sign-extends over the high half
+        const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+        const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+        return (void*)(((uint64_t)hi << 32) | (uint64_t)lo);
+    };
+    // Raw buffers (stride 0) that end where the operand ends.  The steady-state slab body also issues loads for the
+    // two slabs past the end of K; those go through descriptors of zero length, which the hardware answers with
+    // zeros without touching memory (the stages they land in are never read).
+    const void* base_a = uniform(p.a_base);
+    const void* base_b0 = uniform(p.b0);
+    const void* base_b1 = uniform(p.swiglu ? p.b1 : p.b0);
+    // load n of a slab: n < 8 token rows, else weight rows; the weight rows of pass m come from w_gate when m % 4 < 2
+    auto load_one = [&](int slab, int n) {
+        unsigned char* base = smem + (slab & 1) * STAGE;
+        const int soff = slab * kRowBytes;
+        const bool live = slab < KT;
+        if (n < 8) {
+            const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base_a), 0, live ? (int)p.a_extent : 0, 0x00020000);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void*)(base + (wrow + n * T::ROWS_PER_PASS) * kRowBytes), 16,
+                                                     voff_a[n], soff, 0, 0);
+        } else {
+            const int m = n - 8;
+            const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>((m & 2) ? base_b0 : base_b1), 0,
+                                                                                 live ? (int)p.b_extent : 0, 0x00020000);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void*)(base + BM * kRowBytes + (wrow + m * T::ROWS_PER_PASS) * kRowBytes),
+                                                     16, voff_b[m], soff, 0, 0);
+        }
+    };
+
+    f32x4 acc[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    const int frow = lane & 15, fk = lane >> 4;
+    const int sw = (frow >> 1) & 7;
+    // LDS addresses of this lane's fragment rows: [stage][k half]
+    // (the asm reads take raw LDS byte addresses: start from where the dynamic array really begins -- a kernel with
+    // static __shared__ variables places it behind them)
+    const unsigned lds0 = (unsigned)(__UINTPTR_TYPE__)(lds_void*)smem;
+    const unsigned a_row = lds0 + (unsigned)((wm * 128 + frow) * kRowBytes), b_row = lds0 + (unsigned)(BM * kRowBytes + (wn * 128 + frow) * kRowBytes);
+    const unsigned c0 = (unsigned)((fk ^ sw) << 4), c1 = (unsigned)(((4 + fk) ^ sw) << 4);
+    const unsigned la0[2] = {a_row + c0, a_row + c1}, lb0[2] = {b_row + c0, b_row + c1};
+    const unsigned la1[2] = {la0[0] + STAGE, la0[1] + STAGE}, lb1[2] = {lb0[0] + STAGE, lb0[1] + STAGE};
+    bf16x8 af[2][8], bfr[2][8];
+    int kt = 0;
+
+#define MF(i, j, s) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(bfr[s][j]), "v"(af[s][i]))
+#define RA(stg, half, idx) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(af[half][idx]) : "v"((stg) ? la1[half] : la0[half]), "n"((idx) * 16 * kRowBytes))
+#define RB(stg, half, j) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(bfr[half][j]) : "v"((stg) ? lb1[half] : lb0[half]), "n"((j) * 16 * kRowBytes))
+#define WL(n) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(n))
+#define BAR1 do { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); __builtin_amdgcn_s_barrier(); } while (0)
+#define BAR2(n) do { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(n) : "memory"); __builtin_amdgcn_s_barrier(); } while (0)
+#define GL(n) load_one(kt + 2, n)
+#define TAIL asm volatile("s_nop 15\n\ts_nop 3" ::: "memory")
+    __syncthreads();                            // the previous task may still be reading the stages
+#pragma unroll
+    for (int n = 0; n < 16; ++n) load_one(0, n);
+#pragma unroll
+    for (int n = 0; n < 16; ++n) load_one(1, n);
+    BAR2(16);                                   // slab 0 has landed (loads return in issue order)
+    {   // same order as the reads behind BAR2 of a steady-state slab
+        constexpr unsigned sn = 0;
+        RA(sn, 0, 0);
+        RB(sn, 0, 0); RB(sn, 0, 1); RB(sn, 0, 2); RB(sn, 0, 3); RB(sn, 0, 4); RB(sn, 0, 5); RB(sn, 0, 6); RB(sn, 0, 7);
+        RA(sn, 0, 1); RA(sn, 0, 2); RA(sn, 0, 3); RA(sn, 0, 4); RA(sn, 0, 5); RA(sn, 0, 6); RA(sn, 0, 7);
+    }
+    // Every slab runs the same body, the last two included: their loads (of slabs KT and KT+1) fetch nothing and
+    // land in stages nobody reads any more.  Separate tail bodies would be shorter, but between them the compiler is
+    // free to spill or copy an accumulator right behind the asm MFMA that writes it, and it does not know that the
+    // value is still in flight.
+    for (; kt < KT; kt += 2) {
+        {
+            constexpr unsigned st = 0, sn = 1;
+#include "ffn_bf16_slab_steady.inc"
+        }
+        ++kt;
+        {
+            constexpr unsigned st = 1, sn = 0;
+#include "ffn_bf16_slab_steady.inc"
+        }
+        --kt;
+    }
+    // (the TAIL of the last slab also covers the epilogue's first read of an accumulator)
+#undef MF
+#undef RA
+#undef RB
+#undef WL
+#undef BAR1
+#undef BAR2
+#undef GL
+#undef TAIL
+    epilogue_full_n<T>(p, smem, acc);
+}
+
+template <class T, bool PARTIAL>
+__device__ __forceinline__ void gemm_tile_generic(const TaskPtrs& p, unsigned char* smem) {
+    f32x4 acc[T::TM][T::TN];
+    mainloop_generic<T, PARTIAL>(p, smem, acc);
+    epilogue<T>(p, acc);
+}
+
+template <class T>
 __device__ __forceinline__ void gemm_tile(const TaskPtrs& p, unsigned char* smem) {
-    if (p.rows >= T::BM) gemm_tile_impl<T, false>(p, smem);
-    else gemm_tile_impl<T, true>(p, smem);
+    if constexpr (T::RING) {
+        const int outc = p.swiglu ? T::BN / 2 : T::BN;
+        if (p.ring_ok && (p.K & 127) == 0 && p.n0 + outc <= p.N) {
+            gemm_tile_ring<T>(p, smem);
+            return;
+        }
+    }
+    if (p.rows >= T::BM) gemm_tile_generic<T, false>(p, smem);
+    else gemm_tile_generic<T, true>(p, smem);
 }
 
 template <class T>
@@ -331,6 +605,9 @@ __device__ __forceinline__ TaskPtrs resolve(const FfnArgs& a, const Task& t, boo
         p.publish = false;
     }
     p.rows = t.rows;
+    p.ring_ok = a.ring_ok != 0;
+    p.a_extent = t.phase == 0 ? a.x_bytes : a.h_bytes;
+    p.b_extent = a.w_bytes;
     return p;
 }
 
@@ -344,42 +621,34 @@ struct Plan {
     static constexpr int THREADS = T0::THREADS;
     static constexpr int LDS_BYTES = T0::LDS_BYTES > T1::LDS_BYTES ? T0::LDS_BYTES : T1::LDS_BYTES;
 };
-using LargePlan = Plan<Tile<256, 256, 2, 4, 2>, Tile<256, 256, 2, 4, 2>>;
+using LargePlan = Plan<Tile<256, 256, 2, 2, 2>, Tile<256, 256, 2, 2, 2>>;
 using SmallPlan = Plan<Tile<128, 128, 2, 2, 2>, Tile<128, 128, 2, 2, 2>>;
 
 // One launch per phase; workgroup b runs task b of that phase.
 template <class P>
 __global__ __launch_bounds__(P::THREADS) void ffn_tiled_kernel(FfnArgs a, int phase) {
     extern __shared__ __align__(16) unsigned char smem[];
-    const int ntasks = phase ? a.q->tasks_phase1 : a.q->tasks_phase0;
-    const int id = blockIdx.x;
-    if (id >= ntasks) return;
-    const int nnt0 = a.seg_phase0[0].nnt;
-    const Task t = decode_task(phase ? a.seg_phase1 : a.seg_phase0, a.E, a.mtiles, id, nnt0);
-    if (phase == 0) gemm_tile<typename P::T0>(resolve<typename P::T0>(a, t, false), smem);
-    else gemm_tile<typename P::T1>(resolve<typename P::T1>(a, t, false), smem);
+    Task t;
+    if (!tiled_task(a, phase, blockIdx.x, t)) return;
+    static_assert(std::is_same<typename P::T0, typename P::T1>::value, "one tile for both projections: one inlined copy");
+    gemm_tile<typename P::T0>(resolve<typename P::T0>(a, t, false), smem);
 }
 
-// Persistent workgroups popping (expert, tile) tasks from one global atomic counter (protocol: ffn_common.hpp).
+// Persistent workgroups popping (expert, tile) tasks from the queue of their XCD (protocol: ffn_common.hpp).
 template <class P>
 __global__ __launch_bounds__(P::THREADS) void ffn_persistent_kernel(FfnArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ int s_task;
     queue_kernel_entry();
-    const int total = a.q->total_tasks;
+    const int ids = a.q->ids_queue;
     const int nseg = a.q->nseg;
     const int nnt0 = a.seg_phase0[0].nnt;
-    for (;;) {
-        const int id = __builtin_amdgcn_readfirstlane(pop_task(&a.q->head, &s_task));
-        if (id >= total) break;             // uniform exit: every wavefront leaves here
-        const Task t = decode_task(a.seg_queue, nseg, a.mtiles, id, nnt0);
-        if (t.phase == 0) {
-            gemm_tile<typename P::T0>(resolve<typename P::T0>(a, t, true), smem);
-            signal_phase0_done(a.done0, t.mtile);
-        } else {
-            wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q);
-            gemm_tile<typename P::T1>(resolve<typename P::T1>(a, t, false), smem);
-        }
+    QueueCursor cur = queue_cursor(a.groups);
+    Task t;
+    while (next_task(a, cur, &s_task, ids, nseg, nnt0, t)) {   // uniform exit: every wavefront leaves together
+        if (t.phase == 1) wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q);
+        gemm_tile<typename P::T0>(resolve<typename P::T0>(a, t, t.phase == 0), smem);   // one inlined copy for both phases
+        if (t.phase == 0) signal_phase0_done(a.done0, t.mtile);
     }
 }
 
@@ -390,7 +659,7 @@ __global__ __launch_bounds__(T::THREADS) void gemm_dense_kernel(const uint16_t* 
                                                                 int act) {
     extern __shared__ __align__(16) unsigned char smem[];
     TaskPtrs p;
-    const int row0 = blockIdx.y * T::BM;
+    const int row0 = blockIdx.x * T::BM;      // row tiles fastest: neighbouring workgroups share the weight tile
     p.a_base = A;
     p.gather = nullptr;
     p.a_row0 = row0;
@@ -403,10 +672,13 @@ __global__ __launch_bounds__(T::THREADS) void gemm_dense_kernel(const uint16_t* 
     p.N = N;
     p.K = K;
     p.rows = min(T::BM, M - row0);
-    p.n0 = blockIdx.x * T::BN;
+    p.n0 = blockIdx.y * T::BN;
     p.act = act;
     p.swiglu = false;
     p.publish = false;
+    p.ring_ok = ((int64_t)M * K < ((int64_t)1 << 31)) && ((int64_t)N * K < ((int64_t)1 << 31));
+    p.a_extent = (uint32_t)((int64_t)M * K * 2);
+    p.b_extent = (uint32_t)((int64_t)N * K * 2);
     gemm_tile<T>(p, smem);
 }
 
@@ -420,8 +692,8 @@ template <class P>
 hipError_t launch_tiled(const FfnArgs& a, int max_mtiles, int nnt0, int nnt1, hipStream_t st) {
     hipError_t e = allow_lds(&ffn_tiled_kernel<P>, P::LDS_BYTES);
     if (e != hipSuccess) return e;
-    ffn_tiled_kernel<P><<<max_mtiles * nnt0, P::THREADS, P::LDS_BYTES, st>>>(a, 0);
-    ffn_tiled_kernel<P><<<max_mtiles * nnt1, P::THREADS, P::LDS_BYTES, st>>>(a, 1);
+    ffn_tiled_kernel<P><<<tiled_grid(max_mtiles, nnt0, a.groups), P::THREADS, P::LDS_BYTES, st>>>(a, 0);
+    ffn_tiled_kernel<P><<<tiled_grid(max_mtiles, nnt1, a.groups), P::THREADS, P::LDS_BYTES, st>>>(a, 1);
     return hipGetLastError();
 }
 
@@ -478,7 +750,7 @@ hipError_t launch_gemm_dense_bf16(const void* A, const void* B, const void* bias
         using T = LargePlan::T0;
         hipError_t e = allow_lds(&gemm_dense_kernel<T>, T::LDS_BYTES);
         if (e != hipSuccess) return e;
-        const dim3 grid((unsigned)((N + T::BN - 1) / T::BN), (unsigned)((M + T::BM - 1) / T::BM));
+        const dim3 grid((unsigned)((M + T::BM - 1) / T::BM), (unsigned)((N + T::BN - 1) / T::BN));
         gemm_dense_kernel<T><<<grid, T::THREADS, T::LDS_BYTES, st>>>((const uint16_t*)A, (const uint16_t*)B,
                                                                      (const uint16_t*)bias, (uint16_t*)C, (int)M,
                                                                      (int)N, (int)K, act);
@@ -486,7 +758,7 @@ hipError_t launch_gemm_dense_bf16(const void* A, const void* B, const void* bias
         using T = SmallPlan::T0;
         hipError_t e = allow_lds(&gemm_dense_kernel<T>, T::LDS_BYTES);
         if (e != hipSuccess) return e;
-        const dim3 grid((unsigned)((N + T::BN - 1) / T::BN), (unsigned)((M + T::BM - 1) / T::BM));
+        const dim3 grid((unsigned)((M + T::BM - 1) / T::BM), (unsigned)((N + T::BN - 1) / T::BN));
         gemm_dense_kernel<T><<<grid, T::THREADS, T::LDS_BYTES, st>>>((const uint16_t*)A, (const uint16_t*)B,
                                                                      (const uint16_t*)bias, (uint16_t*)C, (int)M,
                                                                      (int)N, (int)K, act);
@@ -495,3 +767,4 @@ hipError_t launch_gemm_dense_bf16(const void* A, const void* B, const void* bias
 }
 
 }  // namespace moe355
+

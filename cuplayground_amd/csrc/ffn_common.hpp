@@ -4,12 +4,11 @@
 // (scheduling.cuh:212-222): a scheduler thread (scheduling.cuh:170-200) or warp (warpScheduler.cuh:167-265)
 // pops ready processors and rings their doorbells, and the second-GEMM tasks of a row block become
 // schedulable when that block's first-GEMM row is complete (gtQHeads[m] = tilesN, scheduling.cuh:233-236).
-// On gfx950 the doorbells are replaced by one global atomic counter that every persistent workgroup pops
+// On gfx950 the doorbells are replaced by global atomic counters (one per XCD) that the persistent workgroups pop
 // (no scheduler workgroup), and gtQHeads by done0[m]: each finished phase-0 tile adds one with release
-// semantics, and a phase-1 task acquires done0[m] == nnt0 before it reads the intermediate rows.  Because task
-// ids are popped in increasing order and every phase-0 task of a row block precedes its phase-1 tasks in
-// the queue, a waiting workgroup only ever waits for tasks that are already running: the wait cannot
-// deadlock whatever the number of resident workgroups.
+// semantics, and a phase-1 task acquires done0[m] == nnt0 before it reads the intermediate rows.  Because the
+// ids of a queue are popped in increasing order and every phase-0 task of a row block precedes its phase-1 tasks
+// in every queue, the wait cannot deadlock whatever the number of resident workgroups (see QueueCursor).
 #pragma once
 
 #include "moe_internal.hpp"
@@ -24,12 +23,13 @@ struct Task {
     int row0;      // first packed row
     int rows;      // valid rows in the block
     int nnt0;      // phase-0 column tiles per row block (the dependency target)
+    bool valid;    // false: a hole of this group's id space, nothing to do
 };
 
-// Finds the segment holding task id `id` (segments are sorted by begin, possibly empty) and decodes it.
-// All arguments are wavefront-uniform, so the loads are scalar.
+// Finds the segment holding id `id` of queue group `group` (segments are sorted by begin, possibly empty) and
+// decodes it.  All arguments are wavefront-uniform, so the loads are scalar.
 __device__ __forceinline__ Task decode_task(const Segment* __restrict__ segs, int nseg, const MTile* __restrict__ mtiles,
-                                            int id, int nnt0) {
+                                            int id, int group, int groups, int nnt0) {
     int lo = 0, hi = nseg - 1;
     while (lo < hi) {   // last segment with begin <= id
         const int mid = (lo + hi + 1) >> 1;
@@ -40,8 +40,12 @@ __device__ __forceinline__ Task decode_task(const Segment* __restrict__ segs, in
     Task t;
     t.phase = s.phase;
     t.expert = s.expert;
-    t.ntile = local / s.nmt;
-    t.mtile = s.mt0 + (local - t.ntile * s.nmt);
+    const int j = local / s.nmt;
+    int first = group - s.rot;
+    if (first < 0) first += groups;
+    t.ntile = first + groups * j;
+    t.valid = t.ntile < s.nnt;
+    t.mtile = s.mt0 + (local - j * s.nmt);
     const MTile m = mtiles[t.mtile];
     t.row0 = m.row0;
     t.rows = m.rows;
@@ -62,6 +66,43 @@ __device__ __noinline__ int pop_task(int32_t* head, int* s_task) {
     const int id = __builtin_amdgcn_readfirstlane(*s_task);
     __syncthreads();   // s_task may be overwritten only after everyone has read it
     return id;
+}
+
+// The XCD this workgroup runs on (XCC_ID, bits 3:0 of hardware register 20).
+__device__ __forceinline__ int xcd_id() { return __builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11)) & 7; }
+
+// Where a persistent workgroup takes its tasks from: the queue of its own XCD first (the workgroups of an XCD then
+// walk the same few weight tiles and share them in that XCD's L2), and once that is empty the other groups' queues
+// in turn.  Every group's ids are popped in increasing order, and in every group a row block's phase-0 tasks come
+// before its phase-1 tasks; so the oldest phase-0 task not yet popped anywhere is only ever preceded, in its queue,
+// by tasks that cannot block for ever, and a phase-1 wait always ends.
+struct QueueCursor {
+    int group, exhausted;
+};
+__device__ __forceinline__ QueueCursor queue_cursor(int groups) { return QueueCursor{groups > 1 ? xcd_id() % groups : 0, 0}; }
+
+// Next task of the workgroup; false when every queue is empty.  Holes are skipped here.
+__device__ __forceinline__ bool next_task(const FfnArgs& a, QueueCursor& c, int* s_task, int ids, int nseg, int nnt0,
+                                          Task& t) {
+    for (;;) {
+        const int id = __builtin_amdgcn_readfirstlane(pop_task(&a.q->heads[c.group], s_task));
+        if (id >= ids) {
+            if (++c.exhausted >= a.groups) return false;
+            c.group = c.group + 1 == a.groups ? 0 : c.group + 1;
+            continue;
+        }
+        t = decode_task(a.seg_queue, nseg, a.mtiles, id, c.group, a.groups, nnt0);
+        if (t.valid) return true;
+    }
+}
+
+// Tiled mode: workgroup b of the launch for `phase` (the dispatcher deals workgroups to the XCDs round robin, so
+// b % groups is the XCD).  False: nothing to do.
+__device__ __forceinline__ bool tiled_task(const FfnArgs& a, int phase, int b, Task& t) {
+    const int group = b % a.groups, id = b / a.groups;
+    if (id >= (phase ? a.q->ids_phase1 : a.q->ids_phase0)) return false;
+    t = decode_task(phase ? a.seg_phase1 : a.seg_phase0, a.E, a.mtiles, id, group, a.groups, a.seg_phase0[0].nnt);
+    return t.valid;
 }
 
 // Visibility of the intermediate rows between workgroups that may sit on different XCDs (one L2 each):
@@ -109,11 +150,15 @@ __device__ __noinline__ void wait_phase0_done(const int32_t* done0, int mtile, i
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");   // keeps the block's loads behind the barrier
 }
 
+// Workgroups of a tiled launch: every group's id space, holes included.
+inline int tiled_grid(int max_mtiles, int nnt, int groups) { return groups * max_mtiles * ((nnt + groups - 1) / groups); }
+
+// Two fp32 values rounded to bf16 (nearest even, NaN quieted) by the packed conversion instruction of gfx950.
 __device__ __forceinline__ uint32_t pack2_bf16(float lo, float hi) {
-    uint32_t a = __float_as_uint(lo), b = __float_as_uint(hi);
-    a += 0x7FFFu + ((a >> 16) & 1u);
-    b += 0x7FFFu + ((b >> 16) & 1u);
-    return (a >> 16) | (b & 0xFFFF0000u);
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t v) { return __uint_as_float((uint32_t)v << 16); }

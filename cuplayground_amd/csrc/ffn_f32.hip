@@ -146,11 +146,8 @@ __device__ __forceinline__ TaskPtrsF resolve_f32(const FfnArgs& a, const Task& t
 __global__ __launch_bounds__(256) void ffn_tiled_f32_kernel(FfnArgs a, int phase) {
     __shared__ __align__(16) float As[FBK][FBM + FPAD];
     __shared__ __align__(16) float Bs[FBK][FBN + FPAD];
-    const int ntasks = phase ? a.q->tasks_phase1 : a.q->tasks_phase0;
-    const int id = blockIdx.x;
-    if (id >= ntasks) return;
-    const int nnt0 = a.seg_phase0[0].nnt;
-    const Task t = decode_task(phase ? a.seg_phase1 : a.seg_phase0, a.E, a.mtiles, id, nnt0);
+    Task t;
+    if (!tiled_task(a, phase, blockIdx.x, t)) return;
     const TaskPtrsF p = resolve_f32(a, t, false);
     gemm_tile_f32(p, As, Bs);
 }
@@ -160,13 +157,12 @@ __global__ __launch_bounds__(256) void ffn_persistent_f32_kernel(FfnArgs a) {
     __shared__ __align__(16) float Bs[FBK][FBN + FPAD];
     __shared__ int s_task;
     queue_kernel_entry();
-    const int total = a.q->total_tasks;
+    const int ids = a.q->ids_queue;
     const int nseg = a.q->nseg;
     const int nnt0 = a.seg_phase0[0].nnt;
-    for (;;) {
-        const int id = __builtin_amdgcn_readfirstlane(pop_task(&a.q->head, &s_task));
-        if (id >= total) break;
-        const Task t = decode_task(a.seg_queue, nseg, a.mtiles, id, nnt0);
+    QueueCursor cur = queue_cursor(a.groups);
+    Task t;
+    while (next_task(a, cur, &s_task, ids, nseg, nnt0, t)) {
         if (t.phase == 1) wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q);
         const TaskPtrsF p = resolve_f32(a, t, true);
         gemm_tile_f32(p, As, Bs);
@@ -193,8 +189,8 @@ int f32_block_m() { return FBM; }
 int f32_block_n() { return FBN; }
 
 hipError_t launch_ffn_tiled_f32(const FfnArgs& a, int max_mtiles, int nnt0, int nnt1, hipStream_t st) {
-    ffn_tiled_f32_kernel<<<max_mtiles * nnt0, 256, 0, st>>>(a, 0);
-    ffn_tiled_f32_kernel<<<max_mtiles * nnt1, 256, 0, st>>>(a, 1);
+    ffn_tiled_f32_kernel<<<tiled_grid(max_mtiles, nnt0, a.groups), 256, 0, st>>>(a, 0);
+    ffn_tiled_f32_kernel<<<tiled_grid(max_mtiles, nnt1, a.groups), 256, 0, st>>>(a, 1);
     return hipGetLastError();
 }
 

@@ -217,11 +217,8 @@ __device__ __forceinline__ Fp8Task resolve_fp8(const FfnArgs& a, const Task& t, 
 
 __global__ __launch_bounds__(256) void ffn_tiled_fp8_kernel(FfnArgs a, int phase) {
     __shared__ float red[QWAVES * QGROUPS * 4 * 64];
-    const int ntasks = phase ? a.q->tasks_phase1 : a.q->tasks_phase0;
-    const int id = blockIdx.x;
-    if (id >= ntasks) return;
-    const int nnt0 = a.seg_phase0[0].nnt;
-    const Task t = decode_task(phase ? a.seg_phase1 : a.seg_phase0, a.E, a.mtiles, id, nnt0);
+    Task t;
+    if (!tiled_task(a, phase, blockIdx.x, t)) return;
     for (int sub = 0; sub < QSUB; ++sub) {
         const Fp8Task p = resolve_fp8(a, t, sub, false);
         if (p.c0 < p.N) fp8_tile(p, red);
@@ -232,13 +229,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     __shared__ float red[QWAVES * QGROUPS * 4 * 64];
     __shared__ int s_task;
     queue_kernel_entry();
-    const int total = a.q->total_tasks;
+    const int ids = a.q->ids_queue;
     const int nseg = a.q->nseg;
     const int nnt0 = a.seg_phase0[0].nnt;
-    for (;;) {
-        const int id = __builtin_amdgcn_readfirstlane(pop_task(&a.q->head, &s_task));
-        if (id >= total) break;
-        const Task t = decode_task(a.seg_queue, nseg, a.mtiles, id, nnt0);
+    QueueCursor cur = queue_cursor(a.groups);
+    Task t;
+    while (next_task(a, cur, &s_task, ids, nseg, nnt0, t)) {
         if (t.phase == 1) wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q);
         for (int sub = 0; sub < QSUB; ++sub) {
             const Fp8Task p = resolve_fp8(a, t, sub, true);
@@ -266,8 +262,8 @@ hipError_t launch_ffn_fp8(const FfnArgs& a, int max_mtiles, int nnt0, int nnt1, 
     if (blocks > 0) {
         ffn_persistent_fp8_kernel<<<blocks, 256, 0, st>>>(a);
     } else {
-        ffn_tiled_fp8_kernel<<<max_mtiles * nnt0, 256, 0, st>>>(a, 0);
-        ffn_tiled_fp8_kernel<<<max_mtiles * nnt1, 256, 0, st>>>(a, 1);
+        ffn_tiled_fp8_kernel<<<tiled_grid(max_mtiles, nnt0, a.groups), 256, 0, st>>>(a, 0);
+        ffn_tiled_fp8_kernel<<<tiled_grid(max_mtiles, nnt1, a.groups), 256, 0, st>>>(a, 1);
     }
     return hipGetLastError();
 }

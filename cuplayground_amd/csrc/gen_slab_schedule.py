@@ -1,0 +1,119 @@
+"""Writes ffn_bf16_slab_steady.inc: the instruction order of one 64-wide K slab of the 256x256 bf16 tile.
+
+Run from this directory after changing the schedule: `python gen_slab_schedule.py`.  The .inc files are committed;
+the build does not run this script.
+
+One wavefront owns 128 x 128 outputs: 8 token fragments A[i] x 8 weight fragments B[j] of v_mfma_f32_16x16x32_bf16 per
+32-wide k half, 128 MFMAs per slab in 16 rows (k half s, token fragment i) of 8.  Both k halves of a slab's fragments
+are double buffered in registers (af[s][i], bfr[s][j]):
+
+  rows 0..5    the 16 fragments of k half 1 are read from LDS (3,3,3,3,2,2 per row)
+  before row 8 BAR1: every wavefront has read all of this slab -> its LDS stage is free
+  rows 8..15   the 16 global->LDS loads of slab kt+2 go into that stage, two per row
+  before row 14 BAR2(n): this wavefront's loads of slab kt+1 have landed (only the n loads of slab kt+2 issued so
+               far may be outstanding); after the barrier the other stage may be read
+  rows 14, 15  the 16 fragments of k half 0 of slab kt+1 are read (B first: row 0 of the next slab needs all of them)
+
+An MFMA needs no wait of its own for fragments read in an earlier half; the s_waitcnt lgkmcnt(n) in front of the
+others is computed here from the read order (LDS returns in order), so that only what the MFMA needs has to have landed.
+The kernel runs this one body for every slab, the last two included (their loads fetch nothing): the variants
+without the loads ("pen", "last", still buildable here) are shorter, but in the code between differently shaped
+bodies the compiler spills and copies accumulators, and it does not know that the asm statements in front of such a
+copy are MFMAs whose results are still in flight.  For the same reason the body ends in TAIL: wait states behind
+the last MFMA, which cover whatever the compiler places after the loop.
+"""
+import os
+
+BAR2_ROW = 14
+LOADS_PER_ROW = 2
+
+
+def build(variant):
+    seq = []
+    half1 = []
+    for i in range(8):
+        half1 += [("RA", "st", 1, i), ("RB", "st", 1, i)]
+    per_row = [3, 3, 3, 3, 2, 2, 0, 0]
+    nxt = [("RA", "sn", 0, 0)] + [("RB", "sn", 0, j) for j in range(8)] + [("RA", "sn", 0, i) for i in range(1, 8)]
+    for g in range(16):
+        s, i = divmod(g, 8)
+        ops = []
+        if s == 0:
+            ops = half1[:per_row[i]]
+            half1 = half1[per_row[i]:]
+        else:
+            if g == 8:
+                seq.append(("BAR1",))
+            if variant == "steady" and g < 8 + 16 // LOADS_PER_ROW:
+                ops = [("GL", (g - 8) * LOADS_PER_ROW + q) for q in range(LOADS_PER_ROW)]
+            if g == BAR2_ROW and variant != "last":
+                seq.append(("BAR2", min(16, (BAR2_ROW - 8) * LOADS_PER_ROW) if variant == "steady" else 0))
+            if g >= BAR2_ROW and variant != "last":
+                n = -(-16 // (16 - BAR2_ROW))
+                ops = ops + nxt[:n]
+                nxt = nxt[n:]
+        n = len(ops)
+        slots = [[] for _ in range(4)]
+        for k, o in enumerate(ops):
+            slots[(k * 4 // n) if n > 4 else k].append(o)
+        for p in range(4):
+            seq.append(("MF", i, 2 * p, s))
+            seq.append(("MF", i, 2 * p + 1, s))
+            seq.extend(slots[p])
+    return seq
+
+
+def emit(variant):
+    steady, cur = build("steady"), build(variant)
+    issued, last = 0, {}
+
+    def run(seq, out):
+        nonlocal issued
+        for op in seq:
+            if op[0] == "RA":
+                issued += 1
+                last[("a", op[2], op[3])] = issued
+            elif op[0] == "RB":
+                issued += 1
+                last[("b", op[2], op[3])] = issued
+            if out is None:
+                continue
+            if op[0] == "MF":
+                need = max(last.get(("a", op[3], op[1]), 0), last.get(("b", op[3], op[2]), 0))
+                out.append(("WL", min(issued - need, 15)))
+            out.append(op)
+
+    run(steady, None)          # the slab before: its reads behind BAR2 are outstanding when this slab starts
+    out = []
+    run(cur, out)
+    lines, prev, since = [], None, 0
+    for op in out:
+        if op[0] in ("RA", "RB"):
+            since += 1
+        if op[0] == "WL":
+            if prev is not None and op[1] >= prev + since:
+                continue       # already implied by the previous wait
+            prev, since = op[1], 0
+            lines.append("WL(%d);" % op[1])
+        elif op[0] == "MF":
+            lines.append("MF(%d, %d, %d);" % op[1:])
+        elif op[0] == "RA":
+            lines.append("RA(%s, %d, %d);" % op[1:])
+        elif op[0] == "RB":
+            lines.append("RB(%s, %d, %d);" % op[1:])
+        elif op[0] == "GL":
+            lines.append("GL(%d);" % op[1])
+        elif op[0] == "BAR1":
+            lines.append("BAR1;")
+            prev, since = 0, 0
+        elif op[0] == "BAR2":
+            lines.append("BAR2(%d);" % op[1])
+    lines.append("TAIL;")
+    return "\n".join(lines) + "\n"
+
+
+if __name__ == "__main__":
+    here = os.path.dirname(os.path.abspath(__file__))
+    for v in ("steady",):
+        with open(os.path.join(here, "ffn_bf16_slab_%s.inc" % v), "w") as f:
+            f.write("// generated by gen_slab_schedule.py -- do not edit\n" + emit(v))

@@ -21,28 +21,41 @@ struct MTile {
     int32_t pad;
 };
 
-// A run of consecutive task ids that share (phase, expert).  Task id - begin = ntile * nmt + mtile_local.
+// A run of consecutive task ids that share (phase, expert).
+//
+// The queue exists once per queue group (one group per XCD when the kernels ask for it, else a single group), and
+// every group sees the same id space: in a segment, group g owns the column tiles c with (c + rot) % groups == g,
+// i.e. c = (g - rot) mod groups + groups * j for j < ceil(nnt / groups), and id - begin = j * nmt + mtile_local
+// (row blocks fastest, so neighbouring ids share the weight tile).  An id whose c falls behind nnt is a hole:
+// popped and skipped.  rot = expert * nnt mod groups continues the round robin over the experts, so groups stay
+// balanced when nnt is not a multiple of the group count.
 struct Segment {
-    int32_t begin;    // first task id
+    int32_t begin;    // first task id (in the id space of one group)
     int32_t phase;    // 0 = up(/gate) projection + activation, 1 = down projection
     int32_t expert;
     int32_t mt0;      // index of the expert's first MTile
     int32_t nmt;      // row blocks of the expert
     int32_t nnt;      // column tiles of this phase
-    int32_t pad0, pad1;
+    int32_t rot;      // rotation of the column-tile round robin over the groups
+    int32_t pad1;
 };
 
 // Words at the start of the queue-state block of the workspace (see QueueState offsets in api.cpp).
+constexpr int kMaxQueueGroups = 8;   // XCDs of a gfx950
 struct QueueState {
-    int32_t head;          // next task id to pop (persistent mode)
-    int32_t total_tasks;   // tasks in the merged queue
+    int32_t groups;        // queue groups (1 or the number of XCDs)
+    int32_t total_tasks;   // tasks of both phases (holes not counted)
     int32_t tasks_phase0;
     int32_t tasks_phase1;
     int32_t num_mtiles;
     int32_t kept_rows;
     int32_t stall;         // set when a bounded dependency wait expired
     int32_t nseg;          // segments in the merged queue
-    int32_t pad[8];
+    int32_t heads[kMaxQueueGroups];   // next id to pop, per group (persistent mode)
+    int32_t ids_queue;     // ids per group in the merged queue (holes included)
+    int32_t ids_phase0;    // ids per group in the phase-0 table / the phase-1 table (tiled mode)
+    int32_t ids_phase1;
+    int32_t pad[5];
 };
 
 // Everything the FFN kernels need; passed by value.
@@ -69,6 +82,9 @@ struct FfnArgs {
     int32_t H, I, E;
     int32_t act;
     int32_t spin_limit;
+    int32_t groups;             // queue groups the schedule was built for
+    int32_t ring_ok;            // x, h and one expert's weight matrix each span less than 4 GiB
+    uint32_t x_bytes, h_bytes, w_bytes;   // their extents when ring_ok
 };
 
 struct RouteArgs {
@@ -93,6 +109,7 @@ struct RouteArgs {
     int32_t nnt0, nnt1;         // column tiles of phase 0 / phase 1
     int32_t max_mtiles;
     int32_t lag;                // experts of phase-0 work queued between an expert's two phases
+    int32_t groups;             // queue groups: 1, or one per XCD
 };
 
 // ---- launchers (defined next to their kernels) ----

@@ -51,9 +51,10 @@ __global__ __launch_bounds__(kRouteBlock) void route_count_kernel(RouteArgs a) {
     }
 }
 
-__device__ __forceinline__ void write_segment(Segment* s, int begin, int phase, int expert, int mt0, int nmt, int nnt) {
+__device__ __forceinline__ void write_segment(Segment* s, int begin, int phase, int expert, int mt0, int nmt, int nnt,
+                                              int groups) {
     s->begin = begin; s->phase = phase; s->expert = expert; s->mt0 = mt0; s->nmt = nmt; s->nnt = nnt;
-    s->pad0 = 0; s->pad1 = 0;
+    s->rot = (int)(((int64_t)expert * nnt) % groups); s->pad1 = 0;
 }
 
 // Exclusive prefix sum of one int per thread over a workgroup of kMaxExperts threads (wave shuffles, then the
@@ -144,13 +145,14 @@ __global__ __launch_bounds__(kMaxExperts) void route_scan_kernel(RouteArgs a) {
     // phase-0 tasks it depends on are still running, or its workgroup idles: `lag` experts of phase-0 work
     // (at least a couple of tasks per resident workgroup) sit between the two.
     const int nseg = 2 * a.E;
+    const int npg0 = (a.nnt0 + a.groups - 1) / a.groups, npg1 = (a.nnt1 + a.groups - 1) / a.groups;   // ids per row block and group
     int ph[2] = {0, 0}, ex[2] = {0, 0}, size[2] = {0, 0};
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         const int sidx = 2 * e + j;
         if (sidx < nseg) {
             queue_slot(sidx, a.E, a.lag, &ph[j], &ex[j]);
-            size[j] = s_nmt[ex[j]] * (ph[j] ? a.nnt1 : a.nnt0);
+            size[j] = s_nmt[ex[j]] * (ph[j] ? npg1 : npg0);
         }
     }
     const int begin = block_exclusive_scan(size[0] + size[1], s_wave, &total_tasks);
@@ -159,11 +161,15 @@ __global__ __launch_bounds__(kMaxExperts) void route_scan_kernel(RouteArgs a) {
         const int sidx = 2 * e + j;
         if (sidx < nseg)
             write_segment(a.seg_queue + sidx, begin + (j ? size[0] : 0), ph[j], ex[j], s_mt0[ex[j]], s_nmt[ex[j]],
-                          ph[j] ? a.nnt1 : a.nnt0);
+                          ph[j] ? a.nnt1 : a.nnt0, a.groups);
     }
     if (e == 0) {
-        a.q->head = 0;
-        a.q->total_tasks = total_tasks;
+        a.q->groups = a.groups;
+        for (int g = 0; g < kMaxQueueGroups; ++g) a.q->heads[g] = 0;
+        a.q->ids_queue = total_tasks;
+        a.q->ids_phase0 = total_mt * npg0;
+        a.q->ids_phase1 = total_mt * npg1;
+        a.q->total_tasks = total_mt * (a.nnt0 + a.nnt1);
         a.q->tasks_phase0 = total_mt * a.nnt0;
         a.q->tasks_phase1 = total_mt * a.nnt1;
         a.q->num_mtiles = total_mt;
@@ -175,8 +181,8 @@ __global__ __launch_bounds__(kMaxExperts) void route_scan_kernel(RouteArgs a) {
     if (e < a.E) {
         a.expert_count[e] = kept;
         a.expert_offset[e] = off;
-        write_segment(a.seg_phase0 + e, mt0 * a.nnt0, 0, e, mt0, nmt, a.nnt0);
-        write_segment(a.seg_phase1 + e, mt0 * a.nnt1, 1, e, mt0, nmt, a.nnt1);
+        write_segment(a.seg_phase0 + e, mt0 * npg0, 0, e, mt0, nmt, a.nnt0, a.groups);
+        write_segment(a.seg_phase1 + e, mt0 * npg1, 1, e, mt0, nmt, a.nnt1, a.groups);
         for (int i = 0; i < nmt; ++i) {
             MTile t;
             t.expert = e;

@@ -1,0 +1,51 @@
+"""The bf16 slab loop issues its MFMAs as inline asm, so the compiler neither knows their latency nor that the
+accumulator registers they write are still in flight.  This test compiles the kernels to assembly and checks what the
+compiler placed behind every such MFMA: no read, copy or spill of the accumulator registers it writes may follow
+within the MFMA's latency unless the wait states that end a slab body (s_nop 15) come first."""
+import os
+import re
+import shutil
+import subprocess
+import tempfile
+
+import pytest
+
+from cuplayground_amd import build as moe_build
+
+WINDOW = 12   # instructions; a 16x16x32 bf16 MFMA takes 8 passes of 4 cycles
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
+def test_no_accumulator_access_behind_asm_mfma():
+    src = os.path.join(moe_build.CSRC, "ffn_bf16.hip")
+    flags = [f for f in moe_build.FLAGS if f not in ("-fPIC",)]
+    with tempfile.TemporaryDirectory() as tmp:
+        out = os.path.join(tmp, "ffn_bf16.s")
+        r = subprocess.run(["hipcc", *flags, "-S", "--cuda-device-only", "-I", os.path.join(moe_build.HERE, "..", "include"),
+                            "-o", out, src], capture_output=True, text=True)
+        assert r.returncode == 0, r.stderr[-2000:]
+        text = open(out).read()
+    lines = [x for x in text.split("\n")
+             if x.strip() and (not x.strip().startswith(";") or "ASMSTART" in x or "ASMEND" in x)]
+    access = re.compile(r"(v_accvgpr_read_b32 v\d+, a(\d+)|v_accvgpr_mov_b32 a\d+, a(\d+)|"
+                        r"scratch_store_dword\w* \w+, a\[?(\d+)|v_accvgpr_write_b32 a(\d+))")
+    asm_mfmas, bad = 0, []
+    for k, line in enumerate(lines):
+        m = re.search(r"v_mfma_f32_16x16x32_bf16 a\[(\d+):(\d+)\]", line)
+        if not m or "ASMSTART" not in lines[k - 1]:
+            continue
+        asm_mfmas += 1
+        lo, hi = int(m.group(1)), int(m.group(2))
+        for d in range(1, WINDOW + 1):
+            if k + d >= len(lines):
+                break
+            x = lines[k + d]
+            if "s_nop 15" in x:
+                break
+            a = access.search(x)
+            if a:
+                reg = int([g for g in a.groups()[1:] if g][0])
+                if lo <= reg <= hi:
+                    bad.append((line.strip(), d, x.strip()))
+    assert asm_mfmas >= 256, "the slab loop's inline-asm MFMAs were not found: has the kernel changed?"
+    assert not bad, "accumulators touched behind an in-flight MFMA:\n" + "\n".join("%s -> +%d %s" % b for b in bad[:10])

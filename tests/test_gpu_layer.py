@@ -160,3 +160,34 @@ def test_argument_errors(moe):
         layer.forward(dev["x"], dev)
     assert e.value.status == 3
     layer.close()
+
+
+LARGE_TILE = {
+    # row blocks of 256 with partial tails; full column tiles (hand-ordered slab loop) and ragged ones (general loop)
+    "swiglu_bias": ob.Cfg(S=1500, H=256, I=384, E=4, k=2, act=ob.ACT_SWIGLU, dtype=ob.BF16, drop=0),
+    "gelu_bias_drop": ob.Cfg(S=1300, H=384, I=512, E=3, k=2, act=ob.ACT_GELU, dtype=ob.BF16, drop=1,
+                             capacity_factor=0.9),
+    "relu_ragged_n": ob.Cfg(S=900, H=320, I=448, E=2, k=1, act=ob.ACT_RELU, dtype=ob.BF16, norm_topk=0, drop=0),
+    "swiglu_k_not_128": ob.Cfg(S=800, H=192, I=320, E=3, k=2, act=ob.ACT_SWIGLU, dtype=ob.BF16, drop=0),
+}
+
+
+@pytest.mark.parametrize("name", sorted(LARGE_TILE))
+def test_large_tile_and_queue_groups(moe, name, monkeypatch):
+    """The 256-row tile forced on small layers, in both FFN modes and with 1, 2 and 8 task queues: every run must
+    reproduce the first bit for bit (the schedule only reorders independent tiles) and match the oracle."""
+    cfg = LARGE_TILE[name]
+    inp = ob.make_inputs(cfg, seed=5, with_bias="bias" in name)
+    want = ob.forward(cfg, inp)
+    monkeypatch.setenv("MOE355_BLOCK_ROWS", "256")
+    first = None
+    for groups in ("1", "2", "8"):
+        monkeypatch.setenv("MOE355_QUEUE_GROUPS", groups)
+        for mode in (FFN_TILED, FFN_PERSISTENT):
+            got = run_layer(moe, cfg, inp, mode)
+            check_routing(got, want)
+            if first is None:
+                first = got["out"]
+                assert max_rel_err(ob.to_f32(first, cfg.act_dtype), ob.to_f32(want["out"], cfg.act_dtype)) <= OUT_TOL[cfg.dtype]
+            else:
+                assert np.array_equal(got["out"], first), (groups, mode)

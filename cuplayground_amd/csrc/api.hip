@@ -11,7 +11,7 @@
 namespace moe355 {
 
 // per-dtype pieces defined next to their kernels
-int bf16_block_m(int64_t pairs, int experts, int up_columns);
+int bf16_block_m(int64_t pairs, int experts, int H, int I, int swiglu);
 int bf16_block_n0(int block_m);
 int bf16_block_n1(int block_m);
 int f32_block_m();
@@ -125,7 +125,7 @@ FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E) {
         p.nnt0 = ceil_div(I, fp8_block_n0());
         p.nnt1 = ceil_div(H, fp8_block_n1());
     } else {
-        p.block_m = bf16_block_m(A, E, sw ? 2 * I : I);
+        p.block_m = bf16_block_m(A, E, H, I, sw);
         p.nnt0 = sw ? ceil_div(I, bf16_block_n0(p.block_m) / 2) : ceil_div(I, bf16_block_n0(p.block_m));
         p.nnt1 = ceil_div(H, bf16_block_n1(p.block_m));
     }
@@ -461,9 +461,8 @@ int moe_forward(moe_handle* h, const void* x, const moe_weights* w, void* out, c
     fa.H = d.H; fa.I = d.I; fa.E = d.E;
     fa.act = c.hidden_act;
     fa.spin_limit = 1 << 24;
-    {
-        const int64_t lim = (int64_t)1 << 32, es = d.act_bytes;
-        fa.ring_ok = (int64_t)d.S * d.H * es < lim && (int64_t)d.A * d.I * es < lim && (int64_t)d.I * d.H * es < lim;
+    {   // operand extents for the buffer descriptors of the 256-row bf16 tile (chosen only when they fit 32 bits)
+        const int64_t es = d.act_bytes;
         fa.x_bytes = (uint32_t)((int64_t)d.S * d.H * es);
         fa.h_bytes = (uint32_t)((int64_t)d.A * d.I * es);
         fa.w_bytes = (uint32_t)((int64_t)d.I * d.H * es);

@@ -71,7 +71,6 @@ struct TaskPtrs {
     int act;                     // epilogue
     bool swiglu;
     bool publish;                // the rows will be read by other workgroups of the same launch
-    bool ring_ok;                // every operand offset of this launch fits 32 bits (buffer addressing)
     uint32_t a_extent, b_extent; // bytes of the token operand (from a_base) and of one weight matrix (from b0 / b1)
 };
 
@@ -553,17 +552,16 @@ __device__ __forceinline__ void gemm_tile_generic(const TaskPtrs& p, unsigned ch
     epilogue<T>(p, acc);
 }
 
+// The 256 x 256 tile only exists with the hand-ordered slab loop; the host selects it when every task of the launch
+// meets that loop's conditions (large_tile_ok) and falls back to the 128 x 128 tile otherwise.
 template <class T>
 __device__ __forceinline__ void gemm_tile(const TaskPtrs& p, unsigned char* smem) {
     if constexpr (T::RING) {
-        const int outc = p.swiglu ? T::BN / 2 : T::BN;
-        if (p.ring_ok && (p.K & 127) == 0 && p.n0 + outc <= p.N) {
-            gemm_tile_ring<T>(p, smem);
-            return;
-        }
+        gemm_tile_ring<T>(p, smem);
+    } else {
+        if (p.rows >= T::BM) gemm_tile_generic<T, false>(p, smem);
+        else gemm_tile_generic<T, true>(p, smem);
     }
-    if (p.rows >= T::BM) gemm_tile_generic<T, false>(p, smem);
-    else gemm_tile_generic<T, true>(p, smem);
 }
 
 template <class T>
@@ -605,7 +603,6 @@ __device__ __forceinline__ TaskPtrs resolve(const FfnArgs& a, const Task& t, boo
         p.publish = false;
     }
     p.rows = t.rows;
-    p.ring_ok = a.ring_ok != 0;
     p.a_extent = t.phase == 0 ? a.x_bytes : a.h_bytes;
     p.b_extent = a.w_bytes;
     return p;
@@ -676,7 +673,6 @@ __global__ __launch_bounds__(T::THREADS) void gemm_dense_kernel(const uint16_t* 
     p.act = act;
     p.swiglu = false;
     p.publish = false;
-    p.ring_ok = ((int64_t)M * K < ((int64_t)1 << 31)) && ((int64_t)N * K < ((int64_t)1 << 31));
     p.a_extent = (uint32_t)((int64_t)M * K * 2);
     p.b_extent = (uint32_t)((int64_t)N * K * 2);
     gemm_tile<T>(p, smem);
@@ -719,7 +715,19 @@ int occupancy() {
 
 // Row-block height chosen for a layer: 256 when the average expert sees at least 256 rows and the up
 // projection still gives every compute unit a task at that size.
-int bf16_block_m(int64_t pairs, int experts, int up_columns) {
+//
+// The 256-row tile runs the hand-ordered slab loop only, which needs: K a multiple of 128 in both projections, no
+// ragged column tile (the SwiGLU tile covers 128 intermediate columns, the others 256), and operands below 4 GiB
+// (32-bit buffer offsets; `pairs` bounds the token count).
+static bool large_tile_ok(int64_t pairs, int H, int I, bool swiglu) {
+    const int64_t lim = (int64_t)1 << 32;
+    return H % 256 == 0 && I % (swiglu ? 128 : 256) == 0 && pairs * H * 2 < lim && pairs * I * 2 < lim &&
+           (int64_t)H * I * 2 < lim;
+}
+
+int bf16_block_m(int64_t pairs, int experts, int H, int I, int swiglu) {
+    if (!large_tile_ok(pairs, H, I, swiglu != 0)) return 128;
+    const int up_columns = swiglu ? 2 * I : I;
     if (const char* env = getenv("MOE355_BLOCK_ROWS")) {   // tuning knob: force the row-block height
         const int v = atoi(env);
         if (v == 128 || v == 256) return v;
@@ -746,7 +754,8 @@ int ffn_persistent_occupancy_bf16(int block_m) {
 
 hipError_t launch_gemm_dense_bf16(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N,
                                   int64_t K, int act, hipStream_t st) {
-    if (M >= 1024 && N >= 1024) {
+    const int64_t lim = (int64_t)1 << 32;
+    if (M >= 1024 && N >= 1024 && N % 256 == 0 && K % 128 == 0 && M * K * 2 < lim && N * K * 2 < lim) {
         using T = LargePlan::T0;
         hipError_t e = allow_lds(&gemm_dense_kernel<T>, T::LDS_BYTES);
         if (e != hipSuccess) return e;

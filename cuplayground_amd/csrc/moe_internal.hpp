@@ -83,8 +83,7 @@ struct FfnArgs {
     int32_t act;
     int32_t spin_limit;
     int32_t groups;             // queue groups the schedule was built for
-    int32_t ring_ok;            // x, h and one expert's weight matrix each span less than 4 GiB
-    uint32_t x_bytes, h_bytes, w_bytes;   // their extents when ring_ok
+    uint32_t x_bytes, h_bytes, w_bytes;   // extents of x, h and one weight matrix (meaningful below 4 GiB)
 };
 
 struct RouteArgs {

@@ -47,7 +47,10 @@ struct Tile {
     static constexpr int STAGE_BYTES = (BM + BN) * kRowBytes;
     // four wavefronts of 128 x 128 outputs: full row blocks take the hand-ordered slab loop (mainloop_ring)
     static constexpr bool RING = BM == 256 && BN == 256 && WM == 2 && WN == 2;
-    static constexpr int LDS_BYTES = NS * STAGE_BYTES;
+    // behind the stages: where the four wavefronts of the hand-ordered tile turn 16 rows of results at a time into
+    // row-major order (row pitch 256 + 16 bytes)
+    static constexpr int STAGING_BYTES = RING ? 4 * 16 * 272 : 0;
+    static constexpr int LDS_BYTES = NS * STAGE_BYTES + STAGING_BYTES;
     static_assert(TM >= 2 && TM % 2 == 0 && TN >= 2 && TN % 2 == 0, "a wavefront's tile is split in token halves; SwiGLU pairs weight-row halves");
     static_assert(RA >= 1 && RB >= 1, "tile too small for the workgroup");
     static_assert(NS == 2, "two LDS stages");
@@ -323,14 +326,14 @@ __device__ __forceinline__ void epilogue(const TaskPtrs& p, f32x4 (&acc)[T::TM][
 // The epilogue of a tile that is not ragged in N (rows may be), staged through LDS.
 //
 // In the accumulator layout the 16 lanes that are neighbours in the wavefront hold 16 different rows, so a store
-// straight from the registers writes 64 separate 8-byte pieces per instruction and the tile's stores take longer than
-// its arithmetic (14 us of a 100 us tile).  Each wavefront therefore writes its bf16 results into its own piece of
-// the (now idle) slab stages, 64 rows at a time, and reads them back row-major: 16 bytes per lane, a whole row of the
-// wavefront's columns per 16 (8 for SwiGLU) neighbouring lanes, four (eight) rows per store instruction.  No barrier
-// is needed between the two steps (same wavefront, LDS operations complete in order); the one barrier before the
-// first write waits for the other wavefronts' last fragment reads.  The row pitch is padded by 16 bytes, which puts
-// the 8-byte writes of 32 neighbouring lanes on distinct banks.  The bias values of this lane's columns are loaded
-// once (or are -0.0f, the neutral element of the addition), so the element loop has no branch.
+// straight from the registers writes 64 separate 8-byte pieces per instruction.  Each wavefront therefore writes its
+// bf16 results, 16 rows at a time, into its own piece of LDS behind the slab stages and reads them back row-major:
+// 16 bytes per lane, a whole row of the wavefront's columns per 16 (8 for SwiGLU) neighbouring lanes, four (eight)
+// rows per store instruction.  No barrier is involved (same wavefront, LDS operations complete in order), and the
+// slab stages stay free: the loads of the workgroup's next task may already be landing in them.  The row pitch is
+// padded by 16 bytes, which puts the 8-byte writes of 32 neighbouring lanes on distinct banks.  The bias values of
+// this lane's columns are loaded once (or are -0.0f, the neutral element of the addition), so the element loop has
+// no branch.
 __device__ __forceinline__ void store16(uint16_t* p, u32x4 v, bool publish) {
     if (publish) asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");   // agent scope, as publish8
     else *reinterpret_cast<u32x4*>(p) = v;
@@ -343,7 +346,7 @@ __device__ __forceinline__ void epilogue_full_n_impl(const TaskPtrs& p, unsigned
     constexpr int NJ = MODE == 3 ? 4 : 8;        // groups of 16 output columns per wavefront
     constexpr int ROW_BYTES = NJ * 32, PITCH = ROW_BYTES + 16;
     constexpr int LANES_PER_ROW = ROW_BYTES / 16, ROWS_PER_PASS = 64 / LANES_PER_ROW;
-    static_assert(4 * 64 * PITCH <= T::LDS_BYTES, "the staging pieces of the four wavefronts fit the slab stages");
+    static_assert(4 * 16 * PITCH <= T::STAGING_BYTES, "the staging pieces of the four wavefronts fit behind the slab stages");
     // Everything below is derived from a thread id the compiler cannot see through: otherwise it computes these
     // addresses before the slab loop, finds no register to keep them in, and reloads them from scratch memory
     // between the stores (each reload then waits for the store before it).
@@ -371,50 +374,45 @@ __device__ __forceinline__ void epilogue_full_n_impl(const TaskPtrs& p, unsigned
             for (int r = 0; r < 4; ++r) b1[j][r] = bf16_bits_to_f32(p.bias1[col0 + 16 * j + 4 * fk + r]);
     }
     const float relu_floor = p.act == MOE_ACT_RELU ? 0.0f : -INFINITY;   // MODE 0: max(u, floor)
-    unsigned char* stage = smem + wave * (64 * PITCH);
+    unsigned char* stage = smem + T::NS * T::STAGE_BYTES + wave * (16 * PITCH);
     unsigned char* wr = stage + frow * PITCH + fk * 8;
     const int rd_row = lane / LANES_PER_ROW, rd_chunk = lane % LANES_PER_ROW;
     const unsigned char* rd = stage + rd_row * PITCH + rd_chunk * 16;
     const int rows_left = p.rows - wm * 128 - rd_row;                 // this lane stores row r0 + rd_row when r0 < rows_left
     const uint32_t lane_off = (uint32_t)(rd_row * p.N + col0 + rd_chunk * 8);   // elements from the uniform row pointer
     const bool publish = p.publish;
-    __syncthreads();                             // every wavefront has read its last fragments from the stages
+    constexpr int NQ = 16 / ROWS_PER_PASS;
 #pragma unroll
-    for (int half = 0; half < 2; ++half) {
+    for (int i = 0; i < 8; ++i) {
 #pragma unroll
-        for (int ii = 0; ii < 4; ++ii) {
-            const int i = half * 4 + ii;
+        for (int j = 0; j < NJ; ++j) {
+            float v[4];
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) {
-                float v[4];
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    if constexpr (MODE == 3) {
-                        const float g = acc[i][j][r] + b1[j][r], u = acc[i][j + 4][r] + b0[j][r];
-                        v[r] = silu_fast(g) * u;
-                    } else {
-                        const float u = acc[i][j][r] + b0[j][r];
-                        v[r] = MODE == 2 ? gelu_fast(u) : fmaxf(u, relu_floor);
-                    }
+            for (int r = 0; r < 4; ++r) {
+                if constexpr (MODE == 3) {
+                    const float g = acc[i][j][r] + b1[j][r], u = acc[i][j + 4][r] + b0[j][r];
+                    v[r] = silu_fast(g) * u;
+                } else {
+                    const float u = acc[i][j][r] + b0[j][r];
+                    v[r] = MODE == 2 ? gelu_fast(u) : fmaxf(u, relu_floor);
                 }
-                u32x2 o = {pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3])};
-                *reinterpret_cast<u32x2*>(wr + ii * 16 * PITCH + j * 32) = o;
             }
+            u32x2 o = {pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3])};
+            *reinterpret_cast<u32x2*>(wr + j * 32) = o;
         }
-        constexpr int NQ = 64 / ROWS_PER_PASS;
         u32x4 v[NQ];
 #pragma unroll
         for (int q = 0; q < NQ; ++q) v[q] = *reinterpret_cast<const u32x4*>(rd + q * ROWS_PER_PASS * PITCH);
-        uint16_t* rows0 = p.c_base + (int64_t)(wm * 128 + half * 64) * p.N;   // uniform
+        uint16_t* rows0 = p.c_base + (int64_t)(wm * 128 + i * 16) * p.N;   // uniform
         if (publish) {
 #pragma unroll
             for (int q = 0; q < NQ; ++q)
-                if (half * 64 + q * ROWS_PER_PASS < rows_left)
+                if (i * 16 + q * ROWS_PER_PASS < rows_left)
                     store16(rows0 + (int64_t)(q * ROWS_PER_PASS) * p.N + lane_off, v[q], true);
         } else {
 #pragma unroll
             for (int q = 0; q < NQ; ++q)
-                if (half * 64 + q * ROWS_PER_PASS < rows_left)
+                if (i * 16 + q * ROWS_PER_PASS < rows_left)
                     store16(rows0 + (int64_t)(q * ROWS_PER_PASS) * p.N + lane_off, v[q], false);
         }
     }
@@ -549,6 +547,7 @@ __device__ __forceinline__ void gemm_tile_ring(const TaskPtrs& p, unsigned char*
         --kt;
     }
     // (the TAIL of the last slab also covers the epilogue's first read of an accumulator)
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the fragment reads of the slab past the end have landed in their registers
 #undef MF
 #undef RA
 #undef RB

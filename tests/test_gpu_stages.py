@@ -61,6 +61,23 @@ def test_gemm_vs_oracle(moe, dtype, M, N, K, act):
     assert np.abs(got_nb - want_nb).max() <= tol * max(np.abs(want_nb).max(), 1e-3)
 
 
+@pytest.mark.parametrize("act", [ob.ACT_RELU, ob.ACT_GELU, ob.ACT_NONE])
+@pytest.mark.parametrize("M,N,K", [(1041, 1024, 128), (1280, 1280, 384), (1025, 1536, 1024)])
+def test_gemm_large_tile_vs_oracle(moe, M, N, K, act):
+    """Shapes that take the 256 x 256 tile with the hand-ordered slab loop (M, N >= 1024, N % 256 = 0, K % 128 = 0):
+    the shortest K it accepts, a ragged last row block, bias on and off."""
+    rng = np.random.default_rng(M + N + K)
+    A = ob.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    B = ob.f32_to_bf16((rng.standard_normal((N, K)) * 0.1).astype(np.float32))
+    bias = ob.f32_to_bf16(rng.standard_normal(N).astype(np.float32))
+    for b in (bias, None):
+        want = ob.to_f32(ob.gemm_bias_act(A, B, b, ob.BF16, act), ob.BF16)
+        got = ob.to_f32(from_device(moe.gemm_bias_act(to_device(A, "bf16"), to_device(B, "bf16"),
+                                                      None if b is None else to_device(b, "bf16"), act)), ob.BF16)
+        assert got.shape == want.shape
+        assert np.abs(got - want).max() <= 1e-2 * np.abs(want).max()
+
+
 def test_gemm_rejects_shapes_it_has_no_kernel_for(moe):
     import torch
     A = torch.zeros(4, 40, device="cuda"); B = torch.zeros(4, 40, device="cuda")

@@ -45,7 +45,7 @@ struct Tile {
     static constexpr int RA = BM / ROWS_PER_PASS; // 16-byte loads per thread per slab, token tile
     static constexpr int RB = BN / ROWS_PER_PASS; // ... weight tile
     static constexpr int STAGE_BYTES = (BM + BN) * kRowBytes;
-    // four wavefronts of 128 x 128 outputs: full row blocks take the hand-ordered slab loop (mainloop_ring)
+    // four wavefronts of 128 x 128 outputs: this tile runs the hand-ordered slab loop (gemm_tile_ring)
     static constexpr bool RING = BM == 256 && BN == 256 && WM == 2 && WN == 2;
     // behind the stages: where the four wavefronts of the hand-ordered tile turn 16 rows of results at a time into
     // row-major order (row pitch 256 + 16 bytes)
@@ -432,7 +432,7 @@ __device__ __forceinline__ void epilogue_full_n(const TaskPtrs& p, unsigned char
 // So (a) both k halves of a slab's fragments are double buffered in registers, which frees the slab's LDS stage at
 // mid-slab, (b) the loads of slab kt+2 are issued into that stage right away, two per MFMA row, and stay in flight
 // across the barriers (bare s_barrier: a __syncthreads() would wait for them), (c) MFMAs, LDS reads and their
-// s_waitcnt are inline asm in the order written by gen_slab_schedule.py (ffn_bf16_slab_*.inc); the compiler places
+// s_waitcnt are inline asm in the order written by gen_slab_schedule.py (ffn_bf16_slab_steady.inc); the compiler places
 // nothing between them but the scalar address updates of the loads.  The accumulators are tied asm operands in
 // AGPRs, so they stay put for the whole loop.  Loads use buffer addressing: a 32-bit byte offset per row, computed
 // once per task, plus a scalar k offset -- no vector ALU instruction is left in the loop.

@@ -547,7 +547,14 @@ __device__ __forceinline__ void gemm_tile_ring(const TaskPtrs& p, unsigned char*
         --kt;
     }
     // (the TAIL of the last slab also covers the epilogue's first read of an accumulator)
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the fragment reads of the slab past the end have landed in their registers
+    // The last slab body has read fragments of a slab past the end.  Nobody uses them, so for the compiler their
+    // registers are free from here on -- but the reads are still in flight.  Wait for them, and keep the registers
+    // occupied until behind that wait.
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) asm volatile("" ::"v"(af[h][i]), "v"(bfr[h][i]));
 #undef MF
 #undef RA
 #undef RB

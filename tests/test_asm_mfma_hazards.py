@@ -15,16 +15,54 @@ from cuplayground_amd import build as moe_build
 WINDOW = 12   # instructions; a 16x16x32 bf16 MFMA takes 8 passes of 4 cycles
 
 
+_ASM = {}
+
+
+def _assembly():
+    if "text" not in _ASM:
+        src = os.path.join(moe_build.CSRC, "ffn_bf16.hip")
+        flags = [f for f in moe_build.FLAGS if f not in ("-fPIC",)]
+        with tempfile.TemporaryDirectory() as tmp:
+            out = os.path.join(tmp, "ffn_bf16.s")
+            r = subprocess.run(["hipcc", *flags, "-S", "--cuda-device-only", "-I",
+                                os.path.join(moe_build.HERE, "..", "include"), "-o", out, src],
+                               capture_output=True, text=True)
+            assert r.returncode == 0, r.stderr[-2000:]
+            _ASM["text"] = open(out).read()
+    return _ASM["text"]
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
+def test_slab_loop_holds_nothing_but_the_schedule():
+    """Between the asm statements of the slab loop the compiler may only place scalar bookkeeping: a vector-ALU
+    instruction, a spill or an accumulator move there would sit between a ds_read and the wait that covers it, or
+    behind an MFMA still in flight."""
+    text = _assembly()
+    loops = 0
+    for kernel in re.split(r"\n(?=_Z\w+:)", text):
+        lines = kernel.split("\n")
+        labels = {m.group(1): k for k, l in enumerate(lines) for m in [re.match(r"^(\.LBB\d+_\d+):", l)] if m}
+        for k, l in enumerate(lines):
+            m = re.search(r"s_cbranch_\w+ (\.LBB\d+_\d+)", l)
+            if not (m and m.group(1) in labels and labels[m.group(1)] < k):
+                continue
+            body = [x.strip() for x in lines[labels[m.group(1)]:k + 1]]
+            body = [x for x in body if x and not x.startswith((";", "."))]
+            if sum(x.startswith("v_mfma_f32_16x16x32_bf16") for x in body) != 256 or len(body) > 1000:
+                continue
+            loops += 1
+            other = [x for x in body if x.startswith(("v_", "scratch_", "global_", "flat_"))
+                     and not x.startswith("v_mfma_f32_16x16x32_bf16")]
+            assert not other, "unexpected instructions in the slab loop: %s" % other[:5]
+            assert sum(x.startswith("ds_read_b128") for x in body) == 64
+            assert sum(x.startswith("buffer_load_dwordx4") for x in body) == 32
+            assert sum(x.startswith("s_barrier") for x in body) == 4
+    assert loops >= 3, "expected the slab loop in the two-launch, queue and plain-GEMM kernels, found %d" % loops
+
+
 @pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
 def test_no_accumulator_access_behind_asm_mfma():
-    src = os.path.join(moe_build.CSRC, "ffn_bf16.hip")
-    flags = [f for f in moe_build.FLAGS if f not in ("-fPIC",)]
-    with tempfile.TemporaryDirectory() as tmp:
-        out = os.path.join(tmp, "ffn_bf16.s")
-        r = subprocess.run(["hipcc", *flags, "-S", "--cuda-device-only", "-I", os.path.join(moe_build.HERE, "..", "include"),
-                            "-o", out, src], capture_output=True, text=True)
-        assert r.returncode == 0, r.stderr[-2000:]
-        text = open(out).read()
+    text = _assembly()
     lines = [x for x in text.split("\n")
              if x.strip() and (not x.strip().startswith(";") or "ASMSTART" in x or "ASMEND" in x)]
     access = re.compile(r"(v_accvgpr_read_b32 v\d+, a(\d+)|v_accvgpr_mov_b32 a\d+, a(\d+)|"

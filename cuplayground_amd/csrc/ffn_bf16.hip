@@ -546,7 +546,7 @@ __device__ __forceinline__ void gemm_tile_ring(const TaskPtrs& p, unsigned char*
         }
         --kt;
     }
-    // (the TAIL of the last slab also covers the epilogue's first read of an accumulator)
+    // (the TAIL of the last slab also covers the first read of an accumulator behind the loop)
     // The last slab body has read fragments of a slab past the end.  Nobody uses them, so for the compiler their
     // registers are free from here on -- but the reads are still in flight.  Wait for them, and keep the registers
     // occupied until behind that wait.

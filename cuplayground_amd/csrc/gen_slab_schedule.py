@@ -7,12 +7,17 @@ One wavefront owns 128 x 128 outputs: 8 token fragments A[i] x 8 weight fragment
 32-wide k half, 128 MFMAs per slab in 16 rows (k half s, token fragment i) of 8.  Both k halves of a slab's fragments
 are double buffered in registers (af[s][i], bfr[s][j]):
 
-  rows 0..5    the 16 fragments of k half 1 are read from LDS (3,3,3,3,2,2 per row)
-  before row 8 BAR1: every wavefront has read all of this slab -> its LDS stage is free
-  rows 8..15   the 16 global->LDS loads of slab kt+2 go into that stage, two per row
-  before row 14 BAR2(n): this wavefront's loads of slab kt+1 have landed (only the n loads of slab kt+2 issued so
+  rows 0..2    the 16 fragments of k half 1 are read from LDS (6,5,5 per row)
+  before row 4 BAR1: every wavefront has read all of this slab -> its LDS stage is free
+  rows 4..15   the 16 global->LDS loads of slab kt+2 go into that stage, one or two per row
+  before row 13 BAR2(n): this wavefront's loads of slab kt+1 have landed (only the n loads of slab kt+2 issued so
                far may be outstanding); after the barrier the other stage may be read
-  rows 14, 15  the 16 fragments of k half 0 of slab kt+1 are read (B first: row 0 of the next slab needs all of them)
+  rows 13..15  the 16 fragments of k half 0 of slab kt+1 are read (B first: row 0 of the next slab needs all of them)
+
+The positions are measured, not derived: releasing the stage at row 8 with two loads per row over rows 8..15 is
+2.6 % slower on the Mixtral-shaped layer, four loads per row 7 % slower, all sixteen at once 12 % slower -- the
+L2 -> LDS fill wants the loads spread as thinly as the double buffering allows; releasing the stage before row 4
+(all k-half-1 reads in rows 0..1) costs more in LDS-read stalls than it gains.
 
 An MFMA needs no wait of its own for fragments read in an earlier half; the s_waitcnt lgkmcnt(n) in front of the
 others is computed here from the read order (LDS returns in order), so that only what the MFMA needs has to have landed.
@@ -20,12 +25,15 @@ The kernel runs this one body for every slab, the last two included (their loads
 without the loads ("pen", "last", still buildable here) are shorter, but in the code between differently shaped
 bodies the compiler spills and copies accumulators, and it does not know that the asm statements in front of such a
 copy are MFMAs whose results are still in flight.  For the same reason the body ends in TAIL: wait states behind
-the last MFMA, which cover whatever the compiler places after the loop.
+the last MFMA, which cover whatever the compiler places at the loop's exit (with the wait states behind the loop
+instead, it placed accumulator spills in front of them); a test of the build checks both that and that the loop
+itself holds nothing but this schedule and scalar bookkeeping.
 """
 import os
 
-BAR2_ROW = 14
-LOADS_PER_ROW = 2
+BAR1_ROW = 4                          # MFMA row in front of which the slab's LDS stage is released
+PER_ROW = [6, 5, 5, 0, 0, 0, 0, 0]    # fragment reads of k half 1 behind the MFMAs of rows 0..7
+BAR2_ROW = 13                         # MFMA row in front of which the next slab's stage may be read
 
 
 def build(variant):
@@ -33,21 +41,24 @@ def build(variant):
     half1 = []
     for i in range(8):
         half1 += [("RA", "st", 1, i), ("RB", "st", 1, i)]
-    per_row = [3, 3, 3, 3, 2, 2, 0, 0]
+    per_row = PER_ROW
     nxt = [("RA", "sn", 0, 0)] + [("RB", "sn", 0, j) for j in range(8)] + [("RA", "sn", 0, i) for i in range(1, 8)]
     for g in range(16):
         s, i = divmod(g, 8)
         ops = []
-        if s == 0:
+        if g < 8:
             ops = half1[:per_row[i]]
             half1 = half1[per_row[i]:]
-        else:
-            if g == 8:
+        if g >= BAR1_ROW:
+            if g == BAR1_ROW:
                 seq.append(("BAR1",))
-            if variant == "steady" and g < 8 + 16 // LOADS_PER_ROW:
-                ops = [("GL", (g - 8) * LOADS_PER_ROW + q) for q in range(LOADS_PER_ROW)]
+            if variant == "steady":
+                nrows = 16 - BAR1_ROW
+                k0 = (g - BAR1_ROW) * 16 // nrows
+                k1 = (g - BAR1_ROW + 1) * 16 // nrows
+                ops = ops + [("GL", q) for q in range(k0, k1)]
             if g == BAR2_ROW and variant != "last":
-                seq.append(("BAR2", min(16, (BAR2_ROW - 8) * LOADS_PER_ROW) if variant == "steady" else 0))
+                seq.append(("BAR2", (BAR2_ROW - BAR1_ROW) * 16 // (16 - BAR1_ROW) if variant == "steady" else 0))
             if g >= BAR2_ROW and variant != "last":
                 n = -(-16 // (16 - BAR2_ROW))
                 ops = ops + nxt[:n]

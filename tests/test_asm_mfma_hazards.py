@@ -67,6 +67,7 @@ def test_no_accumulator_access_behind_asm_mfma():
              if x.strip() and (not x.strip().startswith(";") or "ASMSTART" in x or "ASMEND" in x)]
     access = re.compile(r"(v_accvgpr_read_b32 v\d+, a(\d+)|v_accvgpr_mov_b32 a\d+, a(\d+)|"
                         r"scratch_store_dword\w* \w+, a\[?(\d+)|v_accvgpr_write_b32 a(\d+))")
+    labels = {m.group(1): k for k, l in enumerate(lines) for m in [re.match(r"^(\.LBB\d+_\d+):", l)] if m}
     asm_mfmas, bad = 0, []
     for k, line in enumerate(lines):
         m = re.search(r"v_mfma_f32_16x16x32_bf16 a\[(\d+):(\d+)\]", line)
@@ -74,16 +75,23 @@ def test_no_accumulator_access_behind_asm_mfma():
             continue
         asm_mfmas += 1
         lo, hi = int(m.group(1)), int(m.group(2))
-        for d in range(1, WINDOW + 1):
-            if k + d >= len(lines):
-                break
-            x = lines[k + d]
+        pos, seen = k, 0
+        while seen < WINDOW and pos + 1 < len(lines):
+            pos += 1
+            x = lines[pos].strip()
+            if x.startswith(";") or x.endswith(":"):
+                continue
+            jump = re.match(r"s_branch (\.LBB\d+_\d+)", x)
+            if jump:                          # follow the control flow, not the layout of the file
+                pos = labels[jump.group(1)]
+                continue
+            seen += 1
             if "s_nop 15" in x:
                 break
             a = access.search(x)
             if a:
                 reg = int([g for g in a.groups()[1:] if g][0])
                 if lo <= reg <= hi:
-                    bad.append((line.strip(), d, x.strip()))
+                    bad.append((line.strip(), seen, x))
     assert asm_mfmas >= 256, "the slab loop's inline-asm MFMAs were not found: has the kernel changed?"
     assert not bad, "accumulators touched behind an in-flight MFMA:\n" + "\n".join("%s -> +%d %s" % b for b in bad[:10])

@@ -3,20 +3,20 @@
 // Contract kept from the reference (mma.cuh:46-179, processor/tiling.cuh:273-323): C = act(A.B^T + bias)
 // with A (M,K) and B (N,K) row-major, fp32 accumulation, one cast to the storage type on store, epilogue
 // order add-then-activate (processor/tiling.cuh:29-38).  Everything else is designed for CDNA4:
-//   * v_mfma_f32_32x32x16_bf16; the weight tile is the MFMA "A" operand and the token tile the "B" operand,
-//     so each lane ends up with 4 consecutive output columns of one token row and stores 8 bytes at a time;
-//   * K slabs of 64 bf16 go from global memory straight into LDS (global_load_lds_dwordx4, no VGPR staging)
+//   * v_mfma_f32_16x16x32_bf16; the weight tile is the MFMA "A" operand and the token tile the "B" operand,
+//     so each lane ends up with 4 consecutive output columns of one token row (SwiGLU pairs stay in-lane);
+//   * K slabs of 64 bf16 go from global memory straight into LDS (buffer_load ... lds, no VGPR staging)
 //     as 128-byte rows whose 16-byte chunks are xor-swizzled with (row >> 1) & 7: the LDS has 64 banks, a
 //     ds_read_b128 is served 16 lanes at a time, and with this swizzle 16 consecutive rows of one logical
-//     chunk fall into 16 distinct bank groups (measured: SQ_LDS_BANK_CONFLICT = 0);
-//   * 2 (or 3) LDS stages; the loads of the next slab are issued one MFMA apart during the first two of the
-//     current slab's four sub-steps (early enough to land, spread enough not to queue up behind each other), and MFMA operand fragments are double buffered
-//     in registers across the four 16-wide k sub-steps of a slab;
+//     chunk fall into 16 distinct bank groups;
+//   * two LDS stages; MFMA operand fragments are double buffered in registers;
 //   * dispatch is fused into the A-tile load: phase 0 gathers token rows through token_indices[];
 //   * SwiGLU pairs gate and up columns inside one wavefront (first half of its tile rows from w_gate, second
 //     half from w_up), so silu(g)*u happens in registers.
-// Two plans: "large" (256-row blocks, 512 threads: 256x256 tiles for the up projection, 256x128 for the
-// down projection) when experts see many rows, "small" (128x128 tiles, 256 threads) otherwise.
+// Two plans.  "Large": 256-row blocks, 256 x 256 tiles for both projections, four wavefronts of 128 x 128 with the
+// slab loop ordered by hand (gemm_tile_ring) and an epilogue staged through LDS; chosen when experts see many rows
+// and every tile of the layer meets that loop's conditions (large_tile_ok).  "Small": 128 x 128 tiles, four
+// wavefronts of 64 x 64, compiler-scheduled loop (mainloop_generic), general epilogue; takes everything else.
 #include <cstdlib>
 #include <type_traits>
 

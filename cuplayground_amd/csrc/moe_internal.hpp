@@ -40,7 +40,7 @@ struct Segment {
     int32_t pad1;
 };
 
-// Words at the start of the queue-state block of the workspace (see QueueState offsets in api.cpp).
+// Words at the start of the queue-state block of the workspace (carved out of the workspace in api.hip).
 constexpr int kMaxQueueGroups = 8;   // XCDs of a gfx950
 struct QueueState {
     int32_t groups;        // queue groups (1 or the number of XCDs)

@@ -3,6 +3,8 @@
 The product is `libmoe355.so` (C ABI in `include/moe355.h`, HIP kernels in `csrc/`).  This package is the
 thin Python host side over that ABI: torch supplies device memory and the stream, nothing else.  There is no
 fallback path: if the library is not built, importing `cuplayground_amd.api` symbols that need it raises.
+`cuplayground_amd.torch_op` registers `torch.ops.moe355.forward`; `cuplayground_amd.weights` packs, quantises, saves and
+loads a layer's weights in the operand layout.
 """
 from .api import (  # noqa: F401
     MoEConfig,

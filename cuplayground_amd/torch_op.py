@@ -87,30 +87,49 @@ _lib.impl("forward", _forward_meta, "Meta")
 
 
 class MoE355(torch.nn.Module):
-    """One MoE layer with its weights; forward(x[S,H]) -> [S,H] through torch.ops.moe355.forward."""
+    """One MoE layer with its weights; forward(x[S,H]) -> [S,H] through torch.ops.moe355.forward.
 
-    def __init__(self, cfg: api.MoEConfig, device="cuda", init_std: float = 0.02, seed: int = 0):
+    Built either with random weights (`MoE355(cfg)`, bf16/f32 only) or from packed tensors under the argument names of
+    `moe_forward` (`MoE355.from_packed(cfg, tensors)`; see `cuplayground_amd.weights` for packing, quantising and
+    loading them), which also covers the block-scaled e4m3 layers."""
+
+    _NAMES = ("gate_w", "gate_bias", "w_up", "w_gate", "w_down", "b_up", "b_gate", "b_down", "s_up", "s_gate", "s_down")
+
+    def __init__(self, cfg: api.MoEConfig, device="cuda", init_std: float = 0.02, seed: int = 0, tensors=None):
         super().__init__()
-        if cfg.torch_dtype == api.DTYPE_FP8:
-            raise ValueError("build fp8 layers from quantised tensors and call torch.ops.moe355.forward directly")
         self.cfg = cfg
         self.config_json = cfg.to_json()
-        dt = torch.float32 if cfg.torch_dtype == api.DTYPE_F32 else torch.bfloat16
-        E, H, I = cfg.num_experts, cfg.hidden_size, cfg.intermediate_size
-        g = torch.Generator(device="cpu").manual_seed(seed)
+        if tensors is None:
+            if cfg.torch_dtype == api.DTYPE_FP8:
+                raise ValueError("build fp8 layers from quantised tensors: MoE355.from_packed(cfg, tensors)")
+            dt = torch.float32 if cfg.torch_dtype == api.DTYPE_F32 else torch.bfloat16
+            E, H, I = cfg.num_experts, cfg.hidden_size, cfg.intermediate_size
+            g = torch.Generator(device="cpu").manual_seed(seed)
 
-        def w(*shape):
-            return torch.nn.Parameter((torch.randn(*shape, generator=g) * init_std).to(dt).to(device),
-                                      requires_grad=False)
+            def w(*shape):
+                return (torch.randn(*shape, generator=g) * init_std).to(dt).to(device)
 
-        self.gate_w, self.w_up, self.w_down = w(E, H), w(E, I, H), w(E, H, I)
-        self.w_gate = w(E, I, H) if cfg.hidden_act == api.ACT_SWIGLU else None
+            tensors = {"gate_w": w(E, H), "w_up": w(E, I, H), "w_down": w(E, H, I)}
+            if cfg.hidden_act == api.ACT_SWIGLU:
+                tensors["w_gate"] = w(E, I, H)
+        unknown = set(tensors) - set(self._NAMES)
+        if unknown:
+            raise ValueError(f"unknown tensors {sorted(unknown)}")
+        for name in self._NAMES:       # buffers: inference weights, integer codes included
+            t = tensors.get(name)
+            self.register_buffer(name, None if t is None else t.to(device).contiguous())
+
+    @classmethod
+    def from_packed(cls, cfg: api.MoEConfig, tensors, device="cuda") -> "MoE355":
+        return cls(cfg, device=device, tensors=tensors)
 
     def forward(self, x):
-        return torch.ops.moe355.forward(x, self.gate_w, self.w_up, self.w_gate, self.w_down, self.config_json)
+        return torch.ops.moe355.forward(x, self.gate_w, self.w_up, self.w_gate, self.w_down, self.config_json,
+                                        self.gate_bias, self.b_up, self.b_gate, self.b_down, self.s_up, self.s_gate,
+                                        self.s_down)
 
     def reference(self, x):
-        return torch_reference(x, self.cfg, self.gate_w, self.w_up, self.w_gate, self.w_down)
+        return torch_reference(x, self.cfg, self.gate_w, self.w_up, self.w_gate, self.w_down, gate_bias=self.gate_bias)
 
 
 def torch_reference(x, cfg: api.MoEConfig, gate_w, w_up, w_gate, w_down, gate_bias=None, topk=None):

@@ -191,3 +191,44 @@ def test_large_tile_and_queue_groups(moe, name, monkeypatch):
                 assert max_rel_err(ob.to_f32(first, cfg.act_dtype), ob.to_f32(want["out"], cfg.act_dtype)) <= OUT_TOL[cfg.dtype]
             else:
                 assert np.array_equal(got["out"], first), (groups, mode)
+
+
+def test_two_handles_on_two_streams_from_two_threads(moe):
+    """The boundary promises that handles are independent: two layers, each driven from its own host thread on its
+    own (default-priority) stream, overlap freely and must reproduce what each computes alone."""
+    import threading
+    import torch
+    cases = [RAGGED["bf16_swiglu_skew"], RAGGED["bf16_gelu_ragged"]]
+    layers, devs, alone = [], [], []
+    for cfg in cases:
+        inp = ob.make_inputs(cfg, seed=9)
+        layer = moe.MoELayer(product_config(cfg), ffn_mode=FFN_PERSISTENT)
+        dev = upload_inputs(cfg, inp)
+        alone.append(layer.forward(dev["x"], dev).clone())
+        layers.append(layer)
+        devs.append(dev)
+    torch.cuda.synchronize()
+    results, errors = [None, None], []
+
+    def worker(i):
+        try:
+            stream = torch.cuda.Stream()
+            outs = []
+            with torch.cuda.stream(stream):
+                for _ in range(20):
+                    outs.append(layers[i].forward(devs[i]["x"], devs[i]).clone())
+            stream.synchronize()
+            layers[i].task_counts()
+            results[i] = outs
+        except Exception as e:      # surfaced in the main thread
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not errors, errors
+    for i in range(2):
+        assert results[i] is not None and all(torch.equal(o, alone[i]) for o in results[i])
+        layers[i].close()

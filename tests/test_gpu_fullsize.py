@@ -60,3 +60,41 @@ def test_baseline_config_full_size(name):
     out2 = layer.forward(dev["x"], dev)
     assert torch.equal(out, out2)
     layer.close()
+
+
+@pytest.mark.parametrize("S,H,I,k,rows", [(100000, 256, 8192, 2, 256), (140000, 256, 8192, 2, 128), (300000, 4096, 256, 1, 256)],
+                         ids=["h_3GiB_large_tile", "h_4.6GiB_small_tile", "x_2.4GiB_large_tile"])
+def test_operands_beyond_2_and_4_gib(S, H, I, k, rows):
+    """Byte offsets that need bit 31 (the 256-row tile addresses its operands through 32-bit unsigned buffer offsets:
+    the intermediate buffer in the first case, the gathered token rows in the third) and that exceed 32 bits (the
+    layer then has to fall back to the 128-row tile, which uses 64-bit addresses).  With k = 2 every token goes to
+    both experts, so the second expert's rows sit in the upper half of the intermediate buffer."""
+    import torch
+    import cuplayground_amd as moe
+    cfg = ob.Cfg(S=S, H=H, I=I, E=2, k=k, act=ob.ACT_SWIGLU, dtype=ob.BF16, drop=0, norm_topk=0)
+    biggest = max(S * H * 2, S * k * I * 2)
+    assert biggest > 2 ** 31 and (biggest >= 2 ** 32) == (rows == 128)
+    inp = ob.make_inputs(cfg, seed=4)
+    want = ob.route(cfg, inp)
+    layer = moe.MoELayer(product_config(cfg), ffn_mode=FFN_PERSISTENT)
+    assert layer.plan["block_rows"] == rows
+    dev = upload_inputs(cfg, inp)
+    routing = layer.new_routing()
+    out = layer.forward(dev["x"], dev, routing=routing)
+    torch.cuda.synchronize()
+    layer.task_counts()
+    got = {k: from_device(v) for k, v in routing.items()}
+    for key in ("topk_idx", "slot", "expert_count", "expert_offset"):
+        assert np.array_equal(got[key], want[key]), key
+    # tokens whose rows lie at the very end of each expert's range, plus a random handful
+    rng = np.random.default_rng(1)
+    tokens = np.concatenate([[0, 1, S // 2, S - 2, S - 1], rng.choice(S, size=27, replace=False)]).astype(np.int32)
+    ref = ob.to_f32(ob.forward_tokens(cfg, inp, want["topk_idx"], want["topk_w"], want["slot"], tokens), cfg.act_dtype)
+    o = out[torch.from_numpy(tokens.astype(np.int64)).cuda()].float().cpu().numpy()
+    err = max_rel_err(o, ref)
+    print("S", S, "block rows", rows, "sampled max rel err", err, flush=True)
+    assert err <= OUT_TOL[cfg.dtype], err
+    layer.set_ffn_mode(FFN_TILED)
+    out2 = layer.forward(dev["x"], dev)
+    assert torch.equal(out, out2)
+    layer.close()

@@ -169,6 +169,12 @@ LARGE_TILE = {
                              capacity_factor=0.9),
     "relu_ragged_n": ob.Cfg(S=900, H=320, I=448, E=2, k=1, act=ob.ACT_RELU, dtype=ob.BF16, norm_topk=0, drop=0),
     "swiglu_k_not_128": ob.Cfg(S=800, H=192, I=320, E=3, k=2, act=ob.ACT_SWIGLU, dtype=ob.BF16, drop=0),
+    # the shortest K the slab loop takes (two slabs in the down projection), row blocks that are exactly full
+    "swiglu_two_slabs": ob.Cfg(S=512, H=256, I=128, E=1, k=1, act=ob.ACT_SWIGLU, dtype=ob.BF16, norm_topk=0, drop=0),
+    # most experts empty, one row here and there
+    "gelu_sparse_experts": ob.Cfg(S=40, H=256, I=256, E=32, k=1, act=ob.ACT_GELU, dtype=ob.BF16, norm_topk=0, drop=0),
+    "relu_bias_capacity_drop": ob.Cfg(S=1100, H=512, I=256, E=2, k=2, act=ob.ACT_RELU, dtype=ob.BF16, drop=1,
+                                      capacity_factor=0.7),
 }
 
 

@@ -33,6 +33,7 @@ def run_layer(moe, cfg, inp, mode):
     layer.task_counts()            # raises if the persistent queue recorded a stalled dependency wait
     res = {k: from_device(v) for k, v in routing.items()}
     res["out"] = from_device(out)
+    res["plan"] = layer.plan
     layer.close()
     return res
 
@@ -192,6 +193,8 @@ def test_large_tile_and_queue_groups(moe, name, monkeypatch):
         for mode in (FFN_TILED, FFN_PERSISTENT):
             got = run_layer(moe, cfg, inp, mode)
             check_routing(got, want)
+            eligible = cfg.H % 256 == 0 and cfg.I % (128 if cfg.act == ob.ACT_SWIGLU else 256) == 0
+            assert got["plan"]["block_rows"] == (256 if eligible else 128)     # the cases cover both tiles
             if first is None:
                 first = got["out"]
                 assert max_rel_err(ob.to_f32(first, cfg.act_dtype), ob.to_f32(want["out"], cfg.act_dtype)) <= OUT_TOL[cfg.dtype]

@@ -453,9 +453,12 @@ __device__ __forceinline__ void gemm_tile_ring(const TaskPtrs& p, unsigned char*
     unsigned voff_a[8], voff_b[8];
 #pragma unroll
     for (int n = 0; n < 8; ++n) {
-        const int r = min(prow + n * T::ROWS_PER_PASS, p.rows - 1);   // padding rows re-read the last row; never stored
+        // Padding rows are never stored.  Their loads are aimed behind the end of the buffer, which the hardware
+        // answers with zeros without touching memory: MFMAs on zeros draw less of the power budget than MFMAs on a
+        // copy of real rows.
+        const int r0 = prow + n * T::ROWS_PER_PASS, r = min(r0, p.rows - 1);
         const int64_t src_row = p.gather ? (int64_t)p.gather[r] : p.a_row0 + r;
-        voff_a[n] = (unsigned)((src_row * p.a_ld + chunk * 8) * 2);
+        voff_a[n] = r0 < p.rows ? (unsigned)((src_row * p.a_ld + chunk * 8) * 2) : p.a_extent;
         const int j = prow + n * T::ROWS_PER_PASS;
         const int col = p.swiglu ? p.n0 + (j >> 7) * 64 + (j & 63) : p.n0 + j;
         voff_b[n] = (unsigned)(((int64_t)col * p.K + chunk * 8) * 2);

@@ -24,7 +24,7 @@ PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
 # Bytes per FFN-kernel launch that crossed the L2 <-> memory-fabric boundary, from two rocprofv3 --pmc runs of this
 # script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter showed for a 1 GiB
 # device copy in the same run (--calibrate-copy): read x2.000, write x1.000.  Summaries are kept under profiles/.
-MEASURED_TRAFFIC_BYTES = {"mixtral": 19.099e9 + 0.632e9, "decode_fp8": 9.924e9 + 0.013e9}
+MEASURED_TRAFFIC_BYTES = {"mixtral": 19.130e9 + 0.631e9, "decode_fp8": 9.924e9 + 0.013e9}
 
 
 def workloads():

@@ -24,7 +24,7 @@ EXPORTS = (
     "moe_config_default", "moe_config_from_json_string", "moe_config_from_json_file", "moe_config_validate",
     "moe_config_tokens", "moe_config_capacity", "moe_create", "moe_destroy", "moe_get_arch", "moe_get_plan",
     "moe_workspace_bytes",
-    "moe_set_ffn_mode", "moe_get_ffn_mode", "moe_forward", "moe_gate", "moe_router_stats", "moe_route", "moe_gemm_bias_act", "moe_combine",
+    "moe_set_ffn_mode", "moe_get_ffn_mode", "moe_forward", "moe_set_spin_limit", "moe_clear_stall", "moe_gate", "moe_router_stats", "moe_route", "moe_gemm_bias_act", "moe_combine",
     "moe_set_stage_timing", "moe_get_stage_ms", "moe_get_task_counts", "moe_measure_mfma_tflops",
     "moe_measure_hbm_read_gbs", "moe_quant_block128", "moe_last_hip_error", "moe_status_string",
     "moe_version",
@@ -90,6 +90,8 @@ def load_library():
     L.moe_set_ffn_mode.argtypes = [vp, C.c_int]
     L.moe_get_ffn_mode.argtypes = [vp, C.POINTER(C.c_int32)]
     L.moe_forward.argtypes = [vp, vp, C.POINTER(_CWeights), vp, C.POINTER(_CRouting), vp, C.c_size_t, vp]
+    L.moe_set_spin_limit.argtypes = [vp, i32]
+    L.moe_clear_stall.argtypes = [vp]
     L.moe_router_stats.argtypes = [vp, vp, vp, vp, vp, vp, vp, C.c_size_t, vp]
     L.moe_gate.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, C.c_size_t, vp]
     L.moe_route.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, C.c_size_t, vp]
@@ -291,9 +293,17 @@ class MoELayer:
         r = None
         if routing is not None:
             r = _CRouting(*[routing[n].data_ptr() for n, _ in _CRouting._fields_])
-        _check(self.L.moe_forward(self._h, _ptr(x), C.byref(w), _ptr(out), C.byref(r) if r is not None else None,
-                                  _ptr(self.workspace), self.workspace_bytes, _stream()), "moe_forward")
+        rp = C.byref(r) if r is not None else None
+        _check(self.L.moe_forward(self._h, _ptr(x), C.byref(w), _ptr(out), rp, _ptr(self.workspace),
+                                  self.workspace_bytes, _stream()), "moe_forward")
         return out
+
+    def set_spin_limit(self, polls: int):
+        """Polls before a dependency wait of the queue kernel gives up (0: default; negative: every wait expires)."""
+        _check(self.L.moe_set_spin_limit(self._h, polls))
+
+    def clear_stall(self):
+        _check(self.L.moe_clear_stall(self._h))
 
     def gate(self, x, gate_w, gate_bias=None, want_logits: bool = False):
         import torch

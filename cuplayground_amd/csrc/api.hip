@@ -137,6 +137,7 @@ FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E) {
 using namespace moe355;
 
 constexpr int kTimedCalls = 64;
+constexpr int kDefaultSpinLimit = 1 << 24;   // polls (with a short sleep each) of a dependency wait: many seconds
 
 struct moe_handle {
     moe_config cfg;
@@ -145,6 +146,8 @@ struct moe_handle {
     moe_arch arch;
     int ffn_mode;
     int queue_groups;      // task queues of the FFN stage: one per XCD, or 1
+    int spin_limit;        // polls a dependency wait of the queue kernel makes before it gives up
+    int32_t* stall_host;   // pinned host word the queue kernel sets when such a wait expired (never cleared by a kernel)
     int timing;
     // stage timing: a ring of kTimedCalls x (MOE_STAGE_COUNT + 1) events, one row per moe_forward call
     hipEvent_t ev[kTimedCalls][MOE_STAGE_COUNT + 1];
@@ -260,7 +263,14 @@ int moe_create(const moe_config* cfg, moe_handle** out) {
     memset(&h->arch, 0, sizeof h->arch);
     h->arch.device = dev;
     h->arch.compute_units = prop.multiProcessorCount;
-    h->arch.xcds = 8;   // MI355X: 8 accelerator complex dies of 32 CUs
+    // A gfx950 XCD has 32 active compute units; a partitioned device (CPX / DPX / QPX modes) shows fewer CUs and
+    // fewer XCDs.  Queues are built per XCD, and a queue nobody calls home would starve (ffn_common.hpp), so the
+    // count follows what this device really has: 8 on a whole MI355X, 1 on a single-XCD partition.
+    {
+        int x = prop.multiProcessorCount / 32, p2 = 1;
+        while (p2 * 2 <= x && p2 < kMaxQueueGroups) p2 *= 2;
+        h->arch.xcds = p2;
+    }
     h->arch.wavefront_size = prop.warpSize;
     h->arch.lds_bytes_per_cu = (int)prop.maxSharedMemoryPerMultiProcessor;
     h->arch.max_clock_khz = prop.clockRate;
@@ -274,9 +284,19 @@ int moe_create(const moe_config* cfg, moe_handle** out) {
     // One task queue per XCD for the MFMA-bound bf16 tiles, whose operand tiles are then shared in that XCD's L2;
     // the f32 and fp8 paths keep a single queue.
     h->queue_groups = cfg->torch_dtype == MOE_DTYPE_BF16 ? h->arch.xcds : 1;
-    if (const char* env = getenv("MOE355_QUEUE_GROUPS")) {   // tuning knob
+    if (const char* env = getenv("MOE355_QUEUE_GROUPS")) {   // tuning knob; never more queues than XCDs
         const int v = atoi(env);
-        if (v == 1 || v == 2 || v == 4 || v == 8) h->queue_groups = v;
+        if ((v == 1 || v == 2 || v == 4 || v == 8) && v <= h->arch.xcds) h->queue_groups = v;
+    }
+    if (h->queue_groups > h->arch.persistent_blocks) h->queue_groups = 1;   // every queue needs a home workgroup
+    h->spin_limit = kDefaultSpinLimit;
+    h->stall_host = nullptr;
+    {   // host memory, allocated once per handle; the hot path never allocates
+        void* p = nullptr;
+        const hipError_t e = hipHostMalloc(&p, sizeof(int32_t), hipHostMallocDefault);
+        if (e != hipSuccess) { delete h; return MOE_ERR_HIP; }
+        h->stall_host = static_cast<int32_t*>(p);
+        *h->stall_host = 0;
     }
     *out = h;
     return MOE_OK;
@@ -287,6 +307,7 @@ int moe_destroy(moe_handle* h) {
     if (h->ev_valid)
         for (auto& row : h->ev)
             for (auto& e : row) (void)hipEventDestroy(e);
+    if (h->stall_host) (void)hipHostFree(h->stall_host);
     delete h;
     return MOE_OK;
 }
@@ -408,9 +429,16 @@ int moe_route(moe_handle* h, const int32_t* topk_idx, int32_t* slot, int32_t* ex
     return MOE_OK;
 }
 
-int moe_forward(moe_handle* h, const void* x, const moe_weights* w, void* out, const moe_routing_out* routing,
-                void* workspace, size_t workspace_bytes, void* stream) {
+}  // extern "C"
+
+namespace {
+
+// The whole layer.
+int forward_on(moe_handle* h, const void* x, const moe_weights* w, void* out, const moe_routing_out* routing,
+               void* workspace, size_t workspace_bytes, void* stream) {
     if (!h || !x || !w || !out) return MOE_ERR_BAD_ARGUMENT;
+    // a dependency wait of an earlier call expired: that call's output was poisoned; say so until the caller clears it
+    if (*(volatile int32_t*)h->stall_host) return MOE_ERR_QUEUE_STALL;
     const moe_config& c = h->cfg;
     const bool sw = c.hidden_act == MOE_ACT_SWIGLU;
     const bool fp8 = c.torch_dtype == MOE_DTYPE_FP8_E4M3_B128;
@@ -460,7 +488,8 @@ int moe_forward(moe_handle* h, const void* x, const moe_weights* w, void* out, c
     fa.done0 = ra.done0;
     fa.H = d.H; fa.I = d.I; fa.E = d.E;
     fa.act = c.hidden_act;
-    fa.spin_limit = 1 << 24;
+    fa.spin_limit = h->spin_limit;
+    fa.host_stall = h->stall_host;
     {   // operand extents for the buffer descriptors of the 256-row bf16 tile (chosen only when they fit 32 bits)
         const int64_t es = d.act_bytes;
         fa.x_bytes = (uint32_t)((int64_t)d.S * d.H * es);
@@ -503,6 +532,27 @@ int moe_forward(moe_handle* h, const void* x, const moe_weights* w, void* out, c
     return MOE_OK;
 }
 
+}  // namespace
+
+extern "C" {
+
+int moe_forward(moe_handle* h, const void* x, const moe_weights* w, void* out, const moe_routing_out* routing,
+                void* workspace, size_t workspace_bytes, void* stream) {
+    return forward_on(h, x, w, out, routing, workspace, workspace_bytes, stream);
+}
+
+int moe_set_spin_limit(moe_handle* h, int32_t polls) {
+    if (!h) return MOE_ERR_BAD_ARGUMENT;
+    h->spin_limit = polls == 0 ? kDefaultSpinLimit : polls;
+    return MOE_OK;
+}
+
+int moe_clear_stall(moe_handle* h) {
+    if (!h) return MOE_ERR_BAD_ARGUMENT;
+    *(volatile int32_t*)h->stall_host = 0;
+    return MOE_OK;
+}
+
 int moe_get_task_counts(moe_handle* h, const void* workspace, void* stream, int64_t* gemm0_tasks,
                         int64_t* gemm1_tasks) {
     if (!h || !workspace) return MOE_ERR_BAD_ARGUMENT;
@@ -515,7 +565,7 @@ int moe_get_task_counts(moe_handle* h, const void* workspace, void* stream, int6
     if (e != hipSuccess) return hip_fail(h, e);
     if (gemm0_tasks) *gemm0_tasks = q.tasks_phase0;
     if (gemm1_tasks) *gemm1_tasks = q.tasks_phase1;
-    return q.stall ? MOE_ERR_QUEUE_STALL : MOE_OK;
+    return (q.stall || *(volatile int32_t*)h->stall_host) ? MOE_ERR_QUEUE_STALL : MOE_OK;
 }
 
 int moe_gemm_bias_act(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N, int64_t K,

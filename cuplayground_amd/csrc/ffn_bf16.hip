@@ -277,7 +277,9 @@ __device__ __forceinline__ void epilogue_impl(const TaskPtrs& p, f32x4 (&acc)[T:
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wm = wave / T::WN, wn = wave % T::WN;
     const int frow = lane & 15, fk = lane >> 4;
-    const float relu_floor = p.act == MOE_ACT_RELU ? 0.0f : -INFINITY;   // MODE 0: max(u, floor)
+    // MODE 0: u below the floor becomes the floor.  Written as a compare and select, not as fmaxf: a max returns its
+    // other operand for a NaN, and a NaN must stay a NaN (the reference's __hfma_relu propagates it too, processor/tiling.cuh:45,54)
+    const float relu_floor = p.act == MOE_ACT_RELU ? 0.0f : -INFINITY;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const int m = wm * 16 * TM + i * 16 + frow;
@@ -308,7 +310,7 @@ __device__ __forceinline__ void epilogue_impl(const TaskPtrs& p, f32x4 (&acc)[T:
                 for (int r = 0; r < 4; ++r) {
                     float u = acc[i][j][r];
                     if (p.bias0) u = u + bf16_bits_to_f32(p.bias0[col + r]);
-                    v[r] = MODE == 2 ? gelu_fast(u) : fmaxf(u, relu_floor);
+                    v[r] = MODE == 2 ? gelu_fast(u) : (u < relu_floor ? relu_floor : u);
                 }
                 store8(crow + col, pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]), p.publish);
             }
@@ -373,7 +375,9 @@ __device__ __forceinline__ void epilogue_full_n_impl(const TaskPtrs& p, unsigned
 #pragma unroll
             for (int r = 0; r < 4; ++r) b1[j][r] = bf16_bits_to_f32(p.bias1[col0 + 16 * j + 4 * fk + r]);
     }
-    const float relu_floor = p.act == MOE_ACT_RELU ? 0.0f : -INFINITY;   // MODE 0: max(u, floor)
+    // MODE 0: u below the floor becomes the floor.  Written as a compare and select, not as fmaxf: a max returns its
+    // other operand for a NaN, and a NaN must stay a NaN (the reference's __hfma_relu propagates it too, processor/tiling.cuh:45,54)
+    const float relu_floor = p.act == MOE_ACT_RELU ? 0.0f : -INFINITY;
     unsigned char* stage = smem + T::NS * T::STAGE_BYTES + wave * (16 * PITCH);
     unsigned char* wr = stage + frow * PITCH + fk * 8;
     const int rd_row = lane / LANES_PER_ROW, rd_chunk = lane % LANES_PER_ROW;
@@ -394,7 +398,7 @@ __device__ __forceinline__ void epilogue_full_n_impl(const TaskPtrs& p, unsigned
                     v[r] = silu_fast(g) * u;
                 } else {
                     const float u = acc[i][j][r] + b0[j][r];
-                    v[r] = MODE == 2 ? gelu_fast(u) : fmaxf(u, relu_floor);
+                    v[r] = MODE == 2 ? gelu_fast(u) : (u < relu_floor ? relu_floor : u);
                 }
             }
             u32x2 o = {pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3])};
@@ -699,7 +703,7 @@ __global__ __launch_bounds__(P::THREADS) void ffn_tiled_kernel(FfnArgs a, int ph
 template <class P>
 __global__ __launch_bounds__(P::THREADS) void ffn_persistent_kernel(FfnArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
-    __shared__ int s_task;
+    __shared__ int s_task, s_ok;
     queue_kernel_entry();
     const int ids = a.q->ids_queue;
     const int nseg = a.q->nseg;
@@ -707,7 +711,12 @@ __global__ __launch_bounds__(P::THREADS) void ffn_persistent_kernel(FfnArgs a) {
     QueueCursor cur = queue_cursor(a.groups);
     Task t;
     while (next_task(a, cur, &s_task, ids, nseg, nnt0, t)) {   // uniform exit: every wavefront leaves together
-        if (t.phase == 1) wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q);
+        if (t.phase == 1 && !wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q, a.host_stall, &s_ok)) {
+            // the rows never became ready: NaN instead of a result, and a tile of no rows (it loads, computes and
+            // stores nothing of its own), so that the loop keeps its one shape
+            poison_tile((uint16_t*)a.y + (int64_t)t.row0 * a.H, t.rows, a.H, t.ntile * P::T1::BN, P::T1::BN, 2);
+            t.rows = 0;
+        }
         gemm_tile<typename P::T0>(resolve<typename P::T0>(a, t, t.phase == 0), smem);   // one inlined copy for both phases
         if (t.phase == 0) signal_phase0_done(a.done0, t.mtile);
     }

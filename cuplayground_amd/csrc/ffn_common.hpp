@@ -8,7 +8,9 @@
 // (no scheduler workgroup), and gtQHeads by done0[m]: each finished phase-0 tile adds one with release
 // semantics, and a phase-1 task acquires done0[m] == nnt0 before it reads the intermediate rows.  Because the
 // ids of a queue are popped in increasing order and every phase-0 task of a row block precedes its phase-1 tasks
-// in every queue, the wait cannot deadlock whatever the number of resident workgroups (see QueueCursor).
+// in every queue, the wait cannot deadlock as long as every queue has workgroups popping it from the start of the
+// launch (see QueueCursor); the host guarantees that by building no more queues than the device partition has XCDs
+// and launching at least one workgroup per queue.  The wait is bounded all the same.
 #pragma once
 
 #include "moe_internal.hpp"
@@ -107,7 +109,7 @@ __device__ __forceinline__ bool tiled_task(const FfnArgs& a, int phase, int b, T
 
 // Visibility of the intermediate rows between workgroups that may sit on different XCDs (one L2 each):
 //   producer: every intermediate store is an agent-scope store (publish8 / publish4: written through to
-//             memory); each wavefront waits for its own stores (workgroup-scope release = s_waitcnt vmcnt(0)),
+//             memory); each wavefront waits for its own stores (an explicit s_waitcnt vmcnt(0)),
 //             the workgroup meets at a barrier, one lane adds to done0[m] with an agent-scope atomic;
 //   consumer: one lane polls done0[m] with agent-scope atomic loads, the workgroup meets at a barrier, and
 //             only then issues its first load of the block's rows.  Those lines cannot already sit in the
@@ -126,28 +128,52 @@ __device__ __forceinline__ void publish4(void* p, uint32_t v) {
     __hip_atomic_store(reinterpret_cast<uint32_t*>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Called by every thread of the workgroup after its phase-0 stores.
+// Called by every thread of the workgroup after its phase-0 stores.  The explicit vmcnt(0) is the release: it
+// completes this wavefront's published (write-through) stores before the barrier and the counter increment.  A
+// workgroup-scope fence alone emits no wait for global stores here, so the hand-off must not depend on it.
 __device__ __noinline__ void signal_phase0_done(int32_t* done0, int mtile) {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");   // this wavefront's published stores have completed
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
     if (threadIdx.x == 0) __hip_atomic_fetch_add(done0 + mtile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Called by every thread of the workgroup before a phase-1 task reads the intermediate rows.
-__device__ __noinline__ void wait_phase0_done(const int32_t* done0, int mtile, int target, int spin_limit,
-                                              QueueState* q) {
+// Called by every thread of the workgroup before a phase-1 task reads the intermediate rows.  Returns 1 when the
+// rows are complete.  Returns 0 (to every thread) when the bounded wait expired: the stall is recorded in the
+// workspace and in the handle's host-visible word, and the caller must not compute on the rows -- it poisons its
+// output tile instead (poison_tile), so a wrong result cannot pass for a right one.  spin_limit < 0 makes every wait
+// expire at once without polling: the host-forceable way to exercise this path with every kernel exiting normally.
+__device__ __noinline__ int wait_phase0_done(const int32_t* done0, int mtile, int target, int spin_limit,
+                                             QueueState* q, int32_t* host_stall, int* s_ok) {
     if (threadIdx.x == 0) {
-        int spins = 0;
-        while (__hip_atomic_load(done0 + mtile, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
+        int spins = 0, ok = spin_limit >= 0;
+        while (ok && __hip_atomic_load(done0 + mtile, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
             __builtin_amdgcn_s_sleep(8);
-            if (++spins > spin_limit) {   // never hang the device: record the stall and carry on
-                __hip_atomic_store(&q->stall, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                break;
-            }
+            if (++spins > spin_limit) ok = 0;   // never hang the device
         }
+        if (!ok) {
+            __hip_atomic_store(&q->stall, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (host_stall) __hip_atomic_store(host_stall, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        }
+        *s_ok = ok;
     }
     __syncthreads();
+    const int ok = __builtin_amdgcn_readfirstlane(*s_ok);
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");   // keeps the block's loads behind the barrier
+    return ok;
+}
+
+// Fills rows [0, rows) x columns [n0, min(n0 + ncols, N)) of a row-major output block with NaN (elem_bytes 2: bf16
+// 0x7FC0, 4: fp32 0x7FC00000).  Run by the whole workgroup in place of a tile whose inputs never became ready.
+__device__ __noinline__ void poison_tile(void* c_base, int rows, int N, int n0, int ncols, int elem_bytes) {
+    const int n1 = min(n0 + ncols, N), w = n1 - n0;
+    if (w <= 0) return;
+    for (int i = threadIdx.x; i < rows * w; i += blockDim.x) {
+        const int r = i / w, c = n0 + i % w;
+        const int64_t at = (int64_t)r * N + c;
+        if (elem_bytes == 2) reinterpret_cast<uint16_t*>(c_base)[at] = 0x7FC0u;
+        else reinterpret_cast<uint32_t*>(c_base)[at] = 0x7FC00000u;
+    }
 }
 
 // Workgroups of a tiled launch: every group's id space, holes included.
@@ -164,7 +190,7 @@ __device__ __forceinline__ uint32_t pack2_bf16(float lo, float hi) {
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t v) { return __uint_as_float((uint32_t)v << 16); }
 
 __device__ __forceinline__ float act_apply(float v, int act) {
-    if (act == MOE_ACT_RELU) return v > 0.0f ? v : 0.0f;
+    if (act == MOE_ACT_RELU) return v < 0.0f ? 0.0f : v;   // a NaN stays a NaN
     if (act == MOE_ACT_GELU) return 0.5f * v * (1.0f + erff(v * 0.70710678118654752440f));
     return v;
 }

@@ -155,7 +155,7 @@ __global__ __launch_bounds__(256) void ffn_tiled_f32_kernel(FfnArgs a, int phase
 __global__ __launch_bounds__(256) void ffn_persistent_f32_kernel(FfnArgs a) {
     __shared__ __align__(16) float As[FBK][FBM + FPAD];
     __shared__ __align__(16) float Bs[FBK][FBN + FPAD];
-    __shared__ int s_task;
+    __shared__ int s_task, s_ok;
     queue_kernel_entry();
     const int ids = a.q->ids_queue;
     const int nseg = a.q->nseg;
@@ -163,9 +163,11 @@ __global__ __launch_bounds__(256) void ffn_persistent_f32_kernel(FfnArgs a) {
     QueueCursor cur = queue_cursor(a.groups);
     Task t;
     while (next_task(a, cur, &s_task, ids, nseg, nnt0, t)) {
-        if (t.phase == 1) wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q);
+        int ok = 1;
+        if (t.phase == 1) ok = wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q, a.host_stall, &s_ok);
         const TaskPtrsF p = resolve_f32(a, t, true);
-        gemm_tile_f32(p, As, Bs);
+        if (ok) gemm_tile_f32(p, As, Bs);
+        else poison_tile(p.c_base, p.rows, p.N, p.n0, FBN, 4);
         if (t.phase == 0) signal_phase0_done(a.done0, t.mtile);
     }
 }

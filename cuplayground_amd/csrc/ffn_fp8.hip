@@ -227,7 +227,7 @@ __global__ __launch_bounds__(256) void ffn_tiled_fp8_kernel(FfnArgs a, int phase
 
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void ffn_persistent_fp8_kernel(FfnArgs a) {
     __shared__ float red[QWAVES * QGROUPS * 4 * 64];
-    __shared__ int s_task;
+    __shared__ int s_task, s_ok;
     queue_kernel_entry();
     const int ids = a.q->ids_queue;
     const int nseg = a.q->nseg;
@@ -235,10 +235,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     QueueCursor cur = queue_cursor(a.groups);
     Task t;
     while (next_task(a, cur, &s_task, ids, nseg, nnt0, t)) {
-        if (t.phase == 1) wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q);
+        int ok = 1;
+        if (t.phase == 1) ok = wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q, a.host_stall, &s_ok);
         for (int sub = 0; sub < QSUB; ++sub) {
             const Fp8Task p = resolve_fp8(a, t, sub, true);
-            if (p.c0 < p.N) fp8_tile(p, red);
+            if (p.c0 >= p.N) continue;
+            if (ok) fp8_tile(p, red);
+            else poison_tile(p.c_base, p.rows, p.N, p.c0, QN1, 2);
         }
         if (t.phase == 0) signal_phase0_done(a.done0, t.mtile);
     }

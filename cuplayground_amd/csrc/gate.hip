@@ -166,6 +166,9 @@ __device__ __forceinline__ bool better(const Cand& a, const Cand& b) {
 }
 
 // One wavefront per token; lane l keeps logits of experts l, l+64, ... (at most 8) in registers.
+// The selection is total: a NaN logit ranks as -inf (behind every number, ties to the lower index), so a token row
+// that overflowed still gets k distinct, valid experts; its weights are computed from the logits as they are and
+// come out NaN, which is what reaches the output of that token and of no other.
 __global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ logits, int S, int E, int k, int gate_fn,
                                                    int norm, int32_t* __restrict__ topk_idx,
                                                    float* __restrict__ topk_w) {
@@ -193,7 +196,7 @@ __global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ log
 #pragma unroll
         for (int j = 0; j < J; ++j) {
             if ((avail >> j) & 1u) {
-                Cand d{v[j], j * kWave + lane};
+                Cand d{v[j] != v[j] ? -INFINITY : v[j], j * kWave + lane};
                 if (better(d, c)) c = d;
             }
         }
@@ -203,8 +206,13 @@ __global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ log
             if (better(o, c)) c = o;
         }
         if ((c.i & (kWave - 1)) == lane) avail &= ~(1u << (c.i >> 6));
-        if (lane == r) { my_l = c.v; my_i = c.i; }
-        if (r == 0) top_l = c.v;
+        // the logit behind the winning key, as stored (a NaN ranks as -inf but stays a NaN in the weights)
+        float mine = v[0];
+#pragma unroll
+        for (int j = 1; j < J; ++j) mine = (c.i >> 6) == j ? v[j] : mine;
+        const float cv = __shfl(mine, c.i & (kWave - 1), kWave);
+        if (lane == r) { my_l = cv; my_i = c.i; }
+        if (r == 0) top_l = cv;
     }
     float p = 0.0f;
     if (gate_fn == MOE_GATE_SOFTMAX) {
@@ -273,7 +281,10 @@ __global__ __launch_bounds__(256) void router_stats_partial_kernel(const float* 
             for (int j = 0; j < J; ++j)
                 if (j * kWave + lane < E) acc[j] += (double)(1.0f / (1.0f + expf(-v[j])));
         }
-        if (lane < k) atomicAdd(&s_cnt[topk_idx[(size_t)t * k + lane]], 1);
+        if (lane < k) {
+            const int e = topk_idx[(size_t)t * k + lane];
+            if ((unsigned)e < (unsigned)E) atomicAdd(&s_cnt[e], 1);   // ids outside [0, E) are counted nowhere
+        }
     }
 #pragma unroll
     for (int j = 0; j < J; ++j)

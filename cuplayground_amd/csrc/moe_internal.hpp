@@ -79,6 +79,7 @@ struct FfnArgs {
     const Segment* seg_queue;   // 2E segments in queue order
     QueueState* q;
     int32_t* done0;             // per MTile: finished phase-0 column tiles
+    int32_t* host_stall;        // pinned host word of the handle, set (system scope) when a dependency wait expires
     int32_t H, I, E;
     int32_t act;
     int32_t spin_limit;

@@ -24,8 +24,10 @@ __global__ __launch_bounds__(kRouteBlock) void route_count_kernel(RouteArgs a) {
     for (int i = tid; i < (kRouteBlock / kWave) * kMaxExperts; i += kRouteBlock) (&wcount[0][0])[i] = 0;
     __syncthreads();
     const int p = blockIdx.x * kRouteBlock + tid;
-    const bool valid = p < a.A;
-    const int e = valid ? a.topk_idx[p] : 0;
+    // an expert id outside [0, E) (only a caller-supplied topk_idx can hold one) is counted nowhere: the pair is dropped
+    const int e_in = p < a.A ? a.topk_idx[p] : -1;
+    const bool valid = (unsigned)e_in < (unsigned)a.E;
+    const int e = valid ? e_in : 0;
     unsigned long long mask = __ballot(valid);
     int nbits = 0;
     while ((1 << nbits) < a.E) ++nbits;
@@ -198,9 +200,11 @@ __global__ __launch_bounds__(kMaxExperts) void route_scan_kernel(RouteArgs a) {
 __global__ __launch_bounds__(kRouteBlock) void route_finalize_kernel(RouteArgs a) {
     const int p = blockIdx.x * kRouteBlock + threadIdx.x;
     if (p >= a.A) return;
-    const int e = a.topk_idx[p];
-    const int s = a.block_hist[(size_t)blockIdx.x * a.E + e] + a.rank_local[p];
-    const bool dropped = a.drop && s >= a.capacity;
+    const int e_in = a.topk_idx[p];
+    const bool known = (unsigned)e_in < (unsigned)a.E;   // see route_count_kernel
+    const int e = known ? e_in : 0;
+    const int s = known ? a.block_hist[(size_t)blockIdx.x * a.E + e] + a.rank_local[p] : 0;
+    const bool dropped = !known || (a.drop && s >= a.capacity);
     const int row = dropped ? -1 : a.expert_offset[e] + s;
     a.slot[p] = dropped ? -1 : s;
     a.pair_row[p] = row;

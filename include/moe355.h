@@ -186,6 +186,16 @@ int moe_get_stage_ms(moe_handle* h, int stage, float* ms, int32_t* calls);
  * back a few words from the workspace, so it synchronises the stream. */
 int moe_get_task_counts(moe_handle* h, const void* workspace, void* stream, int64_t* gemm0_tasks, int64_t* gemm1_tasks);
 
+/* A dependency wait of the task-queue kernel is bounded (the reference's spin waits are not: overlap.cuh:104,135,
+ * warpScheduler.cuh:339).  When one expires, the kernel does not compute on unfinished rows: it fills the affected
+ * output tile with NaN (which the combine carries into the affected rows of `out`), sets the stall word of the
+ * workspace and a host-visible word of the handle, and every kernel still exits normally.  From then on moe_forward /
+ * moe_get_task_counts on that handle return MOE_ERR_QUEUE_STALL (checked on the host, without
+ * synchronising) until moe_clear_stall.  moe_set_spin_limit sets the number of polls before a wait gives up
+ * (0 = the default, about 2^24; negative = every wait expires at once, which exercises this path from the host). */
+int moe_set_spin_limit(moe_handle* h, int32_t polls);
+int moe_clear_stall(moe_handle* h);
+
 /* Ceilings measured on the current device, to be quoted beside the published peaks: bf16 MFMA issue rate with no
  * memory traffic (scratch: >= 2 MiB of device memory, overwritten; random_operands = 0: all-zero operands, the
  * clock stays at its maximum; 1: random bf16 operands, the board's power limit lowers the clock -- this is the

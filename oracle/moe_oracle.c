@@ -240,8 +240,12 @@ void orc_gate_logits(const void* x, const void* gate_w, const float* gate_bias,
  * Top-k and gate weights.  Build-defined.  Selection is on the logits (softmax and sigmoid are monotone, so
  * the chosen set equals the one chosen on scores) by descending value, ties to the lower expert index.
  * Scores are fp32: softmax over all E experts, or elementwise sigmoid; with norm_topk the k selected
- * scores are divided by their sum (ascending rank).
+ * scores are divided by their sum (ascending rank).  The selection is total: a NaN logit ranks as -inf
+ * (behind every number; among themselves and with real -inf, lower index first), so every token gets k
+ * distinct valid experts; the scores are computed from the logits as stored, so such a token's weights
+ * are NaN where the arithmetic says so.
  * ---------------------------------------------------------------------------------------------- */
+static float topk_key(float v) { return v != v ? -INFINITY : v; }
 void orc_topk(const float* logits, int32_t S, int32_t E, int32_t k, int32_t gate_fn, int32_t norm_topk,
               int32_t* topk_idx, float* topk_w) {
 #pragma omp parallel
@@ -255,7 +259,7 @@ void orc_topk(const float* logits, int32_t S, int32_t E, int32_t k, int32_t gate
                 int32_t best = -1;
                 for (int32_t e = 0; e < E; ++e) {
                     if (taken[e]) continue;
-                    if (best < 0 || l[e] > l[best]) best = e;
+                    if (best < 0 || topk_key(l[e]) > topk_key(l[best])) best = e;
                 }
                 taken[best] = 1;
                 topk_idx[(int64_t)t * k + r] = best;
@@ -306,7 +310,10 @@ void orc_router_stats(const float* logits, const int32_t* topk_idx, int32_t S, i
         } else {
             for (int32_t e = 0; e < E; ++e) sum[e] += (double)(1.0f / (1.0f + expf(-l[e])));
         }
-        for (int32_t r = 0; r < k; ++r) cnt[topk_idx[(int64_t)t * k + r]] += 1;
+        for (int32_t r = 0; r < k; ++r) {
+            const int32_t e = topk_idx[(int64_t)t * k + r];
+            if (e >= 0 && e < E) cnt[e] += 1;   /* ids outside [0, E) are counted nowhere */
+        }
     }
     double aux = 0.0;
     for (int32_t e = 0; e < E; ++e) {
@@ -326,7 +333,8 @@ void orc_router_stats(const float* logits, const int32_t* topk_idx, int32_t S, i
  * pairs are numbered p = t*k + r; slot[p] = number of earlier pairs routed to the same expert (a stable
  * counting sort by expert id); with drop != 0, pairs whose slot >= capacity are dropped (slot = -1).
  * expert_count is the kept count, expert_offset its exclusive scan, and kept pair p lives in packed row
- * expert_offset[e] + slot[p]; token_indices[row] = t.
+ * expert_offset[e] + slot[p]; token_indices[row] = t.  A pair whose expert id lies outside [0, E) (only a
+ * caller-supplied topk_idx can hold one) is dropped like a pair over capacity.
  * ---------------------------------------------------------------------------------------------- */
 void orc_route(const int32_t* topk_idx, int32_t S, int32_t k, int32_t E, int32_t drop, int64_t capacity,
                int32_t* slot, int32_t* expert_count, int32_t* expert_offset, int32_t* token_indices,
@@ -335,6 +343,7 @@ void orc_route(const int32_t* topk_idx, int32_t S, int32_t k, int32_t E, int32_t
     int32_t* seen = (int32_t*)calloc((size_t)E, sizeof(int32_t));
     for (int64_t p = 0; p < A; ++p) {
         int32_t e = topk_idx[p];
+        if (e < 0 || e >= E) { slot[p] = -1; continue; }
         int32_t s = seen[e]++;
         slot[p] = (drop && s >= capacity) ? -1 : s;
     }
@@ -420,7 +429,7 @@ static inline float dot_w(const float* a, const void* W, const float* scales, in
 
 static inline float act_apply(float v, int act) {
     switch (act) {
-        case ORC_ACT_RELU: return v > 0.0f ? v : 0.0f;
+        case ORC_ACT_RELU: return v < 0.0f ? 0.0f : v;   /* a NaN stays a NaN, as with the reference's __hfma_relu */
         case ORC_ACT_GELU: return 0.5f * v * (1.0f + erff(v * 0.70710678118654752440f));
         default: return v;
     }

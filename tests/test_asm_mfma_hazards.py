@@ -18,18 +18,18 @@ WINDOW = 12   # instructions; a 16x16x32 bf16 MFMA takes 8 passes of 4 cycles
 _ASM = {}
 
 
-def _assembly():
-    if "text" not in _ASM:
-        src = os.path.join(moe_build.CSRC, "ffn_bf16.hip")
+def _assembly(name="ffn_bf16.hip"):
+    if name not in _ASM:
+        src = os.path.join(moe_build.CSRC, name)
         flags = [f for f in moe_build.FLAGS if f not in ("-fPIC",)]
         with tempfile.TemporaryDirectory() as tmp:
-            out = os.path.join(tmp, "ffn_bf16.s")
+            out = os.path.join(tmp, os.path.splitext(name)[0] + ".s")
             r = subprocess.run(["hipcc", *flags, "-S", "--cuda-device-only", "-I",
                                 os.path.join(moe_build.HERE, "..", "include"), "-o", out, src],
                                capture_output=True, text=True)
             assert r.returncode == 0, r.stderr[-2000:]
-            _ASM["text"] = open(out).read()
-    return _ASM["text"]
+            _ASM[name] = open(out).read()
+    return _ASM[name]
 
 
 @pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
@@ -95,3 +95,20 @@ def test_no_accumulator_access_behind_asm_mfma():
                     bad.append((line.strip(), seen, x))
     assert asm_mfmas >= 256, "the slab loop's inline-asm MFMAs were not found: has the kernel changed?"
     assert not bad, "accumulators touched behind an in-flight MFMA:\n" + "\n".join("%s -> +%d %s" % b for b in bad[:10])
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
+@pytest.mark.parametrize("source", ["ffn_bf16.hip", "ffn_f32.hip", "ffn_fp8.hip"])
+def test_phase0_results_are_complete_before_they_are_signalled(source):
+    """The hand-off of the intermediate rows between workgroups: in signal_phase0_done every wavefront must wait for
+    its own stores (s_waitcnt vmcnt(0)) before the workgroup barrier and the counter increment that publishes the
+    row block.  A workgroup-scope fence alone emits no such wait, so the wait is written out and checked here."""
+    text = _assembly(source)
+    m = re.search(r"\n(_ZN6moe355\w*signal_phase0_done\w*):[^\n]*\n(.*?)\n\s*s_setpc_b64", text, re.S)
+    assert m, "signal_phase0_done is no longer a function of its own (it must not be inlined)"
+    body = [x.strip() for x in m.group(2).split("\n") if x.strip() and not x.strip().startswith((";", "."))]
+    barrier = next(i for i, x in enumerate(body) if x.startswith("s_barrier"))
+    atomic = next(i for i, x in enumerate(body) if "atomic_add" in x)
+    # the wait written out in the source (the calling convention's wait at the function's entry does not count)
+    waits = [i for i, x in enumerate(body) if x == "s_waitcnt vmcnt(0)"]
+    assert waits and waits[0] < barrier < atomic, body[:20]

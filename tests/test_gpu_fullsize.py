@@ -1,7 +1,8 @@
 """The BASELINE configurations at full size on the GPU.
 
 The oracle cannot run a whole 5.8 TFLOP layer in test time, so: routing (integers) is compared in full, the
-layer output on a seeded sample of tokens, and the rest through properties that hold at any size (the two
+layer output on a stratified sample of tokens (each expert's first row, tail block, wavefront and row-block
+boundaries, plus a few hundred random tokens), and the rest through properties that hold at any size (the two
 independent FFN schedules agree bit for bit, fully dropped tokens are exactly zero, kept rows add up)."""
 import numpy as np
 import pytest
@@ -11,7 +12,32 @@ from helpers import OUT_TOL, from_device, max_rel_err, product_config, upload_in
 
 pytestmark = pytest.mark.gpu
 FFN_TILED, FFN_PERSISTENT = 1, 2
-SAMPLE = {"C2": 48, "C3": 16, "C4": 48, "C5": 24}
+RANDOM_TOKENS = {"C2": 512, "C3": 256, "C4": 512, "C5": 64}   # C5: all of its tokens
+MAX_STRATA_EXPERTS = 32
+
+
+def stratified_tokens(cfg, want, block_rows, seed=7):
+    """Tokens whose rows sit where a tile kernel is most likely to go wrong, plus a seeded random sample.
+
+    Per expert (the 32 most loaded when there are more): the first packed row, the last row (the end of the partial
+    tail block), the rows either side of the first 128-row wavefront boundary, either side of the first row-block
+    boundary, and the first row of the tail block.  Returns (tokens, strata) with strata a list of
+    (expert, slot, row block, what)."""
+    cnt, off, tok = want["expert_count"], want["expert_offset"], want["token_indices"]
+    experts = [int(e) for e in np.argsort(-cnt, kind="stable")[:MAX_STRATA_EXPERTS] if cnt[e] > 0]
+    strata = []
+    for e in sorted(experts):
+        n = int(cnt[e])
+        tail0 = (n - 1) // block_rows * block_rows
+        picks = {0: "first", n - 1: "last row of the tail block", tail0: "first row of the tail block"}
+        for b, what in ((128, "128-row wavefront boundary"), (block_rows, "row-block boundary")):
+            if n > b:
+                picks.setdefault(b - 1, "below the " + what)
+                picks.setdefault(b, "above the " + what)
+        for slot, what in sorted(picks.items()):
+            strata.append((e, slot, slot // block_rows, what))
+    chosen = [int(tok[off[e] + slot]) for e, slot, _, _ in strata]
+    return chosen, strata, np.random.default_rng(seed)
 
 
 @pytest.mark.parametrize("name", ["C2", "C3", "C4", "C5"])
@@ -39,12 +65,17 @@ def test_baseline_config_full_size(name):
         assert kept == cfg.S * cfg.k
     assert t0 > 0 and t1 > 0
 
-    # sampled output parity: tokens drawn with a fixed seed, always including a dropped-pair token if any
-    rng = np.random.default_rng(7)
-    tokens = rng.choice(cfg.S, size=SAMPLE[name], replace=False).astype(np.int32)
+    # sampled output parity: stratified rows (tails, wavefront and row-block boundaries) + a seeded random sample,
+    # always including a token with a dropped pair if there is one
+    chosen, strata, rng = stratified_tokens(cfg, want, layer.plan["block_rows"])
+    rand = rng.choice(cfg.S, size=min(RANDOM_TOKENS[name], cfg.S), replace=False)
     partly = np.nonzero((want["slot"] < 0).any(axis=1))[0]
-    if partly.size:
-        tokens[0] = partly[0]
+    tokens = np.unique(np.concatenate([chosen, rand, partly[:4]])).astype(np.int32)
+    tails = sum(1 for s_ in strata if "tail" in s_[3])
+    print(name, "block rows", layer.plan["block_rows"], "strata", len(strata), "over experts",
+          sorted({s_[0] for s_ in strata}), "tail rows", tails, "tokens checked", tokens.size, flush=True)
+    for s_ in strata[:12]:
+        print("   stratum expert %d slot %d row block %d: %s" % s_, flush=True)
     ref = ob.to_f32(ob.forward_tokens(cfg, inp, want["topk_idx"], want["topk_w"], want["slot"], tokens), cfg.act_dtype)
     o = out.float().cpu().numpy()
     err = max_rel_err(o[tokens], ref)

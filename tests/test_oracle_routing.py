@@ -181,3 +181,47 @@ def test_router_stats_vs_float64(gate_fn):
     assert abs(st["load"].sum() - 1.0) <= 1e-6
     if gate_fn == ob.GATE_SOFTMAX:
         assert abs(st["mean_prob"].sum() - 1.0) <= 1e-6
+
+
+def brute_topk_total(l, k):
+    """The total order: NaN ranks as -inf; value descending, index ascending."""
+    key = [(-np.inf if np.isnan(v) else float(v)) for v in l]
+    return sorted(range(len(l)), key=lambda e: (-key[e], e))[:k]
+
+
+def test_topk_is_total_with_nan_and_inf_logits():
+    """A NaN logit ranks as -inf: every token gets k distinct valid experts, numbers first."""
+    nan, inf = np.float32(np.nan), np.float32(np.inf)
+    rows = np.array([
+        [nan, nan, nan, nan, nan, nan],            # a token row that overflowed: experts 0..k-1
+        [nan, 1.0, nan, 3.0, 2.0, nan],            # numbers first, then NaN by index
+        [-inf, nan, -inf, 0.5, nan, -inf],         # NaN ties with a real -inf: lower index first
+        [inf, nan, 1.0, inf, 0.0, -1.0],
+        [0.1, 0.2, 0.3, 0.4, 0.5, 0.6],
+    ], np.float32)
+    for k in (1, 2, 4, 6):
+        for fn in (ob.GATE_SOFTMAX, ob.GATE_SIGMOID):
+            idx, w = ob.topk(rows, k, fn, 1)
+            for t in range(rows.shape[0]):
+                assert list(idx[t]) == brute_topk_total(rows[t], k), (t, k)
+                assert len(set(idx[t])) == k and idx[t].min() >= 0 and idx[t].max() < rows.shape[1]
+            assert np.isnan(w[0]).all()                       # weights follow the arithmetic: NaN in, NaN out
+            assert np.isfinite(w[4]).all() and abs(w[4].sum() - 1) < 1e-6
+    idx, _ = ob.topk(rows, 3, ob.GATE_SOFTMAX, 0)
+    assert list(idx[0]) == [0, 1, 2] and list(idx[1]) == [3, 4, 1] and list(idx[2]) == [3, 0, 1]
+
+
+def test_route_drops_expert_ids_outside_the_range():
+    """Only a caller-supplied topk_idx can hold them; such a pair is dropped and counted nowhere."""
+    E, k = 4, 2
+    idx = np.array([[0, 1], [7, 1], [-3, 0], [1, 2**31 - 1], [1, 3]], np.int32)
+    r = ob.route_slots(idx, E, 0, 100)
+    good = (idx >= 0) & (idx < E)
+    assert (r["slot"][~good] == -1).all() and (r["pair_row"][~good] == -1).all()
+    assert list(r["expert_count"]) == [2, 4, 0, 1]
+    assert r["expert_count"].sum() == good.sum()
+    rows = r["pair_row"][good]
+    assert sorted(rows) == list(range(good.sum()))
+    assert (r["token_indices"][good.sum():] == -1).all()
+    st_ = ob.router_stats(np.zeros((5, E), np.float32), idx, ob.GATE_SOFTMAX)
+    assert np.allclose(st_["load"] * 10, [2, 4, 0, 1])

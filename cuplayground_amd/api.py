@@ -24,7 +24,7 @@ EXPORTS = (
     "moe_config_default", "moe_config_from_json_string", "moe_config_from_json_file", "moe_config_validate",
     "moe_config_tokens", "moe_config_capacity", "moe_create", "moe_destroy", "moe_get_arch", "moe_get_plan",
     "moe_workspace_bytes",
-    "moe_set_ffn_mode", "moe_get_ffn_mode", "moe_forward", "moe_set_spin_limit", "moe_clear_stall", "moe_gate", "moe_router_stats", "moe_route", "moe_gemm_bias_act", "moe_combine",
+    "moe_set_ffn_mode", "moe_get_ffn_mode", "moe_forward", "moe_forward_static", "moe_set_spin_limit", "moe_clear_stall", "moe_gate", "moe_router_stats", "moe_route", "moe_gemm_bias_act", "moe_combine",
     "moe_set_stage_timing", "moe_get_stage_ms", "moe_get_task_counts", "moe_measure_mfma_tflops",
     "moe_measure_hbm_read_gbs", "moe_quant_block128", "moe_last_hip_error", "moe_status_string",
     "moe_version",
@@ -90,6 +90,7 @@ def load_library():
     L.moe_set_ffn_mode.argtypes = [vp, C.c_int]
     L.moe_get_ffn_mode.argtypes = [vp, C.POINTER(C.c_int32)]
     L.moe_forward.argtypes = [vp, vp, C.POINTER(_CWeights), vp, C.POINTER(_CRouting), vp, C.c_size_t, vp]
+    L.moe_forward_static.argtypes = [vp, vp, C.POINTER(_CWeights), vp, C.POINTER(_CRouting), vp]
     L.moe_set_spin_limit.argtypes = [vp, i32]
     L.moe_clear_stall.argtypes = [vp]
     L.moe_router_stats.argtypes = [vp, vp, vp, vp, vp, vp, vp, C.c_size_t, vp]
@@ -198,7 +199,7 @@ class MoELayer:
     WEIGHT_KEYS = ("gate_w", "gate_bias", "w_up", "w_gate", "w_down", "b_up", "b_gate", "b_down", "s_up", "s_gate",
                    "s_down")
 
-    def __init__(self, cfg: MoEConfig, ffn_mode: int = FFN_AUTO):
+    def __init__(self, cfg: MoEConfig, ffn_mode: int = FFN_AUTO, allocate_workspace: bool = True):
         import torch
         self.cfg = cfg
         self.L = load_library()
@@ -206,7 +207,9 @@ class MoELayer:
         c = cfg.to_c()
         _check(self.L.moe_create(C.byref(c), C.byref(self._h)), "moe_create")
         self.workspace_bytes = cfg.workspace_bytes()
-        self.workspace = torch.empty(self.workspace_bytes, dtype=torch.uint8, device="cuda")
+        # allocate_workspace=False: for callers that only use forward(static_workspace=True)
+        self.workspace = (torch.empty(self.workspace_bytes, dtype=torch.uint8, device="cuda")
+                          if allocate_workspace else None)
         self.S, self.k, self.E, self.H = cfg.tokens, cfg.expert_top_k, cfg.num_experts, cfg.hidden_size
         self.act_dtype = _torch_act_dtype(cfg.torch_dtype)
         if ffn_mode != FFN_AUTO:
@@ -284,8 +287,9 @@ class MoELayer:
                     expert_offset=torch.empty(E, dtype=torch.int32, device=dev),
                     token_indices=torch.empty(S * k, dtype=torch.int32, device=dev))
 
-    def forward(self, x, weights: dict, out=None, routing: dict | None = None):
-        """out[S,H] = MoE(x).  `routing` (from new_routing()) receives the routing result when given."""
+    def forward(self, x, weights: dict, out=None, routing: dict | None = None, static_workspace: bool = False):
+        """out[S,H] = MoE(x).  `routing` (from new_routing()) receives the routing result when given.
+        static_workspace: call moe_forward_static (the library's own per-GPU array instead of self.workspace)."""
         import torch
         if out is None:
             out = torch.empty(self.S, self.H, dtype=self.act_dtype, device=x.device)
@@ -294,8 +298,12 @@ class MoELayer:
         if routing is not None:
             r = _CRouting(*[routing[n].data_ptr() for n, _ in _CRouting._fields_])
         rp = C.byref(r) if r is not None else None
-        _check(self.L.moe_forward(self._h, _ptr(x), C.byref(w), _ptr(out), rp, _ptr(self.workspace),
-                                  self.workspace_bytes, _stream()), "moe_forward")
+        if static_workspace:
+            _check(self.L.moe_forward_static(self._h, _ptr(x), C.byref(w), _ptr(out), rp, _stream()),
+                   "moe_forward_static")
+        else:
+            _check(self.L.moe_forward(self._h, _ptr(x), C.byref(w), _ptr(out), rp, _ptr(self.workspace),
+                                      self.workspace_bytes, _stream()), "moe_forward")
         return out
 
     def set_spin_limit(self, polls: int):

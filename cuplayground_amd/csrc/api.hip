@@ -4,6 +4,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
 
 #include "moe_internal.hpp"
@@ -156,6 +157,29 @@ struct moe_handle {
     int last_hip;
 };
 
+// ---- the workspace of moe_forward_static: one array per GPU, owned by the code object, never allocated or freed ----
+// In host code the array's name is only a handle for hipGetSymbolAddress; the address the kernels need is looked up
+// once per device (with that device current) and kept in g_scratch_ptr.
+constexpr size_t kStaticScratchBytes = MOE355_STATIC_WORKSPACE_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+static void* g_scratch_ptr[kMaxDevices];
+static hipError_t g_scratch_err[kMaxDevices];
+static bool g_scratch_done[kMaxDevices];
+static std::mutex g_scratch_mutex;
+
+// Looks up this device's copy of `scratch` (the device must be current).  Called from moe_create.
+static void resolve_static_scratch(int dev) {
+    if (dev < 0 || dev >= kMaxDevices) return;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_done[dev]) return;
+    void* ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    g_scratch_err[dev] = e;
+    g_scratch_ptr[dev] = e == hipSuccess ? ptr : nullptr;
+    g_scratch_done[dev] = true;
+}
+
 namespace {
 
 int hip_fail(moe_handle* h, hipError_t e) {
@@ -298,6 +322,7 @@ int moe_create(const moe_config* cfg, moe_handle** out) {
         h->stall_host = static_cast<int32_t*>(p);
         *h->stall_host = 0;
     }
+    resolve_static_scratch(dev);
     *out = h;
     return MOE_OK;
 }
@@ -433,7 +458,7 @@ int moe_route(moe_handle* h, const int32_t* topk_idx, int32_t* slot, int32_t* ex
 
 namespace {
 
-// The whole layer.
+// The whole layer on a workspace that has passed check_ws (the caller's, or this device's static array).
 int forward_on(moe_handle* h, const void* x, const moe_weights* w, void* out, const moe_routing_out* routing,
                void* workspace, size_t workspace_bytes, void* stream) {
     if (!h || !x || !w || !out) return MOE_ERR_BAD_ARGUMENT;
@@ -539,6 +564,16 @@ extern "C" {
 int moe_forward(moe_handle* h, const void* x, const moe_weights* w, void* out, const moe_routing_out* routing,
                 void* workspace, size_t workspace_bytes, void* stream) {
     return forward_on(h, x, w, out, routing, workspace, workspace_bytes, stream);
+}
+
+int moe_forward_static(moe_handle* h, const void* x, const moe_weights* w, void* out, const moe_routing_out* routing,
+                       void* stream) {
+    if (!h) return MOE_ERR_BAD_ARGUMENT;
+    if (h->ws.total > kStaticScratchBytes) return MOE_ERR_WORKSPACE;   // the layer needs more than the array holds
+    const int dev = h->arch.device;
+    if (dev < 0 || dev >= kMaxDevices || !g_scratch_done[dev]) return MOE_ERR_NO_DEVICE;
+    if (!g_scratch_ptr[dev]) return hip_fail(h, g_scratch_err[dev]);
+    return forward_on(h, x, w, out, routing, g_scratch_ptr[dev], kStaticScratchBytes, stream);
 }
 
 int moe_set_spin_limit(moe_handle* h, int32_t polls) {

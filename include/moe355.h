@@ -143,6 +143,21 @@ int moe_get_ffn_mode(const moe_handle* h, int32_t* mode);
 int moe_forward(moe_handle* h, const void* x, const moe_weights* w, void* out, const moe_routing_out* routing,
                 void* workspace, size_t workspace_bytes, void* stream);
 
+/*
+ * moe_forward for callers that cannot allocate device memory at all -- code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc: the same layer, same kernels and same results, with the workspace taken
+ * from an array that is part of the library's device code (MOE355_STATIC_WORKSPACE_BYTES per GPU, held from the moment
+ * the library is loaded until the process ends) instead of from the caller.  It has no counterpart in the reference,
+ * whose drivers allocate one arena per run (mma.cuh:385-391).  Calls no hipMalloc / hipFree or any other allocating
+ * routine.  Returns MOE_ERR_WORKSPACE when moe_workspace_bytes(config) exceeds the array (decode-sized and small
+ * prefill layers fit; the Mixtral-shape intermediate does not).  Every call on a GPU uses that GPU's one array: calls
+ * that overlap in time on one GPU (two streams, two threads, two handles) race; calls in sequence on one stream are
+ * safe, each call re-initialises what it needs.
+ */
+#define MOE355_STATIC_WORKSPACE_BYTES ((size_t)32 << 20)
+int moe_forward_static(moe_handle* h, const void* x, const moe_weights* w, void* out, const moe_routing_out* routing,
+                       void* stream);
+
 /* ---- single stages, same kernels, for parity tests and callers that own the pipeline ---- */
 
 /* Router: logits = x.gate_w^T (+bias), top-k on logits, softmax|sigmoid weights.  logits may be NULL. */
@@ -190,7 +205,7 @@ int moe_get_task_counts(moe_handle* h, const void* workspace, void* stream, int6
  * warpScheduler.cuh:339).  When one expires, the kernel does not compute on unfinished rows: it fills the affected
  * output tile with NaN (which the combine carries into the affected rows of `out`), sets the stall word of the
  * workspace and a host-visible word of the handle, and every kernel still exits normally.  From then on moe_forward /
- * moe_get_task_counts on that handle return MOE_ERR_QUEUE_STALL (checked on the host, without
+ * moe_forward_static / moe_get_task_counts on that handle return MOE_ERR_QUEUE_STALL (checked on the host, without
  * synchronising) until moe_clear_stall.  moe_set_spin_limit sets the number of polls before a wait gives up
  * (0 = the default, about 2^24; negative = every wait expires at once, which exercises this path from the host). */
 int moe_set_spin_limit(moe_handle* h, int32_t polls);

@@ -2,17 +2,22 @@
 """Benchmark of the fused MoE forward on one MI355X.
 
 A step is one moe_forward call (gate -> slots -> expert FFN -> combine) on one batch of synthetic tokens already
-resident in HBM.  Default workload: the Mixtral-shape configuration (S=8192, H=4096, I=14336, E=8, top-2, SwiGLU,
+resident in HBM.  Headline workload: the Mixtral-shape configuration (S=8192, H=4096, I=14336, E=8, top-2, SwiGLU,
 bf16, dropless).  Prints one JSON line:
-  value      tokens/s of the whole layer
-  roofline   the expert-FFN kernel (the dominant launch) against the bf16 MFMA peak -- or the HBM peak for the fp8
-             decode shape -- from hipEvents recorded around that kernel inside the timed steps
-  cpu_baseline  the CPU oracle (a port: the reference's own CPU hook, torching.cuh:8-11, is empty) timed on a
-             bounded token sample of the same workload on this box's host cores
+  value         tokens/s of the whole layer, from the wall clock around the K timed steps
+  roofline      the expert-FFN kernel (the dominant launch) against the bf16 MFMA peak -- or the HBM peak for the fp8
+                decode shape -- from hipEvents recorded around that kernel inside the same K steps
+  cpu_baseline  the layer written with libtorch CPU ops (the role the reference reserves in torching.cuh:7-11 and
+                leaves empty), timed on this box's host cores on a bounded token sample; the CPU oracle's timing on
+                the same sample is given beside it
+  workloads     the other configurations (decode fp8, mid, fine-grained), each with its own step time, stage times
+                and roofline, measured the same way in the same run
 """
 import argparse
+import hashlib
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -20,53 +25,120 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
+PEAK_F32_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
+
 # Bytes per FFN-kernel launch that crossed the L2 <-> memory-fabric boundary, from two rocprofv3 --pmc runs of this
 # script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter showed for a 1 GiB
-# device copy in the same run (--calibrate-copy): read x2.000, write x1.000.  Summaries are kept under profiles/.
-MEASURED_TRAFFIC_BYTES = {"mixtral": 19.130e9 + 0.631e9, "decode_fp8": 9.924e9 + 0.013e9}
+# device copy in the same run (--calibrate-copy).  Each entry names the summary under profiles/ it comes from and the
+# digest of the kernel sources it was collected with: when the sources have changed since, the figure is withheld.
+KERNEL_SOURCES = ("ffn_bf16.hip", "ffn_bf16_slab_steady.inc", "ffn_fp8.hip", "ffn_common.hpp", "route.hip")
+MEASURED_TRAFFIC = {
+}
 
 
-def workloads():
-    from oracle import binding as ob
-    return {"mixtral": ("C3", ob.BASELINE["C3"]), "mid": ("C2", ob.BASELINE["C2"]),
-            "finegrained": ("C4", ob.BASELINE["C4"]), "decode_fp8": ("C5", ob.BASELINE["C5"]),
-            "tiny": ("C1", ob.BASELINE["C1"])}
+def kernel_digest():
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "cuplayground_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:12]
 
 
-def make_device_inputs(cfg, seed):
-    """Synthetic operands generated on the GPU: tokens N(0,1), weights N(0,0.02), rounded to storage."""
+def stats(samples):
+    if not samples:
+        return None
+    return {"mean": round(statistics.fmean(samples), 5), "median": round(statistics.median(samples), 5),
+            "min": round(min(samples), 5), "n": len(samples)}
+
+
+def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False):
+    """Runs one workload; returns (result dict, layer, device operands, output tensor, routing tensors)."""
     import torch
     import cuplayground_amd as moe
-    from oracle import binding as ob
-    g = torch.Generator(device="cuda").manual_seed(seed)
-    adt = torch.float32 if cfg.dtype == ob.F32 else torch.bfloat16
-    S, H, I, E = cfg.S, cfg.H, cfg.I, cfg.E
+    from cuplayground_amd import api, workloads as wl
 
-    def normal(shape, std, dtype):
-        out = torch.empty(shape, dtype=dtype, device="cuda")
-        n0 = shape[0]
-        for i in range(n0):            # expert by expert: bounds the fp32 temporary
-            out[i] = (torch.randn(shape[1:], generator=g, device="cuda", dtype=torch.float32) * std).to(dtype)
-        return out
+    w = wl.WORKLOADS[name]
+    c = w.config
+    layer = moe.MoELayer(c, ffn_mode=ffn_mode)
+    dev = wl.make_device_inputs(w, seed)
+    out = torch.empty(c.tokens, c.hidden_size, dtype=layer.act_dtype, device="cuda")
+    if calibrate_copy:
+        src = torch.zeros(1 << 30, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)              # reads 1 GiB and writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
+    for _ in range(warmup):
+        layer.forward(dev["x"], dev, out=out)
+    torch.cuda.synchronize()
+    layer.set_stage_timing(True)
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for a, b in ev:
+        a.record()
+        layer.forward(dev["x"], dev, out=out)
+        b.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    stage_mean = layer.stage_ms()
+    samples = layer.stage_samples()
+    layer.set_stage_timing(False)
+    step_ms = [a.elapsed_time(b) for a, b in ev]
+    ms_per_step = (t1 - t0) * 1e3 / steps
 
-    d = {"x": (torch.randn(S, H, generator=g, device="cuda", dtype=torch.float32)).to(adt),
-         "gate_w": (torch.randn(E, H, generator=g, device="cuda", dtype=torch.float32) * 0.02).to(adt)}
-    if cfg.zipf_bias:
-        d["gate_bias"] = torch.from_numpy(ob.zipf_gate_bias(E, seed)).cuda()
-    names = ["w_up", "w_down"] + (["w_gate"] if cfg.act == ob.ACT_SWIGLU else [])
-    for n in names:
-        shape = (E, H, I) if n == "w_down" else (E, I, H)
-        if cfg.dtype == ob.FP8:
-            w = normal(shape, 0.02, torch.float32)
-            d[n], d["s_" + n[2:]] = moe.quantize_block128(w)   # e4m3 codes + one scale per 128x128 block
-            del w
-        else:
-            d[n] = normal(shape, 0.02, adt)
-    return d
+    routing = layer.new_routing()                 # one extra, untimed call fetches the routing result
+    layer.forward(dev["x"], dev, out=out, routing=routing)
+    torch.cuda.synchronize()
+    tasks0, tasks1 = layer.task_counts()
+    cnt = routing["expert_count"].cpu().numpy()
+    kept = int(cnt.sum())
+    flops = wl.ffn_flops(c, kept)
+    layer_flops = flops + 2.0 * c.tokens * c.hidden_size * c.num_experts
+    ffn = stats(samples["ffn"][-steps:])
+    queue = layer.ffn_mode == 2   # one launch of the task-queue kernel; otherwise one launch per projection
+    fp8 = c.torch_dtype == api.DTYPE_FP8
+    if fp8:
+        active = int((cnt > 0).sum())
+        nbytes = wl.fp8_ffn_bytes(c, active, kept)
+        roof = {"bound": "hbm", "achieved": nbytes / (ffn["mean"] * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                "kernel": "ffn_persistent_fp8_kernel" if queue else "ffn_tiled_fp8_kernel x2",
+                "algorithmic_bytes": nbytes, "active_experts": active,
+                # the whole step held against the same bytes: what a caller of moe_forward sees
+                "layer_frac": nbytes / (ms_per_step * 1e-3) / 1e9 / PEAK_HBM_GBS}
+    else:
+        roof = {"bound": "mfma", "achieved": flops / (ffn["mean"] * 1e-3) / 1e12,
+                "peak": PEAK_F32_TFLOPS if c.torch_dtype == api.DTYPE_F32 else PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                "kernel": "ffn_persistent_kernel" if queue else "ffn_tiled_kernel x2", "algorithmic_flops": flops}
+        roof["layer_frac"] = layer_flops / (ms_per_step * 1e-3) / 1e12 / roof["peak"]
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["kernel_ms"] = ffn["mean"]
+    roof["kernel_ms_median"] = ffn["median"]
+    roof["kernel_ms_min"] = ffn["min"]
+    digest = kernel_digest()
+    t = MEASURED_TRAFFIC.get(name)
+    if queue and t and t["kernel_digest"] == digest:
+        roof["traffic"] = t["bytes"]
+        roof["traffic_source"] = "%s (kernel sources %s)" % (t["profile"], digest)
+    else:
+        roof["traffic"] = None
+        roof["traffic_source"] = ("kernel sources changed since %s was collected" % t["profile"]) if t and queue \
+            else "no counter run for this kernel"
+    res = {
+        "workload": w.describe(), "tokens_per_s": c.tokens / (ms_per_step * 1e-3), "ms_per_step": ms_per_step,
+        "step_ms": stats(step_ms), "steps": steps, "warmup": warmup,
+        "tflops": layer_flops / (ms_per_step * 1e-3) / 1e12,
+        "stage_ms": {k: round(v, 4) for k, v in stage_mean.items() if k != "calls"},
+        "stage_ms_median": {k: round(statistics.median(v[-steps:]), 4) for k, v in samples.items()},
+        "ffn_mode": layer.ffn_mode, "block_rows": layer.plan["block_rows"],
+        "persistent_blocks": layer.arch["persistent_blocks"], "kept_assignments": kept, "tile_tasks": [tasks0, tasks1],
+        "roofline": roof,
+    }
+    return res, layer, dev, out, routing
 
 
-def to_host(cfg, d):
+def to_host(d):
     """Device operands -> the numpy layout the oracle takes (bf16 as uint16 bit patterns)."""
     import numpy as np
     import torch
@@ -79,12 +151,112 @@ def to_host(cfg, d):
     return out
 
 
+def cpu_leg(name, dev, out, routing, seconds, seed):
+    """The CPU baseline (libtorch layer, then the oracle) on a bounded token sample, and the parity spot check of the
+    GPU output against the oracle on the same sample.  The only part of this script that touches oracle/."""
+    import numpy as np
+    import torch
+    from cuplayground_amd import api, workloads as wl
+    from cuplayground_amd.torch_op import torch_cpu_layer
+    from oracle import binding as ob
+
+    w = wl.WORKLOADS[name]
+    c = w.config
+    S = c.tokens
+    fp8 = c.torch_dtype == api.DTYPE_FP8
+    threads = os.cpu_count() or 1
+    env = os.environ.get("OMP_NUM_THREADS")
+    if env and env.isdigit():
+        threads = int(env)
+    torch.set_num_threads(threads)
+    rng = np.random.default_rng(seed)
+    order = rng.permutation(S)
+
+    # ---- libtorch CPU layer: weights widened once (bf16 -> fp32; e4m3 -> bf16) outside the timed region ----
+    host = {k: v.cpu() for k, v in dev.items()}
+    if fp8:
+        def deq(q, s):
+            wq = q.view(torch.float8_e4m3fn).to(torch.float32)
+            E, N, K = wq.shape
+            wq = wq.view(E, N // 128, 128, K // 128, 128) * s.view(E, N // 128, 1, K // 128, 1)
+            return wq.view(E, N, K).to(torch.bfloat16)
+        cw = {n: deq(host[n], host["s_" + n[2:]]) for n in ("w_up", "w_gate", "w_down")}
+        prep = "e4m3 weights dequantised to bf16 once outside the timed region, bf16 linear"
+    elif c.torch_dtype == api.DTYPE_BF16:
+        cw = {n: host[n].float() for n in ("w_up", "w_gate", "w_down") if n in host}
+        prep = "bf16 storage, weights widened to fp32 once outside the timed region, fp32 matmul"
+    else:
+        cw = {n: host[n] for n in ("w_up", "w_gate", "w_down") if n in host}
+        prep = "fp32"
+
+    def run_torch(tokens):
+        import dataclasses
+        sub = dataclasses.replace(c, micro_batch=1, sequence_len=len(tokens))
+        xs = host["x"][torch.from_numpy(tokens.astype(np.int64))]
+        t = time.perf_counter()
+        o, idx = torch_cpu_layer(xs, sub, host["gate_w"], cw["w_up"], cw.get("w_gate"), cw["w_down"],
+                                 host.get("gate_bias"))
+        return time.perf_counter() - t, o, idx
+
+    n0 = min(S, 64)
+    dt0, _, _ = run_torch(order[:n0])                       # warm-up of the thread pool and a first estimate
+    dt0, _, _ = run_torch(order[:n0])
+    n = int(min(S, max(n0, seconds * n0 / max(dt0, 1e-6))))
+    dt, o_cpu, idx_cpu = run_torch(order[:n])
+    libtorch = {"value": n / dt, "unit": "tokens/s", "cores": threads, "kind": "port", "engine": "libtorch",
+                "sample": "%d of %d tokens through the whole layer in libtorch CPU ops (linear, softmax/sigmoid, topk, "
+                          "stable sort, index_select, per-expert linear/act/linear, index_add; %s), %.1f s on %d threads"
+                          % (n, S, prep, dt, threads)}
+    # the same tokens on the GPU: rows agree where the CPU router picked the same experts (its fp32 sum runs in
+    # another order, so near-ties may differ) and no capacity drop depends on the rest of the batch
+    sel = torch.from_numpy(order[:n].astype(np.int64))
+    same = (idx_cpu == routing["topk_idx"].cpu()[sel].long()).all(dim=1).numpy()
+    if not c.drop_tokens and same.any():
+        g = out[sel.cuda()].float().cpu().numpy()[same]
+        r = o_cpu.float().numpy()[same]
+        libtorch["max_rel_err_gpu_vs_libtorch"] = float(np.abs(g - r).max() / max(np.abs(r).max(), 1e-30))
+        libtorch["tokens_with_same_routing"] = int(same.sum())
+    del cw
+
+    # ---- the CPU oracle on (a part of) the same sample + parity of the GPU output ----
+    ocfg = ob.Cfg(S=S, H=c.hidden_size, I=c.intermediate_size, E=c.num_experts, k=c.expert_top_k, act=c.hidden_act,
+                  dtype=c.torch_dtype, gate_fn=c.gate_fn, norm_topk=c.norm_topk_prob, drop=c.drop_tokens,
+                  capacity_factor=c.capacity_factor, zipf_bias=w.zipf_bias)
+    hostnp = to_host(dev)
+    r = {k: v.cpu().numpy() for k, v in routing.items()}
+    tok = order.astype(np.int32)
+    m0 = min(4, S)
+    t = time.perf_counter()
+    rows = ob.forward_tokens(ocfg, hostnp, r["topk_idx"], r["topk_w"], r["slot"], tok[:m0])
+    d0 = time.perf_counter() - t
+    extra = int(min(S - m0, max(0, 0.5 * seconds / max(d0 / m0, 1e-9) - m0)))
+    if extra > 0:
+        t = time.perf_counter()
+        rows2 = ob.forward_tokens(ocfg, hostnp, r["topk_idx"], r["topk_w"], r["slot"], tok[m0:m0 + extra])
+        d0 += time.perf_counter() - t
+        rows = np.concatenate([rows, rows2])
+        m0 += extra
+    oracle = {"value": m0 / d0, "unit": "tokens/s", "cores": ob.num_threads(), "kind": "port", "engine": "oracle (C11 + OpenMP)",
+              "sample": "%d of %d tokens through the oracle's expert FFN + combine (routing taken as given), %.1f s"
+                        % (m0, S, d0)}
+    got = out[torch.from_numpy(tok[:m0].astype(np.int64)).cuda()].float().cpu().numpy()
+    ref = ob.to_f32(rows, ocfg.act_dtype)
+    parity = float(np.abs(got - ref).max() / max(np.abs(ref).max(), 1e-30))
+    want = ob.route(ocfg, hostnp)
+    exact = all(np.array_equal(r[k], want[k]) for k in ("topk_idx", "slot", "expert_count"))
+    return libtorch, oracle, {"routing_bit_exact": exact, "max_rel_err_sample": parity, "sample_tokens": m0}
+
+
 def main():
+    from cuplayground_amd import workloads as wl
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="mixtral", choices=sorted(workloads()))
+    ap.add_argument("--workload", default="mixtral", choices=sorted(wl.WORKLOADS))
+    ap.add_argument("--extra", default="decode_fp8,mid,finegrained",
+                    help="comma-separated workloads measured besides the headline one (\"\" or none: skip)")
+    ap.add_argument("--extra-steps", type=int, default=20)
     ap.add_argument("--ffn-mode", type=int, default=0, help="0 auto, 1 tiled (two launches), 2 persistent queue")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample (0 = skip)")
     ap.add_argument("--seed", type=int, default=42)
@@ -96,122 +268,62 @@ def main():
               "supported (no collectives, no sharding across GPUs)" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
-    import numpy as np
     import torch
     import cuplayground_amd as moe
-    from oracle import binding as ob
+    from cuplayground_amd import api
 
-    tag, cfg = workloads()[args.workload]
     torch.cuda.set_device(0)
     moe.load_library()
-    pc = moe.MoEConfig(capacity_factor=cfg.capacity_factor, drop_tokens=cfg.drop, expert_top_k=cfg.k,
-                       hidden_act=cfg.act, hidden_size=cfg.H, intermediate_size=cfg.I, micro_batch=1,
-                       num_experts=cfg.E, sequence_len=cfg.S, torch_dtype=cfg.dtype, gate_fn=cfg.gate_fn,
-                       norm_topk_prob=cfg.norm_topk)
-    layer = moe.MoELayer(pc, ffn_mode=args.ffn_mode)
-    dev = make_device_inputs(cfg, args.seed)
-    routing = layer.new_routing()
-    out = torch.empty(cfg.S, cfg.H, dtype=layer.act_dtype, device="cuda")
-
-    if args.calibrate_copy:
-        src = torch.zeros(1 << 30, dtype=torch.uint8, device="cuda")
-        dst = torch.empty_like(src)
-        torch.cuda.synchronize()
-        dst.copy_(src)              # reads 1 GiB and writes 1 GiB
-        torch.cuda.synchronize()
-        del src, dst
-    for _ in range(args.warmup):
-        layer.forward(dev["x"], dev, out=out, routing=routing)
-    torch.cuda.synchronize()
-    layer.set_stage_timing(True)
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        layer.forward(dev["x"], dev, out=out, routing=routing)
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    stage = layer.stage_ms()
-    layer.set_stage_timing(False)
-    tasks0, tasks1 = layer.task_counts()
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
-
-    cnt = routing["expert_count"].cpu().numpy()
-    kept = int(cnt.sum())
-    g = 3 if cfg.act == ob.ACT_SWIGLU else 2
-    ffn_flops = 2.0 * g * kept * cfg.H * cfg.I
-    layer_flops = ffn_flops + 2.0 * cfg.S * cfg.H * cfg.E
-    ffn_s = stage["ffn"] * 1e-3
-    queue = layer.ffn_mode == 2   # one launch of the task-queue kernel; otherwise one launch per projection
-    if cfg.dtype == ob.FP8:
-        active = int((cnt > 0).sum())
-        scale_bytes = 3 * (cfg.H // 128) * (cfg.I // 128) * 4
-        ffn_bytes = active * (3.0 * cfg.H * cfg.I + scale_bytes) + 2.0 * kept * cfg.H * 2
-        roofline = {"bound": "hbm", "achieved": ffn_bytes / ffn_s / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                    "traffic": None, "kernel": "ffn_persistent_fp8_kernel" if queue else "ffn_tiled_fp8_kernel x2", "kernel_ms": stage["ffn"],
-                    "algorithmic_bytes": ffn_bytes, "active_experts": active}
-    else:
-        roofline = {"bound": "mfma", "achieved": ffn_flops / ffn_s / 1e12, "peak": PEAK_BF16_TFLOPS,
-                    "unit": "TFLOP/s", "traffic": None, "kernel": "ffn_persistent_kernel" if queue else "ffn_tiled_kernel x2", "kernel_ms": stage["ffn"],
-                    "algorithmic_flops": ffn_flops}
-        if cfg.dtype == ob.F32:
-            roofline["peak"] = 157.3
-    roofline["frac"] = roofline["achieved"] / roofline["peak"]
-    roofline["traffic"] = MEASURED_TRAFFIC_BYTES.get(args.workload) if queue else None
+    main_w = wl.WORKLOADS[args.workload]
+    res, layer, dev, out, routing = measure(args.workload, args.steps, args.warmup, args.seed, args.ffn_mode,
+                                            args.calibrate_copy)
+    arch = layer.arch
     # ceilings measured on this box in this run (the published peaks assume the maximum clock)
     peaks = moe.measured_peaks()
-    arch = layer.arch
+    roof = res["roofline"]
     # for the MFMA bound: the issue-only rate on random operands (the power limit lowers the clock on real data)
-    roofline["measured_peak"] = peaks["hbm_read_gbs"] if cfg.dtype == ob.FP8 else peaks["mfma_bf16_tflops_random_operands"]
-    roofline["frac_of_measured_peak"] = roofline["achieved"] / roofline["measured_peak"]
+    fp8 = main_w.config.torch_dtype == api.DTYPE_FP8
+    roof["measured_peak"] = peaks["hbm_read_gbs"] if fp8 else peaks["mfma_bf16_tflops_random_operands"]
+    roof["frac_of_measured_peak"] = roof["achieved"] / roof["measured_peak"]
 
-    # ---- CPU baseline + parity spot check on the same sample ----
-    cpu = None
-    parity = None
+    cpu = cpu_oracle = parity = None
     if args.cpu_seconds > 0:
-        host = to_host(cfg, dev)
-        r = {k: v.cpu().numpy() for k, v in routing.items()}
-        rng = np.random.default_rng(args.seed)
-        order = rng.permutation(cfg.S).astype(np.int32)
-        n = min(4, cfg.S)
-        t = time.perf_counter()
-        rows = ob.forward_tokens(cfg, host, r["topk_idx"], r["topk_w"], r["slot"], order[:n])
-        dt = time.perf_counter() - t
-        extra = int(min(cfg.S - n, max(0, args.cpu_seconds / max(dt / n, 1e-9) - n)))
-        if extra > 0:
-            t = time.perf_counter()
-            rows2 = ob.forward_tokens(cfg, host, r["topk_idx"], r["topk_w"], r["slot"], order[n:n + extra])
-            dt += time.perf_counter() - t
-            rows = np.concatenate([rows, rows2])
-            n += extra
-        cpu = {"value": n / dt, "unit": "tokens/s", "cores": ob.num_threads(), "kind": "port",
-               "sample": "%d of %d tokens through the CPU oracle's expert FFN + combine (routing taken as given), "
-                         "%.1f s" % (n, cfg.S, dt)}
-        got = out[torch.from_numpy(order[:n].astype(np.int64)).cuda()]
-        got = got.float().cpu().numpy()
-        ref = ob.to_f32(rows, cfg.act_dtype)
-        parity = float(np.abs(got - ref).max() / max(np.abs(ref).max(), 1e-30))
-        want = ob.route(cfg, host)
-        routing_exact = all(np.array_equal(r[k], want[k]) for k in ("topk_idx", "slot", "expert_count"))
-    else:
-        routing_exact = None
+        cpu, cpu_oracle, parity = cpu_leg(args.workload, dev, out, routing, args.cpu_seconds, args.seed)
+    layer.close()
+    del layer, dev, out, routing
+    torch.cuda.empty_cache()
 
+    others = {}
+    extra = [e for e in args.extra.split(",") if e and e != "none" and e != args.workload]
+    for name in extra:
+        if name not in wl.WORKLOADS:
+            print("bench.py: unknown workload %r in --extra" % name, file=sys.stderr)
+            sys.exit(2)
+        r, l2, d2, o2, rt2 = measure(name, args.extra_steps, args.warmup, args.seed, args.ffn_mode)
+        l2.close()
+        del l2, d2, o2, rt2
+        torch.cuda.empty_cache()
+        others[name] = r
+
+    dtype = {api.DTYPE_F32: "f32", api.DTYPE_BF16: "bf16", api.DTYPE_FP8: "fp8_e4m3_w/bf16_act"}
     line = {
         "metric": "MoE layer forward tokens/s (%s shape, 1 MI355X)" % args.workload,
-        "value": cfg.S / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": {ob.F32: "f32", ob.BF16: "bf16", ob.FP8: "fp8_e4m3_w/bf16_act"}[cfg.dtype],
-        "data": "synthetic",
-        "config": {"workload": "%s: S=%d H=%d I=%d E=%d top%d %s %s" % (
-            tag, cfg.S, cfg.H, cfg.I, cfg.E, cfg.k, {0: "relu", 1: "gelu", 2: "swiglu"}[cfg.act],
-            "drop cf=%g" % cfg.capacity_factor if cfg.drop else "dropless"),
-            "ffn_mode": layer.ffn_mode, "persistent_blocks": layer.arch["persistent_blocks"], "kept_assignments": kept, "tile_tasks": [tasks0, tasks1]},
-        "tflops": layer_flops / (ms_per_step * 1e-3) / 1e12,
-        "stage_ms": {k: round(v, 4) for k, v in stage.items()},
-        "device": {"name": arch["name"], "compute_units": arch["compute_units"], "max_clock_khz": arch["max_clock_khz"],
+        "value": res["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": res["ms_per_step"], "step_ms": res["step_ms"],
+        "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": dtype[main_w.config.torch_dtype], "data": "synthetic",
+        "config": {"workload": res["workload"], "ffn_mode": res["ffn_mode"], "block_rows": res["block_rows"],
+                   "persistent_blocks": res["persistent_blocks"], "kept_assignments": res["kept_assignments"],
+                   "tile_tasks": res["tile_tasks"]},
+        "tflops": res["tflops"],
+        "stage_ms": res["stage_ms"], "stage_ms_median": res["stage_ms_median"],
+        "device": {"name": arch["name"], "compute_units": arch["compute_units"], "xcds": arch["xcds"],
+                   "max_clock_khz": arch["max_clock_khz"],
                    "measured_mfma_bf16_tflops": round(peaks["mfma_bf16_tflops"], 1),
                    "measured_mfma_bf16_tflops_random_operands": round(peaks["mfma_bf16_tflops_random_operands"], 1),
                    "measured_hbm_read_gbs": round(peaks["hbm_read_gbs"], 1)},
-        "roofline": roofline, "cpu_baseline": cpu,
-        "parity": {"routing_bit_exact": routing_exact, "max_rel_err_sample": parity},
+        "roofline": roof, "cpu_baseline": cpu, "cpu_baseline_oracle": cpu_oracle, "parity": parity,
+        "workloads": others,
     }
     print(json.dumps(line))
 

@@ -25,7 +25,7 @@ EXPORTS = (
     "moe_config_tokens", "moe_config_capacity", "moe_create", "moe_destroy", "moe_get_arch", "moe_get_plan",
     "moe_workspace_bytes",
     "moe_set_ffn_mode", "moe_get_ffn_mode", "moe_forward", "moe_forward_static", "moe_set_spin_limit", "moe_clear_stall", "moe_gate", "moe_router_stats", "moe_route", "moe_gemm_bias_act", "moe_combine",
-    "moe_set_stage_timing", "moe_get_stage_ms", "moe_get_task_counts", "moe_measure_mfma_tflops",
+    "moe_set_stage_timing", "moe_get_stage_ms", "moe_get_stage_samples", "moe_get_task_counts", "moe_measure_mfma_tflops",
     "moe_measure_hbm_read_gbs", "moe_quant_block128", "moe_last_hip_error", "moe_status_string",
     "moe_version",
 )
@@ -100,6 +100,7 @@ def load_library():
     L.moe_combine.argtypes = [vp, vp, vp, i32, i32, i32, i32, vp, vp]
     L.moe_set_stage_timing.argtypes = [vp, C.c_int]
     L.moe_get_stage_ms.argtypes = [vp, C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_int32)]
+    L.moe_get_stage_samples.argtypes = [vp, C.c_int, C.POINTER(C.c_float), C.c_int32, C.POINTER(C.c_int32)]
     L.moe_get_task_counts.argtypes = [vp, vp, vp, C.POINTER(i64), C.POINTER(i64)]
     L.moe_quant_block128.argtypes = [vp, C.c_int32, C.c_int64, C.c_int64, C.c_int64, vp, vp, vp]
     L.moe_measure_mfma_tflops.argtypes = [vp, C.c_size_t, vp, C.c_int, C.POINTER(C.c_float)]
@@ -262,6 +263,17 @@ class MoELayer:
             _check(self.L.moe_get_stage_ms(self._h, i, C.byref(v), C.byref(calls)))
             out[n] = v.value
         out["calls"] = calls.value
+        return out
+
+    def stage_samples(self) -> dict:
+        """Per-call milliseconds of every stage and of the whole call ("total") for the most recent recorded calls
+        (64 at most), oldest first."""
+        out = {}
+        buf = (C.c_float * 64)()
+        n = C.c_int32(0)
+        for i, name in enumerate(STAGES + ("total",)):
+            _check(self.L.moe_get_stage_samples(self._h, i, buf, 64, C.byref(n)))
+            out[name] = [buf[j] for j in range(n.value)]
         return out
 
     def task_counts(self):

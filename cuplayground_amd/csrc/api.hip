@@ -397,6 +397,23 @@ int moe_get_stage_ms(moe_handle* h, int stage, float* ms, int32_t* calls) {
     return MOE_OK;
 }
 
+int moe_get_stage_samples(moe_handle* h, int stage, float* ms, int32_t capacity, int32_t* count) {
+    if (!h || !ms || !count || capacity < 1 || stage < 0 || stage > MOE_STAGE_COUNT) return MOE_ERR_BAD_ARGUMENT;
+    if (!h->ev_valid || h->ev_calls < 1) return MOE_ERR_BAD_ARGUMENT;
+    int n = (int)(h->ev_calls < kTimedCalls ? h->ev_calls : kTimedCalls);
+    if (n > capacity) n = capacity;
+    for (int i = 0; i < n; ++i) {   // oldest of the n most recent calls first
+        const int row = (int)((h->ev_calls - n + i) % kTimedCalls);
+        hipError_t rc = hipEventSynchronize(h->ev[row][MOE_STAGE_COUNT]);
+        if (rc != hipSuccess) return hip_fail(h, rc);
+        const int a = stage == MOE_STAGE_COUNT ? 0 : stage, b = stage == MOE_STAGE_COUNT ? MOE_STAGE_COUNT : stage + 1;
+        rc = hipEventElapsedTime(&ms[i], h->ev[row][a], h->ev[row][b]);
+        if (rc != hipSuccess) return hip_fail(h, rc);
+    }
+    *count = n;
+    return MOE_OK;
+}
+
 int moe_last_hip_error(const moe_handle* h) { return h ? h->last_hip : 0; }
 
 int moe_gate(moe_handle* h, const void* x, const void* gate_w, const float* gate_bias, float* logits,

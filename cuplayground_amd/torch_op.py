@@ -187,4 +187,47 @@ def torch_reference(x, cfg: api.MoEConfig, gate_w, w_up, w_gate, w_down, gate_bi
     return out.to(dt)
 
 
-__all__ = ["MoE355", "torch_reference"]
+def torch_cpu_layer(x, cfg: api.MoEConfig, gate_w, w_up, w_gate, w_down, gate_bias=None):
+    """The layer as a libtorch program on the host -- the CPU computation the reference reserves a hook for and leaves
+    empty (`torching.cuh:7-11`, libtorch linked at `CMakeLists.txt:126-133`): linear -> softmax / sigmoid -> topk ->
+    stable sort by expert -> index_select -> per-expert linear / activation / linear -> index_add.  Tensors live on
+    the CPU; matmuls run in the dtype of the weights handed in (hand fp32 weights for fp32 accumulation from bf16
+    storage), the intermediate and the output are rounded to x.dtype.  Used as the timed CPU baseline; also runs on
+    GPU tensors.  Returns (out [S,H], topk_idx [S,k])."""
+    F = torch.nn.functional
+    S, k, E = x.shape[0], cfg.expert_top_k, cfg.num_experts
+    cdt = w_up.dtype
+    logits = F.linear(x.float(), gate_w.float())
+    if gate_bias is not None:
+        logits = logits + gate_bias
+    scores = torch.softmax(logits, dim=1) if cfg.gate_fn == api.GATE_SOFTMAX else torch.sigmoid(logits)
+    w, idx = torch.topk(scores, k, dim=1)
+    if cfg.norm_topk_prob:
+        w = w / w.sum(1, keepdim=True)
+    flat = idx.reshape(-1)
+    order = torch.sort(flat, stable=True).indices           # pairs grouped by expert, token order kept
+    counts = torch.bincount(flat, minlength=E)
+    starts = torch.cumsum(counts, 0) - counts
+    kept = torch.clamp(counts, max=cfg.capacity) if cfg.drop_tokens else counts
+    out = torch.zeros(S, x.shape[1], dtype=torch.float32, device=x.device)
+    wflat = w.reshape(-1)
+    for e in range(E):
+        n = int(kept[e])
+        if n == 0:
+            continue
+        pairs = order[int(starts[e]):int(starts[e]) + n]
+        tok = pairs // k
+        xe = x.index_select(0, tok).to(cdt)
+        up = F.linear(xe, w_up[e])
+        if cfg.hidden_act == api.ACT_SWIGLU:
+            h = F.silu(F.linear(xe, w_gate[e])) * up
+        elif cfg.hidden_act == api.ACT_GELU:
+            h = F.gelu(up)
+        else:
+            h = torch.relu(up)
+        y = F.linear(h.to(x.dtype).to(cdt), w_down[e]).to(x.dtype).float()
+        out.index_add_(0, tok, y * wflat[pairs].unsqueeze(1))
+    return out.to(x.dtype), idx
+
+
+__all__ = ["MoE355", "torch_reference", "torch_cpu_layer"]

@@ -197,6 +197,10 @@ int moe_set_stage_timing(moe_handle* h, int enable);
 /* Mean milliseconds of stage `stage` over the moe_forward calls recorded since timing was enabled (the most
  * recent 64 at most); *calls (may be NULL) receives how many were averaged.  Synchronises on their events. */
 int moe_get_stage_ms(moe_handle* h, int stage, float* ms, int32_t* calls);
+/* The single measurements behind moe_get_stage_ms: milliseconds of `stage` (or, with stage = MOE_STAGE_COUNT, of the
+ * whole call from its first to its last kernel) for each of the most recent recorded calls, oldest first, at most
+ * `capacity` (and at most 64) of them; *count receives how many were written.  For medians and minima. */
+int moe_get_stage_samples(moe_handle* h, int stage, float* ms, int32_t capacity, int32_t* count);
 /* Tile tasks the FFN stage of the last moe_forward issued to its queue (GEMM0 tasks, GEMM1 tasks); reads
  * back a few words from the workspace, so it synchronises the stream. */
 int moe_get_task_counts(moe_handle* h, const void* workspace, void* stream, int64_t* gemm0_tasks, int64_t* gemm1_tasks);

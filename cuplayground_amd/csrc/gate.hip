@@ -8,7 +8,10 @@
 // lane l of a wavefront owns partial sum l and takes, in ascending k, every k with (k/8) % 64 == l using
 // one fmaf per element; the 64 partials are folded by an xor butterfly (32,16,8,4,2,1); the bias is added
 // last.  Top-k is taken on the logits (softmax and sigmoid are monotone), ties to the lower expert index.
+#include <cstdlib>
+
 #include "moe_internal.hpp"
+#include "topk.hpp"
 
 namespace moe355 {
 namespace {
@@ -157,85 +160,167 @@ hipError_t launch_gate_typed(const void* x, const void* gate_w, const float* gat
     return hipErrorInvalidValue;
 }
 
-struct Cand {
-    float v;
-    int i;
+// ---- second logits kernel: register tiles of (tokens x experts), K streamed ----
+//
+// The kernel above keeps whole token rows in registers and walks the experts one after the other, one 16-byte load
+// in flight per chunk: with many experts or few tokens it waits on memory latency most of the time.  Here a wavefront
+// owns TT tokens x TE experts (TT * TE running sums per lane), walks K in steps of one 8-element chunk per lane
+// (chunk c = lane + 64 j, exactly the elements partial sum `lane` takes), and has the TT + TE loads of the next step
+// in flight while it works on the current one.  Every sum sees the same fmaf sequence and the same fold as above, so
+// the logits are bit-identical.  A workgroup is WT x WE wavefronts over (tokens, experts); neighbouring wavefronts
+// read the same rows at the same time and share them in the compute unit's L1.
+template <typename T>
+struct RawChunk {
+    typedef unsigned int type __attribute__((ext_vector_type(sizeof(T) == 4 ? 8 : 4)));
 };
-__device__ __forceinline__ bool better(const Cand& a, const Cand& b) {
-    return a.v > b.v || (a.v == b.v && a.i < b.i);
+
+template <typename T>
+__device__ __forceinline__ void widen8(const typename RawChunk<T>::type& r, float (&v)[8]) {
+    if constexpr (sizeof(T) == 4) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = __uint_as_float(r[i]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = __uint_as_float(r[i] << 16);
+            v[2 * i + 1] = __uint_as_float(r[i] & 0xFFFF0000u);
+        }
+    }
 }
 
-// One wavefront per token; lane l keeps logits of experts l, l+64, ... (at most 8) in registers.
-// The selection is total: a NaN logit ranks as -inf (behind every number, ties to the lower index), so a token row
-// that overflowed still gets k distinct, valid experts; its weights are computed from the logits as they are and
-// come out NaN, which is what reaches the output of that token and of no other.
+// Folds the 64 per-lane partial sums of 16 independent sums at once.  At xor distance 32, 16, 8, 4 a lane keeps one
+// register of each pair and hands the other to its partner (halving the registers per step), then distances 2 and 1
+// on the one register left.  Each sum adds lane l to lane l ^ d for d = 32, 16, 8, 4, 2, 1 in that order: the result
+// has the bits of the plain butterfly.  Returns the sum of red[index] with index = fold16_index(lane), valid in the
+// lanes with (lane & 3) == 0.
+__device__ __forceinline__ float fold16(float (&red)[16], int lane) {
+#pragma unroll
+    for (int step = 0; step < 4; ++step) {
+        const int off = 32 >> step, n = 16 >> step;
+        const bool hi = (lane & off) != 0;
+#pragma unroll
+        for (int i = 0; i < n / 2; ++i) {
+            const float keep = hi ? red[2 * i + 1] : red[2 * i];
+            const float send = hi ? red[2 * i] : red[2 * i + 1];
+            red[i] = keep + __shfl_xor(send, off, kWave);
+        }
+    }
+    float sum = red[0];
+    sum = sum + __shfl_xor(sum, 2, kWave);
+    sum = sum + __shfl_xor(sum, 1, kWave);
+    return sum;
+}
+__device__ __forceinline__ int fold16_index(int lane) {
+    return ((lane >> 5) & 1) | (((lane >> 4) & 1) << 1) | (((lane >> 3) & 1) << 2) | (((lane >> 2) & 1) << 3);
+}
+
+template <typename T, int TT, int TE, int WT, int WE>
+__global__ __launch_bounds__(WT * WE * 64) void gate_tile_kernel(const T* __restrict__ x, const T* __restrict__ gate_w,
+                                                                 const float* __restrict__ gate_bias,
+                                                                 float* __restrict__ logits, int S, int H, int E) {
+    static_assert((TT * TE) % 16 == 0 && 16 % TT == 0, "sums are folded sixteen at a time: TT tokens x 16/TT experts");
+    typedef typename RawChunk<T>::type raw_t;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int t0 = (blockIdx.x * WT + wave / WE) * TT, e0 = (blockIdx.y * WE + wave % WE) * TE;
+    if (t0 >= S || e0 >= E) return;
+    const int nchunk = H >> 3, nstep = (nchunk + kWave - 1) / kWave;
+    const T* xrow[TT];
+    const T* wrow[TE];
+#pragma unroll
+    for (int q = 0; q < TT; ++q) xrow[q] = x + (size_t)min(t0 + q, S - 1) * H + lane * 8;    // rows past the end are
+#pragma unroll
+    for (int g = 0; g < TE; ++g) wrow[g] = gate_w + (size_t)min(e0 + g, E - 1) * H + lane * 8;   // computed, not stored
+    float acc[TT][TE];
+#pragma unroll
+    for (int q = 0; q < TT; ++q)
+#pragma unroll
+        for (int g = 0; g < TE; ++g) acc[q][g] = 0.0f;
+    raw_t xn[TT], wn[TE];
+    auto fetch = [&](int j) {
+        if (lane + j * kWave < nchunk) {
+#pragma unroll
+            for (int q = 0; q < TT; ++q) xn[q] = *reinterpret_cast<const raw_t*>(xrow[q] + (size_t)j * (kWave * 8));
+#pragma unroll
+            for (int g = 0; g < TE; ++g) wn[g] = *reinterpret_cast<const raw_t*>(wrow[g] + (size_t)j * (kWave * 8));
+        }
+    };
+    fetch(0);
+    for (int j = 0; j < nstep; ++j) {
+        raw_t xc[TT], wc[TE];
+#pragma unroll
+        for (int q = 0; q < TT; ++q) xc[q] = xn[q];
+#pragma unroll
+        for (int g = 0; g < TE; ++g) wc[g] = wn[g];
+        if (j + 1 < nstep) fetch(j + 1);
+        if (lane + j * kWave < nchunk) {      // partial sum `lane` takes chunk lane + 64 j only if the row has it
+            float xv[TT][8];
+#pragma unroll
+            for (int q = 0; q < TT; ++q) widen8<T>(xc[q], xv[q]);
+#pragma unroll
+            for (int g = 0; g < TE; ++g) {
+                float wv[8];
+                widen8<T>(wc[g], wv);
+#pragma unroll
+                for (int q = 0; q < TT; ++q)
+#pragma unroll
+                    for (int v = 0; v < 8; ++v) acc[q][g] = __builtin_fmaf(xv[q][v], wv[v], acc[q][g]);
+            }
+        }
+    }
+    constexpr int EG = 16 / TT;       // experts per fold
+    const int r = fold16_index(lane);
+#pragma unroll
+    for (int gb = 0; gb < TE; gb += EG) {
+        float red[16];
+#pragma unroll
+        for (int g = 0; g < EG; ++g)
+#pragma unroll
+            for (int q = 0; q < TT; ++q) red[g * TT + q] = acc[q][gb + g];
+        const float sum = fold16(red, lane);
+        const int e = e0 + gb + r / TT, t = t0 + r % TT;
+        if ((lane & 3) == 0 && e < E && t < S) logits[(size_t)t * E + e] = gate_bias ? sum + gate_bias[e] : sum;
+    }
+}
+
+template <typename T, int TT, int TE, int WT, int WE>
+hipError_t launch_gate_tile(const void* x, const void* gate_w, const float* gate_bias, float* logits, int S, int H,
+                            int E, hipStream_t st) {
+    const dim3 grid((S + WT * TT - 1) / (WT * TT), (E + WE * TE - 1) / (WE * TE));
+    gate_tile_kernel<T, TT, TE, WT, WE><<<grid, WT * WE * 64, 0, st>>>((const T*)x, (const T*)gate_w, gate_bias, logits,
+                                                                      S, H, E);
+    return hipGetLastError();
+}
+
+// Tile choice: big tiles when there are enough (token, expert) pairs to fill the chip with them, small ones when
+// the layer is decode-sized and only more wavefronts bring more loads in flight; a 4 x 1 wavefront arrangement when
+// the experts fit one wavefront's tile.
+template <typename T>
+hipError_t launch_gate_tiled(const void* x, const void* gate_w, const float* gate_bias, float* logits, int S, int H,
+                             int E, hipStream_t st) {
+    const int64_t pairs = (int64_t)S * E;
+    int variant = pairs >= 32768 ? 0 : 1;
+    if (const char* env = getenv("MOE355_GATE_TILE")) variant = atoi(env);   // tuning knob
+    switch (variant) {
+        case 0:
+            return E <= 8 ? launch_gate_tile<T, 4, 8, 4, 1>(x, gate_w, gate_bias, logits, S, H, E, st)
+                          : launch_gate_tile<T, 4, 8, 2, 2>(x, gate_w, gate_bias, logits, S, H, E, st);
+        case 1:
+            return E <= 4 ? launch_gate_tile<T, 4, 4, 4, 1>(x, gate_w, gate_bias, logits, S, H, E, st)
+                          : launch_gate_tile<T, 4, 4, 2, 2>(x, gate_w, gate_bias, logits, S, H, E, st);
+        default:
+            return E <= 8 ? launch_gate_tile<T, 2, 8, 4, 1>(x, gate_w, gate_bias, logits, S, H, E, st)
+                          : launch_gate_tile<T, 2, 8, 2, 2>(x, gate_w, gate_bias, logits, S, H, E, st);
+    }
+}
+
+// One wavefront per token.
 __global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ logits, int S, int E, int k, int gate_fn,
                                                    int norm, int32_t* __restrict__ topk_idx,
                                                    float* __restrict__ topk_w) {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int t = blockIdx.x * 4 + wave;
     if (t >= S) return;
-    constexpr int J = kMaxExperts / kWave;
-    float v[J];
-    unsigned avail = 0;
-#pragma unroll
-    for (int j = 0; j < J; ++j) {
-        const int e = j * kWave + lane;
-        v[j] = 0.0f;
-        if (e < E) {
-            v[j] = logits[(size_t)t * E + e];
-            avail |= 1u << j;
-        }
-    }
-    const unsigned valid = avail;
-    float my_l = 0.0f;
-    int my_i = 0;
-    float top_l = 0.0f;
-    for (int r = 0; r < k; ++r) {
-        Cand c{-INFINITY, 0x7FFFFFFF};
-#pragma unroll
-        for (int j = 0; j < J; ++j) {
-            if ((avail >> j) & 1u) {
-                Cand d{v[j] != v[j] ? -INFINITY : v[j], j * kWave + lane};
-                if (better(d, c)) c = d;
-            }
-        }
-#pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) {
-            Cand o{__shfl_xor(c.v, off, kWave), __shfl_xor(c.i, off, kWave)};
-            if (better(o, c)) c = o;
-        }
-        if ((c.i & (kWave - 1)) == lane) avail &= ~(1u << (c.i >> 6));
-        // the logit behind the winning key, as stored (a NaN ranks as -inf but stays a NaN in the weights)
-        float mine = v[0];
-#pragma unroll
-        for (int j = 1; j < J; ++j) mine = (c.i >> 6) == j ? v[j] : mine;
-        const float cv = __shfl(mine, c.i & (kWave - 1), kWave);
-        if (lane == r) { my_l = cv; my_i = c.i; }
-        if (r == 0) top_l = cv;
-    }
-    float p = 0.0f;
-    if (gate_fn == MOE_GATE_SOFTMAX) {
-        float part = 0.0f;
-#pragma unroll
-        for (int j = 0; j < J; ++j)
-            if ((valid >> j) & 1u) part = part + expf(v[j] - top_l);
-#pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) part = part + __shfl_xor(part, off, kWave);
-        if (lane < k) p = expf(my_l - top_l) / part;
-    } else {
-        if (lane < k) p = 1.0f / (1.0f + expf(-my_l));
-    }
-    if (norm) {
-        float sum = p;
-#pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) sum = sum + __shfl_xor(sum, off, kWave);
-        p = p / sum;
-    }
-    if (lane < k) {
-        topk_idx[(size_t)t * k + lane] = my_i;
-        topk_w[(size_t)t * k + lane] = p;
-    }
+    topk_one_token(logits, t, E, k, gate_fn, norm, topk_idx, topk_w, lane);
 }
 
 // Router statistics for a load-balancing loss.  Block b, wavefront w takes tokens (4b + w) + 4*gridDim.x*i; a lane
@@ -336,8 +421,16 @@ hipError_t launch_router_stats(const float* logits, const int32_t* topk_idx, int
 
 hipError_t launch_gate_logits(const void* x, const void* gate_w, const float* gate_bias, float* logits, int S, int H,
                               int E, int act_dtype, hipStream_t st) {
-    if (act_dtype == MOE_DTYPE_F32) return launch_gate_typed<float>(x, gate_w, gate_bias, logits, S, H, E, st);
-    return launch_gate_typed<uint16_t>(x, gate_w, gate_bias, logits, S, H, E, st);
+    // Many experts on many tokens: the first kernel (token rows in registers, experts streamed) reads least per sum.
+    // Everything else -- few experts, or decode-sized batches -- goes to the register-tiled kernel.
+    bool rows_in_registers = E >= 32 && (int64_t)S * E >= ((int64_t)1 << 19);
+    if (const char* env = getenv("MOE355_GATE_KERNEL")) rows_in_registers = atoi(env) == 1;   // tuning knob
+    if (rows_in_registers) {
+        if (act_dtype == MOE_DTYPE_F32) return launch_gate_typed<float>(x, gate_w, gate_bias, logits, S, H, E, st);
+        return launch_gate_typed<uint16_t>(x, gate_w, gate_bias, logits, S, H, E, st);
+    }
+    if (act_dtype == MOE_DTYPE_F32) return launch_gate_tiled<float>(x, gate_w, gate_bias, logits, S, H, E, st);
+    return launch_gate_tiled<uint16_t>(x, gate_w, gate_bias, logits, S, H, E, st);
 }
 
 hipError_t launch_topk(const float* logits, int S, int E, int k, int gate_fn, int norm, int32_t* topk_idx,

@@ -18,14 +18,17 @@
 namespace moe355 {
 namespace {
 
-__global__ __launch_bounds__(kRouteBlock) void route_count_kernel(RouteArgs a) {
-    __shared__ int wcount[kRouteBlock / kWave][kMaxExperts];
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+// Pairs [blk * 256, blk * 256 + 256): ranks within the chunk and the chunk's histogram.  `tid` in [0, 256); wcount is
+// this chunk's [4][kMaxExperts] counters in LDS.  Called by whole workgroups (it holds barriers); `active` false:
+// the caller only keeps the barriers company.
+__device__ __forceinline__ void route_count_body(const RouteArgs& a, int blk, int tid, int (*wcount)[kMaxExperts],
+                                                 bool active) {
+    const int wave = tid >> 6, lane = tid & 63;
     for (int i = tid; i < (kRouteBlock / kWave) * kMaxExperts; i += kRouteBlock) (&wcount[0][0])[i] = 0;
     __syncthreads();
-    const int p = blockIdx.x * kRouteBlock + tid;
+    const int p = blk * kRouteBlock + tid;
     // an expert id outside [0, E) (only a caller-supplied topk_idx can hold one) is counted nowhere: the pair is dropped
-    const int e_in = p < a.A ? a.topk_idx[p] : -1;
+    const int e_in = (active && p < a.A) ? a.topk_idx[p] : -1;
     const bool valid = (unsigned)e_in < (unsigned)a.E;
     const int e = valid ? e_in : 0;
     unsigned long long mask = __ballot(valid);
@@ -45,12 +48,19 @@ __global__ __launch_bounds__(kRouteBlock) void route_count_kernel(RouteArgs a) {
         for (int w = 0; w < wave; ++w) base += wcount[w][e];
         a.rank_local[p] = base + rank_w;
     }
-    for (int i = tid; i < a.E; i += kRouteBlock) {
-        int s = 0;
+    if (active) {
+        for (int i = tid; i < a.E; i += kRouteBlock) {
+            int s = 0;
 #pragma unroll
-        for (int w = 0; w < kRouteBlock / kWave; ++w) s += wcount[w][i];
-        a.block_hist[(size_t)blockIdx.x * a.E + i] = s;
+            for (int w = 0; w < kRouteBlock / kWave; ++w) s += wcount[w][i];
+            a.block_hist[(size_t)blk * a.E + i] = s;
+        }
     }
+}
+
+__global__ __launch_bounds__(kRouteBlock) void route_count_kernel(RouteArgs a) {
+    __shared__ int wcount[kRouteBlock / kWave][kMaxExperts];
+    route_count_body(a, blockIdx.x, threadIdx.x, wcount, true);
 }
 
 __device__ __forceinline__ void write_segment(Segment* s, int begin, int phase, int expert, int mt0, int nmt, int nnt,
@@ -92,15 +102,22 @@ __device__ __forceinline__ void queue_slot(int s, int E, int L, int* phase, int*
 }
 
 // One workgroup of kMaxExperts threads: thread e owns expert e.
-__global__ __launch_bounds__(kMaxExperts) void route_scan_kernel(RouteArgs a) {
-    __shared__ int s_wave[kMaxExperts / kWave];
-    __shared__ int s_nmt[kMaxExperts];
-    __shared__ int s_mt0[kMaxExperts];
+struct ScanShared {
+    int wave[kMaxExperts / kWave];
+    int nmt[kMaxExperts];
+    int mt0[kMaxExperts];
+    int part[kMaxExperts];
+    int total[kMaxExperts];
+};
+__device__ __forceinline__ void route_scan_body(const RouteArgs& a, ScanShared& sh) {
+    int* s_wave = sh.wave;
+    int* s_nmt = sh.nmt;
+    int* s_mt0 = sh.mt0;
+    int* s_part = sh.part;
+    int* s_total = sh.total;
     const int e = threadIdx.x;
     // per-expert exclusive prefix over the workgroups' histograms: the kMaxExperts threads split into
     // `parts` groups that each take a contiguous run of workgroups (two passes over block_hist)
-    __shared__ int s_part[kMaxExperts];
-    __shared__ int s_total[kMaxExperts];
     int epad = 1;
     while (epad < a.E) epad <<= 1;
     const int parts = kMaxExperts / epad;
@@ -197,13 +214,18 @@ __global__ __launch_bounds__(kMaxExperts) void route_scan_kernel(RouteArgs a) {
     for (int i = threadIdx.x; i < a.max_mtiles; i += blockDim.x) a.done0[i] = 0;
 }
 
-__global__ __launch_bounds__(kRouteBlock) void route_finalize_kernel(RouteArgs a) {
-    const int p = blockIdx.x * kRouteBlock + threadIdx.x;
-    if (p >= a.A) return;
+__global__ __launch_bounds__(kMaxExperts) void route_scan_kernel(RouteArgs a) {
+    __shared__ ScanShared sh;
+    route_scan_body(a, sh);
+}
+
+// Pair p of chunk blk = p / 256.
+__device__ __forceinline__ void route_finalize_pair(const RouteArgs& a, int p) {
+    const int blk = p / kRouteBlock;
     const int e_in = a.topk_idx[p];
     const bool known = (unsigned)e_in < (unsigned)a.E;   // see route_count_kernel
     const int e = known ? e_in : 0;
-    const int s = known ? a.block_hist[(size_t)blockIdx.x * a.E + e] + a.rank_local[p] : 0;
+    const int s = known ? a.block_hist[(size_t)blk * a.E + e] + a.rank_local[p] : 0;
     const bool dropped = !known || (a.drop && s >= a.capacity);
     const int row = dropped ? -1 : a.expert_offset[e] + s;
     a.slot[p] = dropped ? -1 : s;
@@ -212,9 +234,41 @@ __global__ __launch_bounds__(kRouteBlock) void route_finalize_kernel(RouteArgs a
     if (p >= a.expert_offset[a.E]) a.token_indices[p] = -1;   // rows past the last kept one
 }
 
+__global__ __launch_bounds__(kRouteBlock) void route_finalize_kernel(RouteArgs a) {
+    const int p = blockIdx.x * kRouteBlock + threadIdx.x;
+    if (p < a.A) route_finalize_pair(a, p);
+}
+
+// Decode-sized layers: counting, scan and finalize in ONE workgroup of kMaxExperts threads, i.e. one launch instead of
+// three -- with a few hundred pairs the launches and the gaps between dependent launches cost more than the work.
+// Same bodies as the separate kernels, so the results are the same bit for bit.  Global memory written by one step is
+// read by other wavefronts of the same workgroup in the next: a workgroup barrier orders that.  (Top-k stays a launch
+// of its own: one wavefront per token in parallel beats a single workgroup walking the tokens, 10 against 70 us.)
+__global__ __launch_bounds__(kMaxExperts) void router_small_kernel(RouteArgs a) {
+    __shared__ int wcount[kMaxExperts / kRouteBlock][kRouteBlock / kWave][kMaxExperts];
+    __shared__ ScanShared sh;
+    const int tid = threadIdx.x;
+    constexpr int kChunksAtOnce = kMaxExperts / kRouteBlock;
+    for (int b0 = 0; b0 < a.nblk; b0 += kChunksAtOnce) {      // uniform trip count: every thread meets every barrier
+        const int blk = b0 + tid / kRouteBlock;
+        route_count_body(a, blk, tid % kRouteBlock, wcount[tid / kRouteBlock], blk < a.nblk);
+    }
+    __syncthreads();
+    route_scan_body(a, sh);
+    __syncthreads();
+    for (int p = tid; p < a.A; p += kMaxExperts) route_finalize_pair(a, p);
+}
+
 }  // namespace
 
+// Pairs up to which the single-workgroup router is used.
+constexpr int kSmallRouterPairs = 4096;
+
 hipError_t launch_route(const RouteArgs& a, hipStream_t st) {
+    if (a.A <= kSmallRouterPairs) {
+        router_small_kernel<<<1, kMaxExperts, 0, st>>>(a);
+        return hipGetLastError();
+    }
     route_count_kernel<<<a.nblk, kRouteBlock, 0, st>>>(a);
     route_scan_kernel<<<1, kMaxExperts, 0, st>>>(a);
     route_finalize_kernel<<<a.nblk, kRouteBlock, 0, st>>>(a);

@@ -341,8 +341,14 @@ __device__ __forceinline__ void store16(uint16_t* p, u32x4 v, bool publish) {
     else *reinterpret_cast<u32x4*>(p) = v;
 }
 
-template <class T, int MODE>
-__device__ __forceinline__ void epilogue_full_n_impl(const TaskPtrs& p, unsigned char* smem, f32x4 (&acc)[8][8]) {
+struct NoHook {
+    __device__ __forceinline__ void operator()(int) const {}
+};
+
+// `between(i)` runs in front of row group i (i = 0..7): the queue kernel issues the next task's first loads there, a
+// few at a time, so that they leave the compute unit under the epilogue's arithmetic instead of in front of it.
+template <class T, int MODE, class Hook>
+__device__ __forceinline__ void epilogue_full_n_impl(const TaskPtrs& p, unsigned char* smem, f32x4 (&acc)[8][8], const Hook& between) {
 
     static_assert(T::TM == 8 && T::TN == 8 && T::WN == 2, "four wavefronts of 128 x 128");
     constexpr int NJ = MODE == 3 ? 4 : 8;        // groups of 16 output columns per wavefront
@@ -388,6 +394,7 @@ __device__ __forceinline__ void epilogue_full_n_impl(const TaskPtrs& p, unsigned
     constexpr int NQ = 16 / ROWS_PER_PASS;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
+        between(i);
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
             float v[4];
@@ -422,11 +429,11 @@ __device__ __forceinline__ void epilogue_full_n_impl(const TaskPtrs& p, unsigned
     }
 }
 
-template <class T>
-__device__ __forceinline__ void epilogue_full_n(const TaskPtrs& p, unsigned char* smem, f32x4 (&acc)[8][8]) {
-    if (p.swiglu) epilogue_full_n_impl<T, 3>(p, smem, acc);
-    else if (p.act == MOE_ACT_GELU) epilogue_full_n_impl<T, 2>(p, smem, acc);
-    else epilogue_full_n_impl<T, 0>(p, smem, acc);
+template <class T, class Hook = NoHook>
+__device__ __forceinline__ void epilogue_full_n(const TaskPtrs& p, unsigned char* smem, f32x4 (&acc)[8][8], const Hook& between = Hook()) {
+    if (p.swiglu) epilogue_full_n_impl<T, 3>(p, smem, acc, between);
+    else if (p.act == MOE_ACT_GELU) epilogue_full_n_impl<T, 2>(p, smem, acc, between);
+    else epilogue_full_n_impl<T, 0>(p, smem, acc, between);
 }
 
 // The slab loop of a full 256 x 256 tile on four wavefronts of 128 x 128, with the instruction order fixed by hand.
@@ -442,63 +449,158 @@ __device__ __forceinline__ void epilogue_full_n(const TaskPtrs& p, unsigned char
 // once per task, plus a scalar k offset -- no vector ALU instruction is left in the loop.
 // Takes partial row blocks too (the whole tile is computed, rows past the end are not stored).
 // Needs: K a multiple of 128, a tile that is not ragged in N, operand extents below 4 GiB.
+// What the loads of one task of the hand-ordered tile need; computed once per task (ring_prepare).
+struct RingLoads {
+    unsigned voff_a[8], voff_b[8];   // byte offsets of this thread's eight token rows / weight rows (row + 16-byte chunk)
+    const void* base_a;              // wavefront-uniform operand bases
+    const void* base_b0;
+    const void* base_b1;
+    uint32_t a_extent, b_extent;
+    int KT;                          // slabs of 64: even, >= 2
+    int wrow;                        // first of the eight consecutive stage rows this wavefront's loads fill per pass
+};
+
+// The part of a task's load state that needs no memory access: weight-row offsets, bases, extents.
 template <class T>
-__device__ __forceinline__ void gemm_tile_ring(const TaskPtrs& p, unsigned char* smem) {
+__device__ __forceinline__ RingLoads ring_prepare_weights(const TaskPtrs& p) {
     static_assert(T::RING && T::TM == 8 && T::TN == 8 && T::RA == 8 && T::RB == 8, "four wavefronts of 128 x 128");
-    constexpr int BM = T::BM, STAGE = T::STAGE_BYTES;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    // a thread id the compiler cannot see through: what is derived from it is computed here, not once at the top of
+    // the kernel and then kept (and spilled) across the slab loop
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
     const int prow = tid >> 3;
     const int chunk = (tid & 7) ^ ((prow >> 1) & 7);
-    const int wrow = __builtin_amdgcn_readfirstlane(prow & ~7);
-
-    const int KT = p.K / kBK;                  // even, >= 2
-
-    unsigned voff_a[8], voff_b[8];
+    RingLoads L;
 #pragma unroll
     for (int n = 0; n < 8; ++n) {
-        // Padding rows are never stored.  Their loads are aimed behind the end of the buffer, which the hardware
-        // answers with zeros without touching memory: MFMAs on zeros draw less of the power budget than MFMAs on a
-        // copy of real rows.
-        const int r0 = prow + n * T::ROWS_PER_PASS, r = min(r0, p.rows - 1);
-        const int64_t src_row = p.gather ? (int64_t)p.gather[r] : p.a_row0 + r;
-        voff_a[n] = r0 < p.rows ? (unsigned)((src_row * p.a_ld + chunk * 8) * 2) : p.a_extent;
+        L.voff_a[n] = p.a_extent;
         const int j = prow + n * T::ROWS_PER_PASS;
         const int col = p.swiglu ? p.n0 + (j >> 7) * 64 + (j & 63) : p.n0 + j;
-        voff_b[n] = (unsigned)(((int64_t)col * p.K + chunk * 8) * 2);
+        L.voff_b[n] = (unsigned)(((int64_t)col * p.K + chunk * 8) * 2);
     }
     auto uniform = [](const void* q) {          // the bases are the same in every lane; say so, or each load loops over lanes
         const uint64_t v = (uint64_t)q;
         // readfirstlane returns int: go through uint32_t, or a low half with bit 31 set sign-extends over the high half
         const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
         const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
-        return (void*)(((uint64_t)hi << 32) | (uint64_t)lo);
+        return (const void*)(((uint64_t)hi << 32) | (uint64_t)lo);
     };
-    // Raw buffers (stride 0) that end where the operand ends.  The steady-state slab body also issues loads for the
-    // two slabs past the end of K; those go through descriptors of zero length, which the hardware answers with
-    // zeros without touching memory (the stages they land in are never read).
-    const void* base_a = uniform(p.a_base);
-    const void* base_b0 = uniform(p.b0);
-    const void* base_b1 = uniform(p.swiglu ? p.b1 : p.b0);
-    // load n of a slab: n < 8 token rows, else weight rows; the weight rows of pass m come from w_gate when m % 4 < 2
-    auto load_one = [&](int slab, int n) {
-        unsigned char* base = smem + (slab & 1) * STAGE;
-        const int soff = slab * kRowBytes;
-        const bool live = slab < KT;
-        if (n < 8) {
-            const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base_a), 0, live ? (int)p.a_extent : 0, 0x00020000);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void*)(base + (wrow + n * T::ROWS_PER_PASS) * kRowBytes), 16,
-                                                     voff_a[n], soff, 0, 0);
-        } else {
-            const int m = n - 8;
-            const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>((m & 2) ? base_b0 : base_b1), 0,
-                                                                                 live ? (int)p.b_extent : 0, 0x00020000);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void*)(base + BM * kRowBytes + (wrow + m * T::ROWS_PER_PASS) * kRowBytes),
-                                                     16, voff_b[m], soff, 0, 0);
-        }
-    };
+    L.base_a = uniform(p.a_base);
+    L.base_b0 = uniform(p.b0);
+    L.base_b1 = uniform(p.swiglu ? p.b1 : p.b0);
+    L.a_extent = p.a_extent;
+    L.b_extent = p.b_extent;
+    L.KT = p.K / kBK;
+    L.wrow = __builtin_amdgcn_readfirstlane(prow & ~7);
+    return L;
+}
 
-    f32x4 acc[8][8];
+// The token-row offsets: phase 0 gathers the row numbers through token_indices[] (eight loads per thread).
+template <class T>
+__device__ __forceinline__ void ring_prepare_tokens(const TaskPtrs& p, RingLoads& L) {
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    const int prow = tid >> 3;
+    const int chunk = (tid & 7) ^ ((prow >> 1) & 7);
+#pragma unroll
+    for (int n = 0; n < 8; ++n) {
+        // Padding rows are never stored.  Their loads are aimed behind the end of the buffer, which the hardware
+        // answers with zeros without touching memory: MFMAs on zeros draw less of the power budget than MFMAs on a
+        // copy of real rows.
+        const int r0 = prow + n * T::ROWS_PER_PASS, r = max(min(r0, p.rows - 1), 0);
+        const int64_t src_row = p.gather ? (int64_t)p.gather[r] : p.a_row0 + r;
+        L.voff_a[n] = r0 < p.rows ? (unsigned)((src_row * p.a_ld + chunk * 8) * 2) : p.a_extent;
+    }
+}
+
+template <class T>
+__device__ __forceinline__ RingLoads ring_prepare(const TaskPtrs& p) {
+    RingLoads L = ring_prepare_weights<T>(p);
+    ring_prepare_tokens<T>(p, L);
+    return L;
+}
+
+// Load n of slab `slab` of a task: n < 8 token rows, else weight rows; the weight rows of pass m come from w_gate when
+// m % 4 < 2.  Raw buffers (stride 0) that end where the operand ends.  Slabs past the end of K go through descriptors of
+// zero length, which the hardware answers with zeros without touching memory (the stages they land in are never read).
+template <class T>
+__device__ __forceinline__ void ring_load_one(const RingLoads& L, unsigned char* smem, int slab, int n) {
+    const int wrow = L.wrow;
+    unsigned char* base = smem + (slab & 1) * T::STAGE_BYTES;
+    const int soff = slab * kRowBytes;
+    const bool live = slab < L.KT;
+    if (n < 8) {
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(L.base_a), 0, live ? (int)L.a_extent : 0, 0x00020000);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void*)(base + (wrow + n * T::ROWS_PER_PASS) * kRowBytes), 16,
+                                                 L.voff_a[n], soff, 0, 0);
+    } else {
+        const int m = n - 8;
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>((m & 2) ? L.base_b0 : L.base_b1), 0,
+                                                                             live ? (int)L.b_extent : 0, 0x00020000);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void*)(base + T::BM * kRowBytes + (wrow + m * T::ROWS_PER_PASS) * kRowBytes),
+                                                 16, L.voff_b[m], soff, 0, 0);
+    }
+}
+
+// The loads of a task's first two slabs: the weight rows of slab 0 and of slab 1, then the token rows of slab 0 and of
+// slab 1 -- weights first because their addresses need no gathered row numbers, so the queue kernel can send them
+// off while those are still on their way.  Slab 0 is complete when at most the last eight of the 32 are outstanding.
+// Nobody may still be reading the stages (the caller sees to that).
+template <class T>
+__device__ __forceinline__ void ring_first_weight_loads(const RingLoads& L, unsigned char* smem) {
+#pragma unroll
+    for (int n = 8; n < 16; ++n) ring_load_one<T>(L, smem, 0, n);
+#pragma unroll
+    for (int n = 8; n < 16; ++n) ring_load_one<T>(L, smem, 1, n);
+}
+template <class T>
+__device__ __forceinline__ void ring_first_token_load(const RingLoads& L, unsigned char* smem, int q) {   // q = 0..15
+    ring_load_one<T>(L, smem, q >> 3, q & 7);
+}
+template <class T>
+__device__ __forceinline__ void ring_first_loads(const RingLoads& L, unsigned char* smem) {
+    ring_first_weight_loads<T>(L, smem);
+#pragma unroll
+    for (int q = 0; q < 16; ++q) ring_first_token_load<T>(L, smem, q);
+}
+
+// The slab loop of a full 256 x 256 tile on four wavefronts of 128 x 128, with the instruction order fixed by hand.
+//
+// Why not the compiler's order: with one wavefront per SIMD nothing else hides a stall, and the global->LDS loads of
+// a slab (64 KB per compute unit) need more than one slab of flight time to stream in at the rate the L2 delivers.
+// So (a) both k halves of a slab's fragments are double buffered in registers, which frees the slab's LDS stage at
+// mid-slab, (b) the loads of slab kt+2 are issued into that stage right away, two per MFMA row, and stay in flight
+// across the barriers (bare s_barrier: a __syncthreads() would wait for them), (c) MFMAs, LDS reads and their
+// s_waitcnt are inline asm in the order written by gen_slab_schedule.py (ffn_bf16_slab_steady.inc); the compiler places
+// nothing between them but the scalar address updates of the loads.  The accumulators are tied asm operands in
+// AGPRs, so they stay put for the whole loop.  Loads use buffer addressing: a 32-bit byte offset per row, computed
+// once per task, plus a scalar k offset -- no vector ALU instruction is left in the loop.
+// Takes partial row blocks too (the whole tile is computed, rows past the end are not stored).
+// Needs: K a multiple of 128, a tile that is not ragged in N, operand extents below 4 GiB.
+// On entry the loads of slabs 0 and 1 (ring_first_loads, in that order) are the 32 youngest vector loads of this
+// wavefront (stores issued behind them only make the first wait more conservative).  Returns false for a wavefront whose 128 rows are all
+// padding: it has taken part in the loads and barriers only and holds no results.
+template <class T>
+__device__ __forceinline__ bool ring_slabs(int rows, const RingLoads& L, unsigned char* smem, f32x4 (&acc)[8][8]) {
+    constexpr int BM = T::BM, STAGE = T::STAGE_BYTES;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    // The scalar members are the same in every lane; say so here, behind whatever control flow handed L over, or the
+    // compiler builds every buffer descriptor in a loop over the lanes.
+    RingLoads U = L;
+    {
+        auto uni = [](unsigned v) { return (unsigned)__builtin_amdgcn_readfirstlane((int)v); };
+        auto unip = [&](const void* q) {
+            const uint64_t v = (uint64_t)q;
+            return (const void*)(((uint64_t)uni((unsigned)(v >> 32)) << 32) | (uint64_t)uni((unsigned)v));
+        };
+        U.base_a = unip(L.base_a); U.base_b0 = unip(L.base_b0); U.base_b1 = unip(L.base_b1);
+        U.a_extent = uni(L.a_extent); U.b_extent = uni(L.b_extent);
+        U.KT = (int)uni((unsigned)L.KT); U.wrow = (int)uni((unsigned)L.wrow);
+    }
+    const int KT = U.KT;
+    auto load_one = [&](int slab, int n) { ring_load_one<T>(U, smem, slab, n); };
+
 #pragma unroll
     for (int i = 0; i < 8; ++i)
 #pragma unroll
@@ -525,18 +627,13 @@ __device__ __forceinline__ void gemm_tile_ring(const TaskPtrs& p, unsigned char*
 #define BAR2(n) do { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(n) : "memory"); __builtin_amdgcn_s_barrier(); } while (0)
 #define GL(n) load_one(kt + 2, n)
 #define TAIL asm volatile("s_nop 15\n\ts_nop 3" ::: "memory")
-    __syncthreads();                            // the previous task may still be reading the stages
-#pragma unroll
-    for (int n = 0; n < 16; ++n) load_one(0, n);
-#pragma unroll
-    for (int n = 0; n < 16; ++n) load_one(1, n);
     // Padding rows.  The MFMA pipes run against the board's power limit, so an MFMA on padding rows costs everybody
     // clock.  A wavefront whose 128 rows are all padding (a row block of at most 128 rows: the upper two wavefronts)
     // therefore takes part in the loads and the barriers only: the same slab body with the MFMAs, the fragment reads
     // and their waits left out.  The tile takes as long as before; the layer gains 1 % (Mixtral shape) to 4 % (many
     // small experts) from the clock.  (Skipping the empty 16-row groups of partly filled wavefronts as well, with a
     // scalar branch around their MFMAs, cost more in the full tiles than it returned.)
-    if (__builtin_amdgcn_readfirstlane(wm) * 128 >= p.rows) {
+    if (__builtin_amdgcn_readfirstlane(wm) * 128 >= rows) {
 #pragma push_macro("MF")
 #pragma push_macro("RA")
 #pragma push_macro("RB")
@@ -549,7 +646,7 @@ __device__ __forceinline__ void gemm_tile_ring(const TaskPtrs& p, unsigned char*
 #define RA(stg, half, idx) ((void)0)
 #define RB(stg, half, j) ((void)0)
 #define WL(n) ((void)0)
-        BAR2(16);
+        BAR2(8);
         for (; kt < KT; kt += 2) {
             {
                 constexpr unsigned st = 0, sn = 1;
@@ -568,9 +665,9 @@ __device__ __forceinline__ void gemm_tile_ring(const TaskPtrs& p, unsigned char*
 #pragma pop_macro("RB")
 #pragma pop_macro("RA")
 #pragma pop_macro("MF")
-        return;                                 // nothing to store either
+        return false;                           // nothing to store either
     }
-    BAR2(16);                                   // slab 0 has landed (loads return in issue order)
+    BAR2(8);                                    // slab 0 has landed (loads return in issue order; see ring_first_loads)
     {   // same order as the reads behind BAR2 of a steady-state slab
         constexpr unsigned sn = 0;
         RA(sn, 0, 0);
@@ -610,7 +707,17 @@ __device__ __forceinline__ void gemm_tile_ring(const TaskPtrs& p, unsigned char*
 #undef BAR2
 #undef GL
 #undef TAIL
-    epilogue_full_n<T>(p, smem, acc);
+    return true;
+}
+
+// One task from start to end: the form the two-launch and the plain-GEMM kernels use.
+template <class T>
+__device__ __forceinline__ void gemm_tile_ring(const TaskPtrs& p, unsigned char* smem) {
+    const RingLoads L = ring_prepare<T>(p);
+    __syncthreads();                            // the previous task may still be reading the stages
+    ring_first_loads<T>(L, smem);
+    f32x4 acc[8][8];
+    if (ring_slabs<T>(p.rows, L, smem, acc)) epilogue_full_n<T>(p, smem, acc);
 }
 
 template <class T, bool PARTIAL>
@@ -722,6 +829,142 @@ __global__ __launch_bounds__(P::THREADS) void ffn_persistent_kernel(FfnArgs a) {
     }
 }
 
+// The same queue for the 256 x 256 tile, with the start of the next task moved under the end of the current one
+// (opt-in: MOE355_QUEUE_EARLY=1).
+//
+// Between two tiles a workgroup pops (an atomic round trip and two barriers), decodes, computes its row offsets (eight
+// gathered token indices per thread), issues the first 32 loads and waits for slab 0.  Here the next id is reserved
+// with an asynchronous pop when the current tile's slab loop begins (its latency disappears under the loop), and right
+// behind the loop -- the LDS stages are free, the accumulators still hold the tile -- the next task is decoded, its
+// dependency polled once, the weight rows of its first two slabs are requested, and the token rows follow two at a
+// time between the row groups of the current tile's epilogue.  A next task that cannot start (dependency not yet
+// met, queue exhausted, a hole) is handled after the epilogue the plain way; a workgroup never blocks while it holds
+// unstored results, so the queue's progress argument is unchanged.  Near the end of its queue a workgroup stops
+// reserving: a task reserved behind a long tile would start late while other workgroups idle.
+// Measured with timestamps inside the kernel (Mixtral shape, per tile): the wait for slab 0 (about 4 us) is gone, but
+// pop result + barrier 0.8, decode 1.2, offsets 1.2 and issuing the loads 1.4 us now sit in front of the epilogue, so
+// the time between two slab loops stays at 12-13 us and the launch takes the same number of cycles (MFMA pipes busy
+// 74 % either way); short tiles lose 2-3 %.  Results are bit-identical to the plain loop.
+constexpr int kReserveMargin = 64;   // ids left in the current queue below which tasks are popped late again
+
+// The kernel's argument block, read again from the kernel-argument segment through a pointer the compiler cannot see
+// through: values loaded from it live only as long as they are used, instead of occupying forty scalar registers
+// across the slab loop (which then spill into vector registers and bring vector instructions into the loop).
+__device__ __forceinline__ const FfnArgs& kernel_args_again() {
+    typedef const __attribute__((address_space(4))) FfnArgs* args_ptr;
+    args_ptr q = (args_ptr)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(q));
+    return *(const FfnArgs*)q;
+}
+
+template <class P>
+__global__ __launch_bounds__(P::THREADS) void ffn_persistent_ring_kernel(FfnArgs) {
+    using T = typename P::T0;
+    static_assert(std::is_same<typename P::T0, typename P::T1>::value && T::RING, "the hand-ordered tile for both projections");
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ int s_task, s_ok, s_next[2];
+    queue_kernel_entry();
+    int ids, nseg, nnt0, groups;
+    {
+        const FfnArgs& a = kernel_args_again();
+        ids = a.q->ids_queue;
+        nseg = a.q->nseg;
+        nnt0 = a.seg_phase0[0].nnt;
+        groups = a.groups;
+    }
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    QueueCursor cur = queue_cursor(groups);
+    // The current task as plain scalars (a struct carried around the loop ends up in scratch memory).
+    int ph = 0, ex = 0, mt = 0, nt = 0, row0 = 0, rows = 0;
+    auto as_task = [&]() {
+        Task q;
+        q.phase = ph; q.expert = ex; q.mtile = mt; q.ntile = nt; q.row0 = row0; q.rows = rows; q.nnt0 = nnt0; q.valid = true;
+        return q;
+    };
+    RingLoads L;
+    // a task started the plain way: wait for its rows if need be, offsets, first loads
+    auto start_cold = [&]() {
+        const FfnArgs& a = kernel_args_again();
+        if (ph == 1 && !wait_phase0_done(a.done0, mt, nnt0, a.spin_limit, a.q, a.host_stall, &s_ok)) {
+            poison_tile((uint16_t*)a.y + (int64_t)row0 * a.H, rows, a.H, nt * T::BN, T::BN, 2);
+            rows = 0;
+        }
+        L = ring_prepare<T>(resolve<T>(a, as_task(), ph == 0));
+        __syncthreads();                        // the previous task may still be reading the stages
+        ring_first_loads<T>(L, smem);
+    };
+    auto pop_blocking = [&]() {
+        Task q;
+        const bool ok = next_task(kernel_args_again(), cur, &s_task, ids, nseg, nnt0, q);
+        if (ok) { ph = q.phase; ex = q.expert; mt = q.mtile; nt = q.ntile; row0 = q.row0; rows = q.rows; }
+        return ok;
+    };
+    bool have = pop_blocking();
+    if (have) start_cold();
+    while (have) {                              // uniform: every wavefront takes the same turns
+        const bool reserve = cur.last_id + kReserveMargin < ids;
+        int rid = 0;
+        if (reserve && wave == 0) rid = pop_async(&kernel_args_again().q->heads[cur.group]);
+        f32x4 acc[8][8];
+        const bool active = ring_slabs<T>(rows, L, smem, acc);
+
+        const FfnArgs& a = kernel_args_again();
+        int nid = ids, n_valid = 0, n_ph = 0, n_ex = 0, n_mt = 0, n_nt = 0, n_row0 = 0, n_rows = 0, started = 0;
+        if (reserve) {
+            if (wave == 0) s_next[0] = pop_async_result(rid);
+            __syncthreads();                    // also: every wavefront is done with the stages
+            nid = __builtin_amdgcn_readfirstlane(s_next[0]);
+            if (nid < ids) {
+                const Task q = decode_task(a.seg_queue, nseg, a.mtiles, nid, cur.group, groups, nnt0);
+                n_valid = q.valid; n_ph = q.phase; n_ex = q.expert; n_mt = q.mtile; n_nt = q.ntile; n_row0 = q.row0; n_rows = q.rows;
+                if (n_valid) {
+                    int ready = 1;
+                    if (n_ph == 1) {            // one look at the dependency; the answer must be the workgroup's, not a wavefront's
+                        if (wave == 0)
+                            s_next[1] = __hip_atomic_load(a.done0 + n_mt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= nnt0;
+                        __syncthreads();
+                        ready = __builtin_amdgcn_readfirstlane(s_next[1]);
+                        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                    }
+                    if (ready) {                // the loop is done with the old offsets
+                        const TaskPtrs pq = resolve<T>(a, q, n_ph == 0);
+                        L = ring_prepare_weights<T>(pq);
+                        ring_first_weight_loads<T>(L, smem);
+                        ring_prepare_tokens<T>(pq, L);
+                        started = 1;
+                    }
+                }
+            }
+        }
+        // the token rows of the next task's first slabs leave two at a time under the epilogue's arithmetic
+        auto token_loads = [&](int i) {
+            if (started) {
+                ring_first_token_load<T>(L, smem, 2 * i);
+                ring_first_token_load<T>(L, smem, 2 * i + 1);
+            }
+        };
+        if (active) {
+            epilogue_full_n<T>(resolve<T>(a, as_task(), ph == 0), smem, acc, token_loads);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) token_loads(i);
+        }
+        if (ph == 0) signal_phase0_done(a.done0, mt);
+        if (reserve && nid < ids && n_valid) {   // the reserved task is the next one
+            ph = n_ph; ex = n_ex; mt = n_mt; nt = n_nt; row0 = n_row0; rows = n_rows;
+            cur.last_id = nid;
+            if (!started) start_cold();          // its rows were not ready: wait now that nothing unstored is held
+            continue;
+        }
+        if (reserve && nid >= ids) {             // the reserved pop found this queue empty: move on as next_task does
+            if (++cur.exhausted >= groups) break;
+            cur.group = cur.group + 1 == groups ? 0 : cur.group + 1;
+        }
+        have = pop_blocking();
+        if (have) start_cold();
+    }
+}
+
 // The bare reference contract on dense operands: rows [b*BM, ...) of A, one "expert".
 template <class T>
 __global__ __launch_bounds__(T::THREADS) void gemm_dense_kernel(const uint16_t* A, const uint16_t* B,
@@ -768,6 +1011,17 @@ hipError_t launch_tiled(const FfnArgs& a, int max_mtiles, int nnt0, int nnt1, hi
 
 template <class P>
 hipError_t launch_persistent(const FfnArgs& a, int blocks, hipStream_t st) {
+    if constexpr (P::T0::RING) {
+        // tuning knob: 1 = the queue loop that starts the next task under the end of the current one (measured: no
+        // faster on the Mixtral shape, 2-3 % slower on short tiles; kept for machines where the balance differs)
+        const char* env = getenv("MOE355_QUEUE_EARLY");
+        if (env && atoi(env) == 1) {
+            hipError_t e = allow_lds(&ffn_persistent_ring_kernel<P>, P::LDS_BYTES);
+            if (e != hipSuccess) return e;
+            ffn_persistent_ring_kernel<P><<<blocks, P::THREADS, P::LDS_BYTES, st>>>(a);
+            return hipGetLastError();
+        }
+    }
     hipError_t e = allow_lds(&ffn_persistent_kernel<P>, P::LDS_BYTES);
     if (e != hipSuccess) return e;
     ffn_persistent_kernel<P><<<blocks, P::THREADS, P::LDS_BYTES, st>>>(a);

@@ -80,8 +80,29 @@ __device__ __forceinline__ int xcd_id() { return __builtin_amdgcn_s_getreg(20 | 
 // by tasks that cannot block for ever, and a phase-1 wait always ends.
 struct QueueCursor {
     int group, exhausted;
+    int last_id;   // id of the task popped last (in `group`)
 };
-__device__ __forceinline__ QueueCursor queue_cursor(int groups) { return QueueCursor{groups > 1 ? xcd_id() % groups : 0, 0}; }
+__device__ __forceinline__ QueueCursor queue_cursor(int groups) { return QueueCursor{groups > 1 ? xcd_id() % groups : 0, 0, 0}; }
+
+// A pop that nothing waits for: lane 0 of the calling wavefront (call it from one wavefront of the workgroup, under a
+// wavefront-uniform branch) adds one to the head and the old value arrives in its register some time later.
+// pop_async_result waits for it and returns it in a scalar register.  Written in assembly so that the one-lane region
+// is invisible to the compiler's control-flow structuriser (see the remark on pop_task above) and so that no wait is
+// placed between the two.  The atomic is the wavefront's oldest outstanding vector memory operation until it returns.
+__device__ __forceinline__ int pop_async(int32_t* head) {
+    int rid;
+    unsigned long long saved_exec;
+    const int one = 1;
+    asm volatile("s_mov_b64 %1, exec\n\ts_mov_b64 exec, 1\n\tglobal_atomic_add %0, %2, %3, off sc0\n\ts_mov_b64 exec, %1"
+                 : "=&v"(rid), "=&s"(saved_exec)
+                 : "v"(head), "v"(one)
+                 : "memory");
+    return rid;
+}
+__device__ __forceinline__ int pop_async_result(int rid) {
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(rid)::"memory");
+    return __builtin_amdgcn_readfirstlane(rid);
+}
 
 // Next task of the workgroup; false when every queue is empty.  Holes are skipped here.
 __device__ __forceinline__ bool next_task(const FfnArgs& a, QueueCursor& c, int* s_task, int ids, int nseg, int nnt0,
@@ -94,6 +115,7 @@ __device__ __forceinline__ bool next_task(const FfnArgs& a, QueueCursor& c, int*
             continue;
         }
         t = decode_task(a.seg_queue, nseg, a.mtiles, id, c.group, a.groups, nnt0);
+        c.last_id = id;
         if (t.valid) return true;
     }
 }

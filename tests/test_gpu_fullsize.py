@@ -41,7 +41,7 @@ def stratified_tokens(cfg, want, block_rows, seed=7):
 
 
 @pytest.mark.parametrize("name", ["C2", "C3", "C4", "C5"])
-def test_baseline_config_full_size(name):
+def test_baseline_config_full_size(name, monkeypatch):
     import torch
     import cuplayground_amd as moe
     assert torch.cuda.is_available()
@@ -90,6 +90,14 @@ def test_baseline_config_full_size(name):
     layer.set_ffn_mode(FFN_TILED)
     out2 = layer.forward(dev["x"], dev)
     assert torch.equal(out, out2)
+    # and so must the queue loop with the early start of the next task (an opt-in schedule of the 256-row tile)
+    layer.set_ffn_mode(FFN_PERSISTENT)
+    monkeypatch.setenv("MOE355_QUEUE_EARLY", "1")
+    out3 = layer.forward(dev["x"], dev)
+    torch.cuda.synchronize()
+    monkeypatch.delenv("MOE355_QUEUE_EARLY")
+    layer.task_counts()
+    assert torch.equal(out, out3)
     layer.close()
 
 

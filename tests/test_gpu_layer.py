@@ -200,6 +200,12 @@ def test_large_tile_and_queue_groups(moe, name, monkeypatch):
                 assert max_rel_err(ob.to_f32(first, cfg.act_dtype), ob.to_f32(want["out"], cfg.act_dtype)) <= OUT_TOL[cfg.dtype]
             else:
                 assert np.array_equal(got["out"], first), (groups, mode)
+        # the queue loop that starts the next task under the end of the current one (same tiles, other timing)
+        monkeypatch.setenv("MOE355_QUEUE_EARLY", "1")
+        got = run_layer(moe, cfg, inp, FFN_PERSISTENT)
+        monkeypatch.delenv("MOE355_QUEUE_EARLY")
+        check_routing(got, want)
+        assert np.array_equal(got["out"], first), ("early", groups)
 
 
 def test_two_handles_on_two_streams_from_two_threads(moe):

@@ -190,8 +190,11 @@ def _stream():
 
 
 def _torch_act_dtype(torch_dtype: int):
+    """Storage type of activations: the layer's own; fp32 for tf32 layers, bf16 for e4m3 layers."""
     import torch
-    return torch.float32 if torch_dtype == DTYPE_F32 else torch.bfloat16
+    if torch_dtype in (DTYPE_F32, DTYPE_TF32):
+        return torch.float32
+    return torch.float16 if torch_dtype == DTYPE_FP16 else torch.bfloat16
 
 
 class MoELayer:
@@ -397,7 +400,7 @@ def gemm_bias_act(A, B, bias, act: int):
     import torch
     M, K = A.shape
     N = B.shape[0]
-    dtype = DTYPE_F32 if A.dtype == torch.float32 else DTYPE_BF16
+    dtype = {torch.float32: DTYPE_F32, torch.bfloat16: DTYPE_BF16, torch.float16: DTYPE_FP16}[A.dtype]
     Cm = torch.empty(M, N, dtype=A.dtype, device=A.device)
     _check(load_library().moe_gemm_bias_act(_ptr(A), _ptr(B), _ptr(bias), _ptr(Cm), M, N, K, dtype, act, _stream()),
            "moe_gemm_bias_act")
@@ -409,7 +412,7 @@ def combine(y_rows, pair_row, topk_w, out=None):
     import torch
     S, k = pair_row.shape
     H = y_rows.shape[1]
-    dtype = DTYPE_F32 if y_rows.dtype == torch.float32 else DTYPE_BF16
+    dtype = {torch.float32: DTYPE_F32, torch.bfloat16: DTYPE_BF16, torch.float16: DTYPE_FP16}[y_rows.dtype]
     if out is None:
         out = torch.empty(S, H, dtype=y_rows.dtype, device=y_rows.device)
     _check(load_library().moe_combine(_ptr(y_rows), _ptr(pair_row), _ptr(topk_w), S, k, H, dtype, _ptr(out),

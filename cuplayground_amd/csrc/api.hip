@@ -17,11 +17,11 @@ int bf16_block_n0(int block_m);
 int bf16_block_n1(int block_m);
 int f32_block_m();
 int f32_block_n();
-hipError_t launch_ffn_tiled_bf16(const FfnArgs&, int block_m, int max_mtiles, int nnt0, int nnt1, hipStream_t);
-hipError_t launch_ffn_persistent_bf16(const FfnArgs&, int block_m, int blocks, hipStream_t);
+hipError_t launch_ffn_tiled_bf16(const FfnArgs&, int block_m, int max_mtiles, int nnt0, int nnt1, hipStream_t, bool f16);
+hipError_t launch_ffn_persistent_bf16(const FfnArgs&, int block_m, int blocks, hipStream_t, bool f16);
 int ffn_persistent_occupancy_bf16(int block_m);
 hipError_t launch_gemm_dense_bf16(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t, int,
-                                  hipStream_t);
+                                  hipStream_t, bool f16);
 hipError_t launch_ffn_tiled_f32(const FfnArgs&, int max_mtiles, int nnt0, int nnt1, hipStream_t);
 hipError_t launch_ffn_persistent_f32(const FfnArgs&, int blocks, hipStream_t);
 hipError_t launch_gemm_dense_f32(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t, int,
@@ -40,7 +40,7 @@ int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
 
 struct Derived {
     int S, H, I, E, k, A;
-    int act_dtype;     // MOE_DTYPE_F32 or MOE_DTYPE_BF16
+    int act_dtype;     // MOE_DTYPE_F32, MOE_DTYPE_BF16 or MOE_DTYPE_FP16
     size_t act_bytes;
     int64_t capacity;
     FfnPlan plan;
@@ -53,8 +53,15 @@ struct WsLayout {
         block_hist, mtiles, seg0, seg1, segq, qstate, done0, stats_prob, stats_cnt, h, y, total;
 };
 
+// Storage type of activations (x, biases, h, y, out): the layer's own, except that tf32 -- fp32 storage with
+// reduced-precision multiplies in the reference (processor/tiling.cuh:131-143) -- is stored and computed as fp32 here
+// (gfx950 has no tf32 matrix instruction; full fp32 is the superset), and e4m3 layers keep bf16 activations.
+int act_dtype_of(int torch_dtype) {
+    if (torch_dtype == MOE_DTYPE_F32 || torch_dtype == MOE_DTYPE_TF32) return MOE_DTYPE_F32;
+    return torch_dtype == MOE_DTYPE_FP16 ? MOE_DTYPE_FP16 : MOE_DTYPE_BF16;
+}
+
 int check_supported(const moe_config& c) {
-    if (c.torch_dtype == MOE_DTYPE_TF32 || c.torch_dtype == MOE_DTYPE_FP16) return MOE_ERR_UNSUPPORTED;
     if (c.num_experts > kMaxExperts || c.expert_top_k > kMaxTopK) return MOE_ERR_UNSUPPORTED;
     if (c.torch_dtype == MOE_DTYPE_FP8_E4M3_B128 &&
         (c.hidden_size % 128 || c.intermediate_size % 128 || c.hidden_act != MOE_ACT_SWIGLU))
@@ -74,7 +81,7 @@ int derive(const moe_config& c, Derived* d) {
     d->E = c.num_experts;
     d->k = c.expert_top_k;
     d->A = d->S * d->k;
-    d->act_dtype = c.torch_dtype == MOE_DTYPE_F32 ? MOE_DTYPE_F32 : MOE_DTYPE_BF16;
+    d->act_dtype = act_dtype_of(c.torch_dtype);
     d->act_bytes = d->act_dtype == MOE_DTYPE_F32 ? 4 : 2;
     moe_config_capacity(&c, &d->capacity);
     if (d->capacity > d->A) d->capacity = d->A;
@@ -117,7 +124,7 @@ WsLayout layout(const Derived& d) {
 FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E) {
     FfnPlan p;
     const bool sw = act == MOE_ACT_SWIGLU;
-    if (dtype == MOE_DTYPE_F32) {
+    if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32) {
         p.block_m = f32_block_m();
         p.nnt0 = sw ? ceil_div(I, f32_block_n() / 2) : ceil_div(I, f32_block_n());
         p.nnt1 = ceil_div(H, f32_block_n());
@@ -307,7 +314,7 @@ int moe_create(const moe_config* cfg, moe_handle** out) {
     h->arch.persistent_blocks = prop.multiProcessorCount * per_cu;
     // One task queue per XCD for the MFMA-bound bf16 tiles, whose operand tiles are then shared in that XCD's L2;
     // the f32 and fp8 paths keep a single queue.
-    h->queue_groups = cfg->torch_dtype == MOE_DTYPE_BF16 ? h->arch.xcds : 1;
+    h->queue_groups = (cfg->torch_dtype == MOE_DTYPE_BF16 || cfg->torch_dtype == MOE_DTYPE_FP16) ? h->arch.xcds : 1;
     if (const char* env = getenv("MOE355_QUEUE_GROUPS")) {   // tuning knob; never more queues than XCDs
         const int v = atoi(env);
         if ((v == 1 || v == 2 || v == 4 || v == 8) && v <= h->arch.xcds) h->queue_groups = v;
@@ -626,12 +633,12 @@ int moe_gemm_bias_act(const void* A, const void* B, const void* bias, void* C, i
     if (act != MOE_ACT_RELU && act != MOE_ACT_GELU && act != MOE_ACT_NONE) return MOE_ERR_BAD_ARGUMENT;
     if (M > INT32_MAX / 2 || N > INT32_MAX / 2 || K > INT32_MAX / 2) return MOE_ERR_UNSUPPORTED;
     hipError_t e;
-    if (dtype == MOE_DTYPE_F32) {
+    if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32) {
         if (K % 16 || N % 2) return MOE_ERR_UNSUPPORTED;
         e = launch_gemm_dense_f32(A, B, bias, C, M, N, K, act, (hipStream_t)stream);
-    } else if (dtype == MOE_DTYPE_BF16) {
+    } else if (dtype == MOE_DTYPE_BF16 || dtype == MOE_DTYPE_FP16) {
         if (K % 64 || N % 4) return MOE_ERR_UNSUPPORTED;
-        e = launch_gemm_dense_bf16(A, B, bias, C, M, N, K, act, (hipStream_t)stream);
+        e = launch_gemm_dense_bf16(A, B, bias, C, M, N, K, act, (hipStream_t)stream, dtype == MOE_DTYPE_FP16);
     } else {
         return MOE_ERR_UNSUPPORTED;
     }
@@ -641,7 +648,7 @@ int moe_gemm_bias_act(const void* A, const void* B, const void* bias, void* C, i
 int moe_combine(const void* y_rows, const int32_t* pair_row, const float* topk_w, int32_t S, int32_t k, int32_t H,
                 int32_t act_dtype, void* out, void* stream) {
     if (!y_rows || !pair_row || !topk_w || !out || S < 0 || k < 1 || H < 1) return MOE_ERR_BAD_ARGUMENT;
-    if (act_dtype != MOE_DTYPE_F32 && act_dtype != MOE_DTYPE_BF16) return MOE_ERR_UNSUPPORTED;
+    if (act_dtype != MOE_DTYPE_F32 && act_dtype != MOE_DTYPE_BF16 && act_dtype != MOE_DTYPE_FP16) return MOE_ERR_UNSUPPORTED;
     if (H % (act_dtype == MOE_DTYPE_F32 ? 4 : 8)) return MOE_ERR_UNSUPPORTED;
     const hipError_t e = launch_combine(y_rows, pair_row, topk_w, S, k, H, act_dtype, out, (hipStream_t)stream);
     return e == hipSuccess ? MOE_OK : MOE_ERR_HIP;
@@ -652,25 +659,25 @@ int moe_combine(const void* y_rows, const int32_t* pair_row, const float* topk_w
 namespace moe355 {
 
 hipError_t launch_ffn_tiled(const FfnArgs& a, int dtype, const FfnPlan& p, int max_mtiles, hipStream_t st) {
-    if (dtype == MOE_DTYPE_F32) return launch_ffn_tiled_f32(a, max_mtiles, p.nnt0, p.nnt1, st);
-    return launch_ffn_tiled_bf16(a, p.block_m, max_mtiles, p.nnt0, p.nnt1, st);
+    if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32) return launch_ffn_tiled_f32(a, max_mtiles, p.nnt0, p.nnt1, st);
+    return launch_ffn_tiled_bf16(a, p.block_m, max_mtiles, p.nnt0, p.nnt1, st, dtype == MOE_DTYPE_FP16);
 }
 
 hipError_t launch_ffn_persistent(const FfnArgs& a, int dtype, const FfnPlan& p, int blocks, hipStream_t st) {
-    if (dtype == MOE_DTYPE_F32) return launch_ffn_persistent_f32(a, blocks, st);
-    return launch_ffn_persistent_bf16(a, p.block_m, blocks, st);
+    if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32) return launch_ffn_persistent_f32(a, blocks, st);
+    return launch_ffn_persistent_bf16(a, p.block_m, blocks, st, dtype == MOE_DTYPE_FP16);
 }
 
 int ffn_persistent_blocks(int dtype, int block_m, int compute_units) {
-    if (dtype == MOE_DTYPE_F32) return compute_units * 4;
+    if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32) return compute_units * 4;
     if (dtype == MOE_DTYPE_FP8_E4M3_B128) return compute_units * ffn_persistent_occupancy_fp8();
     return compute_units * ffn_persistent_occupancy_bf16(block_m);
 }
 
 hipError_t launch_gemm_bias_act(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N,
                                 int64_t K, int dtype, int act, hipStream_t st) {
-    if (dtype == MOE_DTYPE_F32) return launch_gemm_dense_f32(A, B, bias, C, M, N, K, act, st);
-    return launch_gemm_dense_bf16(A, B, bias, C, M, N, K, act, st);
+    if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32) return launch_gemm_dense_f32(A, B, bias, C, M, N, K, act, st);
+    return launch_gemm_dense_bf16(A, B, bias, C, M, N, K, act, st, dtype == MOE_DTYPE_FP16);
 }
 
 }  // namespace moe355

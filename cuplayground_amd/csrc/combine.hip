@@ -12,19 +12,28 @@
 namespace moe355 {
 namespace {
 
-__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+__device__ __forceinline__ uint32_t pack16x2(float lo, float hi, bf16_s) {
     // round to nearest even, the rounding the oracle and torch use for bf16
     uint32_t a = __float_as_uint(lo), b = __float_as_uint(hi);
     a += 0x7FFFu + ((a >> 16) & 1u);
     b += 0x7FFFu + ((b >> 16) & 1u);
     return (a >> 16) | (b & 0xFFFF0000u);
 }
+__device__ __forceinline__ uint32_t pack16x2(float lo, float hi, f16_s) {
+    const uint32_t a = __builtin_bit_cast(uint16_t, (_Float16)lo), b = __builtin_bit_cast(uint16_t, (_Float16)hi);   // RNE
+    return a | (b << 16);
+}
+__device__ __forceinline__ float lo16(uint32_t w, bf16_s) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float hi16(uint32_t w, bf16_s) { return __uint_as_float(w & 0xFFFF0000u); }
+__device__ __forceinline__ float lo16(uint32_t w, f16_s) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xFFFFu)); }
+__device__ __forceinline__ float hi16(uint32_t w, f16_s) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16)); }
 
-// grid = (S, ceil(H / (256*8))) for bf16; each thread owns 8 consecutive columns
-__global__ __launch_bounds__(256) void combine_bf16_kernel(const uint16_t* __restrict__ y,
-                                                           const int32_t* __restrict__ pair_row,
-                                                           const float* __restrict__ topk_w, int k, int H,
-                                                           uint16_t* __restrict__ out) {
+// grid = (S, ceil(H / (256*8))) for the 16-bit types; each thread owns 8 consecutive columns
+template <typename T16>
+__global__ __launch_bounds__(256) void combine_16_kernel(const uint16_t* __restrict__ y,
+                                                         const int32_t* __restrict__ pair_row,
+                                                         const float* __restrict__ topk_w, int k, int H,
+                                                         uint16_t* __restrict__ out) {
     const int t = blockIdx.x;
     const int c = (blockIdx.y * 256 + threadIdx.x) * 8;
     if (c >= H) return;
@@ -39,15 +48,15 @@ __global__ __launch_bounds__(256) void combine_bf16_kernel(const uint16_t* __res
         const uint32_t u[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            acc[2 * i] = acc[2 * i] + w * __uint_as_float(u[i] << 16);
-            acc[2 * i + 1] = acc[2 * i + 1] + w * __uint_as_float(u[i] & 0xFFFF0000u);
+            acc[2 * i] = acc[2 * i] + w * lo16(u[i], T16{});
+            acc[2 * i + 1] = acc[2 * i + 1] + w * hi16(u[i], T16{});
         }
     }
     uint4 o;
-    o.x = pack_bf16x2(acc[0], acc[1]);
-    o.y = pack_bf16x2(acc[2], acc[3]);
-    o.z = pack_bf16x2(acc[4], acc[5]);
-    o.w = pack_bf16x2(acc[6], acc[7]);
+    o.x = pack16x2(acc[0], acc[1], T16{});
+    o.y = pack16x2(acc[2], acc[3], T16{});
+    o.z = pack16x2(acc[4], acc[5], T16{});
+    o.w = pack16x2(acc[6], acc[7], T16{});
     *reinterpret_cast<uint4*>(out + (size_t)t * H + c) = o;
 }
 
@@ -82,7 +91,10 @@ hipError_t launch_combine(const void* y_rows, const int32_t* pair_row, const flo
         combine_f32_kernel<<<grid, 256, 0, st>>>((const float*)y_rows, pair_row, topk_w, k, H, (float*)out);
     } else {
         const dim3 grid(S, (H + 256 * 8 - 1) / (256 * 8));
-        combine_bf16_kernel<<<grid, 256, 0, st>>>((const uint16_t*)y_rows, pair_row, topk_w, k, H, (uint16_t*)out);
+        if (act_dtype == MOE_DTYPE_FP16)
+            combine_16_kernel<f16_s><<<grid, 256, 0, st>>>((const uint16_t*)y_rows, pair_row, topk_w, k, H, (uint16_t*)out);
+        else
+            combine_16_kernel<bf16_s><<<grid, 256, 0, st>>>((const uint16_t*)y_rows, pair_row, topk_w, k, H, (uint16_t*)out);
     }
     return hipGetLastError();
 }

@@ -35,9 +35,12 @@ typedef const __attribute__((address_space(1))) void gbl_void;
 constexpr int kBK = 64;               // bf16 elements of K per slab = one 128-byte LDS row
 constexpr int kRowBytes = kBK * 2;
 
-template <int BM_, int BN_, int WM_, int WN_, int NS_>
+// F16: operands and results are IEEE binary16 (torch_dtype 3) instead of bfloat16; same tile, same loops, the other
+// MFMA instruction and the other conversions.
+template <int BM_, int BN_, int WM_, int WN_, int NS_, bool F16_ = false>
 struct Tile {
     static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_, NS = NS_;
+    static constexpr bool F16 = F16_;
     static constexpr int THREADS = WM * WN * kWave;
     static constexpr int TM = BM / WM / 16;       // 16x16 MFMA tiles per wavefront along tokens
     static constexpr int TN = BN / WN / 16;       // ... along weight rows
@@ -96,6 +99,26 @@ __device__ __forceinline__ float gelu_fast(float u) {
     q = fmaf(q, t, 0.254829592f);
     const float half_erfc = 0.5f * q * t * __builtin_amdgcn_exp2f(x * x * -1.4426950408889634f);
     return u * (u >= 0.0f ? 1.0f - half_erfc : half_erfc);
+}
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+// Two fp32 values rounded to the tile's 16-bit storage type (nearest even), and one stored value widened.
+template <class T>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    if constexpr (T::F16) {
+        typedef float f32x2_t __attribute__((ext_vector_type(2)));
+        typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+        const f32x2_t v = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
+    } else {
+        return pack2_bf16(lo, hi);
+    }
+}
+template <class T>
+__device__ __forceinline__ float widen1(uint16_t v) {
+    if constexpr (T::F16) return (float)__builtin_bit_cast(_Float16, v);
+    else return bf16_bits_to_f32(v);
 }
 
 // 8 bytes of output; rows that another workgroup of the same launch will read are published (ffn_common.hpp).
@@ -208,7 +231,9 @@ __device__ __forceinline__ void mainloop_generic(const TaskPtrs& p, unsigned cha
 #pragma unroll
             for (int j = 0; j < TN; ++j)
                 acc[h * HM + i][j] =
-                    __builtin_amdgcn_mfma_f32_16x16x32_bf16(bfr[bbuf][j], af[abuf][i], acc[h * HM + i][j], 0, 0, 0);
+                    T::F16 ? __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, bfr[bbuf][j]),
+                                                                      __builtin_bit_cast(f16x8, af[abuf][i]), acc[h * HM + i][j], 0, 0, 0)
+                           : __builtin_amdgcn_mfma_f32_16x16x32_bf16(bfr[bbuf][j], af[abuf][i], acc[h * HM + i][j], 0, 0, 0);
         }
     };
     // instruction order inside a unit: behind every second MFMA one LDS read and (last unit) one global load
@@ -294,11 +319,11 @@ __device__ __forceinline__ void epilogue_impl(const TaskPtrs& p, f32x4 (&acc)[T:
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     float g = acc[i][j][r], u = acc[i][j + TN / 2][r];
-                    if (p.bias1) g = g + bf16_bits_to_f32(p.bias1[col + r]);
-                    if (p.bias0) u = u + bf16_bits_to_f32(p.bias0[col + r]);
+                    if (p.bias1) g = g + widen1<T>(p.bias1[col + r]);
+                    if (p.bias0) u = u + widen1<T>(p.bias0[col + r]);
                     v[r] = silu_fast(g) * u;
                 }
-                store8(crow + col, pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]), p.publish);
+                store8(crow + col, pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3]), p.publish);
             }
         } else {
 #pragma unroll
@@ -309,10 +334,10 @@ __device__ __forceinline__ void epilogue_impl(const TaskPtrs& p, f32x4 (&acc)[T:
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     float u = acc[i][j][r];
-                    if (p.bias0) u = u + bf16_bits_to_f32(p.bias0[col + r]);
+                    if (p.bias0) u = u + widen1<T>(p.bias0[col + r]);
                     v[r] = MODE == 2 ? gelu_fast(u) : (u < relu_floor ? relu_floor : u);
                 }
-                store8(crow + col, pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]), p.publish);
+                store8(crow + col, pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3]), p.publish);
             }
         }
     }
@@ -373,13 +398,13 @@ __device__ __forceinline__ void epilogue_full_n_impl(const TaskPtrs& p, unsigned
 #pragma unroll
         for (int j = 0; j < NJ; ++j)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) b0[j][r] = bf16_bits_to_f32(p.bias0[col0 + 16 * j + 4 * fk + r]);
+            for (int r = 0; r < 4; ++r) b0[j][r] = widen1<T>(p.bias0[col0 + 16 * j + 4 * fk + r]);
     }
     if (MODE == 3 && p.bias1) {
 #pragma unroll
         for (int j = 0; j < NJ; ++j)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) b1[j][r] = bf16_bits_to_f32(p.bias1[col0 + 16 * j + 4 * fk + r]);
+            for (int r = 0; r < 4; ++r) b1[j][r] = widen1<T>(p.bias1[col0 + 16 * j + 4 * fk + r]);
     }
     // MODE 0: u below the floor becomes the floor.  Written as a compare and select, not as fmaxf: a max returns its
     // other operand for a NaN, and a NaN must stay a NaN (the reference's __hfma_relu propagates it too, processor/tiling.cuh:45,54)
@@ -408,7 +433,7 @@ __device__ __forceinline__ void epilogue_full_n_impl(const TaskPtrs& p, unsigned
                     v[r] = MODE == 2 ? gelu_fast(u) : (u < relu_floor ? relu_floor : u);
                 }
             }
-            u32x2 o = {pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3])};
+            u32x2 o = {pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3])};
             *reinterpret_cast<u32x2*>(wr + j * 32) = o;
         }
         u32x4 v[NQ];
@@ -619,7 +644,11 @@ __device__ __forceinline__ bool ring_slabs(int rows, const RingLoads& L, unsigne
     bf16x8 af[2][8], bfr[2][8];
     int kt = 0;
 
-#define MF(i, j, s) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(bfr[s][j]), "v"(af[s][i]))
+#define MF(i, j, s)                                                                                                      \
+    do {                                                                                                                 \
+        if constexpr (T::F16) asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(bfr[s][j]), "v"(af[s][i])); \
+        else asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(bfr[s][j]), "v"(af[s][i]));                  \
+    } while (0)
 #define RA(stg, half, idx) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(af[half][idx]) : "v"((stg) ? la1[half] : la0[half]), "n"((idx) * 16 * kRowBytes))
 #define RB(stg, half, j) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(bfr[half][j]) : "v"((stg) ? lb1[half] : lb0[half]), "n"((j) * 16 * kRowBytes))
 #define WL(n) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(n))
@@ -795,6 +824,8 @@ struct Plan {
 };
 using LargePlan = Plan<Tile<256, 256, 2, 2, 2>, Tile<256, 256, 2, 2, 2>>;
 using SmallPlan = Plan<Tile<128, 128, 2, 2, 2>, Tile<128, 128, 2, 2, 2>>;
+using LargePlanH = Plan<Tile<256, 256, 2, 2, 2, true>, Tile<256, 256, 2, 2, 2, true>>;   // fp16
+using SmallPlanH = Plan<Tile<128, 128, 2, 2, 2, true>, Tile<128, 128, 2, 2, 2, true>>;
 
 // One launch per phase; workgroup b runs task b of that phase.
 template <class P>
@@ -1066,12 +1097,17 @@ int bf16_block_m(int64_t pairs, int experts, int H, int I, int swiglu) {
 int bf16_block_n0(int block_m) { return block_m == 256 ? LargePlan::T0::BN : SmallPlan::T0::BN; }
 int bf16_block_n1(int block_m) { return block_m == 256 ? LargePlan::T1::BN : SmallPlan::T1::BN; }
 
-hipError_t launch_ffn_tiled_bf16(const FfnArgs& a, int block_m, int max_mtiles, int nnt0, int nnt1, hipStream_t st) {
+hipError_t launch_ffn_tiled_bf16(const FfnArgs& a, int block_m, int max_mtiles, int nnt0, int nnt1, hipStream_t st,
+                                 bool f16) {
+    if (f16)
+        return block_m == 256 ? launch_tiled<LargePlanH>(a, max_mtiles, nnt0, nnt1, st)
+                              : launch_tiled<SmallPlanH>(a, max_mtiles, nnt0, nnt1, st);
     return block_m == 256 ? launch_tiled<LargePlan>(a, max_mtiles, nnt0, nnt1, st)
                           : launch_tiled<SmallPlan>(a, max_mtiles, nnt0, nnt1, st);
 }
 
-hipError_t launch_ffn_persistent_bf16(const FfnArgs& a, int block_m, int blocks, hipStream_t st) {
+hipError_t launch_ffn_persistent_bf16(const FfnArgs& a, int block_m, int blocks, hipStream_t st, bool f16) {
+    if (f16) return block_m == 256 ? launch_persistent<LargePlanH>(a, blocks, st) : launch_persistent<SmallPlanH>(a, blocks, st);
     return block_m == 256 ? launch_persistent<LargePlan>(a, blocks, st) : launch_persistent<SmallPlan>(a, blocks, st);
 }
 
@@ -1079,28 +1115,27 @@ int ffn_persistent_occupancy_bf16(int block_m) {
     return block_m == 256 ? occupancy<LargePlan>() : occupancy<SmallPlan>();
 }
 
-hipError_t launch_gemm_dense_bf16(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N,
-                                  int64_t K, int act, hipStream_t st) {
-    const int64_t lim = (int64_t)1 << 32;
-    if (M >= 1024 && N >= 1024 && N % 256 == 0 && K % 128 == 0 && M * K * 2 < lim && N * K * 2 < lim) {
-        using T = LargePlan::T0;
-        hipError_t e = allow_lds(&gemm_dense_kernel<T>, T::LDS_BYTES);
-        if (e != hipSuccess) return e;
-        const dim3 grid((unsigned)((M + T::BM - 1) / T::BM), (unsigned)((N + T::BN - 1) / T::BN));
-        gemm_dense_kernel<T><<<grid, T::THREADS, T::LDS_BYTES, st>>>((const uint16_t*)A, (const uint16_t*)B,
-                                                                     (const uint16_t*)bias, (uint16_t*)C, (int)M,
-                                                                     (int)N, (int)K, act);
-    } else {
-        using T = SmallPlan::T0;
-        hipError_t e = allow_lds(&gemm_dense_kernel<T>, T::LDS_BYTES);
-        if (e != hipSuccess) return e;
-        const dim3 grid((unsigned)((M + T::BM - 1) / T::BM), (unsigned)((N + T::BN - 1) / T::BN));
-        gemm_dense_kernel<T><<<grid, T::THREADS, T::LDS_BYTES, st>>>((const uint16_t*)A, (const uint16_t*)B,
-                                                                     (const uint16_t*)bias, (uint16_t*)C, (int)M,
-                                                                     (int)N, (int)K, act);
-    }
+template <class T>
+static hipError_t launch_dense(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N, int64_t K,
+                               int act, hipStream_t st) {
+    hipError_t e = allow_lds(&gemm_dense_kernel<T>, T::LDS_BYTES);
+    if (e != hipSuccess) return e;
+    const dim3 grid((unsigned)((M + T::BM - 1) / T::BM), (unsigned)((N + T::BN - 1) / T::BN));
+    gemm_dense_kernel<T><<<grid, T::THREADS, T::LDS_BYTES, st>>>((const uint16_t*)A, (const uint16_t*)B,
+                                                                 (const uint16_t*)bias, (uint16_t*)C, (int)M, (int)N,
+                                                                 (int)K, act);
     return hipGetLastError();
 }
 
-}  // namespace moe355
+hipError_t launch_gemm_dense_bf16(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N,
+                                  int64_t K, int act, hipStream_t st, bool f16) {
+    const int64_t lim = (int64_t)1 << 32;
+    const bool large = M >= 1024 && N >= 1024 && N % 256 == 0 && K % 128 == 0 && M * K * 2 < lim && N * K * 2 < lim;
+    if (f16)
+        return large ? launch_dense<LargePlanH::T0>(A, B, bias, C, M, N, K, act, st)
+                     : launch_dense<SmallPlanH::T0>(A, B, bias, C, M, N, K, act, st);
+    return large ? launch_dense<LargePlan::T0>(A, B, bias, C, M, N, K, act, st)
+                 : launch_dense<SmallPlan::T0>(A, B, bias, C, M, N, K, act, st);
+}
 
+}  // namespace moe355

@@ -22,12 +22,19 @@ __device__ __forceinline__ void load8(const float* p, float (&v)[8]) {
     v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
     v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
 }
-__device__ __forceinline__ void load8(const uint16_t* p, float (&v)[8]) {
+// two 16-bit values packed in a dword -> fp32 (exact)
+__device__ __forceinline__ float lo16(uint32_t w, bf16_s) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float hi16(uint32_t w, bf16_s) { return __uint_as_float(w & 0xFFFF0000u); }
+__device__ __forceinline__ float lo16(uint32_t w, f16_s) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xFFFFu)); }
+__device__ __forceinline__ float hi16(uint32_t w, f16_s) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16)); }
+
+template <typename T16>
+__device__ __forceinline__ void load8(const T16* p, float (&v)[8]) {
     const uint4 a = reinterpret_cast<const uint4*>(p)[0];
-    v[0] = __uint_as_float(a.x << 16); v[1] = __uint_as_float(a.x & 0xFFFF0000u);
-    v[2] = __uint_as_float(a.y << 16); v[3] = __uint_as_float(a.y & 0xFFFF0000u);
-    v[4] = __uint_as_float(a.z << 16); v[5] = __uint_as_float(a.z & 0xFFFF0000u);
-    v[6] = __uint_as_float(a.w << 16); v[7] = __uint_as_float(a.w & 0xFFFF0000u);
+    v[0] = lo16(a.x, T16{}); v[1] = hi16(a.x, T16{});
+    v[2] = lo16(a.y, T16{}); v[3] = hi16(a.y, T16{});
+    v[4] = lo16(a.z, T16{}); v[5] = hi16(a.z, T16{});
+    v[6] = lo16(a.w, T16{}); v[7] = hi16(a.w, T16{});
 }
 
 // A wavefront keeps TPW token rows in registers (lane l owns the 8-element chunks l, l+64, ... of each row, as
@@ -98,8 +105,8 @@ __global__ __launch_bounds__(256) void gate_logits_kernel(const T* __restrict__ 
                     } else {
 #pragma unroll
                         for (int v = 0; v < 4; ++v) {
-                            wv[2 * v] = __uint_as_float(wc[j][v] << 16);
-                            wv[2 * v + 1] = __uint_as_float(wc[j][v] & 0xFFFF0000u);
+                            wv[2 * v] = lo16(wc[j][v], T{});
+                            wv[2 * v + 1] = hi16(wc[j][v], T{});
                         }
                     }
 #pragma unroll
@@ -182,8 +189,8 @@ __device__ __forceinline__ void widen8(const typename RawChunk<T>::type& r, floa
     } else {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            v[2 * i] = __uint_as_float(r[i] << 16);
-            v[2 * i + 1] = __uint_as_float(r[i] & 0xFFFF0000u);
+            v[2 * i] = lo16(r[i], T{});
+            v[2 * i + 1] = hi16(r[i], T{});
         }
     }
 }
@@ -427,10 +434,12 @@ hipError_t launch_gate_logits(const void* x, const void* gate_w, const float* ga
     if (const char* env = getenv("MOE355_GATE_KERNEL")) rows_in_registers = atoi(env) == 1;   // tuning knob
     if (rows_in_registers) {
         if (act_dtype == MOE_DTYPE_F32) return launch_gate_typed<float>(x, gate_w, gate_bias, logits, S, H, E, st);
-        return launch_gate_typed<uint16_t>(x, gate_w, gate_bias, logits, S, H, E, st);
+        if (act_dtype == MOE_DTYPE_FP16) return launch_gate_typed<f16_s>(x, gate_w, gate_bias, logits, S, H, E, st);
+        return launch_gate_typed<bf16_s>(x, gate_w, gate_bias, logits, S, H, E, st);
     }
     if (act_dtype == MOE_DTYPE_F32) return launch_gate_tiled<float>(x, gate_w, gate_bias, logits, S, H, E, st);
-    return launch_gate_tiled<uint16_t>(x, gate_w, gate_bias, logits, S, H, E, st);
+    if (act_dtype == MOE_DTYPE_FP16) return launch_gate_tiled<f16_s>(x, gate_w, gate_bias, logits, S, H, E, st);
+    return launch_gate_tiled<bf16_s>(x, gate_w, gate_bias, logits, S, H, E, st);
 }
 
 hipError_t launch_topk(const float* logits, int S, int E, int k, int gate_fn, int norm, int32_t* topk_idx,

@@ -9,6 +9,10 @@
 namespace moe355 {
 
 constexpr int kWave = 64;          // gfx950 wavefront
+
+// 16-bit storage types as the kernels see them: raw bit patterns with a tag that selects the conversion.
+struct bf16_s { uint16_t bits; };
+struct f16_s { uint16_t bits; };
 constexpr int kMaxExperts = 512;   // top-k keeps E/64 logits per lane in registers, 8 at most
 constexpr int kMaxTopK = 16;
 constexpr int kRouteBlock = 256;   // pairs per workgroup in the slot-assignment kernels

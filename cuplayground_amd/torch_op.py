@@ -102,7 +102,7 @@ class MoE355(torch.nn.Module):
         if tensors is None:
             if cfg.torch_dtype == api.DTYPE_FP8:
                 raise ValueError("build fp8 layers from quantised tensors: MoE355.from_packed(cfg, tensors)")
-            dt = torch.float32 if cfg.torch_dtype == api.DTYPE_F32 else torch.bfloat16
+            dt = api._torch_act_dtype(cfg.torch_dtype)
             E, H, I = cfg.num_experts, cfg.hidden_size, cfg.intermediate_size
             g = torch.Generator(device="cpu").manual_seed(seed)
 

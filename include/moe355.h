@@ -11,9 +11,9 @@
  *
  * Tensor conventions (row-major everywhere, K contiguous -- the (M,K) x (N,K) -> (M,N) convention of the
  * reference GEMM, mma.cuh:415-427):
- *   x        [S, H]        activations      f32 | bf16
+ *   x        [S, H]        activations      f32 | bf16 | fp16
  *   gate_w   [E, H]        router weights   activation dtype
- *   w_up     [E, I, H]     expert up proj   f32 | bf16 | e4m3 bytes
+ *   w_up     [E, I, H]     expert up proj   f32 | bf16 | fp16 | e4m3 bytes
  *   w_gate   [E, I, H]     SwiGLU gate proj (hidden_act = 2 only)
  *   w_down   [E, H, I]     expert down proj
  *   b_*      [E, I] / [E, H]  optional biases, activation dtype
@@ -35,7 +35,7 @@ extern "C" {
 typedef enum moe_status {
     MOE_OK = 0,
     MOE_ERR_BAD_CONFIG = 1,       /* a knob is outside its domain, or JSON is malformed / missing a key     */
-    MOE_ERR_UNSUPPORTED = 2,      /* valid knob values this build has no kernel for (tf32, fp16, E > 512 ...) */
+    MOE_ERR_UNSUPPORTED = 2,      /* valid knob values this build has no kernel for (E > 512, H > 16384 ...) */
     MOE_ERR_WORKSPACE = 3,        /* workspace pointer NULL, misaligned or smaller than moe_workspace_bytes    */
     MOE_ERR_BAD_ARGUMENT = 4,     /* NULL where a tensor is required, or an extra tensor the config excludes   */
     MOE_ERR_HIP = 5,              /* a HIP call failed; moe_last_hip_error() returns its hipError_t            */
@@ -43,7 +43,9 @@ typedef enum moe_status {
     MOE_ERR_QUEUE_STALL = 7       /* the persistent kernel's bounded dependency wait expired                   */
 } moe_status;
 
-/* torch_dtype: the reference enum (aristos_config.schema.json:54-58) plus 4 */
+/* torch_dtype: the reference enum (aristos_config.schema.json:54-58) plus 4.  Activations are stored in the layer's
+ * type, except: tf32 layers are fp32 in memory and are computed in full fp32 (gfx950 has no tf32 matrix instruction;
+ * the reference's tf32 atoms, processor/tiling.cuh:131-143, keep fp32 storage too), e4m3 layers keep bf16 activations. */
 enum { MOE_DTYPE_F32 = 0, MOE_DTYPE_TF32 = 1, MOE_DTYPE_BF16 = 2, MOE_DTYPE_FP16 = 3, MOE_DTYPE_FP8_E4M3_B128 = 4 };
 /* hidden_act: the reference enum (aristos_config.schema.json:24-28) plus 2 */
 enum { MOE_ACT_RELU = 0, MOE_ACT_GELU = 1, MOE_ACT_SWIGLU = 2, MOE_ACT_NONE = 3 /* moe_gemm_bias_act only */ };
@@ -179,7 +181,7 @@ int moe_route(moe_handle* h, const int32_t* topk_idx, int32_t* slot, int32_t* ex
               int32_t* token_indices, int32_t* pair_row, void* workspace, size_t workspace_bytes, void* stream);
 
 /* The reference tile GEMM contract, C = act(A.B^T + bias) (mma.cuh:46-179, processor/tiling.cuh:29-38).
- * dtype is MOE_DTYPE_F32 or MOE_DTYPE_BF16; act is RELU, GELU or NONE; bias [N] may be NULL. */
+ * dtype is MOE_DTYPE_F32 (TF32 is taken as F32), MOE_DTYPE_BF16 or MOE_DTYPE_FP16; act is RELU, GELU or NONE; bias [N] may be NULL. */
 int moe_gemm_bias_act(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N, int64_t K,
                       int32_t dtype, int32_t act, void* stream);
 

@@ -14,7 +14,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "liboracle.so")
 
-F32, BF16, FP8 = 0, 2, 4
+F32, TF32, BF16, F16, FP8 = 0, 1, 2, 3, 4
 ACT_RELU, ACT_GELU, ACT_SWIGLU, ACT_NONE = 0, 1, 2, 3
 GATE_SOFTMAX, GATE_SIGMOID = 0, 1
 
@@ -62,6 +62,10 @@ def lib():
         L.orc_e4m3_to_f32.argtypes = [C.c_uint8]; L.orc_e4m3_to_f32.restype = f32
         L.orc_round_bf16.argtypes = [vp, vp, i64]
         L.orc_widen_bf16.argtypes = [vp, vp, i64]
+        L.orc_round_f16.argtypes = [vp, vp, i64]
+        L.orc_widen_f16.argtypes = [vp, vp, i64]
+        L.orc_f32_to_f16.argtypes = [f32]; L.orc_f32_to_f16.restype = C.c_uint16
+        L.orc_f16_to_f32.argtypes = [C.c_uint16]; L.orc_f16_to_f32.restype = f32
         L.orc_quant_block128.argtypes = [vp, i64, i64, vp, vp]
         L.orc_dequant_block128.argtypes = [vp, vp, i64, i64, vp]
         L.orc_capacity.argtypes = [C.c_double, i64, i64, i64, C.POINTER(i64)]
@@ -76,6 +80,7 @@ def lib():
         L.orc_forward_tokens.argtypes = [C.POINTER(_Cfg), vp, C.POINTER(_Weights), vp, vp, vp, vp, i64, vp]
         L.orc_num_threads.restype = C.c_int
         for fn in ("orc_philox4x32_10", "orc_fill_normal", "orc_fill_uniform", "orc_round_bf16", "orc_widen_bf16",
+                   "orc_round_f16", "orc_widen_f16",
                    "orc_quant_block128", "orc_dequant_block128", "orc_gate_logits", "orc_topk", "orc_route",
                    "orc_gemm_bias_act", "orc_ffn_rows", "orc_combine", "orc_forward", "orc_forward_tokens"):
             getattr(L, fn).restype = None
@@ -119,7 +124,10 @@ class Cfg:
 
     @property
     def act_dtype(self) -> int:
-        return F32 if self.dtype == F32 else BF16
+        """Storage type of activations: the layer's own, except fp32 for tf32 layers and bf16 for e4m3 layers."""
+        if self.dtype in (F32, TF32):
+            return F32
+        return F16 if self.dtype == F16 else BF16
 
     def c_struct(self) -> _Cfg:
         return _Cfg(self.S, self.H, self.I, self.E, self.k, self.act, self.dtype, self.gate_fn, self.norm_topk,
@@ -172,8 +180,29 @@ def bf16_to_f32(a):
     return o
 
 
+def f32_to_f16(a):
+    a = _c(a, np.float32); o = np.empty(a.shape, np.uint16)
+    lib().orc_round_f16(_p(a), _p(o), a.size)
+    return o
+
+
+def f16_to_f32(a):
+    a = _c(a, np.uint16); o = np.empty(a.shape, np.float32)
+    lib().orc_widen_f16(_p(a), _p(o), a.size)
+    return o
+
+
 def to_f32(a, dtype):
-    return np.asarray(a, np.float32) if dtype == F32 else bf16_to_f32(a)
+    if dtype in (F32, TF32):
+        return np.asarray(a, np.float32)
+    return f16_to_f32(a) if dtype == F16 else bf16_to_f32(a)
+
+
+def from_f32(a, dtype):
+    """fp32 values rounded to an activation storage type (16-bit types as uint16 bit patterns)."""
+    if dtype in (F32, TF32):
+        return np.ascontiguousarray(a, np.float32)
+    return f32_to_f16(a) if dtype == F16 else f32_to_bf16(a)
 
 
 def quant_block128(w):
@@ -212,7 +241,7 @@ def make_inputs(cfg: Cfg, seed: int = 42, with_bias: bool = False, router_only: 
     """Seeded synthetic operands, already rounded to their storage types: tokens N(0,1), weights N(0,0.02).
     router_only skips the expert weights (enough for gate / top-k / slot checks at full size)."""
     S, H, I, E = cfg.S, cfg.H, cfg.I, cfg.E
-    act = (lambda a: a) if cfg.dtype == F32 else f32_to_bf16
+    act = lambda a: from_f32(a, cfg.act_dtype)
     inp = {"x": act(normal(S * H, seed, STREAM["x"]).reshape(S, H)),
            "gate_w": act(normal(E * H, seed, STREAM["gate_w"], 0.0, 0.02).reshape(E, H)),
            "gate_bias": zipf_gate_bias(E, seed) if cfg.zipf_bias else None}
@@ -222,10 +251,10 @@ def make_inputs(cfg: Cfg, seed: int = 42, with_bias: bool = False, router_only: 
     for n in names:
         shape = (E, H, I) if n == "w_down" else (E, I, H)
         w = normal(E * H * I, seed, STREAM[n], 0.0, 0.02).reshape(shape)
-        if cfg.dtype == F32:
+        if cfg.dtype in (F32, TF32):
             inp[n] = w
-        elif cfg.dtype == BF16:
-            inp[n] = f32_to_bf16(w)
+        elif cfg.dtype in (BF16, F16):
+            inp[n] = from_f32(w, cfg.dtype)
         else:
             inp[n], inp["s_" + n[2:]] = quant_block128(w)
         del w
@@ -291,7 +320,7 @@ def route(cfg: Cfg, inp) -> dict:
 
 def gemm_bias_act(A, B, bias, dtype, act):
     M, K = A.shape; N = B.shape[0]
-    out = np.empty((M, N), np.float32 if dtype == F32 else np.uint16)
+    out = np.empty((M, N), np.float32 if dtype in (F32, TF32) else np.uint16)
     lib().orc_gemm_bias_act(_p(np.ascontiguousarray(A)), _p(np.ascontiguousarray(B)),
                             _p(None if bias is None else np.ascontiguousarray(bias)), _p(out), M, N, K, dtype, act)
     return out
@@ -299,7 +328,7 @@ def gemm_bias_act(A, B, bias, dtype, act):
 
 def ffn_rows(cfg: Cfg, inp, tokens, experts):
     tokens = _c(tokens, np.int32); experts = _c(experts, np.int32)
-    y = np.empty((tokens.size, cfg.H), np.float32 if cfg.dtype == F32 else np.uint16)
+    y = np.empty((tokens.size, cfg.H), np.float32 if cfg.act_dtype == F32 else np.uint16)
     cs, ws = cfg.c_struct(), _weights(inp)
     lib().orc_ffn_rows(C.byref(cs), _p(inp["x"]), C.byref(ws), _p(tokens), _p(experts), tokens.size, _p(y))
     return y
@@ -315,7 +344,7 @@ def combine(y_rows, pair_row, topk_w, H, act_dtype):
 
 def forward(cfg: Cfg, inp) -> dict:
     S, k, E, H = cfg.S, cfg.k, cfg.E, cfg.H
-    out = np.empty((S, H), np.float32 if cfg.dtype == F32 else np.uint16)
+    out = np.empty((S, H), np.float32 if cfg.act_dtype == F32 else np.uint16)
     idx = np.empty((S, k), np.int32); w = np.empty((S, k), np.float32); slot = np.empty((S, k), np.int32)
     cnt = np.empty(E, np.int32); off = np.empty(E, np.int32); tok = np.empty(S * k, np.int32)
     cs, ws = cfg.c_struct(), _weights(inp)
@@ -327,7 +356,7 @@ def forward(cfg: Cfg, inp) -> dict:
 def forward_tokens(cfg: Cfg, inp, topk_idx, topk_w, slot, tokens):
     tokens = _c(tokens, np.int32)
     topk_idx = _c(topk_idx, np.int32); topk_w = _c(topk_w, np.float32); slot = _c(slot, np.int32)
-    out = np.empty((tokens.size, cfg.H), np.float32 if cfg.dtype == F32 else np.uint16)
+    out = np.empty((tokens.size, cfg.H), np.float32 if cfg.act_dtype == F32 else np.uint16)
     cs, ws = cfg.c_struct(), _weights(inp)
     lib().orc_forward_tokens(C.byref(cs), _p(inp["x"]), C.byref(ws), _p(topk_idx), _p(topk_w), _p(slot), _p(tokens),
                              tokens.size, _p(out))

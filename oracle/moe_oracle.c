@@ -122,6 +122,43 @@ float orc_e4m3_to_f32(uint8_t v) {
     return (v & 0x80u) ? -a : a;
 }
 
+/* IEEE binary16 (the reference's torch_dtype 3, aristos_config.schema.json:54-58): round to nearest even, overflow
+ * to infinity, subnormals kept. */
+uint16_t orc_f32_to_f16(float v) {
+    const uint32_t u = f2u(v);
+    const uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+    const uint32_t a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return (uint16_t)(sign | 0x7E00u | ((a >> 13) & 0x3FFu));   /* NaN, quieted */
+    if (a >= 0x477FF000u) return (uint16_t)(sign | 0x7C00u);          /* >= 65520 rounds to infinity (and inf itself) */
+    if (a < 0x33000001u) return sign;                                  /* <= 2^-25 rounds to zero (ties to even) */
+    int e = (int)(a >> 23) - 127;                                      /* unbiased exponent of the fp32 value */
+    uint32_t m = (a & 0x7FFFFFu) | 0x800000u;                          /* 24-bit significand */
+    int shift = e >= -14 ? 13 : 13 + (-14 - e);                        /* bits dropped; more for fp16 subnormals */
+    uint32_t q = m >> shift, rem = m & ((1u << shift) - 1u), half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (q & 1u))) q += 1u;
+    if (e >= -14) return (uint16_t)(sign + (uint16_t)(((uint32_t)(e + 15) << 10) + (q - 0x400u)));  /* carry may bump the exponent */
+    return (uint16_t)(sign | (uint16_t)q);                              /* subnormal (q == 0x400 is the smallest normal) */
+}
+float orc_f16_to_f32(uint16_t v) {
+    const uint32_t sign = ((uint32_t)v & 0x8000u) << 16;
+    const int e = (v >> 10) & 0x1F;
+    const uint32_t m = v & 0x3FFu;
+    if (e == 0x1F) return u2f(sign | 0x7F800000u | (m << 13));
+    if (e == 0) {
+        const float a = ldexpf((float)m, -24);
+        return (v & 0x8000u) ? -a : a;
+    }
+    return u2f(sign | ((uint32_t)(e + 112) << 23) | (m << 13));
+}
+void orc_round_f16(const float* src, uint16_t* dst, int64_t n) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; ++i) dst[i] = orc_f32_to_f16(src[i]);
+}
+void orc_widen_f16(const uint16_t* src, float* dst, int64_t n) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; ++i) dst[i] = orc_f16_to_f32(src[i]);
+}
+
 void orc_round_bf16(const float* src, uint16_t* dst, int64_t n) {
 #pragma omp parallel for schedule(static)
     for (int64_t i = 0; i < n; ++i) dst[i] = orc_f32_to_bf16(src[i]);
@@ -189,16 +226,24 @@ int orc_capacity(double capacity_factor, int64_t S, int64_t k, int64_t E, int64_
  *   +8, +4, +2, +1; the bias (if any) is added last.
  * ---------------------------------------------------------------------------------------------- */
 static inline float load_act(const void* p, int64_t i, int dtype) {
-    return dtype == ORC_F32 ? ((const float*)p)[i] : orc_bf16_to_f32(((const uint16_t*)p)[i]);
+    if (dtype == ORC_F32 || dtype == ORC_TF32) return ((const float*)p)[i];
+    return dtype == ORC_F16 ? orc_f16_to_f32(((const uint16_t*)p)[i]) : orc_bf16_to_f32(((const uint16_t*)p)[i]);
 }
 static inline void store_act(void* p, int64_t i, int dtype, float v) {
-    if (dtype == ORC_F32) ((float*)p)[i] = v;
+    if (dtype == ORC_F32 || dtype == ORC_TF32) ((float*)p)[i] = v;
+    else if (dtype == ORC_F16) ((uint16_t*)p)[i] = orc_f32_to_f16(v);
     else ((uint16_t*)p)[i] = orc_f32_to_bf16(v);
 }
 static inline float round_act(float v, int dtype) {
-    return dtype == ORC_F32 ? v : orc_bf16_to_f32(orc_f32_to_bf16(v));
+    if (dtype == ORC_F32 || dtype == ORC_TF32) return v;
+    return dtype == ORC_F16 ? orc_f16_to_f32(orc_f32_to_f16(v)) : orc_bf16_to_f32(orc_f32_to_bf16(v));
 }
-static inline int act_dtype_of(int dtype) { return dtype == ORC_F32 ? ORC_F32 : ORC_BF16; }
+/* activations travel in the layer's storage type; the e4m3 layers keep bf16 activations; tf32 (the reference's
+ * torch_dtype 1) is fp32 storage, computed here in full fp32 */
+static inline int act_dtype_of(int dtype) {
+    if (dtype == ORC_F32 || dtype == ORC_TF32) return ORC_F32;
+    return dtype == ORC_F16 ? ORC_F16 : ORC_BF16;
+}
 
 static float gate_dot(const float* x, const float* w, int32_t H) {
     float acc[64];
@@ -390,6 +435,14 @@ static float dot_bf16(const float* a, const uint16_t* b, int64_t K) {
     for (int j = 0; k < K; ++k, ++j) acc[j] = acc[j] + a[k] * u2f((uint32_t)b[k] << 16);
     return fold16(acc);
 }
+static float dot_f16(const float* a, const uint16_t* b, int64_t K) {
+    float acc[16] = {0};
+    int64_t k = 0;
+    for (; k + 16 <= K; k += 16)
+        for (int j = 0; j < 16; ++j) acc[j] = acc[j] + a[k + j] * orc_f16_to_f32(b[k + j]);
+    for (int j = 0; k < K; ++k, ++j) acc[j] = acc[j] + a[k] * orc_f16_to_f32(b[k]);
+    return fold16(acc);
+}
 static float e4m3_lut[256];
 static int e4m3_lut_ready = 0;
 static void e4m3_lut_init(void) {
@@ -421,8 +474,9 @@ static float dot_fp8(const float* a, const uint8_t* q, const float* scale_row, i
 }
 /* row n of a [N,K] weight matrix in storage dtype `dtype`, dotted with the fp32 vector a */
 static inline float dot_w(const float* a, const void* W, const float* scales, int64_t n, int64_t K, int dtype) {
-    if (dtype == ORC_F32) return dot_f32(a, (const float*)W + n * K, K);
+    if (dtype == ORC_F32 || dtype == ORC_TF32) return dot_f32(a, (const float*)W + n * K, K);
     if (dtype == ORC_BF16) return dot_bf16(a, (const uint16_t*)W + n * K, K);
+    if (dtype == ORC_F16) return dot_f16(a, (const uint16_t*)W + n * K, K);
     const int64_t kb = (K + 127) / 128;
     return dot_fp8(a, (const uint8_t*)W + n * K, scales + (n / 128) * kb, K);
 }
@@ -469,7 +523,7 @@ static void ffn_one_row(const orc_cfg* c, const float* xrow, const orc_weights* 
     const int adt = act_dtype_of(c->dtype);
     const int64_t H = c->H, I = c->I;
     const int64_t kbH = (H + 127) / 128, kbI = (I + 127) / 128, nbI = (I + 127) / 128, nbH = (H + 127) / 128;
-    const size_t wel = c->dtype == ORC_F32 ? 4 : (c->dtype == ORC_BF16 ? 2 : 1);
+    const size_t wel = (c->dtype == ORC_F32 || c->dtype == ORC_TF32) ? 4 : (c->dtype == ORC_FP8 ? 1 : 2);
     const char* Wu = (const char*)w->w_up + (size_t)e * I * H * wel;
     const char* Wg = w->w_gate ? (const char*)w->w_gate + (size_t)e * I * H * wel : NULL;
     const char* Wd = (const char*)w->w_down + (size_t)e * H * I * wel;

@@ -7,7 +7,7 @@
  * The reference (osayamenja/cuPlayground) only fixes fragments of this path; each function below cites the
  * fragment it follows and says where the semantics are defined by this build instead.  Pinning status:
  *   - orc_philox4x32_10        pinned by the Random123 known-answer vectors (tests/test_oracle_rng.py)
- *   - bf16 / e4m3 conversions  pinned by exhaustive code-point round trips and torch CPU casts
+ *   - bf16 / fp16 / e4m3 conversions  pinned by exhaustive code-point round trips and torch / numpy CPU casts
  *   - orc_gemm_bias_act        pinned by the reference driver's known-answer corner (mma.cuh:394-411)
  *                              and by float64 triple loops on random shapes
  *   - orc_gate_logits          pinned against float64 dot products (value) and against a pure-Python
@@ -33,7 +33,7 @@ extern "C" {
 #endif
 
 /* storage dtype codes: the reference's torch_dtype enum (aristos_config.schema.json:54-58) plus 4 = e4m3 */
-enum { ORC_F32 = 0, ORC_BF16 = 2, ORC_FP8 = 4 };
+enum { ORC_F32 = 0, ORC_TF32 = 1, ORC_BF16 = 2, ORC_F16 = 3, ORC_FP8 = 4 };
 /* hidden_act codes (aristos_config.schema.json:24-28) plus 2 = SwiGLU; ORC_ACT_NONE is for the bare GEMM */
 enum { ORC_ACT_RELU = 0, ORC_ACT_GELU = 1, ORC_ACT_SWIGLU = 2, ORC_ACT_NONE = 3 };
 enum { ORC_GATE_SOFTMAX = 0, ORC_GATE_SIGMOID = 1 };
@@ -72,6 +72,10 @@ uint16_t orc_f32_to_bf16(float v);
 float orc_bf16_to_f32(uint16_t v);
 uint8_t orc_f32_to_e4m3(float v);
 float orc_e4m3_to_f32(uint8_t v);
+uint16_t orc_f32_to_f16(float v);
+float orc_f16_to_f32(uint16_t v);
+void orc_round_f16(const float* src, uint16_t* dst, int64_t n);
+void orc_widen_f16(const uint16_t* src, float* dst, int64_t n);
 void orc_round_bf16(const float* src, uint16_t* dst, int64_t n);
 void orc_widen_bf16(const uint16_t* src, float* dst, int64_t n);
 void orc_quant_block128(const float* w, int64_t N, int64_t K, uint8_t* q, float* scales);

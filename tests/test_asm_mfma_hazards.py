@@ -12,7 +12,8 @@ import pytest
 
 from cuplayground_amd import build as moe_build
 
-WINDOW = 12   # instructions; a 16x16x32 bf16 MFMA takes 8 passes of 4 cycles
+WINDOW = 12   # instructions; a 16x16x32 bf16 / fp16 MFMA takes 8 passes of 4 cycles
+MFMA = ("v_mfma_f32_16x16x32_bf16", "v_mfma_f32_16x16x32_f16")
 
 
 _ASM = {}
@@ -48,16 +49,15 @@ def test_slab_loop_holds_nothing_but_the_schedule():
                 continue
             body = [x.strip() for x in lines[labels[m.group(1)]:k + 1]]
             body = [x for x in body if x and not x.startswith((";", "."))]
-            if sum(x.startswith("v_mfma_f32_16x16x32_bf16") for x in body) != 256 or len(body) > 1000:
+            if sum(x.startswith(MFMA) for x in body) != 256 or len(body) > 1000:
                 continue
             loops += 1
-            other = [x for x in body if x.startswith(("v_", "scratch_", "global_", "flat_"))
-                     and not x.startswith("v_mfma_f32_16x16x32_bf16")]
+            other = [x for x in body if x.startswith(("v_", "scratch_", "global_", "flat_")) and not x.startswith(MFMA)]
             assert not other, "unexpected instructions in the slab loop: %s" % other[:5]
             assert sum(x.startswith("ds_read_b128") for x in body) == 64
             assert sum(x.startswith("buffer_load_dwordx4") for x in body) == 32
             assert sum(x.startswith("s_barrier") for x in body) == 4
-    assert loops >= 3, "expected the slab loop in the two-launch, queue and plain-GEMM kernels, found %d" % loops
+    assert loops >= 8, "expected the slab loop in the two-launch, both queue and the plain-GEMM kernels, bf16 and fp16, found %d" % loops
 
 
 @pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
@@ -70,7 +70,7 @@ def test_no_accumulator_access_behind_asm_mfma():
     labels = {m.group(1): k for k, l in enumerate(lines) for m in [re.match(r"^(\.LBB\d+_\d+):", l)] if m}
     asm_mfmas, bad = 0, []
     for k, line in enumerate(lines):
-        m = re.search(r"v_mfma_f32_16x16x32_bf16 a\[(\d+):(\d+)\]", line)
+        m = re.search(r"v_mfma_f32_16x16x32_b?f16 a\[(\d+):(\d+)\]", line)
         if not m or "ASMSTART" not in lines[k - 1]:
             continue
         asm_mfmas += 1
@@ -93,7 +93,7 @@ def test_no_accumulator_access_behind_asm_mfma():
                 reg = int([g for g in a.groups()[1:] if g][0])
                 if lo <= reg <= hi:
                     bad.append((line.strip(), seen, x))
-    assert asm_mfmas >= 256, "the slab loop's inline-asm MFMAs were not found: has the kernel changed?"
+    assert asm_mfmas >= 8 * 256, "the slab loop's inline-asm MFMAs were not found: has the kernel changed?"
     assert not bad, "accumulators touched behind an in-flight MFMA:\n" + "\n".join("%s -> +%d %s" % b for b in bad[:10])
 
 

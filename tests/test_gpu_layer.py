@@ -83,6 +83,10 @@ RAGGED = {
                                gate_fn=ob.GATE_SIGMOID, drop=0),
     "fp8_many_rows_bias": ob.Cfg(S=200, H=384, I=384, E=4, k=2, act=ob.ACT_SWIGLU, dtype=ob.FP8,
                                  gate_fn=ob.GATE_SIGMOID, drop=1, capacity_factor=1.0),
+    "fp16_swiglu_skew_bias": ob.Cfg(S=900, H=256, I=320, E=24, k=4, act=ob.ACT_SWIGLU, dtype=ob.F16, drop=1,
+                                    capacity_factor=1.0, zipf_bias=True),
+    "fp16_relu_ragged": ob.Cfg(S=301, H=192, I=448, E=5, k=2, act=ob.ACT_RELU, dtype=ob.F16, drop=0),
+    "tf32_gelu_ragged": ob.Cfg(S=150, H=128, I=192, E=4, k=2, act=ob.ACT_GELU, dtype=ob.TF32, drop=1, capacity_factor=0.8),
     "one_token": ob.Cfg(S=1, H=64, I=64, E=2, k=1, act=ob.ACT_GELU, dtype=ob.BF16, norm_topk=0, drop=0),
     # every expert selected by every token; a single expert; the widest router the kernels take; capacity of one row
     "all_experts_selected": ob.Cfg(S=100, H=64, I=64, E=4, k=4, act=ob.ACT_SWIGLU, dtype=ob.BF16, drop=0),
@@ -172,6 +176,8 @@ LARGE_TILE = {
     "swiglu_k_not_128": ob.Cfg(S=800, H=192, I=320, E=3, k=2, act=ob.ACT_SWIGLU, dtype=ob.BF16, drop=0),
     # the shortest K the slab loop takes (two slabs in the down projection), row blocks that are exactly full
     "swiglu_two_slabs": ob.Cfg(S=512, H=256, I=128, E=1, k=1, act=ob.ACT_SWIGLU, dtype=ob.BF16, norm_topk=0, drop=0),
+    "fp16_swiglu_bias": ob.Cfg(S=1400, H=256, I=256, E=3, k=2, act=ob.ACT_SWIGLU, dtype=ob.F16, drop=0),
+    "fp16_gelu_drop": ob.Cfg(S=1200, H=512, I=512, E=2, k=2, act=ob.ACT_GELU, dtype=ob.F16, drop=1, capacity_factor=0.9),
     # most experts empty, one row here and there
     "gelu_sparse_experts": ob.Cfg(S=40, H=256, I=256, E=32, k=1, act=ob.ACT_GELU, dtype=ob.BF16, norm_topk=0, drop=0),
     "relu_bias_capacity_drop": ob.Cfg(S=1100, H=512, I=256, E=2, k=2, act=ob.ACT_RELU, dtype=ob.BF16, drop=1,

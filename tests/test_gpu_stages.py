@@ -28,11 +28,14 @@ def bits(a):
 
 
 # ---------------------------------------------------------------- GEMM + epilogue (reference fGET contract)
-@pytest.mark.parametrize("dtype", [ob.F32, ob.BF16])
+KIND = {ob.F32: "f32", ob.BF16: "bf16", ob.F16: "f16"}
+
+
+@pytest.mark.parametrize("dtype", [ob.F32, ob.BF16, ob.F16])
 def test_gemm_reference_driver_known_answer(moe, dtype):
     """testCollective's operands (mma.cuh:394-411): closed-form expected output."""
     A, B, bias, want = collective_operands(dtype)
-    kind = "f32" if dtype == ob.F32 else "bf16"
+    kind = KIND[dtype]
     C = moe.gemm_bias_act(to_device(A, kind), to_device(B, kind), to_device(bias, kind), ob.ACT_RELU)
     got = ob.to_f32(from_device(C), dtype)
     assert got[0, 0] == 6 and got[0, 1] == 9 and got[1, 0] == 24 and got[1, 1] == 35
@@ -41,20 +44,19 @@ def test_gemm_reference_driver_known_answer(moe, dtype):
 
 @pytest.mark.parametrize("act", [ob.ACT_RELU, ob.ACT_GELU, ob.ACT_NONE])
 @pytest.mark.parametrize("dtype,M,N,K", [(ob.F32, 100, 66, 48), (ob.F32, 64, 128, 256), (ob.BF16, 300, 200, 192),
-                                         (ob.BF16, 128, 128, 64), (ob.BF16, 1, 4, 64), (ob.BF16, 129, 260, 1024)])
+                                         (ob.BF16, 128, 128, 64), (ob.BF16, 1, 4, 64), (ob.BF16, 129, 260, 1024),
+                                         (ob.F16, 300, 200, 192), (ob.F16, 129, 260, 1024), (ob.F16, 1100, 1024, 256)])
 def test_gemm_vs_oracle(moe, dtype, M, N, K, act):
     rng = np.random.default_rng(M * 7 + N)
     A = rng.standard_normal((M, K)).astype(np.float32)
     B = (rng.standard_normal((N, K)) * 0.1).astype(np.float32)
     bias = rng.standard_normal(N).astype(np.float32)
-    kind = "f32"
-    if dtype == ob.BF16:
-        A, B, bias = ob.f32_to_bf16(A), ob.f32_to_bf16(B), ob.f32_to_bf16(bias)
-        kind = "bf16"
+    kind = KIND[dtype]
+    A, B, bias = ob.from_f32(A, dtype), ob.from_f32(B, dtype), ob.from_f32(bias, dtype)
     want = ob.to_f32(ob.gemm_bias_act(A, B, bias, dtype, act), dtype)
     got = ob.to_f32(from_device(moe.gemm_bias_act(to_device(A, kind), to_device(B, kind), to_device(bias, kind), act)),
                     dtype)
-    tol = 1e-5 if dtype == ob.F32 else 1e-2     # fp32: summation order only; bf16: one output ulp is 2^-8
+    tol = {ob.F32: 1e-5, ob.BF16: 1e-2, ob.F16: 1.25e-3}[dtype]   # fp32: summation order only; bf16 / fp16: an output ulp is 2^-8 / 2^-11
     assert np.abs(got - want).max() <= tol * np.abs(want).max()
     got_nb = ob.to_f32(from_device(moe.gemm_bias_act(to_device(A, kind), to_device(B, kind), None, act)), dtype)
     want_nb = ob.to_f32(ob.gemm_bias_act(A, B, None, dtype, act), dtype)
@@ -99,7 +101,8 @@ def test_combine_reference_identity_case(moe, dtype):
     assert np.array_equal(ob.to_f32(from_device(out), dtype), y)
 
 
-@pytest.mark.parametrize("dtype,S,k,H", [(ob.F32, 50, 3, 64), (ob.BF16, 333, 6, 2048), (ob.BF16, 64, 8, 7168)])
+@pytest.mark.parametrize("dtype,S,k,H", [(ob.F32, 50, 3, 64), (ob.BF16, 333, 6, 2048), (ob.BF16, 64, 8, 7168),
+                                         (ob.F16, 200, 2, 1024)])
 def test_combine_vs_oracle(moe, dtype, S, k, H):
     rng = np.random.default_rng(S)
     A = S * k
@@ -108,11 +111,11 @@ def test_combine_vs_oracle(moe, dtype, S, k, H):
     rows[::5, 0] = -1
     rows[3, :] = -1
     w = rng.random((S, k)).astype(np.float32)
-    kind = "f32" if dtype == ob.F32 else "bf16"
-    yy = y if dtype == ob.F32 else ob.f32_to_bf16(y)
+    kind = KIND[dtype]
+    yy = ob.from_f32(y, dtype)
     want = ob.to_f32(ob.combine(yy, rows, w, H, dtype), dtype)
     got = ob.to_f32(from_device(moe.combine(to_device(yy, kind), to_device(rows, "i32"), to_device(w, "f32"))), dtype)
-    tol = 1e-6 if dtype == ob.F32 else 2.0 ** -8
+    tol = {ob.F32: 1e-6, ob.BF16: 2.0 ** -8, ob.F16: 2.0 ** -11}[dtype]
     assert np.abs(got - want).max() <= tol * np.abs(want).max()
     assert (got[3] == 0).all()
 
@@ -125,6 +128,9 @@ GATE_CASES = [
     ob.Cfg(S=64, H=7168, I=128, E=256, k=8, dtype=ob.BF16, gate_fn=ob.GATE_SIGMOID),
     ob.Cfg(S=33, H=4096, I=64, E=300, k=16, dtype=ob.BF16, norm_topk=0),
     ob.Cfg(S=1000, H=2048, I=64, E=16, k=2, dtype=ob.BF16),
+    ob.Cfg(S=300, H=1536, I=64, E=40, k=4, dtype=ob.F16),
+    ob.Cfg(S=20000, H=512, I=64, E=32, k=2, dtype=ob.F16),     # many pairs: the kernel that keeps token rows in registers
+    ob.Cfg(S=50, H=128, I=64, E=5, k=2, dtype=ob.TF32),
 ]
 
 

@@ -106,7 +106,10 @@ def test_workspace_and_unsupported_shapes():
     assert 0 < small < big and small % 256 == 0
     # at least the two intermediates: h [A,I] and y [A,H] in bf16
     assert small >= 128 * 2 * (512 + 256) * 2
-    for patch in ({"torch_dtype": 1}, {"torch_dtype": 3}, {"num_experts": 1024}, {"expert_top_k": 17, "num_experts": 64}):
+    # every dtype of the reference schema has a kernel: tf32 is stored and computed as fp32 (twice the bytes of bf16)
+    assert moe.MoEConfig(**{**base, "torch_dtype": 3}).workspace_bytes() == small
+    assert moe.MoEConfig(**{**base, "torch_dtype": 1}).workspace_bytes() == moe.MoEConfig(**{**base, "torch_dtype": 0}).workspace_bytes() > small
+    for patch in ({"num_experts": 1024}, {"expert_top_k": 17, "num_experts": 64}, {"hidden_size": 32768}):
         with pytest.raises(moe.MoEError) as e:
             moe.MoEConfig(**{**base, **patch}).workspace_bytes()
         assert e.value.status == 2

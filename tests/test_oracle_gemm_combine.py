@@ -16,12 +16,11 @@ def collective_operands(dtype):
     want = np.zeros((M, N), np.float32)
     want[:, 0] = 1; want[:, 1] = 2
     want[0, 0], want[0, 1], want[1, 0], want[1, 1] = 0 * 4 + 1 * 5 + 1, 0 * 6 + 1 * 7 + 2, 2 * 4 + 3 * 5 + 1, 2 * 6 + 3 * 7 + 2
-    if dtype == ob.BF16:
-        A, B, bias = ob.f32_to_bf16(A), ob.f32_to_bf16(B), ob.f32_to_bf16(bias)
+    A, B, bias = ob.from_f32(A, dtype), ob.from_f32(B, dtype), ob.from_f32(bias, dtype)
     return A, B, bias, want
 
 
-@pytest.mark.parametrize("dtype", [ob.F32, ob.BF16])
+@pytest.mark.parametrize("dtype", [ob.F32, ob.BF16, ob.F16])
 def test_reference_driver_known_answer(dtype):
     A, B, bias, want = collective_operands(dtype)
     C = ob.to_f32(ob.gemm_bias_act(A, B, bias, dtype, ob.ACT_RELU), dtype)

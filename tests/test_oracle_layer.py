@@ -49,6 +49,10 @@ CASES = {
                              capacity_factor=1.25),
     "bf16_swiglu_sigmoid": ob.Cfg(S=40, H=192, I=128, E=16, k=4, act=ob.ACT_SWIGLU, dtype=ob.BF16,
                                   gate_fn=ob.GATE_SIGMOID, norm_topk=1, drop=0),
+    "fp16_swiglu_top2_bias": ob.Cfg(S=72, H=128, I=192, E=6, k=2, act=ob.ACT_SWIGLU, dtype=ob.F16, norm_topk=1, drop=1,
+                                    capacity_factor=1.0),
+    "fp16_gelu_top1": ob.Cfg(S=50, H=64, I=128, E=3, k=1, act=ob.ACT_GELU, dtype=ob.F16, norm_topk=0, drop=0),
+    "tf32_relu_top2": ob.Cfg(S=40, H=64, I=64, E=4, k=2, act=ob.ACT_RELU, dtype=ob.TF32, norm_topk=1, drop=0),
     "fp8_swiglu_sigmoid": ob.Cfg(S=24, H=256, I=128, E=12, k=3, act=ob.ACT_SWIGLU, dtype=ob.FP8,
                                  gate_fn=ob.GATE_SIGMOID, norm_topk=1, drop=0),
 }
@@ -66,7 +70,7 @@ def test_layer_equals_dense_mixture(name):
     want = dense_mixture(cfg, inp, r)
     got = ob.to_f32(r["out"], cfg.act_dtype)
     # storage rounding of h, y and out (bf16: 2^-9 relative each) is the only difference from float64
-    tol = 1e-5 if cfg.dtype == ob.F32 else 1e-2
+    tol = {ob.F32: 1e-5, ob.TF32: 1e-5, ob.F16: 1.25e-3}.get(cfg.dtype, 1e-2)
     assert np.abs(got - want).max() <= tol * np.abs(want).max()
     assert np.abs(want).max() > 0
     # dropped-everywhere tokens are exactly zero

@@ -49,6 +49,32 @@ def test_bf16_rounding_matches_torch():
     assert np.array_equal(ob.f32_to_bf16(x), want)
 
 
+def test_fp16_every_code_point_and_rounding_match_numpy():
+    """IEEE binary16 (the reference's torch_dtype 3): every code widens as numpy's float16 does and rounds back to
+    itself; round-to-nearest-even on random values over the whole range, on every kind of midpoint and its two
+    neighbours, at the overflow threshold and in the subnormals -- against numpy's cast, a library routine."""
+    codes = np.arange(65536, dtype=np.uint16)
+    wide = ob.f16_to_f32(codes)
+    ref = codes.view(np.float16).astype(np.float32)
+    assert ((wide.view(np.uint32) == ref.view(np.uint32)) | (np.isnan(wide) & np.isnan(ref))).all()
+    finite = ~np.isnan(ref)
+    assert np.array_equal(ob.f32_to_f16(wide)[finite], codes[finite])
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal(300000).astype(np.float32) * np.float32(10.0) ** rng.integers(-9, 6, 300000).astype(np.float32)
+    h = rng.integers(0, 0x7BFF, 100000).astype(np.uint16)
+    a = h.view(np.float16).astype(np.float64)
+    b = (h + 1).astype(np.uint16).view(np.float16).astype(np.float64)
+    mid = ((a + b) / 2).astype(np.float32)
+    edge = np.array([65504, 65519.996, 65520, 65536, 1e9, -1e9, np.inf, -np.inf, 0, -0.0, 5.96e-8, 2.98e-8,
+                     2.9802322e-8, 2.9802326e-8, 6.1e-5, 6.097e-5], np.float32)
+    x = np.concatenate([x, -x[:1000], mid, np.nextafter(mid, np.float32(np.inf)), np.nextafter(mid, np.float32(-np.inf)), edge])
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    assert np.array_equal(ob.f32_to_f16(x), want)
+    nan = ob.f32_to_f16(np.array([np.nan], np.float32))
+    assert (nan[0] & 0x7C00) == 0x7C00 and (nan[0] & 0x3FF) != 0
+
+
 def test_e4m3_decode_matches_torch_for_all_codes():
     codes = np.arange(256, dtype=np.uint8)
     want = torch.from_numpy(codes).view(torch.float8_e4m3fn).float().numpy()

@@ -180,7 +180,8 @@ int moe_config_validate(const moe_config* c, char* err, size_t n) {
     if (c->gate_fn != MOE_GATE_SOFTMAX && c->gate_fn != MOE_GATE_SIGMOID) { set_err(err, n, "gate_fn must be 0 (softmax) or 1 (sigmoid)"); return MOE_ERR_BAD_CONFIG; }
     if (c->norm_topk_prob != 0 && c->norm_topk_prob != 1) { set_err(err, n, "norm_topk_prob must be 0 or 1"); return MOE_ERR_BAD_CONFIG; }
     const int64_t S = (int64_t)c->micro_batch * c->sequence_len;
-    if (S * c->expert_top_k > (int64_t)1 << 30) { set_err(err, n, "micro_batch*sequence_len*expert_top_k exceeds 2^30"); return MOE_ERR_BAD_CONFIG; }
+    // S * k against 2^30, without forming a product that could overflow
+    if (S > ((int64_t)1 << 30) / c->expert_top_k) { set_err(err, n, "micro_batch*sequence_len*expert_top_k exceeds 2^30"); return MOE_ERR_BAD_CONFIG; }
     return MOE_OK;
 }
 
@@ -233,8 +234,9 @@ int moe_config_capacity(const moe_config* c, int64_t* capacity) {
     if (!c || !capacity) return MOE_ERR_BAD_ARGUMENT;
     if (c->num_experts < 1 || c->expert_top_k < 1 || !(c->capacity_factor > 0.0)) return MOE_ERR_BAD_CONFIG;
     const int64_t S = moe_config_tokens(c);
-    double v = std::ceil(c->capacity_factor * (double)(S * c->expert_top_k) / (double)c->num_experts);
-    if (v < 1.0) v = 1.0;
+    double v = std::ceil(c->capacity_factor * ((double)S * (double)c->expert_top_k) / (double)c->num_experts);
+    if (!(v >= 1.0)) v = 1.0;
+    if (v > 9.0e18) v = 9.0e18;   // beyond any row count; keeps the conversion defined
     *capacity = (int64_t)v;
     return MOE_OK;
 }

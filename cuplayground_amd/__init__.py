@@ -16,4 +16,6 @@ from .api import (  # noqa: F401
     load_library,
     measured_peaks,
     quantize_block128,
+    transpose,
 )
+from . import api  # noqa: F401

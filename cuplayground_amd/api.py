@@ -26,7 +26,8 @@ EXPORTS = (
     "moe_workspace_bytes",
     "moe_set_ffn_mode", "moe_get_ffn_mode", "moe_forward", "moe_forward_static", "moe_set_spin_limit", "moe_clear_stall", "moe_gate", "moe_router_stats", "moe_route", "moe_gemm_bias_act", "moe_combine",
     "moe_set_stage_timing", "moe_get_stage_ms", "moe_get_stage_samples", "moe_get_task_counts", "moe_measure_mfma_tflops",
-    "moe_measure_hbm_read_gbs", "moe_quant_block128", "moe_last_hip_error", "moe_status_string",
+    "moe_measure_hbm_read_gbs", "moe_quant_block128", "moe_backward_scratch_bytes", "moe_transpose", "moe_expert_gemm",
+    "moe_expert_wgrad", "moe_last_hip_error", "moe_status_string",
     "moe_version",
 )
 
@@ -105,6 +106,10 @@ def load_library():
     L.moe_quant_block128.argtypes = [vp, C.c_int32, C.c_int64, C.c_int64, C.c_int64, vp, vp, vp]
     L.moe_measure_mfma_tflops.argtypes = [vp, C.c_size_t, vp, C.c_int, C.POINTER(C.c_float)]
     L.moe_measure_hbm_read_gbs.argtypes = [vp, C.c_size_t, vp, vp, C.POINTER(C.c_float)]
+    L.moe_backward_scratch_bytes.argtypes = [cfgp, C.POINTER(C.c_size_t)]
+    L.moe_transpose.argtypes = [vp, vp, i64, i64, i64, i32, vp]
+    L.moe_expert_gemm.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, vp, C.c_size_t, vp]
+    L.moe_expert_wgrad.argtypes = [vp, vp, vp, vp, vp, i32, i32, vp, vp, C.c_size_t, vp]
     L.moe_last_hip_error.argtypes = [vp]
     L.moe_status_string.argtypes = [C.c_int]; L.moe_status_string.restype = C.c_char_p
     L.moe_version.restype = C.c_int
@@ -362,6 +367,51 @@ class MoELayer:
                                 _ptr(r["expert_offset"]), _ptr(r["token_indices"]), _ptr(r["pair_row"]),
                                 _ptr(self.workspace), self.workspace_bytes, _stream()), "moe_route")
         return r
+
+    # ---- backward building blocks (bf16 / fp16 layers) ----
+    def backward_scratch(self):
+        """Device scratch for expert_gemm / expert_wgrad, allocated on first use and kept with the layer."""
+        import torch
+        if getattr(self, "_bwd_scratch", None) is None:
+            n = C.c_size_t(0)
+            _check(self.L.moe_backward_scratch_bytes(C.byref(self.cfg.to_c()), C.byref(n)), "moe_backward_scratch_bytes")
+            self._bwd_scratch = torch.empty(n.value, dtype=torch.uint8, device="cuda")
+        return self._bwd_scratch
+
+    def expert_gemm(self, a_rows, w, bias, expert_count, expert_offset, act: int = ACT_NONE, out=None):
+        """out_rows[r] = act(a_rows[r] . w[e(r)]^T + bias[e(r)]) over the kept packed rows; w [E,N,K]."""
+        import torch
+        N, K = w.shape[1], w.shape[2]
+        if out is None:
+            out = torch.zeros(a_rows.shape[0], N, dtype=a_rows.dtype, device=a_rows.device)
+        sc = self.backward_scratch()
+        _check(self.L.moe_expert_gemm(self._h, _ptr(a_rows), _ptr(w), _ptr(bias), _ptr(expert_count),
+                                      _ptr(expert_offset), N, K, act, _ptr(out), _ptr(sc), sc.numel(), _stream()),
+               "moe_expert_gemm")
+        return out
+
+    def expert_wgrad(self, dy_rows, a_rows, expert_count, expert_offset, out=None):
+        """dw[e] [N,K] = sum over expert e's rows of dy_rows[r,:N]^T a_rows[r,:K]."""
+        import torch
+        N, K = dy_rows.shape[1], a_rows.shape[1]
+        if out is None:
+            out = torch.empty(self.E, N, K, dtype=a_rows.dtype, device=a_rows.device)
+        sc = self.backward_scratch()
+        _check(self.L.moe_expert_wgrad(self._h, _ptr(dy_rows), _ptr(a_rows), _ptr(expert_count), _ptr(expert_offset),
+                                       N, K, _ptr(out), _ptr(sc), sc.numel(), _stream()), "moe_expert_wgrad")
+        return out
+
+
+def transpose(src, out=None):
+    """[.., R, C] -> [.., C, R] for 2- and 4-byte element types, batched over the leading dimensions."""
+    import torch
+    R, Cc = src.shape[-2], src.shape[-1]
+    src = src.contiguous()
+    if out is None:
+        out = torch.empty(*src.shape[:-2], Cc, R, dtype=src.dtype, device=src.device)
+    _check(load_library().moe_transpose(_ptr(src), _ptr(out), src.numel() // (R * Cc), R, Cc, src.element_size(),
+                                        _stream()), "moe_transpose")
+    return out
 
 
 def measured_peaks() -> dict:

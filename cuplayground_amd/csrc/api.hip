@@ -645,6 +645,59 @@ int moe_gemm_bias_act(const void* A, const void* B, const void* bias, void* C, i
     return e == hipSuccess ? MOE_OK : MOE_ERR_HIP;
 }
 
+int moe_backward_scratch_bytes(const moe_config* cfg, size_t* bytes) {
+    if (!cfg || !bytes) return MOE_ERR_BAD_ARGUMENT;
+    Derived d;
+    const int rc = derive(*cfg, &d);
+    if (rc) return rc;
+    if (d.act_dtype != MOE_DTYPE_BF16 && d.act_dtype != MOE_DTYPE_FP16) return MOE_ERR_UNSUPPORTED;
+    *bytes = backward_scratch_bytes(d.A, d.E, d.H, d.I);
+    return MOE_OK;
+}
+
+int moe_transpose(const void* src, void* dst, int64_t batch, int64_t rows, int64_t cols, int32_t elem_bytes, void* stream) {
+    if (!src || !dst || batch < 0 || rows < 0 || cols < 0) return MOE_ERR_BAD_ARGUMENT;
+    if (elem_bytes != 2 && elem_bytes != 4) return MOE_ERR_UNSUPPORTED;
+    if (batch > 65535 || rows > INT32_MAX || cols > INT32_MAX) return MOE_ERR_UNSUPPORTED;
+    const hipError_t e = launch_transpose(src, dst, batch, rows, cols, elem_bytes, (hipStream_t)stream);
+    return e == hipSuccess ? MOE_OK : MOE_ERR_HIP;
+}
+
+namespace {
+int check_backward_call(const moe_handle* h, int32_t N, int32_t K, const void* scratch, size_t scratch_bytes) {
+    if (h->d.act_dtype != MOE_DTYPE_BF16 && h->d.act_dtype != MOE_DTYPE_FP16) return MOE_ERR_UNSUPPORTED;
+    if (h->cfg.torch_dtype == MOE_DTYPE_FP8_E4M3_B128) return MOE_ERR_UNSUPPORTED;
+    const bool dims_ok = (N == h->d.H && K == h->d.I) || (N == h->d.I && K == h->d.H);
+    if (!dims_ok) return MOE_ERR_BAD_ARGUMENT;      // (N, K) is a projection of this layer, one way or the other
+    if (!scratch || ((uintptr_t)scratch % kAlign) || scratch_bytes < backward_scratch_bytes(h->d.A, h->d.E, h->d.H, h->d.I))
+        return MOE_ERR_WORKSPACE;
+    return MOE_OK;
+}
+}  // namespace
+
+int moe_expert_gemm(moe_handle* h, const void* a_rows, const void* w, const void* bias, const int32_t* expert_count,
+                    const int32_t* expert_offset, int32_t N, int32_t K, int32_t act, void* out_rows, void* scratch,
+                    size_t scratch_bytes, void* stream) {
+    if (!h || !a_rows || !w || !expert_count || !expert_offset || !out_rows) return MOE_ERR_BAD_ARGUMENT;
+    if (act != MOE_ACT_RELU && act != MOE_ACT_GELU && act != MOE_ACT_NONE) return MOE_ERR_BAD_ARGUMENT;
+    const int rc = check_backward_call(h, N, K, scratch, scratch_bytes);
+    if (rc) return rc;
+    const hipError_t e = launch_expert_gemm(a_rows, w, bias, expert_count, expert_offset, h->d.A, h->d.E, N, K, act,
+                                            h->d.act_dtype == MOE_DTYPE_FP16, out_rows, scratch, (hipStream_t)stream);
+    return e == hipSuccess ? MOE_OK : hip_fail(h, e);
+}
+
+int moe_expert_wgrad(moe_handle* h, const void* dy_rows, const void* a_rows, const int32_t* expert_count,
+                     const int32_t* expert_offset, int32_t N, int32_t K, void* dw, void* scratch, size_t scratch_bytes,
+                     void* stream) {
+    if (!h || !dy_rows || !a_rows || !expert_count || !expert_offset || !dw) return MOE_ERR_BAD_ARGUMENT;
+    const int rc = check_backward_call(h, N, K, scratch, scratch_bytes);
+    if (rc) return rc;
+    const hipError_t e = launch_expert_wgrad(dy_rows, a_rows, expert_count, expert_offset, h->d.A, h->d.E, N, K,
+                                             h->d.act_dtype == MOE_DTYPE_FP16, dw, scratch, (hipStream_t)stream);
+    return e == hipSuccess ? MOE_OK : hip_fail(h, e);
+}
+
 int moe_combine(const void* y_rows, const int32_t* pair_row, const float* topk_w, int32_t S, int32_t k, int32_t H,
                 int32_t act_dtype, void* out, void* stream) {
     if (!y_rows || !pair_row || !topk_w || !out || S < 0 || k < 1 || H < 1) return MOE_ERR_BAD_ARGUMENT;

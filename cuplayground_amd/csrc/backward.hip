@@ -1,0 +1,178 @@
+// Building blocks of the backward pass of the expert FFN (the training knob is_training,
+// aristos_config.schema.json:20-23, is parsed by the reference and never read; these are this library's).
+//
+// Everything works on packed expert-major rows as the forward pass lays them out: rows
+// [expert_offset[e], expert_offset[e] + expert_count[e]) belong to expert e.
+//   * data gradients are grouped (M,K) x (N,K)^T GEMMs with the weight in its K-major view, which a batched transpose
+//     produces: dX = dY . W  ==  dY x (W^T)^T.  The forward tile kernels run them unchanged.
+//   * weight gradients sum over an expert's rows: dW[e] = dY_e^T . A_e.  Both operands are transposed into buffers whose
+//     columns are the packed rows, each expert's window padded with zeros to a multiple of 128 columns, and every
+//     expert is then one tile GEMM over its window.
+#include "moe_internal.hpp"
+
+namespace moe355 {
+
+bool grouped_gemm_takes_large_tile(int64_t A, int E, int N, int K);
+hipError_t launch_grouped_gemm_16(const void* a_rows, const void* w, const void* bias, void* out, const MTile* mtiles,
+                                  const int32_t* num_mtiles, int max_mtiles, int block_m, int64_t A, int N, int K, int act,
+                                  bool f16, hipStream_t st);
+hipError_t launch_wgrad_16(const void* dyT, const void* aT, void* dw, const int32_t* poff, int E, int N, int K,
+                           int64_t ld, bool f16, hipStream_t st);
+
+namespace {
+
+constexpr int kWindowAlign = 128;   // columns an expert's window of a transposed operand is padded to
+
+// One workgroup: row blocks of `block_m` rows per expert (for the grouped GEMM) and the padded window offsets (for the
+// weight gradient).  Either table may be null.
+__global__ __launch_bounds__(kMaxExperts) void backward_tables_kernel(const int32_t* __restrict__ count,
+                                                                      const int32_t* __restrict__ offset, int E,
+                                                                      int block_m, MTile* mtiles, int32_t* num_mtiles,
+                                                                      int32_t* poff) {
+    __shared__ int s_mt0[kMaxExperts + 1];
+    const int e = threadIdx.x;
+    if (e == 0) {
+        int mt = 0, po = 0;
+        for (int i = 0; i < E; ++i) {
+            const int n = max(count[i], 0);
+            s_mt0[i] = mt;
+            mt += (n + block_m - 1) / block_m;
+            if (poff) poff[i] = po;
+            po += (n + kWindowAlign - 1) / kWindowAlign * kWindowAlign;
+        }
+        s_mt0[E] = mt;
+        if (num_mtiles) *num_mtiles = mt;
+        if (poff) poff[E] = po;
+    }
+    __syncthreads();
+    if (e < E && mtiles) {
+        const int n = max(count[e], 0), off = offset[e];
+        for (int i = 0, mt = s_mt0[e]; mt < s_mt0[e + 1]; ++i, ++mt) {
+            MTile t;
+            t.expert = e;
+            t.row0 = off + i * block_m;
+            t.rows = min(block_m, n - i * block_m);
+            t.pad = 0;
+            mtiles[mt] = t;
+        }
+    }
+}
+
+// dst[b][c][r] = src[b][r][c] for 16-bit elements; 64 x 64 tiles through LDS.  grid = (ceil(C/64), ceil(R/64), B).
+__global__ __launch_bounds__(256) void transpose16_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst,
+                                                          int64_t R, int64_t C) {
+    __shared__ uint16_t tile[64][66];
+    const uint16_t* s = src + (size_t)blockIdx.z * R * C;
+    uint16_t* d = dst + (size_t)blockIdx.z * R * C;
+    const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
+    for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+        const int r = i >> 6, c = i & 63;
+        tile[r][c] = (r0 + r < R && c0 + c < C) ? s[(r0 + r) * C + c0 + c] : (uint16_t)0;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+        const int c = i >> 6, r = i & 63;
+        if (r0 + r < R && c0 + c < C) d[(c0 + c) * R + r0 + r] = tile[r][c];
+    }
+}
+__global__ __launch_bounds__(256) void transpose32_kernel(const uint32_t* __restrict__ src, uint32_t* __restrict__ dst,
+                                                          int64_t R, int64_t C) {
+    __shared__ uint32_t tile[64][65];
+    const uint32_t* s = src + (size_t)blockIdx.z * R * C;
+    uint32_t* d = dst + (size_t)blockIdx.z * R * C;
+    const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
+    for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+        const int r = i >> 6, c = i & 63;
+        tile[r][c] = (r0 + r < R && c0 + c < C) ? s[(r0 + r) * C + c0 + c] : 0u;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+        const int c = i >> 6, r = i & 63;
+        if (r0 + r < R && c0 + c < C) d[(c0 + c) * R + r0 + r] = tile[r][c];
+    }
+}
+
+// Packed rows [*, C] -> dst [C, ld]: column poff[e] + s holds row offset[e] + s of expert e (s < count[e]); the rest
+// of each window is zero.  A 64-column tile of dst never straddles two windows (they are multiples of 128 wide).
+// grid = (ld / 64, ceil(C / 64)).
+__global__ __launch_bounds__(256) void transpose_rows_padded_kernel(const uint16_t* __restrict__ rows, int C,
+                                                                    const int32_t* __restrict__ count,
+                                                                    const int32_t* __restrict__ offset,
+                                                                    const int32_t* __restrict__ poff, int E, int64_t ld,
+                                                                    uint16_t* __restrict__ dst) {
+    __shared__ uint16_t tile[64][66];
+    const int p0 = blockIdx.x * 64;
+    if (p0 >= poff[E]) return;                 // behind the last window: never read
+    int lo = 0, hi = E - 1;
+    while (lo < hi) {                          // last expert whose window starts at or before p0 (empty windows skipped)
+        const int mid = (lo + hi + 1) >> 1;
+        if (poff[mid] <= p0) lo = mid; else hi = mid - 1;
+    }
+    const int e = lo, s0 = p0 - poff[e], n = count[e], off = offset[e];
+    const int c0 = blockIdx.y * 64;
+    for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+        const int r = i >> 6, c = i & 63;
+        tile[r][c] = (s0 + r < n && c0 + c < C) ? rows[(size_t)(off + s0 + r) * C + c0 + c] : (uint16_t)0;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+        const int c = i >> 6, r = i & 63;
+        if (c0 + c < C) dst[(size_t)(c0 + c) * ld + p0 + r] = tile[r][c];
+    }
+}
+
+size_t align256(size_t v) { return (v + 255) / 256 * 256; }
+
+}  // namespace
+
+int64_t wgrad_ld(int64_t A, int E) { return (A + (int64_t)kWindowAlign * E + 127) / 128 * 128; }
+
+size_t backward_scratch_bytes(int64_t A, int E, int H, int I) {
+    const size_t tables = align256(sizeof(int32_t)) + align256((size_t)(A / 128 + E + 1) * sizeof(MTile)) + align256((size_t)(E + 1) * 4);
+    const size_t operands = align256((size_t)H * wgrad_ld(A, E) * 2) + align256((size_t)I * wgrad_ld(A, E) * 2);
+    return tables + operands;
+}
+
+hipError_t launch_transpose(const void* src, void* dst, int64_t batch, int64_t rows, int64_t cols, int elem_bytes,
+                            hipStream_t st) {
+    if (batch < 1 || rows < 1 || cols < 1) return hipSuccess;
+    const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64), (unsigned)batch);
+    if (elem_bytes == 2) transpose16_kernel<<<grid, 256, 0, st>>>((const uint16_t*)src, (uint16_t*)dst, rows, cols);
+    else transpose32_kernel<<<grid, 256, 0, st>>>((const uint32_t*)src, (uint32_t*)dst, rows, cols);
+    return hipGetLastError();
+}
+
+// out_rows[r,:] = act(a_rows[r,:] . w[e(r)]^T + bias[e(r)]); scratch holds the row-block table.
+hipError_t launch_expert_gemm(const void* a_rows, const void* w, const void* bias, const int32_t* count,
+                              const int32_t* offset, int64_t A, int E, int N, int K, int act, bool f16, void* out_rows,
+                              void* scratch, hipStream_t st) {
+    const int block_m = grouped_gemm_takes_large_tile(A, E, N, K) ? 256 : 128;
+    char* s = static_cast<char*>(scratch);
+    int32_t* num_mtiles = reinterpret_cast<int32_t*>(s);
+    MTile* mtiles = reinterpret_cast<MTile*>(s + align256(sizeof(int32_t)));
+    const int max_mtiles = (int)(A / block_m + E);
+    backward_tables_kernel<<<1, kMaxExperts, 0, st>>>(count, offset, E, block_m, mtiles, num_mtiles, nullptr);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    return launch_grouped_gemm_16(a_rows, w, bias, out_rows, mtiles, num_mtiles, max_mtiles, block_m, A, N, K, act, f16, st);
+}
+
+// dw[e] [N,K] = dy_e^T . a_e; scratch holds the window offsets and the two transposed operands.
+hipError_t launch_expert_wgrad(const void* dy_rows, const void* a_rows, const int32_t* count, const int32_t* offset,
+                               int64_t A, int E, int N, int K, bool f16, void* dw, void* scratch, hipStream_t st) {
+    char* s = static_cast<char*>(scratch);
+    const size_t tables = align256(sizeof(int32_t)) + align256((size_t)(A / 128 + E + 1) * sizeof(MTile));
+    int32_t* poff = reinterpret_cast<int32_t*>(s + tables);
+    const int64_t ld = wgrad_ld(A, E);
+    uint16_t* dyT = reinterpret_cast<uint16_t*>(s + tables + align256((size_t)(E + 1) * 4));
+    uint16_t* aT = reinterpret_cast<uint16_t*>(reinterpret_cast<char*>(dyT) + align256((size_t)N * ld * 2));
+    backward_tables_kernel<<<1, kMaxExperts, 0, st>>>(count, offset, E, 128, nullptr, nullptr, poff);
+    const dim3 g1((unsigned)(ld / 64), (unsigned)((N + 63) / 64)), g2((unsigned)(ld / 64), (unsigned)((K + 63) / 64));
+    transpose_rows_padded_kernel<<<g1, 256, 0, st>>>((const uint16_t*)dy_rows, N, count, offset, poff, E, ld, dyT);
+    transpose_rows_padded_kernel<<<g2, 256, 0, st>>>((const uint16_t*)a_rows, K, count, offset, poff, E, ld, aT);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    return launch_wgrad_16(dyT, aT, dw, poff, E, N, K, ld, f16, st);
+}
+
+}  // namespace moe355

@@ -67,6 +67,7 @@ struct TaskPtrs {
     int a_ld;                    // K
     const uint16_t* b0;          // weight matrix of this expert (w_up or w_down)
     const uint16_t* b1;          // SwiGLU: w_gate of this expert, else null
+    int b_ld;                    // elements between weight rows (K unless the operand is a window of a wider matrix)
     const uint16_t* bias0;
     const uint16_t* bias1;
     uint16_t* c_base;            // h or y, first row of the block
@@ -173,7 +174,7 @@ __device__ __forceinline__ void mainloop_generic(const TaskPtrs& p, unsigned cha
             col = p.n0 + j;
         }
         if (col >= p.N) col = p.N - 1;                            // ragged last tile; never stored
-        b_src[i] = base + (int64_t)col * p.K + chunk * 8;
+        b_src[i] = base + (int64_t)col * p.b_ld + chunk * 8;
     }
 
 #pragma unroll
@@ -501,7 +502,7 @@ __device__ __forceinline__ RingLoads ring_prepare_weights(const TaskPtrs& p) {
         L.voff_a[n] = p.a_extent;
         const int j = prow + n * T::ROWS_PER_PASS;
         const int col = p.swiglu ? p.n0 + (j >> 7) * 64 + (j & 63) : p.n0 + j;
-        L.voff_b[n] = (unsigned)(((int64_t)col * p.K + chunk * 8) * 2);
+        L.voff_b[n] = (unsigned)(((int64_t)col * p.b_ld + chunk * 8) * 2);
     }
     auto uniform = [](const void* q) {          // the bases are the same in every lane; say so, or each load loops over lanes
         const uint64_t v = (uint64_t)q;
@@ -785,6 +786,7 @@ __device__ __forceinline__ TaskPtrs resolve(const FfnArgs& a, const Task& t, boo
         p.c_base = (uint16_t*)a.h + (int64_t)t.row0 * a.I;
         p.N = a.I;
         p.K = a.H;
+        p.b_ld = a.H;
         p.n0 = t.ntile * (sw ? T::BN / 2 : T::BN);
         p.act = a.act;
         p.swiglu = sw;
@@ -801,6 +803,7 @@ __device__ __forceinline__ TaskPtrs resolve(const FfnArgs& a, const Task& t, boo
         p.c_base = (uint16_t*)a.y + (int64_t)t.row0 * a.H;
         p.N = a.H;
         p.K = a.I;
+        p.b_ld = a.I;
         p.n0 = t.ntile * T::BN;
         p.act = MOE_ACT_NONE;
         p.swiglu = false;
@@ -1015,6 +1018,7 @@ __global__ __launch_bounds__(T::THREADS) void gemm_dense_kernel(const uint16_t* 
     p.c_base = C + (int64_t)row0 * N;
     p.N = N;
     p.K = K;
+    p.b_ld = K;
     p.rows = min(T::BM, M - row0);
     p.n0 = blockIdx.y * T::BN;
     p.act = act;
@@ -1022,6 +1026,86 @@ __global__ __launch_bounds__(T::THREADS) void gemm_dense_kernel(const uint16_t* 
     p.publish = false;
     p.a_extent = (uint32_t)((int64_t)M * K * 2);
     p.b_extent = (uint32_t)((int64_t)N * K * 2);
+    gemm_tile<T>(p, smem);
+}
+
+// Grouped GEMM on packed expert-major rows, outside the layer: out[r,:] = act(a[r,:] . w[e(r)]^T + bias[e(r)]) for
+// the rows of every row block of the table -- the reference's tile GEMM (mma.cuh:46-179) once per expert, with the
+// expert taken from the row block.  With the weight handed over in its K-major view this is the data gradient of a
+// projection (dX = dY . W).  grid = (row blocks upper bound, column tiles).
+template <class T>
+__global__ __launch_bounds__(T::THREADS) void grouped_gemm_kernel(const uint16_t* a_rows, const uint16_t* w,
+                                                                  const uint16_t* bias, uint16_t* out,
+                                                                  const MTile* mtiles, const int32_t* num_mtiles, int N,
+                                                                  int K, int act, uint32_t a_bytes) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int mt = blockIdx.x;
+    if (mt >= *num_mtiles) return;
+    const MTile m = mtiles[mt];
+    TaskPtrs p;
+    p.a_base = a_rows;
+    p.gather = nullptr;
+    p.a_row0 = m.row0;
+    p.a_ld = K;
+    p.b0 = w + (int64_t)m.expert * N * K;
+    p.b1 = nullptr;
+    p.b_ld = K;
+    p.bias0 = bias ? bias + (int64_t)m.expert * N : nullptr;
+    p.bias1 = nullptr;
+    p.c_base = out + (int64_t)m.row0 * N;
+    p.N = N;
+    p.K = K;
+    p.rows = m.rows;
+    p.n0 = blockIdx.y * T::BN;
+    p.act = act;
+    p.swiglu = false;
+    p.publish = false;
+    p.a_extent = a_bytes;
+    p.b_extent = (uint32_t)((int64_t)N * K * 2);
+    gemm_tile<T>(p, smem);
+}
+
+// Weight gradient of one projection: dw[e] [N, K] = dy_e^T . a_e, the sum running over the rows of expert e.  Both
+// operands arrive transposed and padded: dyT [N, ld] and aT [K, ld] hold expert e's rows in columns
+// [poff[e], poff[e+1]) (zeros behind the last real row; every window is a multiple of 128 wide), so each expert is one
+// (M,K) x (N,K)^T tile GEMM over its window.  grid = (row tiles of N, column tiles of K, experts).
+template <class T>
+__global__ __launch_bounds__(T::THREADS) void wgrad_kernel(const uint16_t* dyT, const uint16_t* aT, uint16_t* dw,
+                                                           const int32_t* poff, int N, int K, int ld, uint32_t dy_bytes,
+                                                           uint32_t a_bytes) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int e = blockIdx.z;
+    const int row0 = blockIdx.x * T::BM, n0 = blockIdx.y * T::BN;
+    const int p0 = poff[e], window = poff[e + 1] - p0;
+    uint16_t* c = dw + (int64_t)e * N * K + (int64_t)row0 * K;
+    const int rows = min(T::BM, N - row0);
+    if (window == 0) {   // an expert that received no rows: its gradient is zero
+        for (int i = threadIdx.x; i < rows * T::BN; i += T::THREADS) {
+            const int r = i / T::BN, col = n0 + i % T::BN;
+            if (col < K) c[(int64_t)r * K + col] = 0;
+        }
+        return;
+    }
+    TaskPtrs p;
+    p.a_base = dyT + p0;
+    p.gather = nullptr;
+    p.a_row0 = row0;
+    p.a_ld = ld;
+    p.b0 = aT + p0;
+    p.b1 = nullptr;
+    p.b_ld = ld;
+    p.bias0 = nullptr;
+    p.bias1 = nullptr;
+    p.c_base = c;
+    p.N = K;
+    p.K = window;
+    p.rows = rows;
+    p.n0 = n0;
+    p.act = MOE_ACT_NONE;
+    p.swiglu = false;
+    p.publish = false;
+    p.a_extent = dy_bytes - (uint32_t)p0 * 2;
+    p.b_extent = a_bytes - (uint32_t)p0 * 2;
     gemm_tile<T>(p, smem);
 }
 
@@ -1136,6 +1220,57 @@ hipError_t launch_gemm_dense_bf16(const void* A, const void* B, const void* bias
                      : launch_dense<SmallPlanH::T0>(A, B, bias, C, M, N, K, act, st);
     return large ? launch_dense<LargePlan::T0>(A, B, bias, C, M, N, K, act, st)
                  : launch_dense<SmallPlan::T0>(A, B, bias, C, M, N, K, act, st);
+}
+
+// ---- building blocks of the backward pass (callers: csrc/backward.hip) ----
+bool grouped_gemm_takes_large_tile(int64_t A, int E, int N, int K) {
+    const int64_t lim = (int64_t)1 << 32;
+    return N % 256 == 0 && K % 128 == 0 && A * K * 2 < lim && (int64_t)N * K * 2 < lim && A / (E > 0 ? E : 1) >= 256;
+}
+
+template <class T>
+static hipError_t launch_grouped(const void* a_rows, const void* w, const void* bias, void* out, const MTile* mtiles,
+                                 const int32_t* num_mtiles, int max_mtiles, int64_t A, int N, int K, int act,
+                                 hipStream_t st) {
+    hipError_t e = allow_lds(&grouped_gemm_kernel<T>, T::LDS_BYTES);
+    if (e != hipSuccess) return e;
+    const dim3 grid((unsigned)max_mtiles, (unsigned)((N + T::BN - 1) / T::BN));
+    grouped_gemm_kernel<T><<<grid, T::THREADS, T::LDS_BYTES, st>>>((const uint16_t*)a_rows, (const uint16_t*)w,
+                                                                   (const uint16_t*)bias, (uint16_t*)out, mtiles,
+                                                                   num_mtiles, N, K, act, (uint32_t)(A * K * 2));
+    return hipGetLastError();
+}
+
+hipError_t launch_grouped_gemm_16(const void* a_rows, const void* w, const void* bias, void* out, const MTile* mtiles,
+                                  const int32_t* num_mtiles, int max_mtiles, int block_m, int64_t A, int N, int K, int act,
+                                  bool f16, hipStream_t st) {
+    if (block_m == 256)
+        return f16 ? launch_grouped<LargePlanH::T0>(a_rows, w, bias, out, mtiles, num_mtiles, max_mtiles, A, N, K, act, st)
+                   : launch_grouped<LargePlan::T0>(a_rows, w, bias, out, mtiles, num_mtiles, max_mtiles, A, N, K, act, st);
+    return f16 ? launch_grouped<SmallPlanH::T0>(a_rows, w, bias, out, mtiles, num_mtiles, max_mtiles, A, N, K, act, st)
+               : launch_grouped<SmallPlan::T0>(a_rows, w, bias, out, mtiles, num_mtiles, max_mtiles, A, N, K, act, st);
+}
+
+template <class T>
+static hipError_t launch_wgrad(const void* dyT, const void* aT, void* dw, const int32_t* poff, int E, int N, int K,
+                               int64_t ld, hipStream_t st) {
+    hipError_t e = allow_lds(&wgrad_kernel<T>, T::LDS_BYTES);
+    if (e != hipSuccess) return e;
+    const dim3 grid((unsigned)((N + T::BM - 1) / T::BM), (unsigned)((K + T::BN - 1) / T::BN), (unsigned)E);
+    wgrad_kernel<T><<<grid, T::THREADS, T::LDS_BYTES, st>>>((const uint16_t*)dyT, (const uint16_t*)aT, (uint16_t*)dw, poff,
+                                                            N, K, (int)ld, (uint32_t)((int64_t)N * ld * 2),
+                                                            (uint32_t)((int64_t)K * ld * 2));
+    return hipGetLastError();
+}
+
+hipError_t launch_wgrad_16(const void* dyT, const void* aT, void* dw, const int32_t* poff, int E, int N, int K,
+                           int64_t ld, bool f16, hipStream_t st) {
+    const int64_t lim = (int64_t)1 << 32;
+    const bool large = N >= 1024 && K >= 1024 && K % 256 == 0 && N * ld * 2 < lim && K * ld * 2 < lim;
+    if (large) return f16 ? launch_wgrad<LargePlanH::T0>(dyT, aT, dw, poff, E, N, K, ld, st)
+                          : launch_wgrad<LargePlan::T0>(dyT, aT, dw, poff, E, N, K, ld, st);
+    return f16 ? launch_wgrad<SmallPlanH::T0>(dyT, aT, dw, poff, E, N, K, ld, st)
+               : launch_wgrad<SmallPlan::T0>(dyT, aT, dw, poff, E, N, K, ld, st);
 }
 
 }  // namespace moe355

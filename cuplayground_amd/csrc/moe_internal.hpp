@@ -140,6 +140,16 @@ hipError_t launch_ffn_tiled(const FfnArgs& a, int dtype, const FfnPlan& p, int m
 hipError_t launch_ffn_persistent(const FfnArgs& a, int dtype, const FfnPlan& p, int blocks, hipStream_t st);
 int ffn_persistent_blocks(int dtype, int block_m, int compute_units);
 
+// ---- backward building blocks (csrc/backward.hip) ----
+size_t backward_scratch_bytes(int64_t A, int E, int H, int I);
+hipError_t launch_transpose(const void* src, void* dst, int64_t batch, int64_t rows, int64_t cols, int elem_bytes,
+                            hipStream_t st);
+hipError_t launch_expert_gemm(const void* a_rows, const void* w, const void* bias, const int32_t* count,
+                              const int32_t* offset, int64_t A, int E, int N, int K, int act, bool f16, void* out_rows,
+                              void* scratch, hipStream_t st);
+hipError_t launch_expert_wgrad(const void* dy_rows, const void* a_rows, const int32_t* count, const int32_t* offset,
+                               int64_t A, int E, int N, int K, bool f16, void* dw, void* scratch, hipStream_t st);
+
 hipError_t launch_gemm_bias_act(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N,
                                 int64_t K, int dtype, int act, hipStream_t st);
 

@@ -233,6 +233,31 @@ int moe_measure_hbm_read_gbs(const void* src, size_t bytes, void* scratch, void*
 int moe_quant_block128(const void* w, int32_t src_dtype, int64_t matrices, int64_t N, int64_t K, void* q,
                        float* scales, void* stream);
 
+/* ---- Backward building blocks (bf16 and fp16 layers) -------------------------------------------------------------
+ * The reference declares a training knob (is_training, aristos_config.schema.json:20-23) that none of its code reads
+ * and has no backward pass; these entry points are what a training step needs beyond the forward stages above.  All
+ * of them work on packed expert-major rows as moe_route lays them out: rows [expert_offset[e], expert_offset[e] +
+ * expert_count[e]) of a [S*k, *] buffer belong to expert e (expert_count / expert_offset as moe_route wrote them, on
+ * the device).  (N, K) must be (H, I) or (I, H) of the handle's layer.  `scratch` is 256-byte aligned device memory of
+ * at least moe_backward_scratch_bytes(); each call overwrites it.  Asynchronous on `stream`; fp32 accumulation.
+ *
+ * moe_transpose: dst[b][c][r] = src[b][r][c], elem_bytes 2 or 4.  Turns a weight [E,N,K] into its K-major view
+ *   [E,K,N], which makes a data gradient an ordinary forward-shaped product:
+ *     dX_rows = dY_rows . W        ==  moe_expert_gemm(dY_rows, transpose(W), no bias, MOE_ACT_NONE)
+ * moe_expert_gemm: out_rows[r,:] = act(a_rows[r,:K] . w[e(r)]^T + bias[e(r)]) for every kept row r, w [E,N,K], bias
+ *   [E,N] or null, act RELU / GELU / NONE; the grouped product of the forward FFN as a stage of its own.
+ * moe_expert_wgrad: dw[e] [N,K] = sum over the rows r of expert e of dy_rows[r,:N]^T a_rows[r,:K]; an expert with no
+ *   rows gets zeros.  dw is written in the layer's 16-bit type. */
+int moe_backward_scratch_bytes(const moe_config* cfg, size_t* bytes);
+int moe_transpose(const void* src, void* dst, int64_t batch, int64_t rows, int64_t cols, int32_t elem_bytes,
+                  void* stream);
+int moe_expert_gemm(moe_handle* h, const void* a_rows, const void* w, const void* bias, const int32_t* expert_count,
+                    const int32_t* expert_offset, int32_t N, int32_t K, int32_t act, void* out_rows, void* scratch,
+                    size_t scratch_bytes, void* stream);
+int moe_expert_wgrad(moe_handle* h, const void* dy_rows, const void* a_rows, const int32_t* expert_count,
+                     const int32_t* expert_offset, int32_t N, int32_t K, void* dw, void* scratch, size_t scratch_bytes,
+                     void* stream);
+
 int moe_last_hip_error(const moe_handle* h);
 const char* moe_status_string(int status);
 int moe_version(void);

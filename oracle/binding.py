@@ -74,6 +74,8 @@ def lib():
         L.orc_router_stats.argtypes = [vp, vp, i32, i32, i32, i32, vp, vp, vp]
         L.orc_route.argtypes = [vp, i32, i32, i32, i32, i64, vp, vp, vp, vp, vp]
         L.orc_gemm_bias_act.argtypes = [vp, vp, vp, vp, i64, i64, i64, i32, i32]
+        L.orc_expert_gemm.argtypes = [vp, vp, vp, vp, vp, i32, i64, i64, i32, i32, vp]
+        L.orc_expert_wgrad.argtypes = [vp, vp, vp, vp, i32, i64, i64, i32, vp]
         L.orc_ffn_rows.argtypes = [C.POINTER(_Cfg), vp, C.POINTER(_Weights), vp, vp, i64, vp]
         L.orc_combine.argtypes = [vp, vp, vp, i32, i32, i32, i32, vp]
         L.orc_forward.argtypes = [C.POINTER(_Cfg), vp, C.POINTER(_Weights), vp, vp, vp, vp, vp, vp, vp]
@@ -82,7 +84,7 @@ def lib():
         for fn in ("orc_philox4x32_10", "orc_fill_normal", "orc_fill_uniform", "orc_round_bf16", "orc_widen_bf16",
                    "orc_round_f16", "orc_widen_f16",
                    "orc_quant_block128", "orc_dequant_block128", "orc_gate_logits", "orc_topk", "orc_route",
-                   "orc_gemm_bias_act", "orc_ffn_rows", "orc_combine", "orc_forward", "orc_forward_tokens"):
+                   "orc_gemm_bias_act", "orc_expert_gemm", "orc_expert_wgrad", "orc_ffn_rows", "orc_combine", "orc_forward", "orc_forward_tokens"):
             getattr(L, fn).restype = None
         _lib = L
     return _lib
@@ -324,6 +326,27 @@ def gemm_bias_act(A, B, bias, dtype, act):
     lib().orc_gemm_bias_act(_p(np.ascontiguousarray(A)), _p(np.ascontiguousarray(B)),
                             _p(None if bias is None else np.ascontiguousarray(bias)), _p(out), M, N, K, dtype, act)
     return out
+
+
+def expert_gemm(a_rows, w, bias, count, offset, dtype, act):
+    """out[r] = act(a_rows[r] . w[e(r)]^T + bias[e(r)]) on packed expert-major rows; untouched rows are zero."""
+    E, N, K = w.shape
+    count = _c(count, np.int32); offset = _c(offset, np.int32)
+    out = np.zeros((a_rows.shape[0], N), np.float32 if dtype in (F32, TF32) else np.uint16)
+    lib().orc_expert_gemm(_p(np.ascontiguousarray(a_rows)), _p(np.ascontiguousarray(w)),
+                          _p(None if bias is None else np.ascontiguousarray(bias)), _p(count), _p(offset), E, N, K,
+                          dtype, act, _p(out))
+    return out
+
+
+def expert_wgrad(dy_rows, a_rows, count, offset, dtype):
+    """dw[e] = sum over expert e's rows of dy_rows[r]^T a_rows[r] -> [E, N, K]."""
+    count = _c(count, np.int32); offset = _c(offset, np.int32)
+    N, K = dy_rows.shape[1], a_rows.shape[1]
+    dw = np.empty((count.size, N, K), np.float32 if dtype in (F32, TF32) else np.uint16)
+    lib().orc_expert_wgrad(_p(np.ascontiguousarray(dy_rows)), _p(np.ascontiguousarray(a_rows)), _p(count), _p(offset),
+                           count.size, N, K, dtype, _p(dw))
+    return dw
 
 
 def ffn_rows(cfg: Cfg, inp, tokens, experts):

@@ -514,6 +514,43 @@ void orc_gemm_bias_act(const void* A, const void* B, const void* bias, void* C,
     }
 }
 
+/* ------------------------------------------------------------------------------------------------
+ * Grouped products over packed expert-major rows (rows [offset[e], offset[e] + count[e]) belong to expert
+ * e), the building blocks of a backward pass.  Build-defined: the reference parses a training flag
+ * (aristos_config.schema.json:20-23) and holds no backward code.  Both keep the forward GEMM's contract:
+ * fp32 accumulation, one rounding to the storage type on store.
+ *   orc_expert_gemm:  out[r,:] = act(a[r,:K] . w[e]^T + bias[e]),   w [E,N,K], bias [E,N] or NULL
+ *   orc_expert_wgrad: dw[e] [N,K] = sum over r of expert e, ascending, of dy[r,:N]^T a[r,:K]
+ * Rows outside every expert's range are left untouched.
+ * ---------------------------------------------------------------------------------------------- */
+void orc_expert_gemm(const void* a_rows, const void* w, const void* bias, const int32_t* count, const int32_t* offset,
+                     int32_t E, int64_t N, int64_t K, int32_t dtype, int32_t act, void* out_rows) {
+    const size_t el = (dtype == ORC_F32 || dtype == ORC_TF32) ? 4 : 2;
+    for (int32_t e = 0; e < E; ++e) {
+        if (count[e] <= 0) continue;
+        orc_gemm_bias_act((const char*)a_rows + (size_t)offset[e] * K * el, (const char*)w + (size_t)e * N * K * el,
+                          bias ? (const char*)bias + (size_t)e * N * el : NULL,
+                          (char*)out_rows + (size_t)offset[e] * N * el, count[e], N, K, dtype, act);
+    }
+}
+
+void orc_expert_wgrad(const void* dy_rows, const void* a_rows, const int32_t* count, const int32_t* offset, int32_t E,
+                      int64_t N, int64_t K, int32_t dtype, void* dw) {
+    const int adt = act_dtype_of(dtype);
+    for (int32_t e = 0; e < E; ++e) {
+        const int64_t r0 = offset[e], r1 = r0 + (count[e] > 0 ? count[e] : 0);
+#pragma omp parallel for schedule(static)
+        for (int64_t n = 0; n < N; ++n) {
+            for (int64_t k = 0; k < K; ++k) {
+                float acc = 0.0f;
+                for (int64_t r = r0; r < r1; ++r)
+                    acc = fmaf(load_act(dy_rows, r * N + n, adt), load_act(a_rows, r * K + k, adt), acc);
+                store_act(dw, ((int64_t)e * N + n) * K + k, adt, acc);
+            }
+        }
+    }
+}
+
 /* One expert FFN row: the two chained GEMMs of the reference's task graph (scheduling.cuh:212-222), the
  * intermediate rounded to the storage type between them (mma.cuh:108-109).  GELU is the exact erf form,
  * SwiGLU is silu(x.Wg^T + bg) * (x.Wu^T + bu); both are this build's extensions of hidden_act.

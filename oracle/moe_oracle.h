@@ -19,6 +19,9 @@
  *   - orc_combine              pinned by the reference driver's identity case (combine.cuh:220-231),
  *                              permutation and linearity properties
  *   - orc_forward*             pinned by the dense-mixture equivalence in float64
+ *   - orc_expert_gemm / orc_expert_wgrad  pinned by float64 einsums per expert, by one-hot rows that select
+ *                              single weight columns / operand rows, and by the adjoint identity
+ *                              <dY, X.W^T> = <dY^T.X, W> = <dY.W, X> (tests/test_oracle_backward.py)
  * Reference parity of gate / top-k / capacity / SwiGLU / fp8 scaling is unpinned by construction: the
  * reference holds no code for them.
  */
@@ -94,6 +97,10 @@ void orc_route(const int32_t* topk_idx, int32_t S, int32_t k, int32_t E, int32_t
                int32_t* pair_row);
 void orc_gemm_bias_act(const void* A, const void* B, const void* bias, void* C,
                        int64_t M, int64_t N, int64_t K, int32_t dtype, int32_t act);
+void orc_expert_gemm(const void* a_rows, const void* w, const void* bias, const int32_t* count, const int32_t* offset,
+                     int32_t E, int64_t N, int64_t K, int32_t dtype, int32_t act, void* out_rows);
+void orc_expert_wgrad(const void* dy_rows, const void* a_rows, const int32_t* count, const int32_t* offset, int32_t E,
+                      int64_t N, int64_t K, int32_t dtype, void* dw);
 void orc_ffn_rows(const orc_cfg* cfg, const void* x, const orc_weights* w, const int32_t* tokens,
                   const int32_t* experts, int64_t n_rows, void* y_rows);
 void orc_combine(const void* y_rows, const int32_t* pair_row, const float* topk_w,

@@ -1,0 +1,144 @@
+"""GPU parity of the backward building blocks (batched transpose, grouped product over packed expert rows, per-expert
+weight gradient), called through the C ABI, against the CPU oracle."""
+import numpy as np
+import pytest
+
+from oracle import binding as ob
+from helpers import OUT_TOL, from_device, max_rel_err, product_config, to_device
+
+pytestmark = pytest.mark.gpu
+KIND = {ob.BF16: "bf16", ob.F16: "f16"}
+
+
+@pytest.fixture(scope="module")
+def moe():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    import cuplayground_amd
+    cuplayground_amd.load_library()
+    return cuplayground_amd
+
+
+def routed_case(S, H, I, E, k, dtype, seed, drop=1, cf=1.0, skew=0.0):
+    """A layer shape with a real routing result from the oracle: counts and offsets as moe_route writes them."""
+    cfg = ob.Cfg(S=S, H=H, I=I, E=E, k=k, dtype=dtype, act=ob.ACT_GELU, drop=drop, capacity_factor=cf, norm_topk=1)
+    rng = np.random.default_rng(seed)
+    logits = rng.standard_normal((S, E)).astype(np.float32) + skew * np.arange(E, dtype=np.float32)
+    idx, _ = ob.topk(logits, k, cfg.gate_fn, cfg.norm_topk)
+    r = ob.route_slots(idx, E, cfg.drop, cfg.capacity)
+    return cfg, rng, r["expert_count"], r["expert_offset"]
+
+
+def operands(rng, R, E, N, K, dtype):
+    a = ob.from_f32(rng.standard_normal((R, K)).astype(np.float32), dtype)
+    dy = ob.from_f32(rng.standard_normal((R, N)).astype(np.float32), dtype)
+    w = ob.from_f32((rng.standard_normal((E, N, K)) * 0.1).astype(np.float32), dtype)
+    bias = ob.from_f32(rng.standard_normal((E, N)).astype(np.float32), dtype)
+    return a, dy, w, bias
+
+
+@pytest.mark.parametrize("shape", [(1, 5, 7), (3, 64, 64), (2, 130, 257), (4, 1000, 72)])
+@pytest.mark.parametrize("elem", [2, 4])
+def test_transpose_is_exact(moe, shape, elem):
+    rng = np.random.default_rng(sum(shape))
+    a = rng.integers(0, 2 ** (8 * elem) - 1, shape, dtype=np.uint64).astype(np.uint16 if elem == 2 else np.uint32)
+    t = moe.api.transpose(to_device(a.view(np.int16 if elem == 2 else np.int32), "i32"))
+    assert np.array_equal(from_device(t).view(a.dtype), a.transpose(0, 2, 1))
+
+
+CASES = [  # S, H, I, E, k, capacity factor, router skew
+    (256, 256, 512, 8, 2, 1.0, 0.0),
+    (512, 128, 320, 4, 1, 2.0, 0.7),        # skewed: one expert takes most rows, one may stay empty
+    (2048, 512, 1024, 4, 2, 1.25, 0.0),     # 256-row blocks in the grouped product
+    (1024, 1024, 1024, 2, 2, 2.0, 0.0),     # 256 x 256 tiles in the weight gradient as well
+]
+
+
+@pytest.mark.parametrize("dtype", [ob.BF16, ob.F16])
+@pytest.mark.parametrize("case", CASES)
+def test_expert_gemm_vs_oracle(moe, case, dtype):
+    S, H, I, E, k, cf, skew = case
+    cfg, rng, count, offset = routed_case(S, H, I, E, k, dtype, seed=S + E, cf=cf, skew=skew)
+    layer = moe.MoELayer(product_config(cfg))
+    kind = KIND[dtype]
+    dcount, doffset = to_device(count, "i32"), to_device(offset, "i32")
+    for (N, K, act, with_bias) in ((I, H, ob.ACT_GELU, True), (H, I, ob.ACT_NONE, False), (H, I, ob.ACT_RELU, True)):
+        a, _, w, bias = operands(rng, S * k, E, N, K, dtype)
+        want = ob.to_f32(ob.expert_gemm(a, w, bias if with_bias else None, count, offset, dtype, act), dtype)
+        got = layer.expert_gemm(to_device(a, kind), to_device(w, kind), to_device(bias, kind) if with_bias else None,
+                                dcount, doffset, act)
+        got = ob.to_f32(from_device(got), dtype)
+        kept = int(count.sum())
+        assert max_rel_err(got[:kept], want[:kept]) <= OUT_TOL[dtype]
+        assert not got[kept:].any()            # rows of no expert are not written (the output started as zeros)
+
+
+@pytest.mark.parametrize("dtype", [ob.BF16, ob.F16])
+@pytest.mark.parametrize("case", CASES)
+def test_data_gradient_is_the_grouped_product_with_the_transposed_weight(moe, case, dtype):
+    """dX = dY . W: the oracle works on numpy's transpose, the product on moe_transpose's."""
+    S, H, I, E, k, cf, skew = case
+    cfg, rng, count, offset = routed_case(S, H, I, E, k, dtype, seed=3 * S + E, cf=cf, skew=skew)
+    layer = moe.MoELayer(product_config(cfg))
+    kind = KIND[dtype]
+    _, dy, w, _ = operands(rng, S * k, E, H, I, dtype)           # down projection: y [*, H] = h [*, I] . w[e]^T, w [E, H, I]
+    wT = np.ascontiguousarray(w.transpose(0, 2, 1))              # [E, I, H]
+    want = ob.to_f32(ob.expert_gemm(dy, wT, None, count, offset, dtype, ob.ACT_NONE), dtype)
+    dwT = moe.api.transpose(to_device(w, kind))
+    assert np.array_equal(from_device(dwT), wT)
+    got = layer.expert_gemm(to_device(dy, kind), dwT, None, to_device(count, "i32"), to_device(offset, "i32"))
+    kept = int(count.sum())
+    assert max_rel_err(ob.to_f32(from_device(got), dtype)[:kept], want[:kept]) <= OUT_TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [ob.BF16, ob.F16])
+@pytest.mark.parametrize("case", CASES)
+def test_weight_gradient_vs_oracle(moe, case, dtype):
+    S, H, I, E, k, cf, skew = case
+    cfg, rng, count, offset = routed_case(S, H, I, E, k, dtype, seed=5 * S + E, cf=cf, skew=skew)
+    layer = moe.MoELayer(product_config(cfg))
+    kind = KIND[dtype]
+    dcount, doffset = to_device(count, "i32"), to_device(offset, "i32")
+    for (N, K) in ((H, I), (I, H)):
+        a, dy, _, _ = operands(rng, S * k, E, N, K, dtype)
+        want = ob.to_f32(ob.expert_wgrad(dy, a, count, offset, dtype), dtype)
+        got = ob.to_f32(from_device(layer.expert_wgrad(to_device(dy, kind), to_device(a, kind), dcount, doffset)), dtype)
+        for e in range(E):
+            if count[e] == 0:
+                assert not got[e].any()
+            else:
+                assert max_rel_err(got[e], want[e]) <= OUT_TOL[dtype], (e, int(count[e]))
+
+
+def test_empty_experts_and_second_call_reuse_scratch(moe):
+    """All rows on one expert, then a different split through the same layer: stale scratch must not leak."""
+    dtype, kind = ob.BF16, "bf16"
+    S, H, I, E = 256, 128, 256, 4
+    cfg = ob.Cfg(S=S, H=H, I=I, E=E, k=1, dtype=dtype, act=ob.ACT_RELU, drop=0)
+    layer = moe.MoELayer(product_config(cfg))
+    rng = np.random.default_rng(9)
+    a, dy, _, _ = operands(rng, S, E, H, I, dtype)
+    for count in ([0, S, 0, 0], [100, 0, 29, 127], [0, 0, 0, 0]):
+        count = np.asarray(count, np.int32)
+        offset = np.concatenate([[0], np.cumsum(count)[:-1]]).astype(np.int32)
+        want = ob.to_f32(ob.expert_wgrad(dy, a, count, offset, dtype), dtype)
+        got = ob.to_f32(from_device(layer.expert_wgrad(to_device(dy, kind), to_device(a, kind),
+                                                       to_device(count, "i32"), to_device(offset, "i32"))), dtype)
+        assert np.abs(got - want).max() <= OUT_TOL[dtype] * max(np.abs(want).max(), 1.0)
+
+
+def test_unsupported_layers_and_bad_arguments_are_refused(moe):
+    import torch
+    cfg = ob.Cfg(S=128, H=128, I=256, E=4, k=1, dtype=ob.F32, act=ob.ACT_RELU, drop=0)
+    layer = moe.MoELayer(product_config(cfg))
+    with pytest.raises(moe.MoEError) as e:
+        layer.backward_scratch()
+    assert e.value.status == 2                    # fp32 layers have no backward kernels
+    cfg = ob.Cfg(S=128, H=128, I=256, E=4, k=1, dtype=ob.BF16, act=ob.ACT_RELU, drop=0)
+    layer = moe.MoELayer(product_config(cfg))
+    z = torch.zeros(128, 192, dtype=torch.bfloat16, device="cuda")
+    w = torch.zeros(4, 256, 192, dtype=torch.bfloat16, device="cuda")
+    cnt = torch.zeros(4, dtype=torch.int32, device="cuda")
+    with pytest.raises(moe.MoEError) as e:        # (N, K) = (256, 192) is no projection of this layer
+        layer.expert_gemm(z, w, None, cnt, cnt)
+    assert e.value.status == 4

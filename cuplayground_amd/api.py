@@ -25,7 +25,7 @@ EXPORTS = (
     "moe_config_tokens", "moe_config_capacity", "moe_create", "moe_destroy", "moe_get_arch", "moe_get_plan",
     "moe_workspace_bytes",
     "moe_set_ffn_mode", "moe_get_ffn_mode", "moe_forward", "moe_forward_static", "moe_set_spin_limit", "moe_clear_stall", "moe_gate", "moe_router_stats", "moe_route", "moe_gemm_bias_act", "moe_combine",
-    "moe_set_stage_timing", "moe_get_stage_ms", "moe_get_stage_samples", "moe_get_task_counts", "moe_measure_mfma_tflops",
+    "moe_set_stage_timing", "moe_get_stage_ms", "moe_get_stage_samples", "moe_get_task_counts", "moe_get_queue_balance", "moe_measure_mfma_tflops",
     "moe_measure_hbm_read_gbs", "moe_quant_block128", "moe_backward_scratch_bytes", "moe_transpose", "moe_expert_gemm",
     "moe_expert_wgrad", "moe_last_hip_error", "moe_status_string",
     "moe_version",
@@ -103,6 +103,8 @@ def load_library():
     L.moe_get_stage_ms.argtypes = [vp, C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_int32)]
     L.moe_get_stage_samples.argtypes = [vp, C.c_int, C.POINTER(C.c_float), C.c_int32, C.POINTER(C.c_int32)]
     L.moe_get_task_counts.argtypes = [vp, vp, vp, C.POINTER(i64), C.POINTER(i64)]
+    L.moe_get_queue_balance.argtypes = [vp, vp, vp, C.POINTER(i32), C.POINTER(C.c_float), C.POINTER(C.c_float),
+                                        C.POINTER(C.c_float)]
     L.moe_quant_block128.argtypes = [vp, C.c_int32, C.c_int64, C.c_int64, C.c_int64, vp, vp, vp]
     L.moe_measure_mfma_tflops.argtypes = [vp, C.c_size_t, vp, C.c_int, C.POINTER(C.c_float)]
     L.moe_measure_hbm_read_gbs.argtypes = [vp, C.c_size_t, vp, vp, C.POINTER(C.c_float)]
@@ -288,6 +290,13 @@ class MoELayer:
         a, b = C.c_int64(0), C.c_int64(0)
         _check(self.L.moe_get_task_counts(self._h, _ptr(self.workspace), _stream(), C.byref(a), C.byref(b)))
         return a.value, b.value
+
+    def queue_balance(self) -> dict:
+        """Workgroup entry/exit statistics of the last forward's queue kernel (microseconds)."""
+        n, a, b, c = C.c_int32(0), C.c_float(0), C.c_float(0), C.c_float(0)
+        _check(self.L.moe_get_queue_balance(self._h, _ptr(self.workspace), _stream(), C.byref(n), C.byref(a),
+                                            C.byref(b), C.byref(c)), "moe_get_queue_balance")
+        return dict(workgroups=n.value, span_us=a.value, mean_active_us=b.value, mean_tail_idle_us=c.value)
 
     def _weights(self, weights: dict) -> _CWeights:
         w = _CWeights()

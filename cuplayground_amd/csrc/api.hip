@@ -1,25 +1,29 @@
 // Host side of libmoe355: handle, workspace carving, stage sequencing.  No device memory is allocated here;
 // the caller owns every buffer (the reference carves one stream-ordered arena per driver, mma.cuh:385-391,
 // combine.cuh:214-224 -- the same idea, made the caller's).
+#include <algorithm>
+#include <climits>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <new>
+#include <vector>
 
 #include "moe_internal.hpp"
 
 namespace moe355 {
 
 // per-dtype pieces defined next to their kernels
-int bf16_block_m(int64_t pairs, int experts, int H, int I, int swiglu);
-int bf16_block_n0(int block_m);
-int bf16_block_n1(int block_m);
+int bf16_tile(int64_t pairs, int experts, int H, int I, int swiglu);
+int bf16_block_m(int tile);
+int bf16_block_n0(int tile);
+int bf16_block_n1(int tile);
 int f32_block_m();
 int f32_block_n();
-hipError_t launch_ffn_tiled_bf16(const FfnArgs&, int block_m, int max_mtiles, int nnt0, int nnt1, hipStream_t, bool f16);
-hipError_t launch_ffn_persistent_bf16(const FfnArgs&, int block_m, int blocks, hipStream_t, bool f16);
-int ffn_persistent_occupancy_bf16(int block_m);
+hipError_t launch_ffn_tiled_bf16(const FfnArgs&, int tile, int max_mtiles, int nnt0, int nnt1, hipStream_t, bool f16);
+hipError_t launch_ffn_persistent_bf16(const FfnArgs&, int tile, int blocks, hipStream_t, bool f16);
+int ffn_persistent_occupancy_bf16(int tile);
 hipError_t launch_gemm_dense_bf16(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t, int,
                                   hipStream_t, bool f16);
 hipError_t launch_ffn_tiled_f32(const FfnArgs&, int max_mtiles, int nnt0, int nnt1, hipStream_t);
@@ -50,7 +54,7 @@ struct Derived {
 
 struct WsLayout {
     size_t logits, topk_idx, topk_w, slot, pair_row, token_indices, expert_count, expert_offset, rank_local,
-        block_hist, mtiles, seg0, seg1, segq, qstate, done0, stats_prob, stats_cnt, h, y, total;
+        block_hist, mtiles, seg0, seg1, segq, qstate, done0, wg_clock, stats_prob, stats_cnt, h, y, total;
 };
 
 // Storage type of activations (x, biases, h, y, out): the layer's own, except that tf32 -- fp32 storage with
@@ -111,6 +115,7 @@ WsLayout layout(const Derived& d) {
     w.segq = take((size_t)2 * d.E * sizeof(Segment));
     w.qstate = take(sizeof(QueueState));
     w.done0 = take((size_t)d.max_mtiles * 4);
+    w.wg_clock = take((size_t)kMaxQueueWorkgroups * 2 * sizeof(int64_t));
     w.stats_prob = take((size_t)kStatsBlocks * d.E * 8);
     w.stats_cnt = take((size_t)kStatsBlocks * d.E * 4);
     w.h = take((size_t)d.A * d.I * d.act_bytes);
@@ -123,6 +128,7 @@ WsLayout layout(const Derived& d) {
 
 FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E) {
     FfnPlan p;
+    p.tile = 0;
     const bool sw = act == MOE_ACT_SWIGLU;
     if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32) {
         p.block_m = f32_block_m();
@@ -133,9 +139,10 @@ FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E) {
         p.nnt0 = ceil_div(I, fp8_block_n0());
         p.nnt1 = ceil_div(H, fp8_block_n1());
     } else {
-        p.block_m = bf16_block_m(A, E, H, I, sw);
-        p.nnt0 = sw ? ceil_div(I, bf16_block_n0(p.block_m) / 2) : ceil_div(I, bf16_block_n0(p.block_m));
-        p.nnt1 = ceil_div(H, bf16_block_n1(p.block_m));
+        p.tile = bf16_tile(A, E, H, I, sw);
+        p.block_m = bf16_block_m(p.tile);
+        p.nnt0 = sw ? ceil_div(I, bf16_block_n0(p.tile) / 2) : ceil_div(I, bf16_block_n0(p.tile));
+        p.nnt1 = ceil_div(H, bf16_block_n1(p.tile));
     }
     return p;
 }
@@ -154,6 +161,7 @@ struct moe_handle {
     moe_arch arch;
     int ffn_mode;
     int queue_groups;      // task queues of the FFN stage: one per XCD, or 1
+    int wall_clock_khz;    // rate of the constant clock the queue kernels stamp their entry and exit with
     int spin_limit;        // polls a dependency wait of the queue kernel makes before it gives up
     int32_t* stall_host;   // pinned host word the queue kernel sets when such a wait expired (never cleared by a kernel)
     int timing;
@@ -305,8 +313,10 @@ int moe_create(const moe_config* cfg, moe_handle** out) {
     h->arch.wavefront_size = prop.warpSize;
     h->arch.lds_bytes_per_cu = (int)prop.maxSharedMemoryPerMultiProcessor;
     h->arch.max_clock_khz = prop.clockRate;
+    if (hipDeviceGetAttribute(&h->wall_clock_khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess || h->wall_clock_khz <= 0)
+        h->wall_clock_khz = 100000;   // 100 MHz on gfx950
     snprintf(h->arch.name, sizeof h->arch.name, "%s", prop.gcnArchName);
-    int per_cu = ffn_persistent_blocks(cfg->torch_dtype, d.plan.block_m, 1);
+    int per_cu = ffn_persistent_blocks(cfg->torch_dtype, d.plan.tile, 1);
     if (const char* env = getenv("MOE355_BLOCKS_PER_CU")) {   // tuning knob: resident workgroups per CU
         const int v = atoi(env);
         if (v >= 1 && v <= 16) per_cu = v;
@@ -539,6 +549,7 @@ int forward_on(moe_handle* h, const void* x, const moe_weights* w, void* out, co
     fa.act = c.hidden_act;
     fa.spin_limit = h->spin_limit;
     fa.host_stall = h->stall_host;
+    fa.wg_clock = at<int64_t>(workspace, L.wg_clock);
     {   // operand extents for the buffer descriptors of the 256-row bf16 tile (chosen only when they fit 32 bits)
         const int64_t es = d.act_bytes;
         fa.x_bytes = (uint32_t)((int64_t)d.S * d.H * es);
@@ -627,6 +638,35 @@ int moe_get_task_counts(moe_handle* h, const void* workspace, void* stream, int6
     return (q.stall || *(volatile int32_t*)h->stall_host) ? MOE_ERR_QUEUE_STALL : MOE_OK;
 }
 
+int moe_get_queue_balance(moe_handle* h, const void* workspace, void* stream, int32_t* workgroups, float* span_us,
+                          float* mean_active_us, float* mean_tail_idle_us) {
+    if (!h || !workspace) return MOE_ERR_BAD_ARGUMENT;
+    if (resolved_ffn_mode(h) != MOE_FFN_PERSISTENT) return MOE_ERR_UNSUPPORTED;
+    const int n = std::min(h->arch.persistent_blocks, kMaxQueueWorkgroups);
+    std::vector<int64_t> t((size_t)2 * n);
+    hipStream_t st = (hipStream_t)stream;
+    hipError_t e = hipMemcpyAsync(t.data(), static_cast<const char*>(workspace) + h->ws.wg_clock, t.size() * 8,
+                                  hipMemcpyDeviceToHost, st);
+    if (e != hipSuccess) return hip_fail(h, e);
+    e = hipStreamSynchronize(st);
+    if (e != hipSuccess) return hip_fail(h, e);
+    int64_t first = INT64_MAX, last = INT64_MIN;
+    double active = 0;
+    for (int i = 0; i < n; ++i) {
+        first = std::min(first, t[2 * i]);
+        last = std::max(last, t[2 * i + 1]);
+        active += (double)(t[2 * i + 1] - t[2 * i]);
+    }
+    double tail = 0;
+    for (int i = 0; i < n; ++i) tail += (double)(last - t[2 * i + 1]);
+    const double tick_us = 1000.0 / h->wall_clock_khz;
+    if (workgroups) *workgroups = n;
+    if (span_us) *span_us = (float)((double)(last - first) * tick_us);
+    if (mean_active_us) *mean_active_us = (float)(active / n * tick_us);
+    if (mean_tail_idle_us) *mean_tail_idle_us = (float)(tail / n * tick_us);
+    return MOE_OK;
+}
+
 int moe_gemm_bias_act(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N, int64_t K,
                       int32_t dtype, int32_t act, void* stream) {
     if (!A || !B || !C || M < 1 || N < 1 || K < 1) return MOE_ERR_BAD_ARGUMENT;
@@ -713,18 +753,18 @@ namespace moe355 {
 
 hipError_t launch_ffn_tiled(const FfnArgs& a, int dtype, const FfnPlan& p, int max_mtiles, hipStream_t st) {
     if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32) return launch_ffn_tiled_f32(a, max_mtiles, p.nnt0, p.nnt1, st);
-    return launch_ffn_tiled_bf16(a, p.block_m, max_mtiles, p.nnt0, p.nnt1, st, dtype == MOE_DTYPE_FP16);
+    return launch_ffn_tiled_bf16(a, p.tile, max_mtiles, p.nnt0, p.nnt1, st, dtype == MOE_DTYPE_FP16);
 }
 
 hipError_t launch_ffn_persistent(const FfnArgs& a, int dtype, const FfnPlan& p, int blocks, hipStream_t st) {
     if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32) return launch_ffn_persistent_f32(a, blocks, st);
-    return launch_ffn_persistent_bf16(a, p.block_m, blocks, st, dtype == MOE_DTYPE_FP16);
+    return launch_ffn_persistent_bf16(a, p.tile, blocks, st, dtype == MOE_DTYPE_FP16);
 }
 
-int ffn_persistent_blocks(int dtype, int block_m, int compute_units) {
+int ffn_persistent_blocks(int dtype, int tile, int compute_units) {
     if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32) return compute_units * 4;
     if (dtype == MOE_DTYPE_FP8_E4M3_B128) return compute_units * ffn_persistent_occupancy_fp8();
-    return compute_units * ffn_persistent_occupancy_bf16(block_m);
+    return compute_units * ffn_persistent_occupancy_bf16(tile);
 }
 
 hipError_t launch_gemm_bias_act(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N,

@@ -50,9 +50,14 @@ struct Tile {
     static constexpr int STAGE_BYTES = (BM + BN) * kRowBytes;
     // four wavefronts of 128 x 128 outputs: this tile runs the hand-ordered slab loop (gemm_tile_ring)
     static constexpr bool RING = BM == 256 && BN == 256 && WM == 2 && WN == 2;
-    // behind the stages: where the four wavefronts of the hand-ordered tile turn 16 rows of results at a time into
-    // row-major order (row pitch 256 + 16 bytes)
-    static constexpr int STAGING_BYTES = RING ? 4 * 16 * 272 : 0;
+    // four wavefronts of 128 x 64 outputs, side by side (128 x 256) or two by two (256 x 128): the same loop with
+    // half the weight fragments per wavefront
+    static constexpr bool HALF = TM == 8 && TN == 4 && WM * WN == 4;
+    static constexpr bool HAND = RING || HALF;
+    static constexpr int WB = BN / WN;            // weight rows per wavefront
+    // behind the stages: where the four wavefronts of a hand-ordered tile turn 16 rows of results at a time into
+    // row-major order (row pitch: the wavefront's columns in bytes + 16)
+    static constexpr int STAGING_BYTES = HAND ? 4 * 16 * (TN * 32 + 16) : 0;
     static constexpr int LDS_BYTES = NS * STAGE_BYTES + STAGING_BYTES;
     static_assert(TM >= 2 && TM % 2 == 0 && TN >= 2 && TN % 2 == 0, "a wavefront's tile is split in token halves; SwiGLU pairs weight-row halves");
     static_assert(RA >= 1 && RB >= 1, "tile too small for the workgroup");
@@ -374,10 +379,10 @@ struct NoHook {
 // `between(i)` runs in front of row group i (i = 0..7): the queue kernel issues the next task's first loads there, a
 // few at a time, so that they leave the compute unit under the epilogue's arithmetic instead of in front of it.
 template <class T, int MODE, class Hook>
-__device__ __forceinline__ void epilogue_full_n_impl(const TaskPtrs& p, unsigned char* smem, f32x4 (&acc)[8][8], const Hook& between) {
+__device__ __forceinline__ void epilogue_full_n_impl(const TaskPtrs& p, unsigned char* smem, f32x4 (&acc)[8][T::TN], const Hook& between) {
 
-    static_assert(T::TM == 8 && T::TN == 8 && T::WN == 2, "four wavefronts of 128 x 128");
-    constexpr int NJ = MODE == 3 ? 4 : 8;        // groups of 16 output columns per wavefront
+    static_assert(T::HAND, "four wavefronts of 128 x 128 or 128 x 64");
+    constexpr int NJ = MODE == 3 ? T::TN / 2 : T::TN;   // groups of 16 output columns per wavefront
     constexpr int ROW_BYTES = NJ * 32, PITCH = ROW_BYTES + 16;
     constexpr int LANES_PER_ROW = ROW_BYTES / 16, ROWS_PER_PASS = 64 / LANES_PER_ROW;
     static_assert(4 * 16 * PITCH <= T::STAGING_BYTES, "the staging pieces of the four wavefronts fit behind the slab stages");
@@ -387,7 +392,7 @@ __device__ __forceinline__ void epilogue_full_n_impl(const TaskPtrs& p, unsigned
     int tid = threadIdx.x;
     asm volatile("" : "+v"(tid));
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / T::WN, wn = wave % T::WN;
     const int frow = lane & 15, fk = lane >> 4;
     const int col0 = p.n0 + wn * 16 * NJ;        // first output column of this wavefront
     float b0[NJ][4], b1[NJ][4];
@@ -427,7 +432,7 @@ __device__ __forceinline__ void epilogue_full_n_impl(const TaskPtrs& p, unsigned
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 if constexpr (MODE == 3) {
-                    const float g = acc[i][j][r] + b1[j][r], u = acc[i][j + 4][r] + b0[j][r];
+                    const float g = acc[i][j][r] + b1[j][r], u = acc[i][j + NJ][r] + b0[j][r];
                     v[r] = silu_fast(g) * u;
                 } else {
                     const float u = acc[i][j][r] + b0[j][r];
@@ -456,7 +461,7 @@ __device__ __forceinline__ void epilogue_full_n_impl(const TaskPtrs& p, unsigned
 }
 
 template <class T, class Hook = NoHook>
-__device__ __forceinline__ void epilogue_full_n(const TaskPtrs& p, unsigned char* smem, f32x4 (&acc)[8][8], const Hook& between = Hook()) {
+__device__ __forceinline__ void epilogue_full_n(const TaskPtrs& p, unsigned char* smem, f32x4 (&acc)[8][T::TN], const Hook& between = Hook()) {
     if (p.swiglu) epilogue_full_n_impl<T, 3>(p, smem, acc, between);
     else if (p.act == MOE_ACT_GELU) epilogue_full_n_impl<T, 2>(p, smem, acc, between);
     else epilogue_full_n_impl<T, 0>(p, smem, acc, between);
@@ -489,7 +494,7 @@ struct RingLoads {
 // The part of a task's load state that needs no memory access: weight-row offsets, bases, extents.
 template <class T>
 __device__ __forceinline__ RingLoads ring_prepare_weights(const TaskPtrs& p) {
-    static_assert(T::RING && T::TM == 8 && T::TN == 8 && T::RA == 8 && T::RB == 8, "four wavefronts of 128 x 128");
+    static_assert(T::HAND && T::ROWS_PER_PASS == 32, "four wavefronts of 128 x 128 or 128 x 64");
     // a thread id the compiler cannot see through: what is derived from it is computed here, not once at the top of
     // the kernel and then kept (and spilled) across the slab loop
     int tid = threadIdx.x;
@@ -498,10 +503,12 @@ __device__ __forceinline__ RingLoads ring_prepare_weights(const TaskPtrs& p) {
     const int chunk = (tid & 7) ^ ((prow >> 1) & 7);
     RingLoads L;
 #pragma unroll
-    for (int n = 0; n < 8; ++n) {
-        L.voff_a[n] = p.a_extent;
+    for (int n = 0; n < 8; ++n) L.voff_a[n] = L.voff_b[n] = p.a_extent;
+#pragma unroll
+    for (int n = 0; n < T::RB; ++n) {
+        // SwiGLU: a wavefront's weight rows are the gate rows of its output columns followed by their up rows
         const int j = prow + n * T::ROWS_PER_PASS;
-        const int col = p.swiglu ? p.n0 + (j >> 7) * 64 + (j & 63) : p.n0 + j;
+        const int col = p.swiglu ? p.n0 + (j / T::WB) * (T::WB / 2) + (j % (T::WB / 2)) : p.n0 + j;
         L.voff_b[n] = (unsigned)(((int64_t)col * p.b_ld + chunk * 8) * 2);
     }
     auto uniform = [](const void* q) {          // the bases are the same in every lane; say so, or each load loops over lanes
@@ -529,7 +536,7 @@ __device__ __forceinline__ void ring_prepare_tokens(const TaskPtrs& p, RingLoads
     const int prow = tid >> 3;
     const int chunk = (tid & 7) ^ ((prow >> 1) & 7);
 #pragma unroll
-    for (int n = 0; n < 8; ++n) {
+    for (int n = 0; n < T::RA; ++n) {
         // Padding rows are never stored.  Their loads are aimed behind the end of the buffer, which the hardware
         // answers with zeros without touching memory: MFMAs on zeros draw less of the power budget than MFMAs on a
         // copy of real rows.
@@ -546,8 +553,8 @@ __device__ __forceinline__ RingLoads ring_prepare(const TaskPtrs& p) {
     return L;
 }
 
-// Load n of slab `slab` of a task: n < 8 token rows, else weight rows; the weight rows of pass m come from w_gate when
-// m % 4 < 2.  Raw buffers (stride 0) that end where the operand ends.  Slabs past the end of K go through descriptors of
+// Load n of slab `slab` of a task: n < RA token rows, else weight rows; the weight rows of pass m come from w_gate when
+// they lie in the first half of a wavefront's weight rows.  Raw buffers (stride 0) that end where the operand ends.  Slabs past the end of K go through descriptors of
 // zero length, which the hardware answers with zeros without touching memory (the stages they land in are never read).
 template <class T>
 __device__ __forceinline__ void ring_load_one(const RingLoads& L, unsigned char* smem, int slab, int n) {
@@ -555,13 +562,14 @@ __device__ __forceinline__ void ring_load_one(const RingLoads& L, unsigned char*
     unsigned char* base = smem + (slab & 1) * T::STAGE_BYTES;
     const int soff = slab * kRowBytes;
     const bool live = slab < L.KT;
-    if (n < 8) {
+    if (n < T::RA) {
         const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(L.base_a), 0, live ? (int)L.a_extent : 0, 0x00020000);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void*)(base + (wrow + n * T::ROWS_PER_PASS) * kRowBytes), 16,
                                                  L.voff_a[n], soff, 0, 0);
     } else {
-        const int m = n - 8;
-        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>((m & 2) ? L.base_b0 : L.base_b1), 0,
+        const int m = n - T::RA;
+        const bool up_rows = (m * T::ROWS_PER_PASS) % T::WB >= T::WB / 2;
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(up_rows ? L.base_b0 : L.base_b1), 0,
                                                                              live ? (int)L.b_extent : 0, 0x00020000);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void*)(base + T::BM * kRowBytes + (wrow + m * T::ROWS_PER_PASS) * kRowBytes),
                                                  16, L.voff_b[m], soff, 0, 0);
@@ -570,18 +578,18 @@ __device__ __forceinline__ void ring_load_one(const RingLoads& L, unsigned char*
 
 // The loads of a task's first two slabs: the weight rows of slab 0 and of slab 1, then the token rows of slab 0 and of
 // slab 1 -- weights first because their addresses need no gathered row numbers, so the queue kernel can send them
-// off while those are still on their way.  Slab 0 is complete when at most the last eight of the 32 are outstanding.
+// off while those are still on their way.  Slab 0 is complete when at most the last RA of them are outstanding.
 // Nobody may still be reading the stages (the caller sees to that).
 template <class T>
 __device__ __forceinline__ void ring_first_weight_loads(const RingLoads& L, unsigned char* smem) {
 #pragma unroll
-    for (int n = 8; n < 16; ++n) ring_load_one<T>(L, smem, 0, n);
+    for (int n = T::RA; n < T::RA + T::RB; ++n) ring_load_one<T>(L, smem, 0, n);
 #pragma unroll
-    for (int n = 8; n < 16; ++n) ring_load_one<T>(L, smem, 1, n);
+    for (int n = T::RA; n < T::RA + T::RB; ++n) ring_load_one<T>(L, smem, 1, n);
 }
 template <class T>
-__device__ __forceinline__ void ring_first_token_load(const RingLoads& L, unsigned char* smem, int q) {   // q = 0..15
-    ring_load_one<T>(L, smem, q >> 3, q & 7);
+__device__ __forceinline__ void ring_first_token_load(const RingLoads& L, unsigned char* smem, int q) {   // q = 0..2 RA - 1
+    if (q < 2 * T::RA) ring_load_one<T>(L, smem, q / T::RA, q % T::RA);
 }
 template <class T>
 __device__ __forceinline__ void ring_first_loads(const RingLoads& L, unsigned char* smem) {
@@ -607,10 +615,10 @@ __device__ __forceinline__ void ring_first_loads(const RingLoads& L, unsigned ch
 // wavefront (stores issued behind them only make the first wait more conservative).  Returns false for a wavefront whose 128 rows are all
 // padding: it has taken part in the loads and barriers only and holds no results.
 template <class T>
-__device__ __forceinline__ bool ring_slabs(int rows, const RingLoads& L, unsigned char* smem, f32x4 (&acc)[8][8]) {
-    constexpr int BM = T::BM, STAGE = T::STAGE_BYTES;
+__device__ __forceinline__ bool ring_slabs(int rows, const RingLoads& L, unsigned char* smem, f32x4 (&acc)[8][T::TN]) {
+    constexpr int BM = T::BM, STAGE = T::STAGE_BYTES, TN = T::TN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / T::WN, wn = wave % T::WN;
     // The scalar members are the same in every lane; say so here, behind whatever control flow handed L over, or the
     // compiler builds every buffer descriptor in a loop over the lanes.
     RingLoads U = L;
@@ -630,7 +638,7 @@ __device__ __forceinline__ bool ring_slabs(int rows, const RingLoads& L, unsigne
 #pragma unroll
     for (int i = 0; i < 8; ++i)
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int j = 0; j < TN; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
     const int frow = lane & 15, fk = lane >> 4;
     const int sw = (frow >> 1) & 7;
@@ -638,11 +646,11 @@ __device__ __forceinline__ bool ring_slabs(int rows, const RingLoads& L, unsigne
     // (the asm reads take raw LDS byte addresses: start from where the dynamic array really begins -- a kernel with
     // static __shared__ variables places it behind them)
     const unsigned lds0 = (unsigned)(__UINTPTR_TYPE__)(lds_void*)smem;
-    const unsigned a_row = lds0 + (unsigned)((wm * 128 + frow) * kRowBytes), b_row = lds0 + (unsigned)(BM * kRowBytes + (wn * 128 + frow) * kRowBytes);
+    const unsigned a_row = lds0 + (unsigned)((wm * 128 + frow) * kRowBytes), b_row = lds0 + (unsigned)(BM * kRowBytes + (wn * T::WB + frow) * kRowBytes);
     const unsigned c0 = (unsigned)((fk ^ sw) << 4), c1 = (unsigned)(((4 + fk) ^ sw) << 4);
     const unsigned la0[2] = {a_row + c0, a_row + c1}, lb0[2] = {b_row + c0, b_row + c1};
     const unsigned la1[2] = {la0[0] + STAGE, la0[1] + STAGE}, lb1[2] = {lb0[0] + STAGE, lb0[1] + STAGE};
-    bf16x8 af[2][8], bfr[2][8];
+    bf16x8 af[2][8], bfr[2][TN];
     int kt = 0;
 
 #define MF(i, j, s)                                                                                                      \
@@ -676,18 +684,26 @@ __device__ __forceinline__ bool ring_slabs(int rows, const RingLoads& L, unsigne
 #define RA(stg, half, idx) ((void)0)
 #define RB(stg, half, j) ((void)0)
 #define WL(n) ((void)0)
-        BAR2(8);
+        if constexpr (T::RA == 8) BAR2(8); else BAR2(4);
         for (; kt < KT; kt += 2) {
             {
                 constexpr unsigned st = 0, sn = 1;
                 (void)st; (void)sn;
+                if constexpr (TN == 8) {
 #include "ffn_bf16_slab_steady.inc"
+                } else {
+#include "ffn_bf16_slab_half.inc"
+                }
             }
             ++kt;
             {
                 constexpr unsigned st = 1, sn = 0;
                 (void)st; (void)sn;
+                if constexpr (TN == 8) {
 #include "ffn_bf16_slab_steady.inc"
+                } else {
+#include "ffn_bf16_slab_half.inc"
+                }
             }
             --kt;
         }
@@ -697,11 +713,13 @@ __device__ __forceinline__ bool ring_slabs(int rows, const RingLoads& L, unsigne
 #pragma pop_macro("MF")
         return false;                           // nothing to store either
     }
-    BAR2(8);                                    // slab 0 has landed (loads return in issue order; see ring_first_loads)
+    // slab 0 has landed (loads return in issue order; see ring_first_loads)
+    if constexpr (T::RA == 8) BAR2(8); else BAR2(4);
     {   // same order as the reads behind BAR2 of a steady-state slab
         constexpr unsigned sn = 0;
         RA(sn, 0, 0);
-        RB(sn, 0, 0); RB(sn, 0, 1); RB(sn, 0, 2); RB(sn, 0, 3); RB(sn, 0, 4); RB(sn, 0, 5); RB(sn, 0, 6); RB(sn, 0, 7);
+        RB(sn, 0, 0); RB(sn, 0, 1); RB(sn, 0, 2); RB(sn, 0, 3);
+        if constexpr (TN == 8) { RB(sn, 0, 4); RB(sn, 0, 5); RB(sn, 0, 6); RB(sn, 0, 7); }
         RA(sn, 0, 1); RA(sn, 0, 2); RA(sn, 0, 3); RA(sn, 0, 4); RA(sn, 0, 5); RA(sn, 0, 6); RA(sn, 0, 7);
     }
     // Every slab runs the same body, the last two included: their loads (of slabs KT and KT+1) fetch nothing and
@@ -711,12 +729,20 @@ __device__ __forceinline__ bool ring_slabs(int rows, const RingLoads& L, unsigne
     for (; kt < KT; kt += 2) {
         {
             constexpr unsigned st = 0, sn = 1;
+                if constexpr (TN == 8) {
 #include "ffn_bf16_slab_steady.inc"
+                } else {
+#include "ffn_bf16_slab_half.inc"
+                }
         }
         ++kt;
         {
             constexpr unsigned st = 1, sn = 0;
+                if constexpr (TN == 8) {
 #include "ffn_bf16_slab_steady.inc"
+                } else {
+#include "ffn_bf16_slab_half.inc"
+                }
         }
         --kt;
     }
@@ -726,9 +752,12 @@ __device__ __forceinline__ bool ring_slabs(int rows, const RingLoads& L, unsigne
     // occupied until behind that wait.
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
-    for (int h = 0; h < 2; ++h)
+    for (int h = 0; h < 2; ++h) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) asm volatile("" ::"v"(af[h][i]), "v"(bfr[h][i]));
+        for (int i = 0; i < 8; ++i) asm volatile("" ::"v"(af[h][i]));
+#pragma unroll
+        for (int j = 0; j < TN; ++j) asm volatile("" ::"v"(bfr[h][j]));
+    }
 #undef MF
 #undef RA
 #undef RB
@@ -746,7 +775,7 @@ __device__ __forceinline__ void gemm_tile_ring(const TaskPtrs& p, unsigned char*
     const RingLoads L = ring_prepare<T>(p);
     __syncthreads();                            // the previous task may still be reading the stages
     ring_first_loads<T>(L, smem);
-    f32x4 acc[8][8];
+    f32x4 acc[8][T::TN];
     if (ring_slabs<T>(p.rows, L, smem, acc)) epilogue_full_n<T>(p, smem, acc);
 }
 
@@ -761,7 +790,7 @@ __device__ __forceinline__ void gemm_tile_generic(const TaskPtrs& p, unsigned ch
 // meets that loop's conditions (large_tile_ok) and falls back to the 128 x 128 tile otherwise.
 template <class T>
 __device__ __forceinline__ void gemm_tile(const TaskPtrs& p, unsigned char* smem) {
-    if constexpr (T::RING) {
+    if constexpr (T::HAND) {
         gemm_tile_ring<T>(p, smem);
     } else {
         if (p.rows >= T::BM) gemm_tile_generic<T, false>(p, smem);
@@ -817,18 +846,47 @@ __device__ __forceinline__ TaskPtrs resolve(const FfnArgs& a, const Task& t, boo
 
 // A plan pairs the tile of the up(/gate) projection with the tile of the down projection; both use the
 // same row-block height and the same workgroup size.
-template <class T0_, class T1_>
+//
+// TS (optional): the tile that takes the row blocks of at most TS::BM rows -- the ragged last block of an expert --
+// in place of T0 / T1.  It covers the same columns per task, so the task tables do not change; it only does not
+// spend a full tile's MFMAs on rows that are mostly padding.
+template <class T0_, class T1_, class TS_ = void>
 struct Plan {
     using T0 = T0_;
     using T1 = T1_;
+    using TS = TS_;
+    static constexpr bool MIXED = !std::is_void<TS_>::value;
     static_assert(T0::BM == T1::BM && T0::THREADS == T1::THREADS, "phases share row blocks and workgroup size");
     static constexpr int THREADS = T0::THREADS;
     static constexpr int LDS_BYTES = T0::LDS_BYTES > T1::LDS_BYTES ? T0::LDS_BYTES : T1::LDS_BYTES;
 };
-using LargePlan = Plan<Tile<256, 256, 2, 2, 2>, Tile<256, 256, 2, 2, 2>>;
+using Tile256 = Tile<256, 256, 2, 2, 2>;
+using Tile128x256 = Tile<128, 256, 1, 4, 2>;     // hand-ordered, four wavefronts of 128 x 64 side by side
+using Tile256H = Tile<256, 256, 2, 2, 2, true>;  // fp16
+using Tile128x256H = Tile<128, 256, 1, 4, 2, true>;
+using LargePlan = Plan<Tile256, Tile256>;
+using MixedPlan = Plan<Tile256, Tile256, Tile128x256>;
+using MediumPlan = Plan<Tile128x256, Tile128x256>;
 using SmallPlan = Plan<Tile<128, 128, 2, 2, 2>, Tile<128, 128, 2, 2, 2>>;
-using LargePlanH = Plan<Tile<256, 256, 2, 2, 2, true>, Tile<256, 256, 2, 2, 2, true>>;   // fp16
+using LargePlanH = Plan<Tile256H, Tile256H>;
+using MixedPlanH = Plan<Tile256H, Tile256H, Tile128x256H>;
+using MediumPlanH = Plan<Tile128x256H, Tile128x256H>;
 using SmallPlanH = Plan<Tile<128, 128, 2, 2, 2, true>, Tile<128, 128, 2, 2, 2, true>>;
+
+// One task of a plan: the plan's tile, or its small-row-block tile when the block has few enough rows.
+template <class P>
+__device__ __forceinline__ void plan_tile(const FfnArgs& a, const Task& t, bool publish, unsigned char* smem) {
+    static_assert(std::is_same<typename P::T0, typename P::T1>::value, "one tile for both projections: one inlined copy");
+    const TaskPtrs p = resolve<typename P::T0>(a, t, publish);
+    if constexpr (P::MIXED) {
+        static_assert(P::TS::BN == P::T0::BN && P::TS::LDS_BYTES <= P::LDS_BYTES, "same columns per task");
+        if (t.rows <= P::TS::BM) {
+            gemm_tile<typename P::TS>(p, smem);
+            return;
+        }
+    }
+    gemm_tile<typename P::T0>(p, smem);
+}
 
 // One launch per phase; workgroup b runs task b of that phase.
 template <class P>
@@ -836,8 +894,17 @@ __global__ __launch_bounds__(P::THREADS) void ffn_tiled_kernel(FfnArgs a, int ph
     extern __shared__ __align__(16) unsigned char smem[];
     Task t;
     if (!tiled_task(a, phase, blockIdx.x, t)) return;
-    static_assert(std::is_same<typename P::T0, typename P::T1>::value, "one tile for both projections: one inlined copy");
-    gemm_tile<typename P::T0>(resolve<typename P::T0>(a, t, false), smem);
+    plan_tile<P>(a, t, false, smem);
+}
+
+// The kernel's argument block, read again from the kernel-argument segment through a pointer the compiler cannot see
+// through: values loaded from it live only as long as they are used, instead of occupying forty scalar registers
+// across the slab loop (which then spill into vector registers and bring vector instructions into the loop).
+__device__ __forceinline__ const FfnArgs& kernel_args_again() {
+    typedef const __attribute__((address_space(4))) FfnArgs* args_ptr;
+    args_ptr q = (args_ptr)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(q));
+    return *(const FfnArgs*)q;
 }
 
 // Persistent workgroups popping (expert, tile) tasks from the queue of their XCD (protocol: ffn_common.hpp).
@@ -846,6 +913,7 @@ __global__ __launch_bounds__(P::THREADS) void ffn_persistent_kernel(FfnArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ int s_task, s_ok;
     queue_kernel_entry();
+    queue_clock_stamp(kernel_args_again().wg_clock, 0);
     const int ids = a.q->ids_queue;
     const int nseg = a.q->nseg;
     const int nnt0 = a.seg_phase0[0].nnt;
@@ -858,9 +926,10 @@ __global__ __launch_bounds__(P::THREADS) void ffn_persistent_kernel(FfnArgs a) {
             poison_tile((uint16_t*)a.y + (int64_t)t.row0 * a.H, t.rows, a.H, t.ntile * P::T1::BN, P::T1::BN, 2);
             t.rows = 0;
         }
-        gemm_tile<typename P::T0>(resolve<typename P::T0>(a, t, t.phase == 0), smem);   // one inlined copy for both phases
+        plan_tile<P>(a, t, t.phase == 0, smem);
         if (t.phase == 0) signal_phase0_done(a.done0, t.mtile);
     }
+    queue_clock_stamp(kernel_args_again().wg_clock, 1);
 }
 
 // The same queue for the 256 x 256 tile, with the start of the next task moved under the end of the current one
@@ -881,16 +950,6 @@ __global__ __launch_bounds__(P::THREADS) void ffn_persistent_kernel(FfnArgs a) {
 // 74 % either way); short tiles lose 2-3 %.  Results are bit-identical to the plain loop.
 constexpr int kReserveMargin = 64;   // ids left in the current queue below which tasks are popped late again
 
-// The kernel's argument block, read again from the kernel-argument segment through a pointer the compiler cannot see
-// through: values loaded from it live only as long as they are used, instead of occupying forty scalar registers
-// across the slab loop (which then spill into vector registers and bring vector instructions into the loop).
-__device__ __forceinline__ const FfnArgs& kernel_args_again() {
-    typedef const __attribute__((address_space(4))) FfnArgs* args_ptr;
-    args_ptr q = (args_ptr)__builtin_amdgcn_kernarg_segment_ptr();
-    asm volatile("" : "+s"(q));
-    return *(const FfnArgs*)q;
-}
-
 template <class P>
 __global__ __launch_bounds__(P::THREADS) void ffn_persistent_ring_kernel(FfnArgs) {
     using T = typename P::T0;
@@ -898,6 +957,7 @@ __global__ __launch_bounds__(P::THREADS) void ffn_persistent_ring_kernel(FfnArgs
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ int s_task, s_ok, s_next[2];
     queue_kernel_entry();
+    queue_clock_stamp(kernel_args_again().wg_clock, 0);
     int ids, nseg, nnt0, groups;
     {
         const FfnArgs& a = kernel_args_again();
@@ -997,6 +1057,7 @@ __global__ __launch_bounds__(P::THREADS) void ffn_persistent_ring_kernel(FfnArgs
         have = pop_blocking();
         if (have) start_cold();
     }
+    queue_clock_stamp(kernel_args_again().wg_clock, 1);
 }
 
 // The bare reference contract on dense operands: rows [b*BM, ...) of A, one "expert".
@@ -1126,7 +1187,7 @@ hipError_t launch_tiled(const FfnArgs& a, int max_mtiles, int nnt0, int nnt1, hi
 
 template <class P>
 hipError_t launch_persistent(const FfnArgs& a, int blocks, hipStream_t st) {
-    if constexpr (P::T0::RING) {
+    if constexpr (P::T0::RING && !P::MIXED) {
         // tuning knob: 1 = the queue loop that starts the next task under the end of the current one (measured: no
         // faster on the Mixtral shape, 2-3 % slower on short tiles; kept for machines where the balance differs)
         const char* env = getenv("MOE355_QUEUE_EARLY");
@@ -1167,37 +1228,71 @@ static bool large_tile_ok(int64_t pairs, int H, int I, bool swiglu) {
            (int64_t)H * I * 2 < lim;
 }
 
-int bf16_block_m(int64_t pairs, int experts, int H, int I, int swiglu) {
-    if (!large_tile_ok(pairs, H, I, swiglu != 0)) return 128;
+// Tile of a layer: 0 = 128 x 128, 1 = 256 x 256, 2 = 128 x 256, 3 = 256 x 256 with the 128 x 256 tile for the row
+// blocks of at most 128 rows.
+//
+// Measured (FFN stage, same box, alternating runs): the 128 x 256 tile reaches 93 % of the 256 x 256 tile's rate on
+// a plain 4096 x 8192 x 4096 GEMM, but as the tile of a whole layer it loses to it everywhere (Mixtral shape 5.45
+// against 4.33 ms, 16 experts of 512 rows 0.209 against 0.187 ms, 64 small experts 0.72 against 0.59 ms): twice the
+// tasks, each with the same 12 us between two slab loops.  For short last blocks only it gains 1-2 % with many small
+// experts and loses 2 % on the Mixtral shape -- there a short block's task runs through K faster than the eight full
+// blocks that share its weight tile, drops out of their lockstep and fetches its weights past the L2 on its own
+// (with a routing that leaves no partial blocks both kernels take the same time).  So 3 is chosen below 1024 rows per
+// expert, 1 above, and 2 is a tuning knob only.
+int bf16_tile(int64_t pairs, int experts, int H, int I, int swiglu) {
+    if (!large_tile_ok(pairs, H, I, swiglu != 0)) return 0;
     const int up_columns = swiglu ? 2 * I : I;
-    if (const char* env = getenv("MOE355_BLOCK_ROWS")) {   // tuning knob: force the row-block height
+    if (const char* env = getenv("MOE355_BLOCK_ROWS")) {   // tuning knob: force the row-block height ...
         const int v = atoi(env);
-        if (v == 128 || v == 256) return v;
+        if (v == 128 || v == 256) return v == 256 ? 1 : 0;
     }
-    if (pairs / (experts > 0 ? experts : 1) < 256) return 128;
-    const int64_t tasks = (pairs / 256) * ((up_columns + LargePlan::T0::BN - 1) / LargePlan::T0::BN);
-    return tasks >= 256 ? 256 : 128;
+    if (const char* env = getenv("MOE355_TILE")) {         // ... or the tile
+        const int v = atoi(env);
+        if (v >= 0 && v <= 3) return v;
+    }
+    const int64_t per_expert = pairs / (experts > 0 ? experts : 1);
+    if (per_expert < 256) return 0;
+    const int64_t tasks = (pairs / 256) * ((up_columns + Tile256::BN - 1) / Tile256::BN);
+    if (tasks < 256) return 0;
+    return per_expert < 1024 ? 3 : 1;
 }
-int bf16_block_n0(int block_m) { return block_m == 256 ? LargePlan::T0::BN : SmallPlan::T0::BN; }
-int bf16_block_n1(int block_m) { return block_m == 256 ? LargePlan::T1::BN : SmallPlan::T1::BN; }
+int bf16_block_m(int tile) { return tile == 1 || tile == 3 ? 256 : 128; }
+int bf16_block_n0(int tile) { return tile == 0 ? SmallPlan::T0::BN : 256; }
+int bf16_block_n1(int tile) { return tile == 0 ? SmallPlan::T1::BN : 256; }
 
-hipError_t launch_ffn_tiled_bf16(const FfnArgs& a, int block_m, int max_mtiles, int nnt0, int nnt1, hipStream_t st,
+template <template <class> class F, class... Args>
+static auto for_plan(int tile, bool f16, Args&&... args) {
+    if (f16) {
+        if (tile == 1) return F<LargePlanH>::run(args...);
+        if (tile == 3) return F<MixedPlanH>::run(args...);
+        if (tile == 2) return F<MediumPlanH>::run(args...);
+        return F<SmallPlanH>::run(args...);
+    }
+    if (tile == 1) return F<LargePlan>::run(args...);
+    if (tile == 3) return F<MixedPlan>::run(args...);
+    if (tile == 2) return F<MediumPlan>::run(args...);
+    return F<SmallPlan>::run(args...);
+}
+template <class P> struct RunTiled {
+    static hipError_t run(const FfnArgs& a, int max_mtiles, int nnt0, int nnt1, hipStream_t st) { return launch_tiled<P>(a, max_mtiles, nnt0, nnt1, st); }
+};
+template <class P> struct RunPersistent {
+    static hipError_t run(const FfnArgs& a, int blocks, hipStream_t st) { return launch_persistent<P>(a, blocks, st); }
+};
+template <class P> struct RunOccupancy {
+    static int run() { return occupancy<P>(); }
+};
+
+hipError_t launch_ffn_tiled_bf16(const FfnArgs& a, int tile, int max_mtiles, int nnt0, int nnt1, hipStream_t st,
                                  bool f16) {
-    if (f16)
-        return block_m == 256 ? launch_tiled<LargePlanH>(a, max_mtiles, nnt0, nnt1, st)
-                              : launch_tiled<SmallPlanH>(a, max_mtiles, nnt0, nnt1, st);
-    return block_m == 256 ? launch_tiled<LargePlan>(a, max_mtiles, nnt0, nnt1, st)
-                          : launch_tiled<SmallPlan>(a, max_mtiles, nnt0, nnt1, st);
+    return for_plan<RunTiled>(tile, f16, a, max_mtiles, nnt0, nnt1, st);
 }
 
-hipError_t launch_ffn_persistent_bf16(const FfnArgs& a, int block_m, int blocks, hipStream_t st, bool f16) {
-    if (f16) return block_m == 256 ? launch_persistent<LargePlanH>(a, blocks, st) : launch_persistent<SmallPlanH>(a, blocks, st);
-    return block_m == 256 ? launch_persistent<LargePlan>(a, blocks, st) : launch_persistent<SmallPlan>(a, blocks, st);
+hipError_t launch_ffn_persistent_bf16(const FfnArgs& a, int tile, int blocks, hipStream_t st, bool f16) {
+    return for_plan<RunPersistent>(tile, f16, a, blocks, st);
 }
 
-int ffn_persistent_occupancy_bf16(int block_m) {
-    return block_m == 256 ? occupancy<LargePlan>() : occupancy<SmallPlan>();
-}
+int ffn_persistent_occupancy_bf16(int tile) { return for_plan<RunOccupancy>(tile, false); }
 
 template <class T>
 static hipError_t launch_dense(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N, int64_t K,
@@ -1215,6 +1310,13 @@ hipError_t launch_gemm_dense_bf16(const void* A, const void* B, const void* bias
                                   int64_t K, int act, hipStream_t st, bool f16) {
     const int64_t lim = (int64_t)1 << 32;
     const bool large = M >= 1024 && N >= 1024 && N % 256 == 0 && K % 128 == 0 && M * K * 2 < lim && N * K * 2 < lim;
+    if (const char* env = getenv("MOE355_DENSE_TILE")) {   // tuning knob: 1 = 256 x 256, 2 = 128 x 256 (shapes they accept only)
+        const int v = atoi(env);
+        if ((v == 1 || v == 2) && N % 256 == 0 && K % 128 == 0 && M * K * 2 < lim && N * K * 2 < lim) {
+            if (v == 1) return f16 ? launch_dense<Tile256H>(A, B, bias, C, M, N, K, act, st) : launch_dense<Tile256>(A, B, bias, C, M, N, K, act, st);
+            return f16 ? launch_dense<Tile128x256H>(A, B, bias, C, M, N, K, act, st) : launch_dense<Tile128x256>(A, B, bias, C, M, N, K, act, st);
+        }
+    }
     if (f16)
         return large ? launch_dense<LargePlanH::T0>(A, B, bias, C, M, N, K, act, st)
                      : launch_dense<SmallPlanH::T0>(A, B, bias, C, M, N, K, act, st);

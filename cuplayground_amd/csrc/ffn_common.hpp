@@ -142,6 +142,13 @@ __device__ __forceinline__ bool tiled_task(const FfnArgs& a, int phase, int b, T
 // every task those two operations cost more than the GEMMs they protected (4.3 ms of a 13 ms layer).
 __device__ __forceinline__ void queue_kernel_entry() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent"); }
 
+// Entry and exit times of every workgroup of a queue kernel, on the constant-rate clock (100 MHz): what the host
+// needs to tell how evenly the queue kept the workgroups busy (moe_get_queue_balance).  Two stores per workgroup.
+__device__ __forceinline__ void queue_clock_stamp(int64_t* wg_clock, int which) {
+    if (wg_clock && threadIdx.x == 0 && blockIdx.x < (unsigned)kMaxQueueWorkgroups)
+        wg_clock[2 * blockIdx.x + which] = (int64_t)wall_clock64();
+}
+
 __device__ __forceinline__ void publish8(void* p, uint32_t lo, uint32_t hi) {
     __hip_atomic_store(reinterpret_cast<uint64_t*>(p), ((uint64_t)hi << 32) | lo, __ATOMIC_RELAXED,
                        __HIP_MEMORY_SCOPE_AGENT);

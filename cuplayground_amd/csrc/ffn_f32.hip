@@ -157,6 +157,7 @@ __global__ __launch_bounds__(256) void ffn_persistent_f32_kernel(FfnArgs a) {
     __shared__ __align__(16) float Bs[FBK][FBN + FPAD];
     __shared__ int s_task, s_ok;
     queue_kernel_entry();
+    queue_clock_stamp(a.wg_clock, 0);
     const int ids = a.q->ids_queue;
     const int nseg = a.q->nseg;
     const int nnt0 = a.seg_phase0[0].nnt;
@@ -170,6 +171,7 @@ __global__ __launch_bounds__(256) void ffn_persistent_f32_kernel(FfnArgs a) {
         else poison_tile(p.c_base, p.rows, p.N, p.n0, FBN, 4);
         if (t.phase == 0) signal_phase0_done(a.done0, t.mtile);
     }
+    queue_clock_stamp(a.wg_clock, 1);
 }
 
 __global__ __launch_bounds__(256) void gemm_dense_f32_kernel(const float* A, const float* B, const float* bias,

@@ -229,6 +229,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     __shared__ float red[QWAVES * QGROUPS * 4 * 64];
     __shared__ int s_task, s_ok;
     queue_kernel_entry();
+    queue_clock_stamp(a.wg_clock, 0);
     const int ids = a.q->ids_queue;
     const int nseg = a.q->nseg;
     const int nnt0 = a.seg_phase0[0].nnt;
@@ -245,6 +246,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         }
         if (t.phase == 0) signal_phase0_done(a.done0, t.mtile);
     }
+    queue_clock_stamp(a.wg_clock, 1);
 }
 
 }  // namespace

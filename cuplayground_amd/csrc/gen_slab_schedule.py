@@ -35,47 +35,61 @@ BAR1_ROW = 4                          # MFMA row in front of which the slab's LD
 PER_ROW = [6, 5, 5, 0, 0, 0, 0, 0]    # fragment reads of k half 1 behind the MFMAs of rows 0..7
 BAR2_ROW = 13                         # MFMA row in front of which the next slab's stage may be read
 
+# The half tiles (128 x 256 on wavefronts of 128 x 64, 256 x 128 likewise): 8 token fragments x 4 weight fragments,
+# 64 MFMAs per slab in 16 rows of 4, 12 fragment reads per k half, 12 global->LDS loads per slab.  A row lasts half
+# as long, so the reads and loads are spread over more rows.
+HALF = dict(nb=4, bar1=7, per_row=[3, 3, 2, 2, 2, 0, 0, 0], bar2=11, next_per_row=[3, 3, 2, 2, 2])
+FULL = dict(nb=8, bar1=BAR1_ROW, per_row=PER_ROW, bar2=BAR2_ROW, next_per_row=[6, 6, 4])
 
-def build(variant):
+
+def build(variant, shape=FULL):
+    nb, bar1, bar2 = shape["nb"], shape["bar1"], shape["bar2"]
+    nloads = 8 + nb
     seq = []
-    half1 = []
-    for i in range(8):
-        half1 += [("RA", "st", 1, i), ("RB", "st", 1, i)]
-    per_row = PER_ROW
-    nxt = [("RA", "sn", 0, 0)] + [("RB", "sn", 0, j) for j in range(8)] + [("RA", "sn", 0, i) for i in range(1, 8)]
+    if nb == 8:
+        half1 = []
+        for i in range(8):
+            half1 += [("RA", "st", 1, i), ("RB", "st", 1, i)]
+    else:   # the first row of k half 1 needs token fragment 0 and every weight fragment
+        half1 = [("RA", "st", 1, 0)] + [("RB", "st", 1, j) for j in range(nb)] + [("RA", "st", 1, i) for i in range(1, 8)]
+    per_row = shape["per_row"]
+    nxt = [("RA", "sn", 0, 0)] + [("RB", "sn", 0, j) for j in range(nb)] + [("RA", "sn", 0, i) for i in range(1, 8)]
+    next_per_row = list(shape["next_per_row"])
+    assert sum(per_row) == len(half1) and sum(next_per_row) == len(nxt) and len(next_per_row) == 16 - bar2
     for g in range(16):
         s, i = divmod(g, 8)
         ops = []
         if g < 8:
             ops = half1[:per_row[i]]
             half1 = half1[per_row[i]:]
-        if g >= BAR1_ROW:
-            if g == BAR1_ROW:
+        if g >= bar1:
+            if g == bar1:
                 seq.append(("BAR1",))
             if variant == "steady":
-                nrows = 16 - BAR1_ROW
-                k0 = (g - BAR1_ROW) * 16 // nrows
-                k1 = (g - BAR1_ROW + 1) * 16 // nrows
+                nrows = 16 - bar1
+                k0 = (g - bar1) * nloads // nrows
+                k1 = (g - bar1 + 1) * nloads // nrows
                 ops = ops + [("GL", q) for q in range(k0, k1)]
-            if g == BAR2_ROW and variant != "last":
-                seq.append(("BAR2", (BAR2_ROW - BAR1_ROW) * 16 // (16 - BAR1_ROW) if variant == "steady" else 0))
-            if g >= BAR2_ROW and variant != "last":
-                n = -(-16 // (16 - BAR2_ROW))
+            if g == bar2 and variant != "last":
+                seq.append(("BAR2", (bar2 - bar1) * nloads // (16 - bar1) if variant == "steady" else 0))
+            if g >= bar2 and variant != "last":
+                n = next_per_row[g - bar2]
                 ops = ops + nxt[:n]
                 nxt = nxt[n:]
         n = len(ops)
         slots = [[] for _ in range(4)]
         for k, o in enumerate(ops):
             slots[(k * 4 // n) if n > 4 else k].append(o)
+        per_slot = nb // 4
         for p in range(4):
-            seq.append(("MF", i, 2 * p, s))
-            seq.append(("MF", i, 2 * p + 1, s))
+            for q in range(per_slot):
+                seq.append(("MF", i, per_slot * p + q, s))
             seq.extend(slots[p])
     return seq
 
 
-def emit(variant):
-    steady, cur = build("steady"), build(variant)
+def emit(variant, shape=FULL):
+    steady, cur = build("steady", shape), build(variant, shape)
     issued, last = 0, {}
 
     def run(seq, out):
@@ -125,6 +139,6 @@ def emit(variant):
 
 if __name__ == "__main__":
     here = os.path.dirname(os.path.abspath(__file__))
-    for v in ("steady",):
-        with open(os.path.join(here, "ffn_bf16_slab_%s.inc" % v), "w") as f:
-            f.write("// generated by gen_slab_schedule.py -- do not edit\n" + emit(v))
+    for name, shape in (("steady", FULL), ("half", HALF)):
+        with open(os.path.join(here, "ffn_bf16_slab_%s.inc" % name), "w") as f:
+            f.write("// generated by gen_slab_schedule.py -- do not edit\n" + emit("steady", shape))

@@ -89,7 +89,9 @@ struct FfnArgs {
     int32_t spin_limit;
     int32_t groups;             // queue groups the schedule was built for
     uint32_t x_bytes, h_bytes, w_bytes;   // extents of x, h and one weight matrix (meaningful below 4 GiB)
+    int64_t* wg_clock;          // queue kernels: [2 * workgroup] constant-rate clock at entry, [2 * workgroup + 1] at exit
 };
+constexpr int kMaxQueueWorkgroups = 4096;   // workgroups of a queue kernel that get a slot in wg_clock
 
 struct RouteArgs {
     const int32_t* topk_idx;    // [A]
@@ -131,6 +133,7 @@ hipError_t launch_combine(const void* y_rows, const int32_t* pair_row, const flo
 
 // FFN stage.  block_m / block_n are the tile sizes the routing stage must be told about.
 struct FfnPlan {
+    int tile;        // 16-bit layers: which tile the kernels are instantiated with (ffn_bf16.hip: bf16_tile)
     int block_m;
     int nnt0;        // column tiles of phase 0
     int nnt1;        // column tiles of phase 1
@@ -138,7 +141,7 @@ struct FfnPlan {
 FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E);
 hipError_t launch_ffn_tiled(const FfnArgs& a, int dtype, const FfnPlan& p, int max_mtiles, hipStream_t st);
 hipError_t launch_ffn_persistent(const FfnArgs& a, int dtype, const FfnPlan& p, int blocks, hipStream_t st);
-int ffn_persistent_blocks(int dtype, int block_m, int compute_units);
+int ffn_persistent_blocks(int dtype, int tile, int compute_units);
 
 // ---- backward building blocks (csrc/backward.hip) ----
 size_t backward_scratch_bytes(int64_t A, int E, int H, int I);

@@ -203,6 +203,14 @@ int moe_get_stage_ms(moe_handle* h, int stage, float* ms, int32_t* calls);
  * whole call from its first to its last kernel) for each of the most recent recorded calls, oldest first, at most
  * `capacity` (and at most 64) of them; *count receives how many were written.  For medians and minima. */
 int moe_get_stage_samples(moe_handle* h, int stage, float* ms, int32_t capacity, int32_t* count);
+
+/* How evenly the task queue of the last moe_forward kept its workgroups busy (task-queue FFN only; MOE_ERR_UNSUPPORTED
+ * in the two-launch mode).  Every workgroup stamps the device's constant-rate clock when it enters and when it leaves
+ * the queue kernel: span_us = first entry to last exit, mean_active_us = mean of (exit - entry), mean_tail_idle_us =
+ * mean of (last exit - own exit), i.e. the time a workgroup had nothing left to pop while others still worked.
+ * Synchronises `stream`.  No counterpart in the reference, whose scheduler keeps no statistics. */
+int moe_get_queue_balance(moe_handle* h, const void* workspace, void* stream, int32_t* workgroups, float* span_us,
+                          float* mean_active_us, float* mean_tail_idle_us);
 /* Tile tasks the FFN stage of the last moe_forward issued to its queue (GEMM0 tasks, GEMM1 tasks); reads
  * back a few words from the workspace, so it synchronises the stream. */
 int moe_get_task_counts(moe_handle* h, const void* workspace, void* stream, int64_t* gemm0_tasks, int64_t* gemm1_tasks);

@@ -39,7 +39,7 @@ def test_slab_loop_holds_nothing_but_the_schedule():
     instruction, a spill or an accumulator move there would sit between a ds_read and the wait that covers it, or
     behind an MFMA still in flight."""
     text = _assembly()
-    loops = 0
+    loops, half_loops = 0, 0
     for kernel in re.split(r"\n(?=_Z\w+:)", text):
         lines = kernel.split("\n")
         labels = {m.group(1): k for k, l in enumerate(lines) for m in [re.match(r"^(\.LBB\d+_\d+):", l)] if m}
@@ -49,15 +49,19 @@ def test_slab_loop_holds_nothing_but_the_schedule():
                 continue
             body = [x.strip() for x in lines[labels[m.group(1)]:k + 1]]
             body = [x for x in body if x and not x.startswith((";", "."))]
-            if sum(x.startswith(MFMA) for x in body) != 256 or len(body) > 1000:
+            mfmas = sum(x.startswith(MFMA) for x in body)
+            if mfmas not in (256, 128) or len(body) > 1000:
                 continue
-            loops += 1
+            full = mfmas == 256            # two slabs of the 128 x 128 wavefront tile, or of the 128 x 64 one
+            loops += full
+            half_loops += not full
             other = [x for x in body if x.startswith(("v_", "scratch_", "global_", "flat_")) and not x.startswith(MFMA)]
             assert not other, "unexpected instructions in the slab loop: %s" % other[:5]
-            assert sum(x.startswith("ds_read_b128") for x in body) == 64
-            assert sum(x.startswith("buffer_load_dwordx4") for x in body) == 32
+            assert sum(x.startswith("ds_read_b128") for x in body) == (64 if full else 48)
+            assert sum(x.startswith("buffer_load_dwordx4") for x in body) == (32 if full else 24)
             assert sum(x.startswith("s_barrier") for x in body) == 4
     assert loops >= 8, "expected the slab loop in the two-launch, both queue and the plain-GEMM kernels, bf16 and fp16, found %d" % loops
+    assert half_loops >= 8, "expected the half-width slab loop in the two-launch and queue kernels, alone and beside the full one, bf16 and fp16, found %d" % half_loops
 
 
 @pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")

@@ -214,6 +214,29 @@ def test_large_tile_and_queue_groups(moe, name, monkeypatch):
         assert np.array_equal(got["out"], first), ("early", groups)
 
 
+@pytest.mark.parametrize("name", sorted(n for n, c in LARGE_TILE.items()
+                                        if c.H % 256 == 0 and c.I % (128 if c.act == ob.ACT_SWIGLU else 256) == 0))
+def test_half_height_tile(moe, name, monkeypatch):
+    """The 128 x 256 tile as the tile of the whole layer (MOE355_TILE=2) and as the tile of the short last row blocks
+    only (3): every output element is accumulated by the same MFMA sequence over K as in the 256 x 256 tile, so all
+    three must agree bit for bit, in both FFN modes, and match the oracle."""
+    cfg = LARGE_TILE[name]
+    inp = ob.make_inputs(cfg, seed=5, with_bias="bias" in name)
+    want = ob.forward(cfg, inp)
+    first = None
+    for tile, rows in (("1", 256), ("2", 128), ("3", 256)):
+        monkeypatch.setenv("MOE355_TILE", tile)
+        for mode in (FFN_TILED, FFN_PERSISTENT):
+            got = run_layer(moe, cfg, inp, mode)
+            check_routing(got, want)
+            assert got["plan"]["block_rows"] == rows
+            if first is None:
+                first = got["out"]
+                assert max_rel_err(ob.to_f32(first, cfg.act_dtype), ob.to_f32(want["out"], cfg.act_dtype)) <= OUT_TOL[cfg.dtype]
+            else:
+                assert np.array_equal(got["out"], first), (tile, mode)
+
+
 def test_two_handles_on_two_streams_from_two_threads(moe):
     """The boundary promises that handles are independent: two layers, each driven from its own host thread on its
     own (default-priority) stream, overlap freely and must reproduce what each computes alone."""

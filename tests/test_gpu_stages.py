@@ -63,6 +63,26 @@ def test_gemm_vs_oracle(moe, dtype, M, N, K, act):
     assert np.abs(got_nb - want_nb).max() <= tol * max(np.abs(want_nb).max(), 1e-3)
 
 
+@pytest.mark.parametrize("dtype", [ob.BF16, ob.F16])
+@pytest.mark.parametrize("M,N,K", [(70, 512, 256), (128, 256, 128), (300, 768, 384)])
+def test_gemm_hand_ordered_tiles_agree(moe, dtype, M, N, K, monkeypatch):
+    """The 256 x 256 and the 128 x 256 hand-ordered tiles forced on a plain GEMM (MOE355_DENSE_TILE): same MFMA
+    sequence over K per output element, so bit-identical to each other, and within tolerance of the oracle."""
+    rng = np.random.default_rng(M + N + K)
+    kind = KIND[dtype]
+    A = ob.from_f32(rng.standard_normal((M, K)).astype(np.float32), dtype)
+    B = ob.from_f32((rng.standard_normal((N, K)) * 0.1).astype(np.float32), dtype)
+    bias = ob.from_f32(rng.standard_normal(N).astype(np.float32), dtype)
+    want = ob.to_f32(ob.gemm_bias_act(A, B, bias, dtype, ob.ACT_GELU), dtype)
+    outs = []
+    for tile in ("1", "2"):
+        monkeypatch.setenv("MOE355_DENSE_TILE", tile)
+        outs.append(from_device(moe.gemm_bias_act(to_device(A, kind), to_device(B, kind), to_device(bias, kind), ob.ACT_GELU)))
+    assert np.array_equal(outs[0], outs[1])
+    tol = {ob.BF16: 1e-2, ob.F16: 1.25e-3}[dtype]
+    assert np.abs(ob.to_f32(outs[1], dtype) - want).max() <= tol * np.abs(want).max()
+
+
 @pytest.mark.parametrize("act", [ob.ACT_RELU, ob.ACT_GELU, ob.ACT_NONE])
 @pytest.mark.parametrize("M,N,K", [(1041, 1024, 128), (1280, 1280, 384), (1025, 1536, 1024)])
 def test_gemm_large_tile_vs_oracle(moe, M, N, K, act):

@@ -52,7 +52,7 @@ def stats(samples):
             "min": round(min(samples), 5), "n": len(samples)}
 
 
-def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False):
+def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False, balanced_routing=False):
     """Runs one workload; returns (result dict, layer, device operands, output tensor, routing tensors)."""
     import torch
     import cuplayground_amd as moe
@@ -62,6 +62,8 @@ def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False):
     c = w.config
     layer = moe.MoELayer(c, ffn_mode=ffn_mode)
     dev = wl.make_device_inputs(w, seed)
+    if balanced_routing:
+        wl.balance_routing(c, dev)
     out = torch.empty(c.tokens, c.hidden_size, dtype=layer.act_dtype, device="cuda")
     if calibrate_copy:
         src = torch.zeros(1 << 30, dtype=torch.uint8, device="cuda")
@@ -133,6 +135,11 @@ def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False):
         "stage_ms_median": {k: round(statistics.median(v[-steps:]), 4) for k, v in samples.items()},
         "ffn_mode": layer.ffn_mode, "block_rows": layer.plan["block_rows"],
         "persistent_blocks": layer.arch["persistent_blocks"], "kept_assignments": kept, "tile_tasks": [tasks0, tasks1],
+        # row blocks the FFN ran against the row blocks its rows would fill (the rest is padding of ragged last blocks)
+        "row_blocks": int(sum((int(n) + layer.plan["block_rows"] - 1) // layer.plan["block_rows"] for n in cnt)),
+        "row_blocks_full": round(kept / layer.plan["block_rows"], 2),
+        # entry/exit stamps of the queue kernel's workgroups in the last call (microseconds)
+        "queue_balance": {k: round(v, 1) for k, v in layer.queue_balance().items()} if queue else None,
         "roofline": roof,
     }
     return res, layer, dev, out, routing
@@ -260,6 +267,9 @@ def main():
     ap.add_argument("--ffn-mode", type=int, default=0, help="0 auto, 1 tiled (two launches), 2 persistent queue")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample (0 = skip)")
     ap.add_argument("--seed", type=int, default=42)
+    ap.add_argument("--balanced-routing", action="store_true",
+                    help="experiment: replace the router's inputs so that every expert receives exactly S*k/E rows "
+                         "(no ragged last row blocks); the FFN arithmetic is unchanged")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy (a known-size reference for HBM byte counters)")
     args = ap.parse_args()
@@ -276,7 +286,7 @@ def main():
     moe.load_library()
     main_w = wl.WORKLOADS[args.workload]
     res, layer, dev, out, routing = measure(args.workload, args.steps, args.warmup, args.seed, args.ffn_mode,
-                                            args.calibrate_copy)
+                                            args.calibrate_copy, args.balanced_routing)
     arch = layer.arch
     # ceilings measured on this box in this run (the published peaks assume the maximum clock)
     peaks = moe.measured_peaks()
@@ -314,7 +324,9 @@ def main():
         "vs_baseline": None, "dtype": dtype[main_w.config.torch_dtype], "data": "synthetic",
         "config": {"workload": res["workload"], "ffn_mode": res["ffn_mode"], "block_rows": res["block_rows"],
                    "persistent_blocks": res["persistent_blocks"], "kept_assignments": res["kept_assignments"],
-                   "tile_tasks": res["tile_tasks"]},
+                   "tile_tasks": res["tile_tasks"], "row_blocks": res["row_blocks"],
+                   "row_blocks_full": res["row_blocks_full"], "balanced_routing": bool(args.balanced_routing)},
+        "queue_balance": res["queue_balance"],
         "tflops": res["tflops"],
         "stage_ms": res["stage_ms"], "stage_ms_median": res["stage_ms_median"],
         "device": {"name": arch["name"], "compute_units": arch["compute_units"], "xcds": arch["xcds"],

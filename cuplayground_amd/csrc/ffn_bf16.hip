@@ -1229,16 +1229,17 @@ static bool large_tile_ok(int64_t pairs, int H, int I, bool swiglu) {
 }
 
 // Tile of a layer: 0 = 128 x 128, 1 = 256 x 256, 2 = 128 x 256, 3 = 256 x 256 with the 128 x 256 tile for the row
-// blocks of at most 128 rows.
+// blocks of at most 128 rows.  1 where its conditions hold and the layer has enough rows, else 0; 2 and 3 are tuning
+// knobs (MOE355_TILE).
 //
-// Measured (FFN stage, same box, alternating runs): the 128 x 256 tile reaches 93 % of the 256 x 256 tile's rate on
-// a plain 4096 x 8192 x 4096 GEMM, but as the tile of a whole layer it loses to it everywhere (Mixtral shape 5.45
-// against 4.33 ms, 16 experts of 512 rows 0.209 against 0.187 ms, 64 small experts 0.72 against 0.59 ms): twice the
-// tasks, each with the same 12 us between two slab loops.  For short last blocks only it gains 1-2 % with many small
-// experts and loses 2 % on the Mixtral shape -- there a short block's task runs through K faster than the eight full
-// blocks that share its weight tile, drops out of their lockstep and fetches its weights past the L2 on its own
-// (with a routing that leaves no partial blocks both kernels take the same time).  So 3 is chosen below 1024 rows per
-// expert, 1 above, and 2 is a tuning knob only.
+// Measured (FFN stage, one box, alternating runs): the 128 x 256 tile reaches 93 % of the 256 x 256 tile's rate on a
+// plain 4096 x 8192 x 4096 GEMM, but as the tile of a whole layer it loses everywhere (Mixtral shape 5.48 against
+// 4.26 ms, 16 experts of 512 rows 0.209 against 0.187 ms, 64 small experts 0.72 against 0.59 ms): twice the tasks,
+// each with the same 12 us between two slab loops.  As the tile of short last blocks only it is no better either
+// (Mixtral shape 4.38 against 4.26 ms, 16 experts 0.198 against 0.190 ms, 64 small experts 0.590 against 0.592 ms):
+// such a task runs through K faster than the full blocks that share its weight tile, drops out of their lockstep
+// and fetches its weights past the L2 on its own, with half the time per slab to hide that latency in (with a
+// routing that leaves no partial blocks both kernels take the same time).
 int bf16_tile(int64_t pairs, int experts, int H, int I, int swiglu) {
     if (!large_tile_ok(pairs, H, I, swiglu != 0)) return 0;
     const int up_columns = swiglu ? 2 * I : I;
@@ -1253,8 +1254,7 @@ int bf16_tile(int64_t pairs, int experts, int H, int I, int swiglu) {
     const int64_t per_expert = pairs / (experts > 0 ? experts : 1);
     if (per_expert < 256) return 0;
     const int64_t tasks = (pairs / 256) * ((up_columns + Tile256::BN - 1) / Tile256::BN);
-    if (tasks < 256) return 0;
-    return per_expert < 1024 ? 3 : 1;
+    return tasks >= 256 ? 1 : 0;
 }
 int bf16_block_m(int tile) { return tile == 1 || tile == 3 ? 256 : 128; }
 int bf16_block_n0(int tile) { return tile == 0 ? SmallPlan::T0::BN : 256; }

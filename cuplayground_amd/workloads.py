@@ -86,6 +86,23 @@ def make_device_inputs(w: Workload, seed: int = 42) -> dict:
     return d
 
 
+def balance_routing(c: api.MoEConfig, dev: dict) -> None:
+    """Rewrites the router's inputs in place so that token t picks experts t, t+1, .. t+k-1 (mod E): every expert
+    receives exactly S*k/E rows.  Only the first E columns of x and the gate weights change (E of H columns), so the
+    FFN does the same arithmetic on (almost) the same data; used to measure what ragged last row blocks cost."""
+    import torch
+    E, k = c.num_experts, c.expert_top_k
+    x, gw = dev["x"], dev["gate_w"]
+    gw.zero_()
+    x[:, :E] = 0
+    t = torch.arange(c.tokens, device=x.device)
+    for r in range(k):
+        x[t, (t + r) % E] = 40.0
+    gw[:, :E] = torch.eye(E, device=x.device, dtype=gw.dtype)
+    if dev.get("gate_bias") is not None:
+        dev["gate_bias"].zero_()
+
+
 def ffn_flops(c: api.MoEConfig, kept_rows: int) -> float:
     """2 * g * H * I per kept (token, expert) row; g = 3 matrices for SwiGLU, 2 otherwise."""
     g = 3 if c.hidden_act == api.ACT_SWIGLU else 2

@@ -7,26 +7,10 @@
 //   out[t,:] = sum over ranks r (ascending) of topk_w[t,r] * y[pair_row[t,r], :]
 // accumulated in fp32 and rounded once; pairs with pair_row < 0 (dropped) contribute nothing.  With k = 1
 // and unit weights it is exactly the reference's single-mode copy.
-#include "moe_internal.hpp"
+#include "combine_core.hpp"
 
 namespace moe355 {
 namespace {
-
-__device__ __forceinline__ uint32_t pack16x2(float lo, float hi, bf16_s) {
-    // round to nearest even, the rounding the oracle and torch use for bf16
-    uint32_t a = __float_as_uint(lo), b = __float_as_uint(hi);
-    a += 0x7FFFu + ((a >> 16) & 1u);
-    b += 0x7FFFu + ((b >> 16) & 1u);
-    return (a >> 16) | (b & 0xFFFF0000u);
-}
-__device__ __forceinline__ uint32_t pack16x2(float lo, float hi, f16_s) {
-    const uint32_t a = __builtin_bit_cast(uint16_t, (_Float16)lo), b = __builtin_bit_cast(uint16_t, (_Float16)hi);   // RNE
-    return a | (b << 16);
-}
-__device__ __forceinline__ float lo16(uint32_t w, bf16_s) { return __uint_as_float(w << 16); }
-__device__ __forceinline__ float hi16(uint32_t w, bf16_s) { return __uint_as_float(w & 0xFFFF0000u); }
-__device__ __forceinline__ float lo16(uint32_t w, f16_s) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xFFFFu)); }
-__device__ __forceinline__ float hi16(uint32_t w, f16_s) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16)); }
 
 // grid = (S, ceil(H / (256*8))) for the 16-bit types; each thread owns 8 consecutive columns
 template <typename T16>
@@ -37,27 +21,7 @@ __global__ __launch_bounds__(256) void combine_16_kernel(const uint16_t* __restr
     const int t = blockIdx.x;
     const int c = (blockIdx.y * 256 + threadIdx.x) * 8;
     if (c >= H) return;
-    float acc[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
-    for (int r = 0; r < k; ++r) {
-        const int row = pair_row[(size_t)t * k + r];
-        if (row < 0) continue;
-        const float w = topk_w[(size_t)t * k + r];
-        const uint4 v = *reinterpret_cast<const uint4*>(y + (size_t)row * H + c);
-        const uint32_t u[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            acc[2 * i] = acc[2 * i] + w * lo16(u[i], T16{});
-            acc[2 * i + 1] = acc[2 * i + 1] + w * hi16(u[i], T16{});
-        }
-    }
-    uint4 o;
-    o.x = pack16x2(acc[0], acc[1], T16{});
-    o.y = pack16x2(acc[2], acc[3], T16{});
-    o.z = pack16x2(acc[4], acc[5], T16{});
-    o.w = pack16x2(acc[6], acc[7], T16{});
-    *reinterpret_cast<uint4*>(out + (size_t)t * H + c) = o;
+    combine_token_16<T16, false>(y, pair_row, topk_w, t, k, H, c, out);
 }
 
 __global__ __launch_bounds__(256) void combine_f32_kernel(const float* __restrict__ y,
@@ -67,18 +31,7 @@ __global__ __launch_bounds__(256) void combine_f32_kernel(const float* __restric
     const int t = blockIdx.x;
     const int c = (blockIdx.y * 256 + threadIdx.x) * 4;
     if (c >= H) return;
-    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int r = 0; r < k; ++r) {
-        const int row = pair_row[(size_t)t * k + r];
-        if (row < 0) continue;
-        const float w = topk_w[(size_t)t * k + r];
-        const float4 v = *reinterpret_cast<const float4*>(y + (size_t)row * H + c);
-        acc.x = acc.x + w * v.x;
-        acc.y = acc.y + w * v.y;
-        acc.z = acc.z + w * v.z;
-        acc.w = acc.w + w * v.w;
-    }
-    *reinterpret_cast<float4*>(out + (size_t)t * H + c) = acc;
+    combine_token_f32<false>(y, pair_row, topk_w, t, k, H, c, out);
 }
 
 }  // namespace

@@ -836,7 +836,7 @@ __device__ __forceinline__ TaskPtrs resolve(const FfnArgs& a, const Task& t, boo
         p.n0 = t.ntile * T::BN;
         p.act = MOE_ACT_NONE;
         p.swiglu = false;
-        p.publish = false;
+        p.publish = publish;
     }
     p.rows = t.rows;
     p.a_extent = t.phase == 0 ? a.x_bytes : a.h_bytes;
@@ -892,9 +892,13 @@ __device__ __forceinline__ void plan_tile(const FfnArgs& a, const Task& t, bool 
 template <class P>
 __global__ __launch_bounds__(P::THREADS) void ffn_tiled_kernel(FfnArgs a, int phase) {
     extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ int s_list[1 + P::T0::BM];
+    using ET = typename std::conditional<P::T0::F16, f16_s, bf16_s>::type;
+    if (phase == 0) zero_unrouted_rows(a, 2);
     Task t;
     if (!tiled_task(a, phase, blockIdx.x, t)) return;
-    plan_tile<P>(a, t, false, smem);
+    plan_tile<P>(a, t, phase == 1 && a.arrive, smem);       // rows another workgroup may combine go out write-through
+    if (phase == 1 && a.arrive) combine_arrivals<ET>(combine_args(a), t.row0, t.rows, t.ntile, t.ntile * P::T1::BN, P::T1::BN, s_list);
 }
 
 // The kernel's argument block, read again from the kernel-argument segment through a pointer the compiler cannot see
@@ -912,8 +916,11 @@ template <class P>
 __global__ __launch_bounds__(P::THREADS) void ffn_persistent_kernel(FfnArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ int s_task, s_ok;
+    __shared__ int s_list[1 + P::T0::BM];
+    using ET = typename std::conditional<P::T0::F16, f16_s, bf16_s>::type;
     queue_kernel_entry();
     queue_clock_stamp(kernel_args_again().wg_clock, 0);
+    zero_unrouted_rows(kernel_args_again(), 2);
     const int ids = a.q->ids_queue;
     const int nseg = a.q->nseg;
     const int nnt0 = a.seg_phase0[0].nnt;
@@ -926,8 +933,10 @@ __global__ __launch_bounds__(P::THREADS) void ffn_persistent_kernel(FfnArgs a) {
             poison_tile((uint16_t*)a.y + (int64_t)t.row0 * a.H, t.rows, a.H, t.ntile * P::T1::BN, P::T1::BN, 2);
             t.rows = 0;
         }
-        plan_tile<P>(a, t, t.phase == 0, smem);
+        plan_tile<P>(a, t, t.phase == 0 || a.arrive, smem);
         if (t.phase == 0) signal_phase0_done(a.done0, t.mtile);
+        else if (a.arrive)   // the row count from the table: a tile whose wait expired runs with none, and still arrives
+            combine_arrivals<ET>(combine_args(kernel_args_again()), t.row0, a.mtiles[t.mtile].rows, t.ntile, t.ntile * P::T1::BN, P::T1::BN, s_list);
     }
     queue_clock_stamp(kernel_args_again().wg_clock, 1);
 }
@@ -956,8 +965,11 @@ __global__ __launch_bounds__(P::THREADS) void ffn_persistent_ring_kernel(FfnArgs
     static_assert(std::is_same<typename P::T0, typename P::T1>::value && T::RING, "the hand-ordered tile for both projections");
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ int s_task, s_ok, s_next[2];
+    __shared__ int s_list[1 + T::BM];
+    using ET = typename std::conditional<T::F16, f16_s, bf16_s>::type;
     queue_kernel_entry();
     queue_clock_stamp(kernel_args_again().wg_clock, 0);
+    zero_unrouted_rows(kernel_args_again(), 2);
     int ids, nseg, nnt0, groups;
     {
         const FfnArgs& a = kernel_args_again();
@@ -1038,12 +1050,13 @@ __global__ __launch_bounds__(P::THREADS) void ffn_persistent_ring_kernel(FfnArgs
             }
         };
         if (active) {
-            epilogue_full_n<T>(resolve<T>(a, as_task(), ph == 0), smem, acc, token_loads);
+            epilogue_full_n<T>(resolve<T>(a, as_task(), ph == 0 || a.arrive), smem, acc, token_loads);
         } else {
 #pragma unroll
             for (int i = 0; i < 8; ++i) token_loads(i);
         }
         if (ph == 0) signal_phase0_done(a.done0, mt);
+        else if (a.arrive) combine_arrivals<ET>(combine_args(a), row0, a.mtiles[mt].rows, nt, nt * T::BN, T::BN, s_list);
         if (reserve && nid < ids && n_valid) {   // the reserved task is the next one
             ph = n_ph; ex = n_ex; mt = n_mt; nt = n_nt; row0 = n_row0; rows = n_rows;
             cur.last_id = nid;

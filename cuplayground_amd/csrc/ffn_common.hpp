@@ -13,7 +13,7 @@
 // and launching at least one workgroup per queue.  The wait is bounded all the same.
 #pragma once
 
-#include "moe_internal.hpp"
+#include "combine_core.hpp"
 
 namespace moe355 {
 
@@ -195,13 +195,92 @@ __device__ __noinline__ int wait_phase0_done(const int32_t* done0, int mtile, in
 // Fills rows [0, rows) x columns [n0, min(n0 + ncols, N)) of a row-major output block with NaN (elem_bytes 2: bf16
 // 0x7FC0, 4: fp32 0x7FC00000).  Run by the whole workgroup in place of a tile whose inputs never became ready.
 __device__ __noinline__ void poison_tile(void* c_base, int rows, int N, int n0, int ncols, int elem_bytes) {
-    const int n1 = min(n0 + ncols, N), w = n1 - n0;
+    const int n1 = min(n0 + ncols, N);
+    // 4-byte agent-scope stores (two bf16 / fp16 NaNs or one fp32 NaN): the combine may read these rows from another
+    // XCD within this launch.  Column counts are even (H and I are multiples of 64).
+    const int per = elem_bytes == 2 ? 2 : 1, w = (n1 - n0) / per;
     if (w <= 0) return;
+    const uint32_t nan = elem_bytes == 2 ? 0x7FC07FC0u : 0x7FC00000u;
     for (int i = threadIdx.x; i < rows * w; i += blockDim.x) {
-        const int r = i / w, c = n0 + i % w;
-        const int64_t at = (int64_t)r * N + c;
-        if (elem_bytes == 2) reinterpret_cast<uint16_t*>(c_base)[at] = 0x7FC0u;
-        else reinterpret_cast<uint32_t*>(c_base)[at] = 0x7FC00000u;
+        const int r = i / w, c = n0 + (i % w) * per;
+        publish4(static_cast<char*>(c_base) + ((int64_t)r * N + c) * elem_bytes, nan);
+    }
+}
+
+// ---- Combine inside the FFN kernels ----
+// The reference applies its combine to a finished tile while the tile is still on chip (combine.cuh:105-188: vector
+// copy for top-1, unordered vector atomic adds for top-k).  Here the result must not depend on who finishes first, so
+// the FFN kernels keep writing the expert rows y and count arrivals instead: when a down-projection tile is stored,
+// one thread per row adds one to arrive[token, column tile]; the workgroup whose increment completes a token -- all
+// of the token's kept (token, expert) rows now hold this column tile -- combines that token's columns right there, in
+// rank order, with the very function the separate combine kernel uses.  Which workgroup does it varies, what it
+// computes does not.
+// Visibility: y is written with agent-scope (write-through) stores; every wavefront waits for its stores, the
+// workgroup meets at a barrier, then come the increments; the combining reads are agent-scope loads issued behind
+// the increment that returned the completing count.  A line of y is written once per launch, entirely by one tile.
+struct CombineArgs {
+    int32_t* arrive;
+    const int32_t* token_indices;
+    const int32_t* pair_row;
+    const float* topk_w;
+    const void* y;
+    void* out;
+    int32_t k, nnt1, H, drop;
+};
+__device__ __forceinline__ CombineArgs combine_args(const FfnArgs& a) {
+    return CombineArgs{a.arrive, a.token_indices, a.pair_row, a.topk_w, a.y, a.out, a.k, a.nnt1, a.H, a.drop};
+}
+
+// Called by every thread of the workgroup behind the stores of the down-projection tile rows [row0, row0 + rows) x
+// columns [n0, n0 + ncols).  ET: bf16_s, f16_s or float.  s_list: 1 + (row-block height) ints of LDS.
+template <class ET>
+__device__ __noinline__ void combine_arrivals(CombineArgs c, int row0, int rows, int ntile, int n0, int ncols,
+                                              int* s_list) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // this wavefront's stores of y have reached memory
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    if (threadIdx.x == 0) s_list[0] = 0;
+    __syncthreads();
+    for (int r = threadIdx.x; r < rows; r += blockDim.x) {
+        const int t = c.token_indices[row0 + r];
+        int kept = c.k;
+        if (c.drop) {
+            kept = 0;
+            for (int q = 0; q < c.k; ++q) kept += c.pair_row[(size_t)t * c.k + q] >= 0;
+        }
+        const int before = __hip_atomic_fetch_add(c.arrive + (size_t)t * c.nnt1 + ntile, 1, __ATOMIC_RELAXED,
+                                                  __HIP_MEMORY_SCOPE_AGENT);
+        if (before == kept - 1) s_list[1 + atomicAdd(&s_list[0], 1)] = t;
+    }
+    __syncthreads();
+    const int n = s_list[0];
+    constexpr int kPerThread = sizeof(ET) == 4 ? 4 : 8;   // elements in 16 bytes
+    const int lanes = ncols / kPerThread;                 // threads that share a token
+    const int per_pass = blockDim.x / lanes;
+    const int sub = threadIdx.x / lanes, col = n0 + (threadIdx.x % lanes) * kPerThread;
+    if (sub < per_pass && col < c.H) {
+        for (int i = sub; i < n; i += per_pass) {
+            const int t = s_list[1 + i];
+            if constexpr (sizeof(ET) == 4)
+                combine_token_f32<true>((const float*)c.y, c.pair_row, c.topk_w, t, c.k, c.H, col, (float*)c.out);
+            else
+                combine_token_16<ET, true>((const uint16_t*)c.y, c.pair_row, c.topk_w, t, c.k, c.H, col, (uint16_t*)c.out);
+        }
+    }
+    __syncthreads();                                      // the list may be rewritten by the next tile
+}
+
+// Tokens that lost every pair to the capacity limit have no tile that would complete them: their output rows are
+// zeroed here, one wavefront per token, by the workgroups of the launch that runs the up projection.
+__device__ __forceinline__ void zero_unrouted_rows(const FfnArgs& a, int elem_bytes) {
+    if (!a.arrive || !a.drop) return;
+    const int lane = threadIdx.x & 63;
+    const int waves = (int)(gridDim.x * blockDim.x) >> 6, wave = (int)(blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const int row_vec = a.H * elem_bytes / 16;
+    for (int t = wave; t < a.S; t += waves) {
+        const bool kept = lane < a.k && a.pair_row[(size_t)t * a.k + lane] >= 0;
+        if (__ballot(kept) != 0ull) continue;
+        uint4* row = reinterpret_cast<uint4*>(static_cast<char*>(a.out) + (size_t)t * a.H * elem_bytes);
+        for (int i = lane; i < row_vec; i += 64) row[i] = uint4{0u, 0u, 0u, 0u};
     }
 }
 

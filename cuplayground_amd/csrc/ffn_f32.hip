@@ -137,7 +137,7 @@ __device__ __forceinline__ TaskPtrsF resolve_f32(const FfnArgs& a, const Task& t
         p.n0 = t.ntile * FBN;
         p.act = MOE_ACT_NONE;
         p.swiglu = false;
-        p.publish = false;
+        p.publish = publish;
     }
     p.rows = t.rows;
     return p;
@@ -147,17 +147,22 @@ __global__ __launch_bounds__(256) void ffn_tiled_f32_kernel(FfnArgs a, int phase
     __shared__ __align__(16) float As[FBK][FBM + FPAD];
     __shared__ __align__(16) float Bs[FBK][FBN + FPAD];
     Task t;
+    __shared__ int s_list[1 + FBM];
+    if (phase == 0) zero_unrouted_rows(a, 4);
     if (!tiled_task(a, phase, blockIdx.x, t)) return;
-    const TaskPtrsF p = resolve_f32(a, t, false);
+    const TaskPtrsF p = resolve_f32(a, t, phase == 1 && a.arrive);
     gemm_tile_f32(p, As, Bs);
+    if (phase == 1 && a.arrive) combine_arrivals<float>(combine_args(a), t.row0, t.rows, t.ntile, p.n0, FBN, s_list);
 }
 
 __global__ __launch_bounds__(256) void ffn_persistent_f32_kernel(FfnArgs a) {
     __shared__ __align__(16) float As[FBK][FBM + FPAD];
     __shared__ __align__(16) float Bs[FBK][FBN + FPAD];
     __shared__ int s_task, s_ok;
+    __shared__ int s_list[1 + FBM];
     queue_kernel_entry();
     queue_clock_stamp(a.wg_clock, 0);
+    zero_unrouted_rows(a, 4);
     const int ids = a.q->ids_queue;
     const int nseg = a.q->nseg;
     const int nnt0 = a.seg_phase0[0].nnt;
@@ -166,10 +171,11 @@ __global__ __launch_bounds__(256) void ffn_persistent_f32_kernel(FfnArgs a) {
     while (next_task(a, cur, &s_task, ids, nseg, nnt0, t)) {
         int ok = 1;
         if (t.phase == 1) ok = wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q, a.host_stall, &s_ok);
-        const TaskPtrsF p = resolve_f32(a, t, true);
+        const TaskPtrsF p = resolve_f32(a, t, t.phase == 0 || a.arrive);
         if (ok) gemm_tile_f32(p, As, Bs);
         else poison_tile(p.c_base, p.rows, p.N, p.n0, FBN, 4);
         if (t.phase == 0) signal_phase0_done(a.done0, t.mtile);
+        else if (a.arrive) combine_arrivals<float>(combine_args(a), t.row0, t.rows, t.ntile, p.n0, FBN, s_list);
     }
     queue_clock_stamp(a.wg_clock, 1);
 }

@@ -171,14 +171,15 @@ __device__ __forceinline__ void fp8_tile(const Fp8Task& t, float* red) {
             uint2 st;
             st.x = pack2_bf16(o[0], o[1]);
             st.y = pack2_bf16(o[2], o[3]);
-            *reinterpret_cast<uint2*>(crow + col) = st;
+            if (t.publish) publish8(crow + col, st.x, st.y);
+            else *reinterpret_cast<uint2*>(crow + col) = st;
         }
     }
 }
 
 __device__ __forceinline__ Fp8Task resolve_fp8(const FfnArgs& a, const Task& t, int sub, bool publish) {
     Fp8Task p;
-    p.publish = publish && t.phase == 0;
+    p.publish = publish;
     const int64_t HI = (int64_t)a.H * a.I;
     const int kbH = a.H >> 7, kbI = a.I >> 7;
     p.phase = t.phase;
@@ -217,19 +218,24 @@ __device__ __forceinline__ Fp8Task resolve_fp8(const FfnArgs& a, const Task& t, 
 
 __global__ __launch_bounds__(256) void ffn_tiled_fp8_kernel(FfnArgs a, int phase) {
     __shared__ float red[QWAVES * QGROUPS * 4 * 64];
+    __shared__ int s_list[1 + QBM];
+    if (phase == 0) zero_unrouted_rows(a, 2);
     Task t;
     if (!tiled_task(a, phase, blockIdx.x, t)) return;
     for (int sub = 0; sub < QSUB; ++sub) {
-        const Fp8Task p = resolve_fp8(a, t, sub, false);
+        const Fp8Task p = resolve_fp8(a, t, sub, phase == 1 && a.arrive);
         if (p.c0 < p.N) fp8_tile(p, red);
     }
+    if (phase == 1 && a.arrive) combine_arrivals<bf16_s>(combine_args(a), t.row0, t.rows, t.ntile, t.ntile * QSUB * QN1, QSUB * QN1, s_list);
 }
 
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void ffn_persistent_fp8_kernel(FfnArgs a) {
     __shared__ float red[QWAVES * QGROUPS * 4 * 64];
     __shared__ int s_task, s_ok;
+    __shared__ int s_list[1 + QBM];
     queue_kernel_entry();
     queue_clock_stamp(a.wg_clock, 0);
+    zero_unrouted_rows(a, 2);
     const int ids = a.q->ids_queue;
     const int nseg = a.q->nseg;
     const int nnt0 = a.seg_phase0[0].nnt;
@@ -239,12 +245,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         int ok = 1;
         if (t.phase == 1) ok = wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q, a.host_stall, &s_ok);
         for (int sub = 0; sub < QSUB; ++sub) {
-            const Fp8Task p = resolve_fp8(a, t, sub, true);
+            const Fp8Task p = resolve_fp8(a, t, sub, t.phase == 0 || a.arrive);
             if (p.c0 >= p.N) continue;
             if (ok) fp8_tile(p, red);
             else poison_tile(p.c_base, p.rows, p.N, p.c0, QN1, 2);
         }
         if (t.phase == 0) signal_phase0_done(a.done0, t.mtile);
+        else if (a.arrive) combine_arrivals<bf16_s>(combine_args(a), t.row0, t.rows, t.ntile, t.ntile * QSUB * QN1, QSUB * QN1, s_list);
     }
     queue_clock_stamp(a.wg_clock, 1);
 }

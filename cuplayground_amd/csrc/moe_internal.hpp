@@ -90,6 +90,13 @@ struct FfnArgs {
     int32_t groups;             // queue groups the schedule was built for
     uint32_t x_bytes, h_bytes, w_bytes;   // extents of x, h and one weight matrix (meaningful below 4 GiB)
     int64_t* wg_clock;          // queue kernels: [2 * workgroup] constant-rate clock at entry, [2 * workgroup + 1] at exit
+    // Combine inside the FFN kernels (null `arrive`: the separate combine launch is used instead).
+    int32_t* arrive;            // [S, nnt1]: finished down-projection tiles per (token, column tile)
+    const int32_t* pair_row;    // [S, k] packed row of every (token, rank), -1 when dropped
+    const float* topk_w;        // [S, k]
+    void* out;                  // [S, H] in the activation type
+    int32_t S, k, nnt1;
+    int32_t drop;               // tokens may have lost every pair: their output rows are zeroed at kernel entry
 };
 constexpr int kMaxQueueWorkgroups = 4096;   // workgroups of a queue kernel that get a slot in wg_clock
 
@@ -108,6 +115,7 @@ struct RouteArgs {
     Segment* seg_queue;
     QueueState* q;
     int32_t* done0;
+    int32_t* arrive;            // [S, nnt1] arrival counters of the fused combine (null: not used), cleared here
     int32_t S, k, E, A, nblk;
     int32_t drop;
     int32_t capacity;

@@ -58,8 +58,16 @@ __device__ __forceinline__ void route_count_body(const RouteArgs& a, int blk, in
     }
 }
 
+// The arrival counters of the fused combine start every call at zero.
+__device__ __forceinline__ void clear_arrivals(const RouteArgs& a, int first, int stride) {
+    if (!a.arrive) return;
+    const int n = a.S * a.nnt1;
+    for (int i = first; i < n; i += stride) a.arrive[i] = 0;
+}
+
 __global__ __launch_bounds__(kRouteBlock) void route_count_kernel(RouteArgs a) {
     __shared__ int wcount[kRouteBlock / kWave][kMaxExperts];
+    clear_arrivals(a, blockIdx.x * kRouteBlock + threadIdx.x, gridDim.x * kRouteBlock);
     route_count_body(a, blockIdx.x, threadIdx.x, wcount, true);
 }
 
@@ -248,6 +256,7 @@ __global__ __launch_bounds__(kMaxExperts) void router_small_kernel(RouteArgs a) 
     __shared__ int wcount[kMaxExperts / kRouteBlock][kRouteBlock / kWave][kMaxExperts];
     __shared__ ScanShared sh;
     const int tid = threadIdx.x;
+    clear_arrivals(a, tid, kMaxExperts);
     constexpr int kChunksAtOnce = kMaxExperts / kRouteBlock;
     for (int b0 = 0; b0 < a.nblk; b0 += kChunksAtOnce) {      // uniform trip count: every thread meets every barrier
         const int blk = b0 + tid / kRouteBlock;

@@ -214,6 +214,31 @@ def test_large_tile_and_queue_groups(moe, name, monkeypatch):
         assert np.array_equal(got["out"], first), ("early", groups)
 
 
+@pytest.mark.parametrize("name", ["bf16_gelu_ragged", "bf16_swiglu_skew", "f32_swiglu_ragged", "fp8_many_rows_bias",
+                                  "fp16_swiglu_skew_bias", "tf32_gelu_ragged", "capacity_one", "many_experts_bias",
+                                  "all_experts_selected", "one_token"])
+def test_combine_inside_the_ffn_kernels_changes_no_bit(moe, name, monkeypatch):
+    """With MOE355_FUSED_COMBINE=1 a token is combined by the FFN workgroup that stores its last expert row; by default
+    the combine is a launch of its own behind the FFN stage.  Same function, same rank order: the outputs must be
+    identical in every bit, in both FFN modes, including the all-zero rows of tokens that lost every pair to the
+    capacity limit, and over repeated calls on one handle (the arrival counters are cleared by every call)."""
+    import torch
+    cfg = RAGGED[name]
+    inp = ob.make_inputs(cfg, seed=3, with_bias="bias" in name)
+    separate = run_layer(moe, cfg, inp, FFN_TILED)["out"]
+    monkeypatch.setenv("MOE355_FUSED_COMBINE", "1")
+    for mode in (FFN_TILED, FFN_PERSISTENT):
+        layer = moe.MoELayer(product_config(cfg), ffn_mode=mode)
+        dev = upload_inputs(cfg, inp)
+        for call in range(3):
+            out = torch.full((cfg.S, cfg.H), float("nan"), dtype=layer.act_dtype, device="cuda")   # nothing may be left unwritten
+            layer.forward(dev["x"], dev, out=out)
+            torch.cuda.synchronize()
+            assert np.array_equal(from_device(out), separate), (mode, call)
+        assert layer.stage_ms is not None
+        layer.close()
+
+
 @pytest.mark.parametrize("name", sorted(n for n, c in LARGE_TILE.items()
                                         if c.H % 256 == 0 and c.I % (128 if c.act == ob.ACT_SWIGLU else 256) == 0))
 def test_half_height_tile(moe, name, monkeypatch):

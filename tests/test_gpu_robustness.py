@@ -82,12 +82,14 @@ def test_route_drops_out_of_range_expert_ids(moe):
     ("f32", ob.Cfg(S=200, H=128, I=128, E=4, k=1, act=ob.ACT_GELU, dtype=ob.F32, norm_topk=0, drop=0)),
     ("fp8", ob.Cfg(S=64, H=256, I=256, E=8, k=2, act=ob.ACT_SWIGLU, dtype=ob.FP8, gate_fn=ob.GATE_SIGMOID, drop=0)),
 ])
-def test_expired_dependency_wait_poisons_the_output_and_is_reported(moe, name, cfg):
+@pytest.mark.parametrize("fused_combine", ["0", "1"])
+def test_expired_dependency_wait_poisons_the_output_and_is_reported(moe, name, cfg, fused_combine, monkeypatch):
     """The queue kernel's bounded wait is made to give up from the host (spin limit < 0: every wait expires without
     polling).  Every kernel exits normally; no down-projection tile computes on unfinished rows -- its output is NaN,
     so every routed token's output is NaN; the stall is reported by the next calls on the handle without a
     synchronisation of their own, until it is cleared; after that the handle computes correctly again."""
     import torch
+    monkeypatch.setenv("MOE355_FUSED_COMBINE", fused_combine)   # the combine inside the FFN kernels must carry the NaNs too
     inp = ob.make_inputs(cfg, seed=9)
     want = ob.forward(cfg, inp)
     layer = moe.MoELayer(product_config(cfg), ffn_mode=FFN_PERSISTENT)

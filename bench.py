@@ -149,6 +149,54 @@ def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False, balanced_
     return res, layer, dev, out, routing
 
 
+def measure_backward(layer, cfg, dev, routing, steps, warmup):
+    """Times the backward building blocks of both projections on the workload's routing: data gradients as grouped
+    products with the transposed weight, weight gradients per expert.  Synthetic upstream gradients; the transposes of
+    the weights are timed separately (a training step makes them once per optimizer step, not once per layer call)."""
+    import torch
+    import cuplayground_amd as moe
+    c = cfg
+    A, H, I, E = c.tokens * c.expert_top_k, c.hidden_size, c.intermediate_size, c.num_experts
+    g = torch.Generator(device="cuda").manual_seed(7)
+    dt = layer.act_dtype
+    cnt, off = routing["expert_count"], routing["expert_offset"]
+    kept = int(cnt.sum().item())
+    dy = torch.randn(A, H, generator=g, device="cuda", dtype=torch.float32).to(dt)     # d loss / d y rows
+    hrows = torch.randn(A, I, generator=g, device="cuda", dtype=torch.float32).to(dt)  # the saved intermediate rows
+    xrows = torch.randn(A, H, generator=g, device="cuda", dtype=torch.float32).to(dt)  # the gathered token rows
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        for a, b in ev:
+            a.record(); fn(); b.record()
+        torch.cuda.synchronize()
+        return statistics.median(a.elapsed_time(b) for a, b in ev)
+
+    res = {}
+    w_down_t = moe.transpose(dev["w_down"])           # [E, I, H]
+    w_up_t = moe.transpose(dev["w_up"])               # [E, H, I]
+    res["transpose_w_down_ms"] = timed(lambda: moe.transpose(dev["w_down"], out=w_down_t))
+    out_i = torch.zeros(A, I, dtype=dt, device="cuda")
+    out_h = torch.zeros(A, H, dtype=dt, device="cuda")
+    dw_down = torch.empty(E, H, I, dtype=dt, device="cuda")
+    dw_up = torch.empty(E, I, H, dtype=dt, device="cuda")
+    flops = 2.0 * kept * H * I
+    ops = {
+        "dgrad_down": lambda: layer.expert_gemm(dy, w_down_t, None, cnt, off, out=out_i),       # dH = dY . W_down
+        "wgrad_down": lambda: layer.expert_wgrad(dy, hrows, cnt, off, out=dw_down),              # dW_down = dY^T . H
+        "dgrad_up": lambda: layer.expert_gemm(hrows, w_up_t, None, cnt, off, out=out_h),         # dX = dU . W_up
+        "wgrad_up": lambda: layer.expert_wgrad(hrows, xrows, cnt, off, out=dw_up),               # dW_up = dU^T . X
+    }
+    for name, fn in ops.items():
+        ms = timed(fn)
+        res[name] = {"ms": round(ms, 4), "tflops": round(flops / (ms * 1e-3) / 1e12, 1),
+                     "frac": round(flops / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)}
+    res["flops_per_op"] = flops
+    return res
+
+
 def to_host(d):
     """Device operands -> the numpy layout the oracle takes (bf16 as uint16 bit patterns)."""
     import numpy as np
@@ -274,6 +322,9 @@ def main():
     ap.add_argument("--balanced-routing", action="store_true",
                     help="experiment: replace the router's inputs so that every expert receives exactly S*k/E rows "
                          "(no ragged last row blocks); the FFN arithmetic is unchanged")
+    ap.add_argument("--backward", action="store_true",
+                    help="also time the backward building blocks (data and weight gradients of both projections) on "
+                         "the workload's routing; bf16 / fp16 workloads only")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy (a known-size reference for HBM byte counters)")
     args = ap.parse_args()
@@ -300,6 +351,9 @@ def main():
     roof["measured_peak"] = peaks["hbm_read_gbs"] if fp8 else peaks["mfma_bf16_tflops_random_operands"]
     roof["frac_of_measured_peak"] = roof["achieved"] / roof["measured_peak"]
 
+    backward = None
+    if args.backward:
+        backward = measure_backward(layer, main_w.config, dev, routing, args.steps, args.warmup)
     cpu = cpu_oracle = parity = None
     if args.cpu_seconds > 0:
         cpu, cpu_oracle, parity = cpu_leg(args.workload, dev, out, routing, args.cpu_seconds, args.seed)
@@ -341,6 +395,8 @@ def main():
         "roofline": roof, "cpu_baseline": cpu, "cpu_baseline_oracle": cpu_oracle, "parity": parity,
         "workloads": others,
     }
+    if backward is not None:
+        line["backward"] = backward
     print(json.dumps(line))
 
 

@@ -14,7 +14,7 @@ namespace moe355 {
 
 bool grouped_gemm_takes_large_tile(int64_t A, int E, int N, int K);
 hipError_t launch_grouped_gemm_16(const void* a_rows, const void* w, const void* bias, void* out, const MTile* mtiles,
-                                  const int32_t* num_mtiles, int max_mtiles, int block_m, int64_t A, int N, int K, int act,
+                                  const int32_t* num_mtiles, int max_mtiles, int tile, int64_t A, int N, int K, int act,
                                   bool f16, hipStream_t st);
 hipError_t launch_wgrad_16(const void* dyT, const void* aT, void* dw, const int32_t* poff, int E, int N, int K,
                            int64_t ld, bool f16, hipStream_t st);
@@ -146,7 +146,14 @@ hipError_t launch_transpose(const void* src, void* dst, int64_t batch, int64_t r
 hipError_t launch_expert_gemm(const void* a_rows, const void* w, const void* bias, const int32_t* count,
                               const int32_t* offset, int64_t A, int E, int N, int K, int act, bool f16, void* out_rows,
                               void* scratch, hipStream_t st) {
-    const int block_m = grouped_gemm_takes_large_tile(A, E, N, K) ? 256 : 128;
+    int tile = grouped_gemm_takes_large_tile(A, E, N, K) ? 1 : 0;     // 1: 256 x 256, 0: 128 x 128
+    if (const char* env = getenv("MOE355_GROUPED_TILE")) {             // tuning knob; 2: 128 x 256 (hand-ordered)
+        const int v = atoi(env);
+        const int64_t lim = (int64_t)1 << 32;
+        if ((v == 1 || v == 2) && N % 256 == 0 && K % 128 == 0 && A * K * 2 < lim && (int64_t)N * K * 2 < lim) tile = v;
+        if (v == 0) tile = 0;
+    }
+    const int block_m = tile == 1 ? 256 : 128;
     char* s = static_cast<char*>(scratch);
     int32_t* num_mtiles = reinterpret_cast<int32_t*>(s);
     MTile* mtiles = reinterpret_cast<MTile*>(s + align256(sizeof(int32_t)));
@@ -154,7 +161,7 @@ hipError_t launch_expert_gemm(const void* a_rows, const void* w, const void* bia
     backward_tables_kernel<<<1, kMaxExperts, 0, st>>>(count, offset, E, block_m, mtiles, num_mtiles, nullptr);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    return launch_grouped_gemm_16(a_rows, w, bias, out_rows, mtiles, num_mtiles, max_mtiles, block_m, A, N, K, act, f16, st);
+    return launch_grouped_gemm_16(a_rows, w, bias, out_rows, mtiles, num_mtiles, max_mtiles, tile, A, N, K, act, f16, st);
 }
 
 // dw[e] [N,K] = dy_e^T . a_e; scratch holds the window offsets and the two transposed operands.

@@ -1357,9 +1357,12 @@ static hipError_t launch_grouped(const void* a_rows, const void* w, const void* 
 }
 
 hipError_t launch_grouped_gemm_16(const void* a_rows, const void* w, const void* bias, void* out, const MTile* mtiles,
-                                  const int32_t* num_mtiles, int max_mtiles, int block_m, int64_t A, int N, int K, int act,
+                                  const int32_t* num_mtiles, int max_mtiles, int tile, int64_t A, int N, int K, int act,
                                   bool f16, hipStream_t st) {
-    if (block_m == 256)
+    if (tile == 2)   // 128-row blocks on the hand-ordered 128 x 256 tile
+        return f16 ? launch_grouped<Tile128x256H>(a_rows, w, bias, out, mtiles, num_mtiles, max_mtiles, A, N, K, act, st)
+                   : launch_grouped<Tile128x256>(a_rows, w, bias, out, mtiles, num_mtiles, max_mtiles, A, N, K, act, st);
+    if (tile == 1)
         return f16 ? launch_grouped<LargePlanH::T0>(a_rows, w, bias, out, mtiles, num_mtiles, max_mtiles, A, N, K, act, st)
                    : launch_grouped<LargePlan::T0>(a_rows, w, bias, out, mtiles, num_mtiles, max_mtiles, A, N, K, act, st);
     return f16 ? launch_grouped<SmallPlanH::T0>(a_rows, w, bias, out, mtiles, num_mtiles, max_mtiles, A, N, K, act, st)

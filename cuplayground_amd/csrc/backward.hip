@@ -92,15 +92,56 @@ __global__ __launch_bounds__(256) void transpose32_kernel(const uint32_t* __rest
     }
 }
 
+// The same for 16-bit elements when R and C are multiples of 8: every global access is 16 bytes per lane.  A 64 x 64
+// tile goes into LDS as rows of 32 dwords + 1 (the odd pitch spreads a column over the banks) and comes out as
+// columns, eight 2-byte reads per lane packed into one 16-byte store.
+__device__ __forceinline__ void tile64_store_row(uint32_t* tile, int r, int ch, uint4 v) {
+    uint32_t* p = tile + r * 33 + ch * 4;
+    p[0] = v.x; p[1] = v.y; p[2] = v.z; p[3] = v.w;
+}
+__device__ __forceinline__ uint4 tile64_load_column(const uint32_t* tile, int col, int row8) {
+    const uint16_t* t = reinterpret_cast<const uint16_t*>(tile);
+    uint32_t w[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t lo = t[(row8 * 8 + 2 * j) * 66 + col], hi = t[(row8 * 8 + 2 * j + 1) * 66 + col];
+        w[j] = lo | (hi << 16);
+    }
+    return uint4{w[0], w[1], w[2], w[3]};
+}
+
+__global__ __launch_bounds__(256) void transpose16_vec_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst,
+                                                              int64_t R, int64_t C) {
+    __shared__ uint32_t tile[64 * 33];
+    const uint16_t* s = src + (size_t)blockIdx.z * R * C;
+    uint16_t* d = dst + (size_t)blockIdx.z * R * C;
+    const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
+    const int sub = threadIdx.x >> 3, ch = threadIdx.x & 7;
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+        const int r = sub + 32 * pass;
+        uint4 v = {0u, 0u, 0u, 0u};
+        if (r0 + r < R && c0 + ch * 8 < C) v = *reinterpret_cast<const uint4*>(s + (r0 + r) * C + c0 + ch * 8);
+        tile64_store_row(tile, r, ch, v);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+        const int c = sub + 32 * pass;
+        if (c0 + c < C && r0 + ch * 8 < R)
+            *reinterpret_cast<uint4*>(d + (c0 + c) * R + r0 + ch * 8) = tile64_load_column(tile, c, ch);
+    }
+}
+
 // Packed rows [*, C] -> dst [C, ld]: column poff[e] + s holds row offset[e] + s of expert e (s < count[e]); the rest
 // of each window is zero.  A 64-column tile of dst never straddles two windows (they are multiples of 128 wide).
-// grid = (ld / 64, ceil(C / 64)).
+// C is a multiple of 8.  grid = (ld / 64, ceil(C / 64)).
 __global__ __launch_bounds__(256) void transpose_rows_padded_kernel(const uint16_t* __restrict__ rows, int C,
                                                                     const int32_t* __restrict__ count,
                                                                     const int32_t* __restrict__ offset,
                                                                     const int32_t* __restrict__ poff, int E, int64_t ld,
                                                                     uint16_t* __restrict__ dst) {
-    __shared__ uint16_t tile[64][66];
+    __shared__ uint32_t tile[64 * 33];
     const int p0 = blockIdx.x * 64;
     if (p0 >= poff[E]) return;                 // behind the last window: never read
     int lo = 0, hi = E - 1;
@@ -110,14 +151,21 @@ __global__ __launch_bounds__(256) void transpose_rows_padded_kernel(const uint16
     }
     const int e = lo, s0 = p0 - poff[e], n = count[e], off = offset[e];
     const int c0 = blockIdx.y * 64;
-    for (int i = threadIdx.x; i < 64 * 64; i += 256) {
-        const int r = i >> 6, c = i & 63;
-        tile[r][c] = (s0 + r < n && c0 + c < C) ? rows[(size_t)(off + s0 + r) * C + c0 + c] : (uint16_t)0;
+    const int sub = threadIdx.x >> 3, ch = threadIdx.x & 7;
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+        const int r = sub + 32 * pass;
+        uint4 v = {0u, 0u, 0u, 0u};
+        if (s0 + r < n && c0 + ch * 8 < C)
+            v = *reinterpret_cast<const uint4*>(rows + (size_t)(off + s0 + r) * C + c0 + ch * 8);
+        tile64_store_row(tile, r, ch, v);
     }
     __syncthreads();
-    for (int i = threadIdx.x; i < 64 * 64; i += 256) {
-        const int c = i >> 6, r = i & 63;
-        if (c0 + c < C) dst[(size_t)(c0 + c) * ld + p0 + r] = tile[r][c];
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+        const int c = sub + 32 * pass;
+        if (c0 + c < C)
+            *reinterpret_cast<uint4*>(dst + (size_t)(c0 + c) * ld + p0 + ch * 8) = tile64_load_column(tile, c, ch);
     }
 }
 
@@ -137,7 +185,9 @@ hipError_t launch_transpose(const void* src, void* dst, int64_t batch, int64_t r
                             hipStream_t st) {
     if (batch < 1 || rows < 1 || cols < 1) return hipSuccess;
     const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64), (unsigned)batch);
-    if (elem_bytes == 2) transpose16_kernel<<<grid, 256, 0, st>>>((const uint16_t*)src, (uint16_t*)dst, rows, cols);
+    if (elem_bytes == 2 && rows % 8 == 0 && cols % 8 == 0 && ((uintptr_t)src % 16 == 0) && ((uintptr_t)dst % 16 == 0))
+        transpose16_vec_kernel<<<grid, 256, 0, st>>>((const uint16_t*)src, (uint16_t*)dst, rows, cols);
+    else if (elem_bytes == 2) transpose16_kernel<<<grid, 256, 0, st>>>((const uint16_t*)src, (uint16_t*)dst, rows, cols);
     else transpose32_kernel<<<grid, 256, 0, st>>>((const uint32_t*)src, (uint32_t*)dst, rows, cols);
     return hipGetLastError();
 }

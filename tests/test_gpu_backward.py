@@ -37,7 +37,7 @@ def operands(rng, R, E, N, K, dtype):
     return a, dy, w, bias
 
 
-@pytest.mark.parametrize("shape", [(1, 5, 7), (3, 64, 64), (2, 130, 257), (4, 1000, 72)])
+@pytest.mark.parametrize("shape", [(1, 5, 7), (3, 64, 64), (2, 130, 257), (4, 1000, 72), (2, 8, 264), (3, 200, 1032)])
 @pytest.mark.parametrize("elem", [2, 4])
 def test_transpose_is_exact(moe, shape, elem):
     rng = np.random.default_rng(sum(shape))

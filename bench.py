@@ -79,20 +79,30 @@ def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False, balanced_
     for _ in range(warmup):
         layer.forward(dev["x"], dev, out=out)
     torch.cuda.synchronize()
+    # the timed region behind `value`: exactly `steps` calls, nothing else on the stream
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        layer.forward(dev["x"], dev, out=out)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / steps
+    # the same `steps` calls again with hipEvents around every stage (recorded by the library on this stream) and
+    # around every call: kernel durations, stage breakdown, medians.  The event records themselves cost about 15 us
+    # per call, which is why they stay out of the region above.
     layer.set_stage_timing(True)
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
-    t0 = time.perf_counter()
+    t2 = time.perf_counter()
     for a, b in ev:
         a.record()
         layer.forward(dev["x"], dev, out=out)
         b.record()
     torch.cuda.synchronize()
-    t1 = time.perf_counter()
+    t3 = time.perf_counter()
     stage_mean = layer.stage_ms()
     samples = layer.stage_samples()
     layer.set_stage_timing(False)
     step_ms = [a.elapsed_time(b) for a, b in ev]
-    ms_per_step = (t1 - t0) * 1e3 / steps
+    ms_per_step_events = (t3 - t2) * 1e3 / steps
 
     routing = layer.new_routing()                 # one extra, untimed call fetches the routing result
     layer.forward(dev["x"], dev, out=out, routing=routing)
@@ -133,7 +143,7 @@ def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False, balanced_
             else "no counter run for this kernel"
     res = {
         "workload": w.describe(), "tokens_per_s": c.tokens / (ms_per_step * 1e-3), "ms_per_step": ms_per_step,
-        "step_ms": stats(step_ms), "steps": steps, "warmup": warmup,
+        "ms_per_step_with_events": ms_per_step_events, "step_ms": stats(step_ms), "steps": steps, "warmup": warmup,
         "tflops": layer_flops / (ms_per_step * 1e-3) / 1e12,
         "stage_ms": {k: round(v, 4) for k, v in stage_mean.items() if k != "calls"},
         "stage_ms_median": {k: round(statistics.median(v[-steps:]), 4) for k, v in samples.items()},
@@ -377,7 +387,9 @@ def main():
     line = {
         "metric": "MoE layer forward tokens/s (%s shape, 1 MI355X)" % args.workload,
         "value": res["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": res["ms_per_step"], "step_ms": res["step_ms"],
+        "warmup": args.warmup, "ms_per_step": res["ms_per_step"],
+        # a second pass over the same steps carries the hipEvents behind step_ms, stage_ms and roofline.kernel_ms
+        "ms_per_step_with_events": res["ms_per_step_with_events"], "step_ms": res["step_ms"],
         "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": dtype[main_w.config.torch_dtype], "data": "synthetic",
         "config": {"workload": res["workload"], "ffn_mode": res["ffn_mode"], "block_rows": res["block_rows"],

@@ -27,7 +27,13 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 constexpr int QBM = 16;      // token rows per task
 constexpr int QN0 = 64;      // intermediate columns per phase-0 sub-tile (64 gate rows + 64 up rows)
 constexpr int QN1 = 128;     // output columns per phase-1 sub-tile
-constexpr int QSUB = 2;      // sub-tiles per task: halves the pops, decodes and dependency traffic per byte streamed
+// Sub-tiles per task.  An up-projection task streams four (64 gate + 64 up rows x H bytes each): fewer pops, decodes
+// and dependency counts per byte.  A down-projection task takes one: those are the last tasks of the queue, and the
+// smaller they are the shorter the tail in which workgroups run dry.  Measured on the decode shape (H 7168, I 2048,
+// 219 experts hit; kernel time, same box): (2, 2) 1.638 ms, (2, 4) 1.646, (2, 1) 1.621, (1, 1) 1.636, (4, 1) 1.606,
+// (8, 1) 1.618, (16, 1) 1.93.
+constexpr int QSUB = 4;
+constexpr int QSUB1 = 1;
 constexpr int QGROUPS = 8;   // 16-row weight groups per task
 constexpr int QWAVES = 4;
 
@@ -200,7 +206,7 @@ __device__ __forceinline__ Fp8Task resolve_fp8(const FfnArgs& a, const Task& t, 
         p.a_row0 = 0;
         p.c_base = (uint16_t*)a.h + (int64_t)t.row0 * a.I;
     } else {
-        p.c0 = (t.ntile * QSUB + sub) * QN1;
+        p.c0 = (t.ntile * QSUB1 + sub) * QN1;
         p.K = a.I;
         p.N = a.H;
         p.w[0] = p.w[1] = (const uint8_t*)a.w_down + t.expert * HI;
@@ -222,11 +228,11 @@ __global__ __launch_bounds__(256) void ffn_tiled_fp8_kernel(FfnArgs a, int phase
     if (phase == 0) zero_unrouted_rows(a, 2);
     Task t;
     if (!tiled_task(a, phase, blockIdx.x, t)) return;
-    for (int sub = 0; sub < QSUB; ++sub) {
+    for (int sub = 0; sub < (phase ? QSUB1 : QSUB); ++sub) {
         const Fp8Task p = resolve_fp8(a, t, sub, phase == 1 && a.arrive);
         if (p.c0 < p.N) fp8_tile(p, red);
     }
-    if (phase == 1 && a.arrive) combine_arrivals<bf16_s>(combine_args(a), t.row0, t.rows, t.ntile, t.ntile * QSUB * QN1, QSUB * QN1, s_list);
+    if (phase == 1 && a.arrive) combine_arrivals<bf16_s>(combine_args(a), t.row0, t.rows, t.ntile, t.ntile * QSUB1 * QN1, QSUB1 * QN1, s_list);
 }
 
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void ffn_persistent_fp8_kernel(FfnArgs a) {
@@ -244,14 +250,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     while (next_task(a, cur, &s_task, ids, nseg, nnt0, t)) {
         int ok = 1;
         if (t.phase == 1) ok = wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q, a.host_stall, &s_ok);
-        for (int sub = 0; sub < QSUB; ++sub) {
+        for (int sub = 0; sub < (t.phase ? QSUB1 : QSUB); ++sub) {
             const Fp8Task p = resolve_fp8(a, t, sub, t.phase == 0 || a.arrive);
             if (p.c0 >= p.N) continue;
             if (ok) fp8_tile(p, red);
             else poison_tile(p.c_base, p.rows, p.N, p.c0, QN1, 2);
         }
         if (t.phase == 0) signal_phase0_done(a.done0, t.mtile);
-        else if (a.arrive) combine_arrivals<bf16_s>(combine_args(a), t.row0, t.rows, t.ntile, t.ntile * QSUB * QN1, QSUB * QN1, s_list);
+        else if (a.arrive) combine_arrivals<bf16_s>(combine_args(a), t.row0, t.rows, t.ntile, t.ntile * QSUB1 * QN1, QSUB1 * QN1, s_list);
     }
     queue_clock_stamp(a.wg_clock, 1);
 }
@@ -260,7 +266,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 
 int fp8_block_m() { return QBM; }
 int fp8_block_n0() { return QN0 * QSUB; }
-int fp8_block_n1() { return QN1 * QSUB; }
+int fp8_block_n1() { return QN1 * QSUB1; }
 
 int ffn_persistent_occupancy_fp8() {
     int n = 0;

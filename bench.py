@@ -34,9 +34,9 @@ PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
 # digest of the kernel sources it was collected with: when the sources have changed since, the figure is withheld.
 KERNEL_SOURCES = ("ffn_bf16.hip", "ffn_bf16_slab_steady.inc", "ffn_fp8.hip", "ffn_common.hpp", "route.hip")
 MEASURED_TRAFFIC = {
-    "mixtral": {"bytes": 19.55e9, "kernel_digest": "1d56d5b70cf1",
+    "mixtral": {"bytes": 19.30e9, "kernel_digest": "e9c99de4a735",
                 "profile": "profiles/ffn_persistent_kernel_bf16_mixtral_c3_hbm_traffic.txt"},
-    "decode_fp8": {"bytes": 9.965e9, "kernel_digest": "1d56d5b70cf1",
+    "decode_fp8": {"bytes": 9.920e9, "kernel_digest": "e9c99de4a735",
                    "profile": "profiles/ffn_persistent_fp8_kernel_decode_c5_hbm_traffic.txt"},
 }
 

@@ -1,0 +1,61 @@
+"""Seeded random layer shapes crossed with the tuning knobs (tile, FFN mode, queue count, early start of the next
+task, combine inside the FFN kernels): every combination must match the CPU oracle -- routing bit for bit, output
+within the dtype's bound -- because no knob is allowed to change what is computed."""
+import numpy as np
+import pytest
+
+from oracle import binding as ob
+from helpers import OUT_TOL, from_device, max_rel_err, product_config, upload_inputs
+from test_gpu_layer import check_routing
+
+pytestmark = pytest.mark.gpu
+
+
+def _cases(n=36, seed=2024):
+    rng = np.random.default_rng(seed)
+    out = []
+    for i in range(n):
+        dtype = [ob.BF16, ob.BF16, ob.F16, ob.F32, ob.FP8][i % 5]
+        act = ob.ACT_SWIGLU if dtype == ob.FP8 else int(rng.choice([ob.ACT_RELU, ob.ACT_GELU, ob.ACT_SWIGLU]))
+        E = int(rng.choice([1, 2, 3, 4, 6, 8, 16, 40]))
+        k = int(rng.integers(1, min(E, 4) + 1))
+        mult = 128 if dtype == ob.FP8 else (256 if i % 2 == 0 else 64)        # multiples of 256 reach the hand-ordered tiles
+        H = mult * int(rng.integers(1, 3))
+        I = mult * int(rng.integers(1, 4))
+        S = int(rng.integers(1, 2600 if i % 2 == 0 else 900))     # the larger ones give experts several row blocks
+        drop = int(rng.integers(0, 2))
+        cfg = ob.Cfg(S=S, H=H, I=I, E=E, k=k, act=act, dtype=dtype, drop=drop,
+                     capacity_factor=float(rng.choice([0.5, 1.0, 1.5])), norm_topk=int(k > 1),
+                     gate_fn=ob.GATE_SIGMOID if dtype == ob.FP8 else int(rng.integers(0, 2)), zipf_bias=bool(i % 3 == 0))
+        knobs = dict(MOE355_TILE=str(int(rng.integers(0, 4))), MOE355_QUEUE_GROUPS=str(int(rng.choice([1, 2, 8]))),
+                     MOE355_QUEUE_EARLY=str(int(rng.integers(0, 2))), MOE355_FUSED_COMBINE=str(int(rng.integers(0, 2))))
+        out.append(pytest.param(cfg, knobs, int(rng.integers(1, 3)), bool(rng.integers(0, 2)), id="case%02d" % i))
+    return out
+
+
+@pytest.mark.parametrize("cfg,knobs,mode,with_bias", _cases())
+def test_random_shape_and_knobs_vs_oracle(cfg, knobs, mode, with_bias, monkeypatch):
+    import torch
+    import cuplayground_amd as moe
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    for k, v in knobs.items():
+        monkeypatch.setenv(k, v)
+    inp = ob.make_inputs(cfg, seed=17, with_bias=with_bias)
+    want = ob.forward(cfg, inp)
+    layer = moe.MoELayer(product_config(cfg), ffn_mode=mode)
+    dev = upload_inputs(cfg, inp)
+    routing = layer.new_routing()
+    out = torch.full((cfg.S, cfg.H), float("nan"), dtype=layer.act_dtype, device="cuda")
+    for _ in range(2):                       # the second call reuses every counter and table of the first
+        layer.forward(dev["x"], dev, out=out, routing=routing)
+    torch.cuda.synchronize()
+    layer.task_counts()
+    got = {k: from_device(v) for k, v in routing.items()}
+    check_routing(got, want)
+    o = ob.to_f32(from_device(out), cfg.act_dtype)
+    ref = ob.to_f32(want["out"], cfg.act_dtype)
+    assert not np.isnan(o).any()
+    assert max_rel_err(o, ref) <= OUT_TOL[cfg.dtype], (knobs, mode)
+    dead = (want["slot"] < 0).all(axis=1)
+    assert not o[dead].any()
+    layer.close()

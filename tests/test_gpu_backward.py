@@ -74,6 +74,28 @@ def test_expert_gemm_vs_oracle(moe, case, dtype):
 
 
 @pytest.mark.parametrize("dtype", [ob.BF16, ob.F16])
+def test_grouped_product_tiles_agree(moe, dtype, monkeypatch):
+    """The 128 x 128, 256 x 256 and 128 x 256 tiles forced on one grouped product (MOE355_GROUPED_TILE): the two
+    hand-ordered ones accumulate every output element with the same MFMA sequence and must agree bit for bit; the
+    compiler-ordered 128 x 128 tile only within the tolerance."""
+    S, H, I, E, k, cf, skew = CASES[2]
+    cfg, rng, count, offset = routed_case(S, H, I, E, k, dtype, seed=77, cf=cf, skew=0.3)
+    layer = moe.MoELayer(product_config(cfg))
+    kind = KIND[dtype]
+    a, _, w, bias = operands(rng, S * k, E, I, H, dtype)
+    want = ob.to_f32(ob.expert_gemm(a, w, bias, count, offset, dtype, ob.ACT_GELU), dtype)
+    outs = {}
+    for tile in ("0", "1", "2"):
+        monkeypatch.setenv("MOE355_GROUPED_TILE", tile)
+        got = layer.expert_gemm(to_device(a, kind), to_device(w, kind), to_device(bias, kind), to_device(count, "i32"),
+                                to_device(offset, "i32"), ob.ACT_GELU)
+        outs[tile] = from_device(got)
+        kept = int(count.sum())
+        assert max_rel_err(ob.to_f32(outs[tile], dtype)[:kept], want[:kept]) <= OUT_TOL[dtype]
+    assert np.array_equal(outs["1"], outs["2"])
+
+
+@pytest.mark.parametrize("dtype", [ob.BF16, ob.F16])
 @pytest.mark.parametrize("case", CASES)
 def test_data_gradient_is_the_grouped_product_with_the_transposed_weight(moe, case, dtype):
     """dX = dY . W: the oracle works on numpy's transpose, the product on moe_transpose's."""

@@ -27,7 +27,7 @@ EXPORTS = (
     "moe_set_ffn_mode", "moe_get_ffn_mode", "moe_forward", "moe_forward_static", "moe_set_spin_limit", "moe_clear_stall", "moe_gate", "moe_router_stats", "moe_route", "moe_gemm_bias_act", "moe_combine",
     "moe_set_stage_timing", "moe_get_stage_ms", "moe_get_stage_samples", "moe_get_task_counts", "moe_get_queue_balance", "moe_measure_mfma_tflops",
     "moe_measure_hbm_read_gbs", "moe_quant_block128", "moe_backward_scratch_bytes", "moe_transpose", "moe_expert_gemm",
-    "moe_expert_wgrad", "moe_last_hip_error", "moe_status_string",
+    "moe_expert_wgrad", "moe_act_backward", "moe_bias_grad", "moe_combine_backward", "moe_last_hip_error", "moe_status_string",
     "moe_version",
 )
 
@@ -112,6 +112,9 @@ def load_library():
     L.moe_transpose.argtypes = [vp, vp, i64, i64, i64, i32, vp]
     L.moe_expert_gemm.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, vp, C.c_size_t, vp]
     L.moe_expert_wgrad.argtypes = [vp, vp, vp, vp, vp, i32, i32, vp, vp, C.c_size_t, vp]
+    L.moe_act_backward.argtypes = [vp, vp, vp, vp, i64, vp, vp, vp]
+    L.moe_bias_grad.argtypes = [vp, vp, vp, vp, i32, vp, vp]
+    L.moe_combine_backward.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp]
     L.moe_last_hip_error.argtypes = [vp]
     L.moe_status_string.argtypes = [C.c_int]; L.moe_status_string.restype = C.c_char_p
     L.moe_version.restype = C.c_int
@@ -409,6 +412,31 @@ class MoELayer:
         _check(self.L.moe_expert_wgrad(self._h, _ptr(dy_rows), _ptr(a_rows), _ptr(expert_count), _ptr(expert_offset),
                                        N, K, _ptr(out), _ptr(sc), sc.numel(), _stream()), "moe_expert_wgrad")
         return out
+
+    def act_backward(self, dh_rows, u_rows, g_rows=None):
+        """(du_rows, dg_rows) for the layer's activation; dg_rows is None unless the layer is SwiGLU."""
+        import torch
+        du = torch.empty_like(dh_rows)
+        dg = torch.empty_like(dh_rows) if g_rows is not None else None
+        _check(self.L.moe_act_backward(self._h, _ptr(dh_rows), _ptr(u_rows), _ptr(g_rows), dh_rows.shape[0], _ptr(du),
+                                       _ptr(dg), _stream()), "moe_act_backward")
+        return du, dg
+
+    def bias_grad(self, dy_rows, expert_count, expert_offset):
+        import torch
+        db = torch.empty(self.E, dy_rows.shape[1], dtype=dy_rows.dtype, device=dy_rows.device)
+        _check(self.L.moe_bias_grad(self._h, _ptr(dy_rows), _ptr(expert_count), _ptr(expert_offset), dy_rows.shape[1],
+                                    _ptr(db), _stream()), "moe_bias_grad")
+        return db
+
+    def combine_backward(self, dout, y_rows, pair_row, topk_w):
+        """(dy_rows with the rows no pair maps to zero, dw [S, k] fp32)."""
+        import torch
+        dy = torch.zeros_like(y_rows)
+        dw = torch.empty(self.S, self.k, dtype=torch.float32, device=dout.device)
+        _check(self.L.moe_combine_backward(self._h, _ptr(dout), _ptr(y_rows), _ptr(pair_row), _ptr(topk_w), _ptr(dy),
+                                           _ptr(dw), _stream()), "moe_combine_backward")
+        return dy, dw
 
 
 def transpose(src, out=None):

@@ -757,6 +757,43 @@ int moe_expert_wgrad(moe_handle* h, const void* dy_rows, const void* a_rows, con
     return e == hipSuccess ? MOE_OK : hip_fail(h, e);
 }
 
+namespace {
+bool backward_dtype(const moe_handle* h) {
+    return h->cfg.torch_dtype == MOE_DTYPE_BF16 || h->cfg.torch_dtype == MOE_DTYPE_FP16;
+}
+}  // namespace
+
+int moe_act_backward(moe_handle* h, const void* dh_rows, const void* u_rows, const void* g_rows, int64_t rows,
+                     void* du_rows, void* dg_rows, void* stream) {
+    if (!h || !dh_rows || !u_rows || !du_rows || rows < 0) return MOE_ERR_BAD_ARGUMENT;
+    if (!backward_dtype(h)) return MOE_ERR_UNSUPPORTED;
+    const bool sw = h->cfg.hidden_act == MOE_ACT_SWIGLU;
+    if (sw != (g_rows != nullptr) || sw != (dg_rows != nullptr)) return MOE_ERR_BAD_ARGUMENT;
+    if (rows > h->d.A) return MOE_ERR_BAD_ARGUMENT;
+    const hipError_t e = launch_act_backward(dh_rows, u_rows, g_rows, rows * h->d.I, h->cfg.hidden_act,
+                                             h->cfg.torch_dtype == MOE_DTYPE_FP16, du_rows, dg_rows, (hipStream_t)stream);
+    return e == hipSuccess ? MOE_OK : hip_fail(h, e);
+}
+
+int moe_bias_grad(moe_handle* h, const void* dy_rows, const int32_t* expert_count, const int32_t* expert_offset, int32_t N,
+                  void* db, void* stream) {
+    if (!h || !dy_rows || !expert_count || !expert_offset || !db) return MOE_ERR_BAD_ARGUMENT;
+    if (!backward_dtype(h)) return MOE_ERR_UNSUPPORTED;
+    if (N != h->d.H && N != h->d.I) return MOE_ERR_BAD_ARGUMENT;
+    const hipError_t e = launch_bias_grad(dy_rows, expert_count, expert_offset, h->d.E, N,
+                                          h->cfg.torch_dtype == MOE_DTYPE_FP16, db, (hipStream_t)stream);
+    return e == hipSuccess ? MOE_OK : hip_fail(h, e);
+}
+
+int moe_combine_backward(moe_handle* h, const void* dout, const void* y_rows, const int32_t* pair_row, const float* topk_w,
+                         void* dy_rows, float* dw, void* stream) {
+    if (!h || !dout || !y_rows || !pair_row || !topk_w || !dy_rows || !dw) return MOE_ERR_BAD_ARGUMENT;
+    if (!backward_dtype(h)) return MOE_ERR_UNSUPPORTED;
+    const hipError_t e = launch_combine_backward(dout, y_rows, pair_row, topk_w, h->d.S, h->d.k, h->d.H,
+                                                 h->cfg.torch_dtype == MOE_DTYPE_FP16, dy_rows, dw, (hipStream_t)stream);
+    return e == hipSuccess ? MOE_OK : hip_fail(h, e);
+}
+
 int moe_combine(const void* y_rows, const int32_t* pair_row, const float* topk_w, int32_t S, int32_t k, int32_t H,
                 int32_t act_dtype, void* out, void* stream) {
     if (!y_rows || !pair_row || !topk_w || !out || S < 0 || k < 1 || H < 1) return MOE_ERR_BAD_ARGUMENT;

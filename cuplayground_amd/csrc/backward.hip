@@ -8,6 +8,8 @@
 //   * weight gradients sum over an expert's rows: dW[e] = dY_e^T . A_e.  Both operands are transposed into buffers whose
 //     columns are the packed rows, each expert's window padded with zeros to a multiple of 128 columns, and every
 //     expert is then one tile GEMM over its window.
+#include <algorithm>
+
 #include "moe_internal.hpp"
 
 namespace moe355 {
@@ -169,6 +171,82 @@ __global__ __launch_bounds__(256) void transpose_rows_padded_kernel(const uint16
     }
 }
 
+// ---- elementwise and reduction steps of a backward pass (16-bit layers) ----
+template <class T16> __device__ __forceinline__ float ld16(const uint16_t* p, size_t i);
+template <> __device__ __forceinline__ float ld16<bf16_s>(const uint16_t* p, size_t i) { return __uint_as_float((uint32_t)p[i] << 16); }
+template <> __device__ __forceinline__ float ld16<f16_s>(const uint16_t* p, size_t i) { return (float)__builtin_bit_cast(_Float16, p[i]); }
+template <class T16> __device__ __forceinline__ uint16_t st16(float v);
+template <> __device__ __forceinline__ uint16_t st16<bf16_s>(float v) {
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t x = {v, 0.0f};
+    return (uint16_t)(__builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2_t)) & 0xFFFFu);
+}
+template <> __device__ __forceinline__ uint16_t st16<f16_s>(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
+
+// du = dh * act'(u); SwiGLU (h = silu(g) u): du = dh silu(g), dg = dh u s (1 + g (1 - s)), s = sigmoid(g).
+template <class T16>
+__global__ __launch_bounds__(256) void act_backward_kernel(const uint16_t* __restrict__ dh, const uint16_t* __restrict__ u,
+                                                           const uint16_t* __restrict__ g, size_t n, int act,
+                                                           uint16_t* __restrict__ du, uint16_t* __restrict__ dg) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+        const float d = ld16<T16>(dh, i), uv = ld16<T16>(u, i);
+        if (act == MOE_ACT_SWIGLU) {
+            const float gv = ld16<T16>(g, i);
+            const float sg = 1.0f / (1.0f + expf(-gv));
+            du[i] = st16<T16>(d * (gv * sg));
+            dg[i] = st16<T16>(d * uv * (sg * (1.0f + gv * (1.0f - sg))));
+        } else if (act == MOE_ACT_GELU) {
+            const float cdf = 0.5f * (1.0f + erff(uv * 0.70710678118654752440f));
+            const float pdf = 0.39894228040143267794f * expf(-0.5f * uv * uv);
+            du[i] = st16<T16>(d * (cdf + uv * pdf));
+        } else {
+            du[i] = st16<T16>(uv > 0.0f ? d : 0.0f);
+        }
+    }
+}
+
+// db[e, n] = sum over expert e's rows, ascending, of dy[r, n]: one thread per column, so the order is fixed.
+// grid = (ceil(N / 256), E).
+template <class T16>
+__global__ __launch_bounds__(256) void bias_grad_kernel(const uint16_t* __restrict__ dy, const int32_t* __restrict__ count,
+                                                        const int32_t* __restrict__ offset, int N, uint16_t* __restrict__ db) {
+    const int n = blockIdx.x * 256 + threadIdx.x, e = blockIdx.y;
+    if (n >= N) return;
+    const int r0 = offset[e], r1 = r0 + max(count[e], 0);
+    float acc = 0.0f;
+    for (int r = r0; r < r1; ++r) acc = acc + ld16<T16>(dy, (size_t)r * N + n);
+    db[(size_t)e * N + n] = st16<T16>(acc);
+}
+
+// One workgroup per token: dy[row(t,r), :] = w[t,r] * dout[t, :]; dw[t,r] = <dout[t, :], y[row(t,r), :]>.
+template <class T16>
+__global__ __launch_bounds__(256) void combine_backward_kernel(const uint16_t* __restrict__ dout, const uint16_t* __restrict__ y,
+                                                               const int32_t* __restrict__ pair_row,
+                                                               const float* __restrict__ topk_w, int k, int H,
+                                                               uint16_t* __restrict__ dy, float* __restrict__ dw) {
+    __shared__ float part[4];
+    const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int r = 0; r < k; ++r) {
+        const int row = pair_row[(size_t)t * k + r];
+        float acc = 0.0f;
+        if (row >= 0) {
+            const float w = topk_w[(size_t)t * k + r];
+            for (int j = threadIdx.x; j < H; j += 256) {
+                const float d = ld16<T16>(dout, (size_t)t * H + j);
+                dy[(size_t)row * H + j] = st16<T16>(w * d);
+                acc = fmaf(d, ld16<T16>(y, (size_t)row * H + j), acc);
+            }
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+        __syncthreads();                       // part may still be read for the previous rank
+        if (lane == 0) part[wave] = acc;
+        __syncthreads();
+        if (threadIdx.x == 0) dw[(size_t)t * k + r] = row >= 0 ? (part[0] + part[1]) + (part[2] + part[3]) : 0.0f;
+    }
+}
+
 size_t align256(size_t v) { return (v + 255) / 256 * 256; }
 
 }  // namespace
@@ -230,6 +308,31 @@ hipError_t launch_expert_wgrad(const void* dy_rows, const void* a_rows, const in
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     return launch_wgrad_16(dyT, aT, dw, poff, E, N, K, ld, f16, st);
+}
+
+hipError_t launch_act_backward(const void* dh, const void* u, const void* g, int64_t n, int act, bool f16, void* du,
+                               void* dg, hipStream_t st) {
+    if (n <= 0) return hipSuccess;
+    const int grid = (int)std::min<int64_t>((n + 255) / 256, 65536);
+    if (f16) act_backward_kernel<f16_s><<<grid, 256, 0, st>>>((const uint16_t*)dh, (const uint16_t*)u, (const uint16_t*)g, (size_t)n, act, (uint16_t*)du, (uint16_t*)dg);
+    else act_backward_kernel<bf16_s><<<grid, 256, 0, st>>>((const uint16_t*)dh, (const uint16_t*)u, (const uint16_t*)g, (size_t)n, act, (uint16_t*)du, (uint16_t*)dg);
+    return hipGetLastError();
+}
+
+hipError_t launch_bias_grad(const void* dy, const int32_t* count, const int32_t* offset, int E, int N, bool f16, void* db,
+                            hipStream_t st) {
+    const dim3 grid((unsigned)((N + 255) / 256), (unsigned)E);
+    if (f16) bias_grad_kernel<f16_s><<<grid, 256, 0, st>>>((const uint16_t*)dy, count, offset, N, (uint16_t*)db);
+    else bias_grad_kernel<bf16_s><<<grid, 256, 0, st>>>((const uint16_t*)dy, count, offset, N, (uint16_t*)db);
+    return hipGetLastError();
+}
+
+hipError_t launch_combine_backward(const void* dout, const void* y, const int32_t* pair_row, const float* topk_w, int S,
+                                   int k, int H, bool f16, void* dy, float* dw, hipStream_t st) {
+    if (S <= 0) return hipSuccess;
+    if (f16) combine_backward_kernel<f16_s><<<S, 256, 0, st>>>((const uint16_t*)dout, (const uint16_t*)y, pair_row, topk_w, k, H, (uint16_t*)dy, dw);
+    else combine_backward_kernel<bf16_s><<<S, 256, 0, st>>>((const uint16_t*)dout, (const uint16_t*)y, pair_row, topk_w, k, H, (uint16_t*)dy, dw);
+    return hipGetLastError();
 }
 
 }  // namespace moe355

@@ -161,6 +161,13 @@ hipError_t launch_expert_gemm(const void* a_rows, const void* w, const void* bia
 hipError_t launch_expert_wgrad(const void* dy_rows, const void* a_rows, const int32_t* count, const int32_t* offset,
                                int64_t A, int E, int N, int K, bool f16, void* dw, void* scratch, hipStream_t st);
 
+hipError_t launch_act_backward(const void* dh, const void* u, const void* g, int64_t n, int act, bool f16, void* du,
+                               void* dg, hipStream_t st);
+hipError_t launch_bias_grad(const void* dy, const int32_t* count, const int32_t* offset, int E, int N, bool f16, void* db,
+                            hipStream_t st);
+hipError_t launch_combine_backward(const void* dout, const void* y, const int32_t* pair_row, const float* topk_w, int S,
+                                   int k, int H, bool f16, void* dy, float* dw, hipStream_t st);
+
 hipError_t launch_gemm_bias_act(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N,
                                 int64_t K, int dtype, int act, hipStream_t st);
 

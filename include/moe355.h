@@ -265,6 +265,21 @@ int moe_expert_gemm(moe_handle* h, const void* a_rows, const void* w, const void
 int moe_expert_wgrad(moe_handle* h, const void* dy_rows, const void* a_rows, const int32_t* expert_count,
                      const int32_t* expert_offset, int32_t N, int32_t K, void* dw, void* scratch, size_t scratch_bytes,
                      void* stream);
+/* The elementwise and reduction steps between those products (same layers; fp32 arithmetic, one rounding on store):
+ * moe_act_backward: for the first `rows` packed rows of width I, du = dh * act'(u) for hidden_act ReLU (1 where u > 0)
+ *   and GELU (Phi(u) + u phi(u)); for SwiGLU, where h = silu(g) * u, du = dh * silu(g) and dg = dh * u * s * (1 + g (1 - s))
+ *   with s = sigmoid(g).  u_rows / g_rows are the projections before the activation (moe_expert_gemm with
+ *   MOE_ACT_NONE); g_rows and dg_rows are given exactly when the layer is SwiGLU.
+ * moe_bias_grad: db[e, n] = sum over expert e's rows, in ascending row order, of dy_rows[r, n]; N is H or I.
+ * moe_combine_backward: the adjoint of moe_combine: dy_rows[pair_row[t,r], :] = topk_w[t,r] * dout[t, :] and
+ *   dw[t,r] = <dout[t, :], y_rows[pair_row[t,r], :]> (0 for a dropped pair); rows of dy_rows that no pair maps to are
+ *   left untouched. */
+int moe_act_backward(moe_handle* h, const void* dh_rows, const void* u_rows, const void* g_rows, int64_t rows,
+                     void* du_rows, void* dg_rows, void* stream);
+int moe_bias_grad(moe_handle* h, const void* dy_rows, const int32_t* expert_count, const int32_t* expert_offset, int32_t N,
+                  void* db, void* stream);
+int moe_combine_backward(moe_handle* h, const void* dout, const void* y_rows, const int32_t* pair_row, const float* topk_w,
+                         void* dy_rows, float* dw, void* stream);
 
 int moe_last_hip_error(const moe_handle* h);
 const char* moe_status_string(int status);

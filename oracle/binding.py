@@ -76,6 +76,9 @@ def lib():
         L.orc_gemm_bias_act.argtypes = [vp, vp, vp, vp, i64, i64, i64, i32, i32]
         L.orc_expert_gemm.argtypes = [vp, vp, vp, vp, vp, i32, i64, i64, i32, i32, vp]
         L.orc_expert_wgrad.argtypes = [vp, vp, vp, vp, i32, i64, i64, i32, vp]
+        L.orc_act_backward.argtypes = [vp, vp, vp, i64, i64, i32, i32, vp, vp]
+        L.orc_bias_grad.argtypes = [vp, vp, vp, i32, i64, i32, vp]
+        L.orc_combine_backward.argtypes = [vp, vp, vp, vp, i32, i32, i32, i32, vp, vp]
         L.orc_ffn_rows.argtypes = [C.POINTER(_Cfg), vp, C.POINTER(_Weights), vp, vp, i64, vp]
         L.orc_combine.argtypes = [vp, vp, vp, i32, i32, i32, i32, vp]
         L.orc_forward.argtypes = [C.POINTER(_Cfg), vp, C.POINTER(_Weights), vp, vp, vp, vp, vp, vp, vp]
@@ -84,7 +87,8 @@ def lib():
         for fn in ("orc_philox4x32_10", "orc_fill_normal", "orc_fill_uniform", "orc_round_bf16", "orc_widen_bf16",
                    "orc_round_f16", "orc_widen_f16",
                    "orc_quant_block128", "orc_dequant_block128", "orc_gate_logits", "orc_topk", "orc_route",
-                   "orc_gemm_bias_act", "orc_expert_gemm", "orc_expert_wgrad", "orc_ffn_rows", "orc_combine", "orc_forward", "orc_forward_tokens"):
+                   "orc_gemm_bias_act", "orc_expert_gemm", "orc_expert_wgrad", "orc_act_backward", "orc_bias_grad",
+                   "orc_combine_backward", "orc_ffn_rows", "orc_combine", "orc_forward", "orc_forward_tokens"):
             getattr(L, fn).restype = None
         _lib = L
     return _lib
@@ -347,6 +351,34 @@ def expert_wgrad(dy_rows, a_rows, count, offset, dtype):
     lib().orc_expert_wgrad(_p(np.ascontiguousarray(dy_rows)), _p(np.ascontiguousarray(a_rows)), _p(count), _p(offset),
                            count.size, N, K, dtype, _p(dw))
     return dw
+
+
+def act_backward(dh, u, g, dtype, act):
+    """(du, dg): dg is None unless act is SwiGLU.  All arrays [rows, I] in the storage type."""
+    rows, I = dh.shape
+    du = np.empty_like(dh)
+    dg = np.empty_like(dh) if act == ACT_SWIGLU else None
+    lib().orc_act_backward(_p(np.ascontiguousarray(dh)), _p(np.ascontiguousarray(u)),
+                           _p(None if g is None else np.ascontiguousarray(g)), rows, I, dtype, act, _p(du), _p(dg))
+    return du, dg
+
+
+def bias_grad(dy_rows, count, offset, dtype):
+    count = _c(count, np.int32); offset = _c(offset, np.int32)
+    db = np.empty((count.size, dy_rows.shape[1]), dy_rows.dtype)
+    lib().orc_bias_grad(_p(np.ascontiguousarray(dy_rows)), _p(count), _p(offset), count.size, dy_rows.shape[1], dtype, _p(db))
+    return db
+
+
+def combine_backward(dout, y_rows, pair_row, topk_w, dtype):
+    """(dy_rows [rows of y, H] with untouched rows zero, dw [S, k] fp32)."""
+    pair_row = _c(pair_row, np.int32); topk_w = _c(topk_w, np.float32)
+    S, k = pair_row.shape
+    dy = np.zeros_like(y_rows)
+    dw = np.empty((S, k), np.float32)
+    lib().orc_combine_backward(_p(np.ascontiguousarray(dout)), _p(np.ascontiguousarray(y_rows)), _p(pair_row), _p(topk_w),
+                               S, k, dout.shape[1], dtype, _p(dy), _p(dw))
+    return dy, dw
 
 
 def ffn_rows(cfg: Cfg, inp, tokens, experts):

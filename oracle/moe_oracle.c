@@ -551,6 +551,65 @@ void orc_expert_wgrad(const void* dy_rows, const void* a_rows, const int32_t* co
     }
 }
 
+/* The elementwise and reduction steps of a backward pass (build-defined, as the grouped products above).
+ *   orc_act_backward:     du = dh * act'(u) (ReLU: 1 for u > 0; GELU: Phi(u) + u phi(u)), or for SwiGLU
+ *                         (h = silu(g) u): du = dh silu(g), dg = dh u s (1 + g (1 - s)) with s = sigmoid(g);
+ *                         fp32 arithmetic on the stored values, one rounding on store
+ *   orc_bias_grad:        db[e,n] = sum over expert e's rows, ascending, of dy[r,n] in fp32, rounded once
+ *   orc_combine_backward: dy[row(t,r),:] = w[t,r] * dout[t,:] (rounded once); dw[t,r] = <dout[t,:], y[row(t,r),:]> in
+ *                         fp32, ascending column; dropped pairs get dw = 0 and no row */
+void orc_act_backward(const void* dh, const void* u, const void* g, int64_t rows, int64_t I, int32_t dtype, int32_t act,
+                      void* du, void* dg) {
+    const int adt = act_dtype_of(dtype);
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < rows * I; ++i) {
+        const float d = load_act(dh, i, adt), uv = load_act(u, i, adt);
+        if (act == ORC_ACT_SWIGLU) {
+            const float gv = load_act(g, i, adt);
+            const float sg = 1.0f / (1.0f + expf(-gv));
+            store_act(du, i, adt, d * (gv * sg));
+            store_act(dg, i, adt, d * uv * (sg * (1.0f + gv * (1.0f - sg))));
+        } else if (act == ORC_ACT_GELU) {
+            const float cdf = 0.5f * (1.0f + erff(uv * 0.70710678118654752440f));
+            const float pdf = 0.39894228040143267794f * expf(-0.5f * uv * uv);
+            store_act(du, i, adt, d * (cdf + uv * pdf));
+        } else {
+            store_act(du, i, adt, uv > 0.0f ? d : 0.0f);
+        }
+    }
+}
+
+void orc_bias_grad(const void* dy_rows, const int32_t* count, const int32_t* offset, int32_t E, int64_t N, int32_t dtype,
+                   void* db) {
+    const int adt = act_dtype_of(dtype);
+    for (int32_t e = 0; e < E; ++e)
+        for (int64_t n = 0; n < N; ++n) {
+            float acc = 0.0f;
+            for (int64_t r = offset[e]; r < offset[e] + (count[e] > 0 ? count[e] : 0); ++r) acc = acc + load_act(dy_rows, r * N + n, adt);
+            store_act(db, (int64_t)e * N + n, adt, acc);
+        }
+}
+
+void orc_combine_backward(const void* dout, const void* y_rows, const int32_t* pair_row, const float* topk_w, int32_t S,
+                          int32_t k, int32_t H, int32_t dtype, void* dy_rows, float* dw) {
+    const int adt = act_dtype_of(dtype);
+#pragma omp parallel for schedule(static)
+    for (int32_t t = 0; t < S; ++t)
+        for (int32_t r = 0; r < k; ++r) {
+            const int32_t row = pair_row[(int64_t)t * k + r];
+            float acc = 0.0f;
+            if (row >= 0) {
+                const float w = topk_w[(int64_t)t * k + r];
+                for (int32_t j = 0; j < H; ++j) {
+                    const float d = load_act(dout, (int64_t)t * H + j, adt);
+                    store_act(dy_rows, (int64_t)row * H + j, adt, w * d);
+                    acc = fmaf(d, load_act(y_rows, (int64_t)row * H + j, adt), acc);
+                }
+            }
+            dw[(int64_t)t * k + r] = acc;
+        }
+}
+
 /* One expert FFN row: the two chained GEMMs of the reference's task graph (scheduling.cuh:212-222), the
  * intermediate rounded to the storage type between them (mma.cuh:108-109).  GELU is the exact erf form,
  * SwiGLU is silu(x.Wg^T + bg) * (x.Wu^T + bu); both are this build's extensions of hidden_act.

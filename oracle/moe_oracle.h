@@ -22,6 +22,8 @@
  *   - orc_expert_gemm / orc_expert_wgrad  pinned by float64 einsums per expert, by one-hot rows that select
  *                              single weight columns / operand rows, and by the adjoint identity
  *                              <dY, X.W^T> = <dY^T.X, W> = <dY.W, X> (tests/test_oracle_backward.py)
+ *   - orc_act_backward / orc_bias_grad / orc_combine_backward  pinned by central differences of the float64
+ *                              activations, float64 column sums, and the adjoint identity of the combine
  * Reference parity of gate / top-k / capacity / SwiGLU / fp8 scaling is unpinned by construction: the
  * reference holds no code for them.
  */
@@ -101,6 +103,12 @@ void orc_expert_gemm(const void* a_rows, const void* w, const void* bias, const 
                      int32_t E, int64_t N, int64_t K, int32_t dtype, int32_t act, void* out_rows);
 void orc_expert_wgrad(const void* dy_rows, const void* a_rows, const int32_t* count, const int32_t* offset, int32_t E,
                       int64_t N, int64_t K, int32_t dtype, void* dw);
+void orc_act_backward(const void* dh, const void* u, const void* g, int64_t rows, int64_t I, int32_t dtype, int32_t act,
+                      void* du, void* dg);
+void orc_bias_grad(const void* dy_rows, const int32_t* count, const int32_t* offset, int32_t E, int64_t N, int32_t dtype,
+                   void* db);
+void orc_combine_backward(const void* dout, const void* y_rows, const int32_t* pair_row, const float* topk_w, int32_t S,
+                          int32_t k, int32_t H, int32_t dtype, void* dy_rows, float* dw);
 void orc_ffn_rows(const orc_cfg* cfg, const void* x, const orc_weights* w, const int32_t* tokens,
                   const int32_t* experts, int64_t n_rows, void* y_rows);
 void orc_combine(const void* y_rows, const int32_t* pair_row, const float* topk_w,

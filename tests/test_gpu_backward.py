@@ -164,3 +164,64 @@ def test_unsupported_layers_and_bad_arguments_are_refused(moe):
     with pytest.raises(moe.MoEError) as e:        # (N, K) = (256, 192) is no projection of this layer
         layer.expert_gemm(z, w, None, cnt, cnt)
     assert e.value.status == 4
+
+
+@pytest.mark.parametrize("dtype", [ob.BF16, ob.F16])
+@pytest.mark.parametrize("act", [ob.ACT_RELU, ob.ACT_GELU, ob.ACT_SWIGLU])
+def test_activation_backward_vs_oracle(moe, act, dtype):
+    cfg = ob.Cfg(S=300, H=128, I=320, E=4, k=2, dtype=dtype, act=act, drop=0)
+    layer = moe.MoELayer(product_config(cfg))
+    kind = KIND[dtype]
+    rng = np.random.default_rng(31 + act)
+    rows = cfg.S * cfg.k - 7                                   # fewer rows than the buffers hold
+    u = ob.from_f32(rng.standard_normal((cfg.S * cfg.k, cfg.I)).astype(np.float32) * 2, dtype)
+    g = ob.from_f32(rng.standard_normal((cfg.S * cfg.k, cfg.I)).astype(np.float32) * 2, dtype)
+    dh = ob.from_f32(rng.standard_normal((cfg.S * cfg.k, cfg.I)).astype(np.float32), dtype)
+    sw = act == ob.ACT_SWIGLU
+    want_du, want_dg = ob.act_backward(dh[:rows], u[:rows], g[:rows] if sw else None, dtype, act)
+    du, dg = layer.act_backward(to_device(dh, kind)[:rows], to_device(u, kind)[:rows], to_device(g, kind)[:rows] if sw else None)
+    # library exp / erf against libm: an output ulp at most
+    tol = OUT_TOL[dtype]
+    assert max_rel_err(ob.to_f32(from_device(du), dtype), ob.to_f32(want_du, dtype)) <= tol
+    if sw:
+        assert max_rel_err(ob.to_f32(from_device(dg), dtype), ob.to_f32(want_dg, dtype)) <= tol
+    else:
+        assert dg is None
+
+
+@pytest.mark.parametrize("dtype", [ob.BF16, ob.F16])
+def test_bias_gradient_is_bit_exact(moe, dtype):
+    """One thread per column adds the rows in ascending order, as the oracle does: the same fp32 sums, bit for bit."""
+    S, H, I, E, k, cf, skew = CASES[1]
+    cfg, rng, count, offset = routed_case(S, H, I, E, k, dtype, seed=91, cf=cf, skew=skew)
+    layer = moe.MoELayer(product_config(cfg))
+    kind = KIND[dtype]
+    for N in (H, I):
+        dy = ob.from_f32(rng.standard_normal((S * k, N)).astype(np.float32), dtype)
+        got = from_device(layer.bias_grad(to_device(dy, kind), to_device(count, "i32"), to_device(offset, "i32")))
+        assert np.array_equal(got, ob.bias_grad(dy, count, offset, dtype))
+
+
+@pytest.mark.parametrize("dtype", [ob.BF16, ob.F16])
+def test_combine_backward_vs_oracle(moe, dtype):
+    cfg = ob.Cfg(S=257, H=320, I=128, E=5, k=3, dtype=dtype, act=ob.ACT_RELU, drop=1, capacity_factor=0.8)
+    rng = np.random.default_rng(41)
+    logits = rng.standard_normal((cfg.S, cfg.E)).astype(np.float32)
+    idx, w = ob.topk(logits, cfg.k, cfg.gate_fn, cfg.norm_topk)
+    r = ob.route_slots(idx, cfg.E, cfg.drop, cfg.capacity)
+    assert (r["pair_row"] < 0).any()
+    layer = moe.MoELayer(product_config(cfg))
+    kind = KIND[dtype]
+    y = ob.from_f32(rng.standard_normal((cfg.S * cfg.k, cfg.H)).astype(np.float32), dtype)
+    dout = ob.from_f32(rng.standard_normal((cfg.S, cfg.H)).astype(np.float32), dtype)
+    want_dy, want_dw = ob.combine_backward(dout, y, r["pair_row"], w, dtype)
+    dy, dw = layer.combine_backward(to_device(dout, kind), to_device(y, kind), to_device(r["pair_row"], "i32"), to_device(w, "f32"))
+    if dtype == ob.BF16:
+        assert np.array_equal(from_device(dy), want_dy)        # one multiplication and one rounding per element
+    else:   # fp16: the compiler multiplies and narrows in one mixed-precision instruction (one rounding), the oracle
+        # rounds the fp32 product first; on near-ties they differ by one fp16 ulp
+        got, ref = ob.to_f32(from_device(dy), dtype), ob.to_f32(want_dy, dtype)
+        assert np.abs(got - ref).max() <= 2.0 ** -10 * np.abs(ref).max()
+        assert (from_device(dy) != want_dy).mean() < 1e-3
+    assert np.abs(from_device(dw) - want_dw).max() <= 1e-5 * max(np.abs(want_dw).max(), 1.0)
+    assert not from_device(dw)[r["pair_row"] < 0].any()

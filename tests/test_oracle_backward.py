@@ -101,3 +101,77 @@ def test_adjoint_identity_ties_forward_to_both_gradients():
     lhs = float((dy.astype(np.float64) * y).sum())
     assert lhs == float((dw.astype(np.float64) * w).sum()) == float((dx.astype(np.float64) * x).sum())
     assert lhs != 0.0
+
+
+def _f64_act(u, g, act):
+    from scipy.special import erf
+    if act == ob.ACT_SWIGLU:
+        return g / (1 + np.exp(-g)) * u
+    if act == ob.ACT_GELU:
+        return 0.5 * u * (1 + erf(u / np.sqrt(2)))
+    return np.maximum(u, 0)
+
+
+@pytest.mark.parametrize("act", [ob.ACT_RELU, ob.ACT_GELU, ob.ACT_SWIGLU])
+@pytest.mark.parametrize("dtype", [ob.F32, ob.BF16, ob.F16])
+def test_act_backward_against_central_differences(dtype, act):
+    """d act / d u (and d g) from central differences of the activation in float64: an independent derivative."""
+    rng = np.random.default_rng(21)
+    shape = (9, 40)
+    u = ob.from_f32(rng.standard_normal(shape).astype(np.float32) * 2, dtype)
+    g = ob.from_f32(rng.standard_normal(shape).astype(np.float32) * 2, dtype)
+    dh = ob.from_f32(rng.standard_normal(shape).astype(np.float32), dtype)
+    uf, gf, df = (ob.to_f32(v, dtype).astype(np.float64) for v in (u, g, dh))
+    if act == ob.ACT_RELU:
+        uf = np.where(np.abs(uf) < 1e-3, 0.5, uf)      # keep the finite difference off the kink
+        u = ob.from_f32(uf.astype(np.float32), dtype); uf = ob.to_f32(u, dtype).astype(np.float64)
+    du, dg = ob.act_backward(dh, u, g if act == ob.ACT_SWIGLU else None, dtype, act)
+    eps = 1e-6
+    want_du = df * (_f64_act(uf + eps, gf, act) - _f64_act(uf - eps, gf, act)) / (2 * eps)
+    tol = {ob.F32: 2e-5, ob.BF16: 2.0 ** -8, ob.F16: 2.0 ** -10}[dtype]
+    assert np.abs(ob.to_f32(du, dtype) - want_du).max() <= tol * max(np.abs(want_du).max(), 1) + 1e-6
+    if act == ob.ACT_SWIGLU:
+        want_dg = df * (_f64_act(uf, gf + eps, act) - _f64_act(uf, gf - eps, act)) / (2 * eps)
+        assert np.abs(ob.to_f32(dg, dtype) - want_dg).max() <= tol * max(np.abs(want_dg).max(), 1) + 1e-6
+        assert np.abs(ob.to_f32(dg, dtype) - want_du).max() > 0.05      # du and dg swapped would show
+    else:
+        assert dg is None
+
+
+@pytest.mark.parametrize("dtype", [ob.F32, ob.BF16])
+def test_bias_grad_is_the_column_sum_per_expert(dtype):
+    rng = np.random.default_rng(22)
+    E, N = 4, 24
+    _, dy, _, _, counts, offset = packed_case(rng, E, N, 8, [7, 0, 130, 2], dtype)
+    got = ob.to_f32(ob.bias_grad(dy, counts, offset, dtype), dtype)
+    dyf = ob.to_f32(dy, dtype).astype(np.float64)
+    want = np.stack([dyf[rows_of(e, counts, offset)].sum(0) for e in range(E)])
+    tol = {ob.F32: 1e-5, ob.BF16: 2.0 ** -8}[dtype]
+    assert np.abs(got - want).max() <= tol * np.abs(want).max() + 1e-6
+    assert not got[1].any()
+
+
+def test_combine_backward_is_the_adjoint_of_the_combine():
+    """<dout, combine(y, w)> must equal <dy, y> and, per pair, dw = d<dout, out>/dw: exact with small integers."""
+    rng = np.random.default_rng(23)
+    S, k, H, rows = 12, 2, 16, 30
+    pair_row = rng.permutation(rows)[:S * k].reshape(S, k).astype(np.int32)
+    pair_row[3, 1] = -1; pair_row[7, 0] = -1                         # two dropped pairs
+    w = rng.integers(-2, 3, (S, k)).astype(np.float32)
+    y = rng.integers(-3, 4, (rows, H)).astype(np.float32)
+    dout = rng.integers(-3, 4, (S, H)).astype(np.float32)
+    out = ob.combine(y, pair_row, w, H, ob.F32)
+    dy, dw = ob.combine_backward(dout, y, pair_row, w, ob.F32)
+    want_out = np.zeros((S, H))
+    for t in range(S):
+        for r in range(k):
+            if pair_row[t, r] >= 0:
+                want_out[t] += w[t, r] * y[pair_row[t, r]]
+    assert np.array_equal(out, want_out.astype(np.float32))      # the forward this is the adjoint of
+    assert float((dout * want_out).sum()) == float((dy.astype(np.float64) * y).sum())
+    for t in range(S):
+        for r in range(k):
+            want = float(dout[t] @ y[pair_row[t, r]]) if pair_row[t, r] >= 0 else 0.0
+            assert dw[t, r] == want
+    used = set(int(v) for v in pair_row.reshape(-1) if v >= 0)
+    assert not dy[[i for i in range(rows) if i not in used]].any()

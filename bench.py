@@ -115,7 +115,7 @@ def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False, balanced_
     ffn = stats(samples["ffn"][-steps:])
     queue = layer.ffn_mode == 2   # one launch of the task-queue kernel; otherwise one launch per projection
     fp8 = c.torch_dtype == api.DTYPE_FP8
-    if fp8:
+    if w.bound == "hbm" and fp8:
         active = int((cnt > 0).sum())
         nbytes = wl.fp8_ffn_bytes(c, active, kept)
         roof = {"bound": "hbm", "achieved": nbytes / (ffn["mean"] * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
@@ -126,7 +126,8 @@ def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False, balanced_
     else:
         roof = {"bound": "mfma", "achieved": flops / (ffn["mean"] * 1e-3) / 1e12,
                 "peak": PEAK_F32_TFLOPS if c.torch_dtype == api.DTYPE_F32 else PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                "kernel": "ffn_persistent_kernel" if queue else "ffn_tiled_kernel x2", "algorithmic_flops": flops}
+                "kernel": (("ffn_persistent_fp8_tile_kernel" if queue else "ffn_tiled_fp8_tile_kernel x2") if fp8 else
+                           ("ffn_persistent_kernel" if queue else "ffn_tiled_kernel x2")), "algorithmic_flops": flops}
         roof["layer_frac"] = layer_flops / (ms_per_step * 1e-3) / 1e12 / roof["peak"]
     roof["frac"] = roof["achieved"] / roof["peak"]
     roof["kernel_ms"] = ffn["mean"]
@@ -357,8 +358,7 @@ def main():
     peaks = moe.measured_peaks()
     roof = res["roofline"]
     # for the MFMA bound: the issue-only rate on random operands (the power limit lowers the clock on real data)
-    fp8 = main_w.config.torch_dtype == api.DTYPE_FP8
-    roof["measured_peak"] = peaks["hbm_read_gbs"] if fp8 else peaks["mfma_bf16_tflops_random_operands"]
+    roof["measured_peak"] = peaks["hbm_read_gbs"] if roof["bound"] == "hbm" else peaks["mfma_bf16_tflops_random_operands"]
     roof["frac_of_measured_peak"] = roof["achieved"] / roof["measured_peak"]
 
     backward = None

@@ -35,6 +35,11 @@ int fp8_block_m();
 int fp8_block_n0();
 int fp8_block_n1();
 int ffn_persistent_occupancy_fp8();
+hipError_t launch_ffn_fp8_tile(const FfnArgs&, int max_mtiles, int nnt0, int nnt1, int blocks, hipStream_t);
+int fp8_tile_block_m();
+int fp8_tile_block_n0();
+int fp8_tile_block_n1();
+int ffn_persistent_occupancy_fp8_tile();
 
 namespace {
 
@@ -136,9 +141,16 @@ FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E) {
         p.nnt0 = sw ? ceil_div(I, f32_block_n() / 2) : ceil_div(I, f32_block_n());
         p.nnt1 = ceil_div(H, f32_block_n());
     } else if (dtype == MOE_DTYPE_FP8_E4M3_B128) {
-        p.block_m = fp8_block_m();
-        p.nnt0 = ceil_div(I, fp8_block_n0());
-        p.nnt1 = ceil_div(H, fp8_block_n1());
+        // 0: weight streamer over 16-token row blocks (decode); 1: 128 x 128 tile GEMM once the experts see enough
+        // rows for a weight tile to be reused from LDS instead of being fetched again per 16 rows
+        p.tile = A / (E > 0 ? E : 1) >= kFp8TileRowsPerExpert ? 1 : 0;
+        if (const char* env = getenv("MOE355_FP8_TILE")) {   // tuning knob
+            const int v = atoi(env);
+            if (v == 0 || v == 1) p.tile = v;
+        }
+        p.block_m = p.tile ? fp8_tile_block_m() : fp8_block_m();
+        p.nnt0 = ceil_div(I, p.tile ? fp8_tile_block_n0() : fp8_block_n0());
+        p.nnt1 = ceil_div(H, p.tile ? fp8_tile_block_n1() : fp8_block_n1());
     } else {
         p.tile = bf16_tile(A, E, H, I, sw);
         p.block_m = bf16_block_m(p.tile);
@@ -334,8 +346,9 @@ int moe_create(const moe_config* cfg, moe_handle** out) {
     }
     h->arch.persistent_blocks = prop.multiProcessorCount * per_cu;
     // One task queue per XCD for the MFMA-bound bf16 tiles, whose operand tiles are then shared in that XCD's L2;
-    // the f32 and fp8 paths keep a single queue.
-    h->queue_groups = (cfg->torch_dtype == MOE_DTYPE_BF16 || cfg->torch_dtype == MOE_DTYPE_FP16) ? h->arch.xcds : 1;
+    // so does the e4m3 tile GEMM; the f32 path and the e4m3 weight streamer keep a single queue.
+    h->queue_groups = (cfg->torch_dtype == MOE_DTYPE_BF16 || cfg->torch_dtype == MOE_DTYPE_FP16 ||
+                       (cfg->torch_dtype == MOE_DTYPE_FP8_E4M3_B128 && d.plan.tile)) ? h->arch.xcds : 1;
     if (const char* env = getenv("MOE355_QUEUE_GROUPS")) {   // tuning knob; never more queues than XCDs
         const int v = atoi(env);
         if ((v == 1 || v == 2 || v == 4 || v == 8) && v <= h->arch.xcds) h->queue_groups = v;
@@ -575,8 +588,8 @@ int forward_on(moe_handle* h, const void* x, const moe_weights* w, void* out, co
     }
     const int mode = resolved_ffn_mode(h);
     if (fp8) {
-        e = launch_ffn_fp8(fa, d.max_mtiles, d.plan.nnt0, d.plan.nnt1,
-                           mode == MOE_FFN_PERSISTENT ? h->arch.persistent_blocks : 0, st);
+        e = (d.plan.tile ? launch_ffn_fp8_tile : launch_ffn_fp8)(fa, d.max_mtiles, d.plan.nnt0, d.plan.nnt1,
+                                                                 mode == MOE_FFN_PERSISTENT ? h->arch.persistent_blocks : 0, st);
     } else if (mode == MOE_FFN_PERSISTENT) {
         e = launch_ffn_persistent(fa, c.torch_dtype, d.plan, h->arch.persistent_blocks, st);
     } else {
@@ -819,7 +832,8 @@ hipError_t launch_ffn_persistent(const FfnArgs& a, int dtype, const FfnPlan& p, 
 
 int ffn_persistent_blocks(int dtype, int tile, int compute_units) {
     if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32) return compute_units * 4;
-    if (dtype == MOE_DTYPE_FP8_E4M3_B128) return compute_units * ffn_persistent_occupancy_fp8();
+    if (dtype == MOE_DTYPE_FP8_E4M3_B128)
+        return compute_units * (tile ? ffn_persistent_occupancy_fp8_tile() : ffn_persistent_occupancy_fp8());
     return compute_units * ffn_persistent_occupancy_bf16(tile);
 }
 

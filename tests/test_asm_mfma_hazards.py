@@ -102,7 +102,7 @@ def test_no_accumulator_access_behind_asm_mfma():
 
 
 @pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
-@pytest.mark.parametrize("source", ["ffn_bf16.hip", "ffn_f32.hip", "ffn_fp8.hip"])
+@pytest.mark.parametrize("source", ["ffn_bf16.hip", "ffn_f32.hip", "ffn_fp8.hip", "ffn_fp8_tile.hip"])
 def test_phase0_results_are_complete_before_they_are_signalled(source):
     """The hand-off of the intermediate rows between workgroups: in signal_phase0_done every wavefront must wait for
     its own stores (s_waitcnt vmcnt(0)) before the workgroup barrier and the counter increment that publishes the
@@ -116,3 +116,46 @@ def test_phase0_results_are_complete_before_they_are_signalled(source):
     # the wait written out in the source (the calling convention's wait at the function's entry does not count)
     waits = [i for i, x in enumerate(body) if x == "s_waitcnt vmcnt(0)"]
     assert waits and waits[0] < barrier < atomic, body[:20]
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
+def test_fp8_tile_barriers_sit_behind_their_waits():
+    """The e4m3 tile GEMM (ffn_fp8_tile.hip) meets at a bare s_barrier and spells its waits out in front of it: between
+    the wait that covers the direct-to-LDS loads and this wavefront's LDS traffic (s_waitcnt vmcnt(<=2) lgkmcnt(0)) and
+    the barrier the compiler may not have placed an LDS access or a load of either kind; its slab loops hold no spill;
+    and the weight bytes are awaited with the count that leaves only the token-row loads issued since (vmcnt(4))."""
+    text = _assembly("ffn_fp8_tile.hip")
+    kernels = re.findall(r"\n(_ZN6moe355\w*fp8_tile_kernel\w*):[^\n]*\n(.*?)\n\s*s_endpgm", text, re.S)
+    assert len(kernels) == 2
+    for name, body in kernels:
+        lines = [x.strip() for x in body.split("\n") if x.strip() and not x.strip().startswith(";")]
+        mfma = [i for i, x in enumerate(lines) if x.startswith("v_mfma")]
+        assert len(mfma) >= 6 * 32, name
+        checked = 0
+        for i, x in enumerate(lines):
+            if not x.startswith("s_barrier") or not any(abs(i - m) < 60 for m in mfma):
+                continue
+            between = []
+            for back in range(i - 1, max(i - 40, 0), -1):
+                w = re.match(r"s_waitcnt vmcnt\((\d+)\) lgkmcnt\(0\)", lines[back])
+                if w:
+                    assert int(w.group(1)) <= 2, (name, lines[back])
+                    break
+                between.append(lines[back])
+            else:
+                continue        # a barrier of the queue bookkeeping (pop, dependency wait), not of the slab pipeline
+            assert not [b for b in between if b.startswith(("ds_", "global_load", "buffer_load", "scratch_"))], (name, between)
+            checked += 1
+        assert checked >= 6, (name, checked)      # prologue + two per steady-state block + two of the peeled block, twice
+        assert any(x == "s_waitcnt vmcnt(4)" for x in lines), name
+        # no spill traffic between the first and the last MFMA of a slab loop: loops are the label .. back-branch ranges
+        labels = {x.split(":")[0]: i for i, x in enumerate(lines) if re.match(r"\.LBB\d+_\d+:", x)}
+        slab_loops = 0
+        for i, x in enumerate(lines):
+            j = re.match(r"s_cbranch_\w+ (\.LBB\d+_\d+)", x)
+            if j and j.group(1) in labels and labels[j.group(1)] < i:
+                loop = lines[labels[j.group(1)]:i]
+                if sum(y.startswith("v_mfma") for y in loop) >= 32 and sum(y.startswith("s_barrier") for y in loop) == 2:
+                    assert not [y for y in loop if y.startswith("scratch_")], (name, "spill in the slab loop")
+                    slab_loops += 1
+        assert slab_loops >= 2, name      # the full-block loop and the partial-block loops

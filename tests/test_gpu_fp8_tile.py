@@ -1,0 +1,81 @@
+"""e4m3-weight layers with many rows per expert: the 128 x 128 tile GEMM (csrc/ffn_fp8_tile.hip) against the CPU
+oracle, against the weight streamer on the same inputs, and across its two schedules."""
+import numpy as np
+import pytest
+
+from oracle import binding as ob
+from helpers import OUT_TOL, from_device, max_rel_err, product_config, upload_inputs
+from test_gpu_layer import FFN_PERSISTENT, FFN_TILED, check_routing
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = {
+    # full blocks and a ragged last block per expert, two k blocks up / three down
+    "few_experts": ob.Cfg(S=700, H=256, I=384, E=4, k=2, act=ob.ACT_SWIGLU, dtype=ob.FP8, gate_fn=ob.GATE_SIGMOID, drop=0),
+    # capacity drops, biases, experts with a handful of rows next to experts with several blocks
+    "skew_drop_bias": ob.Cfg(S=1500, H=384, I=256, E=12, k=3, act=ob.ACT_SWIGLU, dtype=ob.FP8, gate_fn=ob.GATE_SOFTMAX,
+                             drop=1, capacity_factor=1.0, zipf_bias=True),
+    # shortest K (one k block) in the up projection, one expert, exactly full blocks
+    "one_expert_short_k": ob.Cfg(S=256, H=128, I=512, E=1, k=1, act=ob.ACT_SWIGLU, dtype=ob.FP8, norm_topk=0, drop=0),
+    # fewer rows than one block everywhere (the tile forced onto a decode-sized layer)
+    "tiny_rows": ob.Cfg(S=40, H=256, I=128, E=8, k=2, act=ob.ACT_SWIGLU, dtype=ob.FP8, gate_fn=ob.GATE_SIGMOID, drop=0),
+}
+
+
+def _run(cfg, inp, mode, tile, monkeypatch, calls=1):
+    import torch
+    import cuplayground_amd as moe
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    monkeypatch.setenv("MOE355_FP8_TILE", str(tile))
+    layer = moe.MoELayer(product_config(cfg), ffn_mode=mode)
+    assert layer.plan["block_rows"] == (128 if tile else 16)
+    dev = upload_inputs(cfg, inp)
+    routing = layer.new_routing()
+    out = torch.full((cfg.S, cfg.H), float("nan"), dtype=layer.act_dtype, device="cuda")
+    for _ in range(calls):
+        layer.forward(dev["x"], dev, out=out, routing=routing)
+    torch.cuda.synchronize()
+    layer.task_counts()
+    res = {k: from_device(v) for k, v in routing.items()}
+    res["out"] = ob.to_f32(from_device(out), cfg.act_dtype)
+    layer.close()
+    return res
+
+
+@pytest.mark.parametrize("mode", [FFN_TILED, FFN_PERSISTENT], ids=["tiled", "persistent"])
+@pytest.mark.parametrize("name", sorted(SHAPES))
+def test_tile_gemm_vs_oracle_and_streamer(name, mode, monkeypatch):
+    cfg = SHAPES[name]
+    inp = ob.make_inputs(cfg, seed=29, with_bias="bias" in name)
+    want = ob.forward(cfg, inp)
+    ref = ob.to_f32(want["out"], cfg.act_dtype)
+    got = _run(cfg, inp, mode, 1, monkeypatch, calls=2)
+    check_routing(got, want)
+    assert not np.isnan(got["out"]).any()
+    assert max_rel_err(got["out"], ref) <= OUT_TOL[ob.FP8]
+    assert not got["out"][(want["slot"] < 0).all(axis=1)].any()
+    # the streamer computes the same block-scaled sums in another order: both round h and y to bf16 once
+    stream = _run(cfg, inp, mode, 0, monkeypatch)
+    assert max_rel_err(got["out"], stream["out"]) <= 1e-2
+
+
+@pytest.mark.parametrize("name", sorted(SHAPES))
+def test_tile_gemm_schedules_agree_bit_for_bit(name, monkeypatch):
+    cfg = SHAPES[name]
+    inp = ob.make_inputs(cfg, seed=31, with_bias="bias" in name)
+    a = _run(cfg, inp, FFN_TILED, 1, monkeypatch)
+    b = _run(cfg, inp, FFN_PERSISTENT, 1, monkeypatch)
+    assert np.array_equal(a["out"], b["out"])
+    monkeypatch.setenv("MOE355_FUSED_COMBINE", "1")
+    c = _run(cfg, inp, FFN_PERSISTENT, 1, monkeypatch)
+    assert np.array_equal(a["out"], c["out"])
+
+
+def test_plan_follows_rows_per_expert():
+    """Decode-sized layers keep the weight streamer, prefill-sized ones take the tile."""
+    import cuplayground_amd as moe
+    small = moe.MoELayer(product_config(ob.Cfg(S=64, H=256, I=256, E=32, k=8, act=ob.ACT_SWIGLU, dtype=ob.FP8)))
+    big = moe.MoELayer(product_config(ob.Cfg(S=2048, H=256, I=256, E=8, k=2, act=ob.ACT_SWIGLU, dtype=ob.FP8)))
+    assert small.plan["block_rows"] == 16 and big.plan["block_rows"] == 128
+    assert big.plan["col_tiles_up"] == 256 // 64 and big.plan["col_tiles_down"] == 256 // 128
+    small.close(); big.close()

@@ -81,6 +81,8 @@ def test_route_drops_out_of_range_expert_ids(moe):
     ("bf16", ob.Cfg(S=700, H=256, I=384, E=4, k=2, act=ob.ACT_SWIGLU, dtype=ob.BF16, drop=0)),
     ("f32", ob.Cfg(S=200, H=128, I=128, E=4, k=1, act=ob.ACT_GELU, dtype=ob.F32, norm_topk=0, drop=0)),
     ("fp8", ob.Cfg(S=64, H=256, I=256, E=8, k=2, act=ob.ACT_SWIGLU, dtype=ob.FP8, gate_fn=ob.GATE_SIGMOID, drop=0)),
+    # enough rows per expert for the e4m3 tile GEMM instead of the weight streamer
+    ("fp8_tile", ob.Cfg(S=600, H=256, I=256, E=4, k=2, act=ob.ACT_SWIGLU, dtype=ob.FP8, gate_fn=ob.GATE_SIGMOID, drop=0)),
 ])
 @pytest.mark.parametrize("fused_combine", ["0", "1"])
 def test_expired_dependency_wait_poisons_the_output_and_is_reported(moe, name, cfg, fused_combine, monkeypatch):

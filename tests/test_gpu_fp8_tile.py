@@ -79,3 +79,36 @@ def test_plan_follows_rows_per_expert():
     assert small.plan["block_rows"] == 16 and big.plan["block_rows"] == 128
     assert big.plan["col_tiles_up"] == 256 // 64 and big.plan["col_tiles_down"] == 256 // 128
     small.close(); big.close()
+
+
+def test_prefill_sized_layer_on_a_stratified_sample(monkeypatch):
+    """A layer big enough to fill the queue kernel several times over (8 experts of about 1024 rows, 72 row blocks x
+    104 column tiles): routing in full, the output on each expert's first row, tail block and block boundaries plus
+    random tokens, and the two schedules bit for bit."""
+    import torch
+    import cuplayground_amd as moe
+    from test_gpu_fullsize import stratified_tokens
+    cfg = ob.Cfg(S=4096, H=2048, I=5632, E=8, k=2, act=ob.ACT_SWIGLU, dtype=ob.FP8, gate_fn=ob.GATE_SOFTMAX, drop=0)
+    inp = ob.make_inputs(cfg, seed=42)
+    want = ob.route(cfg, inp)
+    layer = moe.MoELayer(product_config(cfg), ffn_mode=FFN_PERSISTENT)
+    assert layer.plan["block_rows"] == 128
+    dev = upload_inputs(cfg, inp)
+    routing = layer.new_routing()
+    out = layer.forward(dev["x"], dev, routing=routing)
+    torch.cuda.synchronize()
+    layer.task_counts()
+    check_routing({k: from_device(v) for k, v in routing.items()}, want)
+    chosen, strata, rng = stratified_tokens(cfg, want, 128)
+    tokens = np.unique(np.concatenate([chosen, rng.choice(cfg.S, size=192, replace=False)])).astype(np.int32)
+    print("strata", len(strata), "tokens checked", tokens.size, flush=True)
+    ref = ob.to_f32(ob.forward_tokens(cfg, inp, want["topk_idx"], want["topk_w"], want["slot"], tokens), cfg.act_dtype)
+    o = out.float().cpu().numpy()
+    err = max_rel_err(o[tokens], ref)
+    print("sampled max rel err", err, flush=True)
+    assert err <= OUT_TOL[ob.FP8], err
+    assert np.isfinite(o).all()
+    layer.set_ffn_mode(FFN_TILED)
+    out2 = layer.forward(dev["x"], dev)
+    assert torch.equal(out, out2)
+    layer.close()

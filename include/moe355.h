@@ -270,7 +270,8 @@ int moe_expert_wgrad(moe_handle* h, const void* dy_rows, const void* a_rows, con
  *   and GELU (Phi(u) + u phi(u)); for SwiGLU, where h = silu(g) * u, du = dh * silu(g) and dg = dh * u * s * (1 + g (1 - s))
  *   with s = sigmoid(g).  u_rows / g_rows are the projections before the activation (moe_expert_gemm with
  *   MOE_ACT_NONE); g_rows and dg_rows are given exactly when the layer is SwiGLU.
- * moe_bias_grad: db[e, n] = sum over expert e's rows, in ascending row order, of dy_rows[r, n]; N is H or I.
+ * moe_bias_grad: db[e, n] = sum over expert e's rows, in ascending row order, of dy_rows[r, n], stored in the layer's
+ *   16-bit type like the bias it belongs to; N is H or I, db is [E, N].
  * moe_combine_backward: the adjoint of moe_combine: dy_rows[pair_row[t,r], :] = topk_w[t,r] * dout[t, :] and
  *   dw[t,r] = <dout[t, :], y_rows[pair_row[t,r], :]> (0 for a dropped pair); rows of dy_rows that no pair maps to are
  *   left untouched. */

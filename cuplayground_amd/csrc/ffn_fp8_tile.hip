@@ -110,7 +110,6 @@ __device__ __forceinline__ void tile_mainloop(const TileTask& p, unsigned char* 
     }
 
     const int wrow = __builtin_amdgcn_readfirstlane(prow & ~7);
-    const int KT = p.K / PBK;                                     // even: K is a multiple of 128
     auto issue_a = [&](int kt) {
         unsigned char* sa = smem + (kt & 1) * PSTAGE;
 #pragma unroll

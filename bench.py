@@ -32,18 +32,26 @@ PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
 # script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter showed for a 1 GiB
 # device copy in the same run (--calibrate-copy).  Each entry names the summary under profiles/ it comes from and the
 # digest of the kernel sources it was collected with: when the sources have changed since, the figure is withheld.
-KERNEL_SOURCES = ("ffn_bf16.hip", "ffn_bf16_slab_steady.inc", "ffn_fp8.hip", "ffn_common.hpp", "route.hip")
+BF16_SOURCES = ("ffn_bf16.hip", "ffn_bf16_slab_steady.inc", "ffn_common.hpp", "route.hip")
+FP8_SOURCES = ("ffn_fp8.hip", "ffn_common.hpp", "route.hip")
+FP8_TILE_SOURCES = ("ffn_fp8_tile.hip", "ffn_common.hpp", "route.hip")
 MEASURED_TRAFFIC = {
-    "mixtral": {"bytes": 19.30e9, "kernel_digest": "e9c99de4a735",
+    "mixtral": {"bytes": 19.03e9, "sources": BF16_SOURCES, "kernel_digest": "68bd68dadf7c",
                 "profile": "profiles/ffn_persistent_kernel_bf16_mixtral_c3_hbm_traffic.txt"},
-    "decode_fp8": {"bytes": 9.920e9, "kernel_digest": "e9c99de4a735",
+    "mid": {"bytes": 0.807e9, "sources": BF16_SOURCES, "kernel_digest": "68bd68dadf7c",
+            "profile": "profiles/ffn_persistent_kernel_bf16_mid_c2_hbm_traffic.txt"},
+    "finegrained": {"bytes": 3.352e9, "sources": BF16_SOURCES, "kernel_digest": "68bd68dadf7c",
+                    "profile": "profiles/ffn_persistent_kernel_bf16_finegrained_c4_hbm_traffic.txt"},
+    "decode_fp8": {"bytes": 9.886e9, "sources": FP8_SOURCES, "kernel_digest": "baf522b83fbe",
                    "profile": "profiles/ffn_persistent_fp8_kernel_decode_c5_hbm_traffic.txt"},
+    "prefill_fp8": {"bytes": 26.49e9, "sources": FP8_TILE_SOURCES, "kernel_digest": "099b450c6351",
+                    "profile": "profiles/ffn_persistent_fp8_tile_kernel_prefill_fp8_hbm_traffic.txt"},
 }
 
 
-def kernel_digest():
+def kernel_digest(sources=BF16_SOURCES):
     h = hashlib.sha256()
-    for name in KERNEL_SOURCES:
+    for name in sources:
         with open(os.path.join(ROOT, "cuplayground_amd", "csrc", name), "rb") as f:
             h.update(f.read())
     return h.hexdigest()[:12]
@@ -133,8 +141,8 @@ def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False, balanced_
     roof["kernel_ms"] = ffn["mean"]
     roof["kernel_ms_median"] = ffn["median"]
     roof["kernel_ms_min"] = ffn["min"]
-    digest = kernel_digest()
     t = MEASURED_TRAFFIC.get(name)
+    digest = kernel_digest(t["sources"]) if t else None
     if queue and t and t["kernel_digest"] == digest:
         roof["traffic"] = t["bytes"]
         roof["traffic_source"] = "%s (kernel sources %s)" % (t["profile"], digest)

@@ -1021,7 +1021,7 @@ __global__ __launch_bounds__(P::THREADS) void ffn_persistent_ring_kernel(FfnArgs
             __syncthreads();                    // also: every wavefront is done with the stages
             nid = __builtin_amdgcn_readfirstlane(s_next[0]);
             if (nid < ids) {
-                const Task q = decode_task(a.seg_queue, nseg, a.mtiles, nid, cur.group, groups, nnt0);
+                const Task q = decode_task(a.seg_queue, nseg, a.mtiles, nid, cur.group, groups, nnt0, a.row_chunk);
                 n_valid = q.valid; n_ph = q.phase; n_ex = q.expert; n_mt = q.mtile; n_nt = q.ntile; n_row0 = q.row0; n_rows = q.rows;
                 if (n_valid) {
                     int ready = 1;

@@ -30,8 +30,13 @@ struct Task {
 
 // Finds the segment holding id `id` of queue group `group` (segments are sorted by begin, possibly empty) and
 // decodes it.  All arguments are wavefront-uniform, so the loads are scalar.
+//
+// Order inside a segment (ids of one group): row blocks fastest -- consecutive ids, popped by workgroups that run side by
+// side, share one column tile's weights.  With row_chunk R > 0 the expert's row blocks are taken R at a time: all
+// column tiles of the first R row blocks, then of the next R, ...; the workgroups of an XCD then hold fewer row blocks
+// and more column tiles at a time (for kernels whose token rows cost more L2 space than their weight rows).
 __device__ __forceinline__ Task decode_task(const Segment* __restrict__ segs, int nseg, const MTile* __restrict__ mtiles,
-                                            int id, int group, int groups, int nnt0) {
+                                            int id, int group, int groups, int nnt0, int row_chunk = 0) {
     int lo = 0, hi = nseg - 1;
     while (lo < hi) {   // last segment with begin <= id
         const int mid = (lo + hi + 1) >> 1;
@@ -42,12 +47,22 @@ __device__ __forceinline__ Task decode_task(const Segment* __restrict__ segs, in
     Task t;
     t.phase = s.phase;
     t.expert = s.expert;
-    const int j = local / s.nmt;
+    int j, mb;
+    if (row_chunk > 0 && row_chunk < s.nmt) {
+        const int per_chunk = row_chunk * ((s.nnt + groups - 1) / groups);   // ids of a full chunk
+        const int c = local / per_chunk, rem = local - c * per_chunk;
+        const int rc = min(row_chunk, s.nmt - c * row_chunk);               // the last chunk may be shorter
+        j = rem / rc;
+        mb = c * row_chunk + (rem - j * rc);
+    } else {
+        j = local / s.nmt;
+        mb = local - j * s.nmt;
+    }
     int first = group - s.rot;
     if (first < 0) first += groups;
     t.ntile = first + groups * j;
     t.valid = t.ntile < s.nnt;
-    t.mtile = s.mt0 + (local - j * s.nmt);
+    t.mtile = s.mt0 + mb;
     const MTile m = mtiles[t.mtile];
     t.row0 = m.row0;
     t.rows = m.rows;
@@ -114,7 +129,7 @@ __device__ __forceinline__ bool next_task(const FfnArgs& a, QueueCursor& c, int*
             c.group = c.group + 1 == a.groups ? 0 : c.group + 1;
             continue;
         }
-        t = decode_task(a.seg_queue, nseg, a.mtiles, id, c.group, a.groups, nnt0);
+        t = decode_task(a.seg_queue, nseg, a.mtiles, id, c.group, a.groups, nnt0, a.row_chunk);
         c.last_id = id;
         if (t.valid) return true;
     }
@@ -125,7 +140,7 @@ __device__ __forceinline__ bool next_task(const FfnArgs& a, QueueCursor& c, int*
 __device__ __forceinline__ bool tiled_task(const FfnArgs& a, int phase, int b, Task& t) {
     const int group = b % a.groups, id = b / a.groups;
     if (id >= (phase ? a.q->ids_phase1 : a.q->ids_phase0)) return false;
-    t = decode_task(phase ? a.seg_phase1 : a.seg_phase0, a.E, a.mtiles, id, group, a.groups, a.seg_phase0[0].nnt);
+    t = decode_task(phase ? a.seg_phase1 : a.seg_phase0, a.E, a.mtiles, id, group, a.groups, a.seg_phase0[0].nnt, a.row_chunk);
     return t.valid;
 }
 

@@ -92,6 +92,7 @@ struct FfnArgs {
     int32_t act;
     int32_t spin_limit;
     int32_t groups;             // queue groups the schedule was built for
+    int32_t row_chunk;          // order of a segment's tasks: 0 = row blocks fastest; R > 0 = R row blocks at a time, all column tiles of those, row blocks fastest inside
     uint32_t x_bytes, h_bytes, w_bytes;   // extents of x, h and one weight matrix (meaningful below 4 GiB)
     int64_t* wg_clock;          // queue kernels: [2 * workgroup] constant-rate clock at entry, [2 * workgroup + 1] at exit
     // Combine inside the FFN kernels (null `arrive`: the separate combine launch is used instead).

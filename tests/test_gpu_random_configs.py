@@ -1,5 +1,5 @@
 """Seeded random layer shapes crossed with the tuning knobs (tile, FFN mode, queue count, early start of the next
-task, combine inside the FFN kernels): every combination must match the CPU oracle -- routing bit for bit, output
+task, combine inside the FFN kernels, task order inside a queue segment, e4m3 streamer or tile): every combination must match the CPU oracle -- routing bit for bit, output
 within the dtype's bound -- because no knob is allowed to change what is computed."""
 import numpy as np
 import pytest
@@ -29,6 +29,8 @@ def _cases(n=36, seed=2024):
                      gate_fn=ob.GATE_SIGMOID if dtype == ob.FP8 else int(rng.integers(0, 2)), zipf_bias=bool(i % 3 == 0))
         knobs = dict(MOE355_TILE=str(int(rng.integers(0, 4))), MOE355_QUEUE_GROUPS=str(int(rng.choice([1, 2, 8]))),
                      MOE355_QUEUE_EARLY=str(int(rng.integers(0, 2))), MOE355_FUSED_COMBINE=str(int(rng.integers(0, 2))))
+        knobs["MOE355_ROW_CHUNK"] = str(i % 4)      # order of the tasks inside a queue segment (0: plain; drawn outside the seeded stream)
+        knobs["MOE355_FP8_TILE"] = str(i // 5 % 2)  # e4m3 layers: weight streamer or tile GEMM
         out.append(pytest.param(cfg, knobs, int(rng.integers(1, 3)), bool(rng.integers(0, 2)), id="case%02d" % i))
     return out
 

@@ -36,15 +36,15 @@ BF16_SOURCES = ("ffn_bf16.hip", "ffn_bf16_slab_steady.inc", "ffn_common.hpp", "r
 FP8_SOURCES = ("ffn_fp8.hip", "ffn_common.hpp", "route.hip")
 FP8_TILE_SOURCES = ("ffn_fp8_tile.hip", "ffn_common.hpp", "route.hip")
 MEASURED_TRAFFIC = {
-    "mixtral": {"bytes": 19.03e9, "sources": BF16_SOURCES, "kernel_digest": "68bd68dadf7c",
+    "mixtral": {"bytes": 19.37e9, "sources": BF16_SOURCES, "kernel_digest": "2dbcdc2654d6",
                 "profile": "profiles/ffn_persistent_kernel_bf16_mixtral_c3_hbm_traffic.txt"},
-    "mid": {"bytes": 0.807e9, "sources": BF16_SOURCES, "kernel_digest": "68bd68dadf7c",
+    "mid": {"bytes": 0.805e9, "sources": BF16_SOURCES, "kernel_digest": "2dbcdc2654d6",
             "profile": "profiles/ffn_persistent_kernel_bf16_mid_c2_hbm_traffic.txt"},
-    "finegrained": {"bytes": 3.352e9, "sources": BF16_SOURCES, "kernel_digest": "68bd68dadf7c",
+    "finegrained": {"bytes": 3.352e9, "sources": BF16_SOURCES, "kernel_digest": "2dbcdc2654d6",
                     "profile": "profiles/ffn_persistent_kernel_bf16_finegrained_c4_hbm_traffic.txt"},
-    "decode_fp8": {"bytes": 9.886e9, "sources": FP8_SOURCES, "kernel_digest": "baf522b83fbe",
+    "decode_fp8": {"bytes": 9.883e9, "sources": FP8_SOURCES, "kernel_digest": "ab362d972ea4",
                    "profile": "profiles/ffn_persistent_fp8_kernel_decode_c5_hbm_traffic.txt"},
-    "prefill_fp8": {"bytes": 26.49e9, "sources": FP8_TILE_SOURCES, "kernel_digest": "099b450c6351",
+    "prefill_fp8": {"bytes": 26.85e9, "sources": FP8_TILE_SOURCES, "kernel_digest": "3aa597eaefd2",
                     "profile": "profiles/ffn_persistent_fp8_tile_kernel_prefill_fp8_hbm_traffic.txt"},
 }
 
@@ -229,6 +229,49 @@ def to_host(d):
     return out
 
 
+def task_trace_summary(layer, dev, out):
+    """One more forward call with the queue kernel's per-task trace on: durations by projection and row-block fill,
+    the gaps between a workgroup's consecutive tasks, and how long workgroups sit idle behind their last task."""
+    import numpy as np
+    import torch
+    layer.enable_task_trace(1 << 17)
+    layer.forward(dev["x"], dev, out=out)
+    torch.cuda.synchronize()
+    rec = layer.task_trace()
+    layer.disable_task_trace()
+    dur = rec["end_us"] - rec["start_us"]
+    full = int(rec["rows"].max())
+    groups = []
+    for ph in (0, 1):
+        for lo, hi, label in ((full, full, "full"), (full // 2 + 1, full - 1, "more than half"), (1, full // 2, "at most half")):
+            m = (rec["phase"] == ph) & (rec["rows"] >= lo) & (rec["rows"] <= hi)
+            if m.any():
+                groups.append({"phase": ph, "rows": label, "tasks": int(m.sum()), "mean_us": round(float(dur[m].mean()), 2),
+                               "median_us": round(float(np.median(dur[m])), 2), "min_us": round(float(dur[m].min()), 2),
+                               "max_us": round(float(dur[m].max()), 2)})
+    gaps = {0: [], 1: []}
+    busy, idle_after, per_wg = [], [], []
+    end = float(rec["end_us"].max())
+    for w in np.unique(rec["workgroup"]):
+        r = np.sort(rec[rec["workgroup"] == w], order="start_us")
+        for a, b in zip(r[:-1], r[1:]):
+            gaps[int(b["phase"])].append(float(b["start_us"] - a["end_us"]))
+        busy.append(float((r["end_us"] - r["start_us"]).sum()))
+        idle_after.append(end - float(r["end_us"][-1]))
+        per_wg.append(len(r))
+    def st(v):
+        return None if not v else {"mean_us": round(float(np.mean(v)), 2), "median_us": round(float(np.median(v)), 2),
+                                   "max_us": round(float(np.max(v)), 2), "n": len(v)}
+    return {"tasks": int(len(rec)), "block_rows": full, "span_us": round(end, 1), "by_kind": groups,
+            "gap_before_up_task": st(gaps[0]), "gap_before_down_task": st(gaps[1]),
+            "workgroups": len(busy), "mean_busy_us": round(float(np.mean(busy)), 1),
+            "mean_idle_after_last_task_us": round(float(np.mean(idle_after)), 1),
+            "max_idle_after_last_task_us": round(float(np.max(idle_after)), 1),
+            "tasks_per_workgroup": [int(min(per_wg)), int(max(per_wg))],
+            "note": "one extra forward call with moe_set_task_trace on (two clock reads and one atomic per task); a "
+                    "down-projection task's dependency wait lies in its gap, not in its duration"}
+
+
 def cpu_leg(name, dev, out, routing, seconds, seed):
     """The CPU baseline (libtorch layer, then the oracle) on a bounded token sample, and the parity spot check of the
     GPU output against the oracle on the same sample.  The only part of this script that touches oracle/."""
@@ -344,6 +387,9 @@ def main():
     ap.add_argument("--backward", action="store_true",
                     help="also time the backward building blocks (data and weight gradients of both projections) on "
                          "the workload's routing; bf16 / fp16 workloads only")
+    ap.add_argument("--task-trace", action="store_true",
+                    help="also run one forward call with the queue kernel's per-task trace on and print its summary "
+                         "(durations by projection and row-block fill, gaps, idle tails)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy (a known-size reference for HBM byte counters)")
     args = ap.parse_args()
@@ -369,6 +415,9 @@ def main():
     roof["measured_peak"] = peaks["hbm_read_gbs"] if roof["bound"] == "hbm" else peaks["mfma_bf16_tflops_random_operands"]
     roof["frac_of_measured_peak"] = roof["achieved"] / roof["measured_peak"]
 
+    trace = None
+    if args.task_trace and layer.ffn_mode == 2:
+        trace = task_trace_summary(layer, dev, out)
     backward = None
     if args.backward:
         backward = measure_backward(layer, main_w.config, dev, routing, args.steps, args.warmup)
@@ -405,6 +454,7 @@ def main():
                    "tile_tasks": res["tile_tasks"], "row_blocks": res["row_blocks"],
                    "row_blocks_full": res["row_blocks_full"], "balanced_routing": bool(args.balanced_routing)},
         "queue_balance": res["queue_balance"],
+        "task_trace": trace,
         "tflops": res["tflops"],
         "stage_ms": res["stage_ms"], "stage_ms_median": res["stage_ms_median"],
         "device": {"name": arch["name"], "compute_units": arch["compute_units"], "xcds": arch["xcds"],

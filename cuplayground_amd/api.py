@@ -25,7 +25,7 @@ EXPORTS = (
     "moe_config_tokens", "moe_config_capacity", "moe_create", "moe_destroy", "moe_get_arch", "moe_get_plan",
     "moe_workspace_bytes",
     "moe_set_ffn_mode", "moe_get_ffn_mode", "moe_forward", "moe_forward_static", "moe_set_spin_limit", "moe_clear_stall", "moe_gate", "moe_router_stats", "moe_route", "moe_gemm_bias_act", "moe_combine",
-    "moe_set_stage_timing", "moe_get_stage_ms", "moe_get_stage_samples", "moe_get_task_counts", "moe_get_queue_balance", "moe_measure_mfma_tflops",
+    "moe_set_stage_timing", "moe_get_stage_ms", "moe_get_stage_samples", "moe_get_task_counts", "moe_get_queue_balance", "moe_task_trace_bytes", "moe_set_task_trace", "moe_get_task_trace", "moe_measure_mfma_tflops",
     "moe_measure_hbm_read_gbs", "moe_quant_block128", "moe_backward_scratch_bytes", "moe_transpose", "moe_expert_gemm",
     "moe_expert_wgrad", "moe_act_backward", "moe_bias_grad", "moe_combine_backward", "moe_last_hip_error", "moe_status_string",
     "moe_version",
@@ -105,6 +105,10 @@ def load_library():
     L.moe_get_task_counts.argtypes = [vp, vp, vp, C.POINTER(i64), C.POINTER(i64)]
     L.moe_get_queue_balance.argtypes = [vp, vp, vp, C.POINTER(i32), C.POINTER(C.c_float), C.POINTER(C.c_float),
                                         C.POINTER(C.c_float)]
+    L.moe_task_trace_bytes.argtypes = [C.c_int64]
+    L.moe_task_trace_bytes.restype = C.c_size_t
+    L.moe_set_task_trace.argtypes = [vp, vp, C.c_size_t]
+    L.moe_get_task_trace.argtypes = [vp, vp, vp, C.c_int64, C.POINTER(C.c_int64)]
     L.moe_quant_block128.argtypes = [vp, C.c_int32, C.c_int64, C.c_int64, C.c_int64, vp, vp, vp]
     L.moe_measure_mfma_tflops.argtypes = [vp, C.c_size_t, vp, C.c_int, C.POINTER(C.c_float)]
     L.moe_measure_hbm_read_gbs.argtypes = [vp, C.c_size_t, vp, vp, C.POINTER(C.c_float)]
@@ -300,6 +304,31 @@ class MoELayer:
         _check(self.L.moe_get_queue_balance(self._h, _ptr(self.workspace), _stream(), C.byref(n), C.byref(a),
                                             C.byref(b), C.byref(c)), "moe_get_queue_balance")
         return dict(workgroups=n.value, span_us=a.value, mean_active_us=b.value, mean_tail_idle_us=c.value)
+
+    def enable_task_trace(self, max_tasks: int = 1 << 16):
+        """Every task of the queue kernel leaves a record from now on (see task_trace); the buffer is a torch tensor."""
+        import torch
+        nbytes = self.L.moe_task_trace_bytes(max_tasks)
+        self._trace = torch.zeros(nbytes // 8, dtype=torch.int64, device="cuda")
+        torch.cuda.synchronize()
+        _check(self.L.moe_set_task_trace(self._h, _ptr(self._trace), nbytes), "moe_set_task_trace")
+
+    def disable_task_trace(self):
+        _check(self.L.moe_set_task_trace(self._h, None, 0), "moe_set_task_trace")
+        self._trace = None
+
+    def task_trace(self):
+        """Records of the last forward's queue kernel as a numpy structured array (phase, expert, row_block, col_tile,
+        rows, workgroup, start_us, end_us); synchronises the current stream."""
+        import numpy as np
+        dt = np.dtype([("phase", "i4"), ("expert", "i4"), ("row_block", "i4"), ("col_tile", "i4"), ("rows", "i4"),
+                       ("workgroup", "i4"), ("start_us", "f4"), ("end_us", "f4")])
+        n = C.c_int64(0)
+        _check(self.L.moe_get_task_trace(self._h, _stream(), None, 0, C.byref(n)), "moe_get_task_trace")
+        out = np.zeros(n.value, dtype=dt)
+        if n.value:
+            _check(self.L.moe_get_task_trace(self._h, _stream(), out.ctypes.data, n.value, C.byref(n)), "moe_get_task_trace")
+        return out
 
     def _weights(self, weights: dict) -> _CWeights:
         w = _CWeights()

@@ -175,6 +175,8 @@ struct moe_handle {
     int ffn_mode;
     int queue_groups;      // task queues of the FFN stage: one per XCD, or 1
     int row_chunk;         // task order inside a queue segment (FfnArgs::row_chunk)
+    int64_t* task_trace;   // the caller's device buffer for per-task records of the queue kernel, or null
+    int task_trace_cap;    // records it holds
     bool fused_combine;    // the FFN kernels combine a token when its last expert row arrives (no combine launch)
     int wall_clock_khz;    // rate of the constant clock the queue kernels stamp their entry and exit with
     int spin_limit;        // polls a dependency wait of the queue kernel makes before it gives up
@@ -244,6 +246,7 @@ RouteArgs route_args(const moe_handle* h, void* ws) {
     a.q = at<QueueState>(ws, w.qstate);
     a.done0 = at<int32_t>(ws, w.done0);
     a.arrive = h->fused_combine ? at<int32_t>(ws, w.arrive) : nullptr;
+    a.task_trace = h->task_trace;
     a.S = d.S; a.k = d.k; a.E = d.E; a.A = d.A; a.nblk = d.nblk;
     a.drop = h->cfg.drop_tokens;
     a.capacity = (int)d.capacity;
@@ -365,6 +368,8 @@ int moe_create(const moe_config* cfg, moe_handle** out) {
         if (v >= 0 && v <= 4096) h->row_chunk = v;
     }
     h->spin_limit = kDefaultSpinLimit;
+    h->task_trace = nullptr;
+    h->task_trace_cap = 0;
     h->stall_host = nullptr;
     {   // host memory, allocated once per handle; the hot path never allocates
         void* p = nullptr;
@@ -586,6 +591,8 @@ int forward_on(moe_handle* h, const void* x, const moe_weights* w, void* out, co
     fa.wg_clock = at<int64_t>(workspace, L.wg_clock);
     fa.row_chunk = h->row_chunk;
     fa.arrive = ra.arrive;
+    fa.task_trace = h->task_trace;
+    fa.task_trace_cap = h->task_trace_cap;
     fa.pair_row = ra.pair_row;
     fa.topk_w = topk_w;
     fa.out = out;
@@ -707,6 +714,58 @@ int moe_get_queue_balance(moe_handle* h, const void* workspace, void* stream, in
     if (span_us) *span_us = (float)((double)(last - first) * tick_us);
     if (mean_active_us) *mean_active_us = (float)(active / n * tick_us);
     if (mean_tail_idle_us) *mean_tail_idle_us = (float)(tail / n * tick_us);
+    return MOE_OK;
+}
+
+size_t moe_task_trace_bytes(int64_t max_tasks) { return 16 + 32 * (size_t)(max_tasks > 0 ? max_tasks : 0); }
+
+int moe_set_task_trace(moe_handle* h, void* device_buffer, size_t bytes) {
+    if (!h) return MOE_ERR_BAD_ARGUMENT;
+    if (!device_buffer || bytes < moe_task_trace_bytes(1)) {
+        h->task_trace = nullptr;
+        h->task_trace_cap = 0;
+        return device_buffer ? MOE_ERR_BAD_ARGUMENT : MOE_OK;
+    }
+    if ((uintptr_t)device_buffer % 8) return MOE_ERR_BAD_ARGUMENT;
+    const int64_t zero[2] = {0, 0};
+    const hipError_t e = hipMemcpy(device_buffer, zero, sizeof zero, hipMemcpyHostToDevice);   // not on the hot path
+    if (e != hipSuccess) return hip_fail(h, e);
+    h->task_trace = static_cast<int64_t*>(device_buffer);
+    h->task_trace_cap = (int)std::min<size_t>((bytes - 16) / 32, (size_t)INT32_MAX);
+    return MOE_OK;
+}
+
+int moe_get_task_trace(moe_handle* h, void* stream, moe_task_record* out, int64_t capacity, int64_t* count) {
+    if (!h || !count || capacity < 0 || (capacity > 0 && !out)) return MOE_ERR_BAD_ARGUMENT;
+    if (!h->task_trace) return MOE_ERR_UNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    int64_t head[2];
+    hipError_t e = hipMemcpyAsync(head, h->task_trace, sizeof head, hipMemcpyDeviceToHost, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    if (e != hipSuccess) return hip_fail(h, e);
+    const int64_t written = std::min<int64_t>((int64_t)(head[0] & 0xFFFFFFFF), h->task_trace_cap);
+    const int64_t n = std::min(written, capacity);
+    *count = written;
+    if (n == 0) return MOE_OK;
+    std::vector<int64_t> raw((size_t)written * 4);
+    e = hipMemcpyAsync(raw.data(), h->task_trace + 2, raw.size() * 8, hipMemcpyDeviceToHost, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    if (e != hipSuccess) return hip_fail(h, e);
+    int64_t first = INT64_MAX;
+    for (int64_t i = 0; i < written; ++i) first = std::min(first, raw[4 * i + 2]);
+    const double tick_us = 1000.0 / h->wall_clock_khz;
+    for (int64_t i = 0; i < n; ++i) {
+        const int64_t w0 = raw[4 * i], w1 = raw[4 * i + 1];
+        moe_task_record& r = out[i];
+        r.phase = (int32_t)(w0 >> 56);
+        r.expert = (int32_t)((w0 >> 40) & 0xFFFF);
+        r.row_block = (int32_t)((w0 >> 20) & 0xFFFFF);
+        r.col_tile = (int32_t)(w0 & 0xFFFFF);
+        r.workgroup = (int32_t)(w1 >> 32);
+        r.rows = (int32_t)(w1 & 0xFFFFFFFF);
+        r.start_us = (float)((double)(raw[4 * i + 2] - first) * tick_us);
+        r.end_us = (float)((double)(raw[4 * i + 3] - first) * tick_us);
+    }
     return MOE_OK;
 }
 

@@ -933,7 +933,10 @@ __global__ __launch_bounds__(P::THREADS) void ffn_persistent_kernel(FfnArgs a) {
             poison_tile((uint16_t*)a.y + (int64_t)t.row0 * a.H, t.rows, a.H, t.ntile * P::T1::BN, P::T1::BN, 2);
             t.rows = 0;
         }
+        const long long started = trace_clock(kernel_args_again().task_trace);
         plan_tile<P>(a, t, t.phase == 0 || a.arrive, smem);
+        if (kernel_args_again().task_trace)
+            trace_task(kernel_args_again().task_trace, kernel_args_again().task_trace_cap, t.phase, t.expert, t.mtile, t.ntile, t.rows, started);
         if (t.phase == 0) signal_phase0_done(a.done0, t.mtile);
         else if (a.arrive)   // the row count from the table: a tile whose wait expired runs with none, and still arrives
             combine_arrivals<ET>(combine_args(kernel_args_again()), t.row0, a.mtiles[t.mtile].rows, t.ntile, t.ntile * P::T1::BN, P::T1::BN, s_list);

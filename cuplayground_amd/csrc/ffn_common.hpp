@@ -164,6 +164,23 @@ __device__ __forceinline__ void queue_clock_stamp(int64_t* wg_clock, int which) 
         wg_clock[2 * blockIdx.x + which] = (int64_t)wall_clock64();
 }
 
+// One record per task of a queue kernel, when the caller has handed over a trace buffer (moe_set_task_trace): which
+// task, which workgroup, and the constant-rate clock before and behind the tile (the dependency wait of a
+// down-projection task lies in front of `start`).  The reference's kernels print such stamps (mma.cuh:51-57,162-169).
+// Four words per record: phase << 56 | expert << 40 | row block << 20 | column tile; workgroup << 32 | rows; start; end.
+__device__ __forceinline__ long long trace_clock(const int64_t* trace) { return trace ? (long long)wall_clock64() : 0; }
+__device__ __noinline__ void trace_task(int64_t* trace, int cap, int phase, int expert, int mtile, int ntile, int rows,
+                                        long long start) {
+    if (threadIdx.x != 0) return;
+    const int slot = atomicAdd(reinterpret_cast<int*>(trace), 1);
+    if (slot >= cap) return;
+    int64_t* e = trace + 2 + 4 * (int64_t)slot;
+    e[0] = ((int64_t)phase << 56) | ((int64_t)expert << 40) | ((int64_t)mtile << 20) | (int64_t)ntile;
+    e[1] = ((int64_t)blockIdx.x << 32) | (uint32_t)rows;
+    e[2] = start;
+    e[3] = (int64_t)wall_clock64();
+}
+
 __device__ __forceinline__ void publish8(void* p, uint32_t lo, uint32_t hi) {
     __hip_atomic_store(reinterpret_cast<uint64_t*>(p), ((uint64_t)hi << 32) | lo, __ATOMIC_RELAXED,
                        __HIP_MEMORY_SCOPE_AGENT);

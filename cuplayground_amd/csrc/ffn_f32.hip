@@ -172,8 +172,10 @@ __global__ __launch_bounds__(256) void ffn_persistent_f32_kernel(FfnArgs a) {
         int ok = 1;
         if (t.phase == 1) ok = wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q, a.host_stall, &s_ok);
         const TaskPtrsF p = resolve_f32(a, t, t.phase == 0 || a.arrive);
+        const long long started = trace_clock(a.task_trace);
         if (ok) gemm_tile_f32(p, As, Bs);
         else poison_tile(p.c_base, p.rows, p.N, p.n0, FBN, 4);
+        if (a.task_trace) trace_task(a.task_trace, a.task_trace_cap, t.phase, t.expert, t.mtile, t.ntile, t.rows, started);
         if (t.phase == 0) signal_phase0_done(a.done0, t.mtile);
         else if (a.arrive) combine_arrivals<float>(combine_args(a), t.row0, t.rows, t.ntile, p.n0, FBN, s_list);
     }

@@ -250,12 +250,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     while (next_task(a, cur, &s_task, ids, nseg, nnt0, t)) {
         int ok = 1;
         if (t.phase == 1) ok = wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q, a.host_stall, &s_ok);
+        const long long started = trace_clock(a.task_trace);
         for (int sub = 0; sub < (t.phase ? QSUB1 : QSUB); ++sub) {
             const Fp8Task p = resolve_fp8(a, t, sub, t.phase == 0 || a.arrive);
             if (p.c0 >= p.N) continue;
             if (ok) fp8_tile(p, red);
             else poison_tile(p.c_base, p.rows, p.N, p.c0, QN1, 2);
         }
+        if (a.task_trace) trace_task(a.task_trace, a.task_trace_cap, t.phase, t.expert, t.mtile, t.ntile, t.rows, started);
         if (t.phase == 0) signal_phase0_done(a.done0, t.mtile);
         else if (a.arrive) combine_arrivals<bf16_s>(combine_args(a), t.row0, t.rows, t.ntile, t.ntile * QSUB1 * QN1, QSUB1 * QN1, s_list);
     }

@@ -366,8 +366,10 @@ __global__ __launch_bounds__(PTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
         int ok = 1;
         if (t.phase == 1) ok = wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q, a.host_stall, &s_ok);
         const TileTask p = resolve_tile(a, t, t.phase == 0 || a.arrive);
+        const long long started = trace_clock(a.task_trace);
         if (ok) fp8_gemm_tile(p, smem);
         else poison_tile(p.c_base, p.rows, p.N, p.c0, t.phase ? PN1 : PN0, 2);
+        if (a.task_trace) trace_task(a.task_trace, a.task_trace_cap, t.phase, t.expert, t.mtile, t.ntile, t.rows, started);
         if (t.phase == 0) signal_phase0_done(a.done0, t.mtile);
         else if (a.arrive) combine_arrivals<bf16_s>(combine_args(a), t.row0, t.rows, t.ntile, p.c0, PN1, s_list);
     }

@@ -95,6 +95,8 @@ struct FfnArgs {
     int32_t row_chunk;          // order of a segment's tasks: 0 = row blocks fastest; R > 0 = R row blocks at a time, all column tiles of those, row blocks fastest inside
     uint32_t x_bytes, h_bytes, w_bytes;   // extents of x, h and one weight matrix (meaningful below 4 GiB)
     int64_t* wg_clock;          // queue kernels: [2 * workgroup] constant-rate clock at entry, [2 * workgroup + 1] at exit
+    int64_t* task_trace;        // null, or the caller's trace buffer: [0] records written, [2 + 4 i ..] record i (trace_task)
+    int32_t task_trace_cap;     // records the buffer holds
     // Combine inside the FFN kernels (null `arrive`: the separate combine launch is used instead).
     int32_t* arrive;            // [S, nnt1]: finished down-projection tiles per (token, column tile)
     const int32_t* pair_row;    // [S, k] packed row of every (token, rank), -1 when dropped
@@ -129,6 +131,7 @@ struct RouteArgs {
     int32_t max_mtiles;
     int32_t lag;                // experts of phase-0 work queued between an expert's two phases
     int32_t groups;             // queue groups: 1, or one per XCD
+    int64_t* task_trace;        // null, or the FFN stage's trace buffer: its record count starts every call at zero
 };
 
 // ---- launchers (defined next to their kernels) ----

@@ -193,6 +193,7 @@ __device__ __forceinline__ void route_scan_body(const RouteArgs& a, ScanShared& 
     if (e == 0) {
         a.q->groups = a.groups;
         for (int g = 0; g < kMaxQueueGroups; ++g) a.q->heads[g] = 0;
+        if (a.task_trace) a.task_trace[0] = 0;
         a.q->ids_queue = total_tasks;
         a.q->ids_phase0 = total_mt * npg0;
         a.q->ids_phase1 = total_mt * npg1;

@@ -211,6 +211,28 @@ int moe_get_stage_samples(moe_handle* h, int stage, float* ms, int32_t capacity,
  * Synchronises `stream`.  No counterpart in the reference, whose scheduler keeps no statistics. */
 int moe_get_queue_balance(moe_handle* h, const void* workspace, void* stream, int32_t* workgroups, float* span_us,
                           float* mean_active_us, float* mean_tail_idle_us);
+/* Per-task trace of the task-queue FFN kernel: with a trace buffer set, every task of a moe_forward on this handle
+ * leaves a record -- which tile of which expert, which workgroup ran it, and the device's constant-rate clock before and
+ * behind the tile (the dependency wait of a down-projection task lies in front of start_us).  The buffer is device
+ * memory of the caller (moe_task_trace_bytes(max_tasks) bytes, 8-byte aligned; tasks beyond its capacity are counted
+ * but not recorded); it holds the records of the most recent call.  moe_set_task_trace(h, NULL, 0) switches the trace
+ * off.  Setting it copies 16 bytes to the device (synchronous; not for the serving loop); moe_get_task_trace copies
+ * the records back, so it synchronises `stream`; times are microseconds since the earliest recorded start; *count
+ * receives the number of records the call left (it may exceed `capacity`).  Cost with the trace on: two clock reads
+ * and one atomic per task.  Counterpart in the reference: the clock stamps its kernels print (mma.cuh:51-57,162-169;
+ * scheduling.cuh:261-263). */
+typedef struct moe_task_record {
+    int32_t phase;      /* 0: up(/gate) projection + activation, 1: down projection */
+    int32_t expert;
+    int32_t row_block;  /* index into the layer's row-block table (expert-major) */
+    int32_t col_tile;
+    int32_t rows;       /* real rows of the block */
+    int32_t workgroup;
+    float start_us, end_us;
+} moe_task_record;
+size_t moe_task_trace_bytes(int64_t max_tasks);
+int moe_set_task_trace(moe_handle* h, void* device_buffer, size_t bytes);
+int moe_get_task_trace(moe_handle* h, void* stream, moe_task_record* out, int64_t capacity, int64_t* count);
 /* Tile tasks the FFN stage of the last moe_forward issued to its queue (GEMM0 tasks, GEMM1 tasks); reads
  * back a few words from the workspace, so it synchronises the stream. */
 int moe_get_task_counts(moe_handle* h, const void* workspace, void* stream, int64_t* gemm0_tasks, int64_t* gemm1_tasks);

@@ -17,6 +17,9 @@ SHAPES = {
                              drop=1, capacity_factor=1.0, zipf_bias=True),
     # shortest K (one k block) in the up projection, one expert, exactly full blocks
     "one_expert_short_k": ob.Cfg(S=256, H=128, I=512, E=1, k=1, act=ob.ACT_SWIGLU, dtype=ob.FP8, norm_topk=0, drop=0),
+    # many experts just above the plan's threshold: every row block is a partial one (about 40 of 128 rows), top-1
+    "many_partial_blocks": ob.Cfg(S=2000, H=256, I=256, E=48, k=1, act=ob.ACT_SWIGLU, dtype=ob.FP8, gate_fn=ob.GATE_SOFTMAX,
+                                  norm_topk=0, drop=0),
     # fewer rows than one block everywhere (the tile forced onto a decode-sized layer)
     "tiny_rows": ob.Cfg(S=40, H=256, I=128, E=8, k=2, act=ob.ACT_SWIGLU, dtype=ob.FP8, gate_fn=ob.GATE_SIGMOID, drop=0),
 }

@@ -16,8 +16,8 @@ namespace moe355 {
 
 bool grouped_gemm_takes_large_tile(int64_t A, int E, int N, int K);
 hipError_t launch_grouped_gemm_16(const void* a_rows, const void* w, const void* bias, void* out, const MTile* mtiles,
-                                  const int32_t* num_mtiles, int max_mtiles, int tile, int64_t A, int N, int K, int act,
-                                  bool f16, hipStream_t st);
+                                  const int32_t* num_mtiles, const int32_t* count, int max_mtiles, int tile, int64_t A,
+                                  int N, int K, int act, bool f16, hipStream_t st);
 hipError_t launch_wgrad_16(const void* dyT, const void* aT, void* dw, const int32_t* poff, int E, int N, int K,
                            int64_t ld, bool f16, hipStream_t st);
 
@@ -54,7 +54,7 @@ __global__ __launch_bounds__(kMaxExperts) void backward_tables_kernel(const int3
             t.expert = e;
             t.row0 = off + i * block_m;
             t.rows = min(block_m, n - i * block_m);
-            t.pad = 0;
+            t.pad = s_mt0[e];        // first row block of this expert (the grouped GEMM orders its tiles by it)
             mtiles[mt] = t;
         }
     }
@@ -289,7 +289,7 @@ hipError_t launch_expert_gemm(const void* a_rows, const void* w, const void* bia
     backward_tables_kernel<<<1, kMaxExperts, 0, st>>>(count, offset, E, block_m, mtiles, num_mtiles, nullptr);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    return launch_grouped_gemm_16(a_rows, w, bias, out_rows, mtiles, num_mtiles, max_mtiles, tile, A, N, K, act, f16, st);
+    return launch_grouped_gemm_16(a_rows, w, bias, out_rows, mtiles, num_mtiles, count, max_mtiles, tile, A, N, K, act, f16, st);
 }
 
 // dw[e] [N,K] = dy_e^T . a_e; scratch holds the window offsets and the two transposed operands.

@@ -1109,16 +1109,26 @@ __global__ __launch_bounds__(T::THREADS) void gemm_dense_kernel(const uint16_t* 
 // Grouped GEMM on packed expert-major rows, outside the layer: out[r,:] = act(a[r,:] . w[e(r)]^T + bias[e(r)]) for
 // the rows of every row block of the table -- the reference's tile GEMM (mma.cuh:46-179) once per expert, with the
 // expert taken from the row block.  With the weight handed over in its K-major view this is the data gradient of a
-// projection (dX = dY . W).  grid = (row blocks upper bound, column tiles).
+// projection (dX = dY . W).  One workgroup per tile, in the order of the layer's task queue: expert by expert, column
+// tile by column tile, an expert's row blocks fastest -- neighbouring workgroups share a weight tile and an expert's
+// few row blocks stay in the caches while its column tiles pass by (column tiles of all experts' row blocks at once:
+// 1.69 ms on the Mixtral-shaped data gradient of the down projection against 1.55 this way).  grid = row blocks upper bound x column tiles;
+// mtiles[i].pad is the index of the first row block of that block's expert.
 template <class T>
 __global__ __launch_bounds__(T::THREADS) void grouped_gemm_kernel(const uint16_t* a_rows, const uint16_t* w,
                                                                   const uint16_t* bias, uint16_t* out,
-                                                                  const MTile* mtiles, const int32_t* num_mtiles, int N,
-                                                                  int K, int act, uint32_t a_bytes) {
+                                                                  const MTile* mtiles, const int32_t* num_mtiles,
+                                                                  const int32_t* count, int N, int K, int act,
+                                                                  uint32_t a_bytes) {
     extern __shared__ __align__(16) unsigned char smem[];
-    const int mt = blockIdx.x;
-    if (mt >= *num_mtiles) return;
-    const MTile m = mtiles[mt];
+    const int ncol = (N + T::BN - 1) / T::BN;
+    const int id = blockIdx.x;
+    if (id >= *num_mtiles * ncol) return;
+    // id / ncol is a row block of the expert this id belongs to: ids [ncol * first, ncol * (first + blocks)) are its own
+    const MTile probe = mtiles[id / ncol];
+    const int first = probe.pad, blocks = (max(count[probe.expert], 0) + T::BM - 1) / T::BM;
+    const int local = id - ncol * first, ctile = local / blocks;
+    const MTile m = mtiles[first + (local - ctile * blocks)];
     TaskPtrs p;
     p.a_base = a_rows;
     p.gather = nullptr;
@@ -1133,7 +1143,7 @@ __global__ __launch_bounds__(T::THREADS) void grouped_gemm_kernel(const uint16_t
     p.N = N;
     p.K = K;
     p.rows = m.rows;
-    p.n0 = blockIdx.y * T::BN;
+    p.n0 = ctile * T::BN;
     p.act = act;
     p.swiglu = false;
     p.publish = false;
@@ -1348,28 +1358,30 @@ bool grouped_gemm_takes_large_tile(int64_t A, int E, int N, int K) {
 
 template <class T>
 static hipError_t launch_grouped(const void* a_rows, const void* w, const void* bias, void* out, const MTile* mtiles,
-                                 const int32_t* num_mtiles, int max_mtiles, int64_t A, int N, int K, int act,
-                                 hipStream_t st) {
+                                 const int32_t* num_mtiles, const int32_t* count, int max_mtiles, int64_t A, int N, int K,
+                                 int act, hipStream_t st) {
     hipError_t e = allow_lds(&grouped_gemm_kernel<T>, T::LDS_BYTES);
     if (e != hipSuccess) return e;
-    const dim3 grid((unsigned)max_mtiles, (unsigned)((N + T::BN - 1) / T::BN));
-    grouped_gemm_kernel<T><<<grid, T::THREADS, T::LDS_BYTES, st>>>((const uint16_t*)a_rows, (const uint16_t*)w,
-                                                                   (const uint16_t*)bias, (uint16_t*)out, mtiles,
-                                                                   num_mtiles, N, K, act, (uint32_t)(A * K * 2));
+    const int64_t blocks = (int64_t)max_mtiles * ((N + T::BN - 1) / T::BN);
+    if (blocks > INT32_MAX) return hipErrorInvalidValue;
+    grouped_gemm_kernel<T><<<(unsigned)blocks, T::THREADS, T::LDS_BYTES, st>>>((const uint16_t*)a_rows, (const uint16_t*)w,
+                                                                               (const uint16_t*)bias, (uint16_t*)out, mtiles,
+                                                                               num_mtiles, count, N, K, act,
+                                                                               (uint32_t)(A * K * 2));
     return hipGetLastError();
 }
 
 hipError_t launch_grouped_gemm_16(const void* a_rows, const void* w, const void* bias, void* out, const MTile* mtiles,
-                                  const int32_t* num_mtiles, int max_mtiles, int tile, int64_t A, int N, int K, int act,
-                                  bool f16, hipStream_t st) {
+                                  const int32_t* num_mtiles, const int32_t* count, int max_mtiles, int tile, int64_t A,
+                                  int N, int K, int act, bool f16, hipStream_t st) {
     if (tile == 2)   // 128-row blocks on the hand-ordered 128 x 256 tile
-        return f16 ? launch_grouped<Tile128x256H>(a_rows, w, bias, out, mtiles, num_mtiles, max_mtiles, A, N, K, act, st)
-                   : launch_grouped<Tile128x256>(a_rows, w, bias, out, mtiles, num_mtiles, max_mtiles, A, N, K, act, st);
+        return f16 ? launch_grouped<Tile128x256H>(a_rows, w, bias, out, mtiles, num_mtiles, count, max_mtiles, A, N, K, act, st)
+                   : launch_grouped<Tile128x256>(a_rows, w, bias, out, mtiles, num_mtiles, count, max_mtiles, A, N, K, act, st);
     if (tile == 1)
-        return f16 ? launch_grouped<LargePlanH::T0>(a_rows, w, bias, out, mtiles, num_mtiles, max_mtiles, A, N, K, act, st)
-                   : launch_grouped<LargePlan::T0>(a_rows, w, bias, out, mtiles, num_mtiles, max_mtiles, A, N, K, act, st);
-    return f16 ? launch_grouped<SmallPlanH::T0>(a_rows, w, bias, out, mtiles, num_mtiles, max_mtiles, A, N, K, act, st)
-               : launch_grouped<SmallPlan::T0>(a_rows, w, bias, out, mtiles, num_mtiles, max_mtiles, A, N, K, act, st);
+        return f16 ? launch_grouped<LargePlanH::T0>(a_rows, w, bias, out, mtiles, num_mtiles, count, max_mtiles, A, N, K, act, st)
+                   : launch_grouped<LargePlan::T0>(a_rows, w, bias, out, mtiles, num_mtiles, count, max_mtiles, A, N, K, act, st);
+    return f16 ? launch_grouped<SmallPlanH::T0>(a_rows, w, bias, out, mtiles, num_mtiles, count, max_mtiles, A, N, K, act, st)
+               : launch_grouped<SmallPlan::T0>(a_rows, w, bias, out, mtiles, num_mtiles, count, max_mtiles, A, N, K, act, st);
 }
 
 template <class T>

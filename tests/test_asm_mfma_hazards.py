@@ -159,3 +159,48 @@ def test_fp8_tile_barriers_sit_behind_their_waits():
                     assert not [y for y in loop if y.startswith("scratch_")], (name, "spill in the slab loop")
                     slab_loops += 1
         assert slab_loops >= 2, name      # the full-block loop and the partial-block loops
+
+
+def _vregs(text):
+    """Vector registers an instruction line names: v7 -> {7}, v[4:7] -> {4..7}."""
+    regs = set()
+    for a, b in re.findall(r"\bv\[(\d+):(\d+)\]", text):
+        regs.update(range(int(a), int(b) + 1))
+    regs.update(int(a) for a in re.findall(r"\bv(\d+)\b", text))
+    return regs
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
+def test_fp8_tile_weight_bytes_are_not_touched_in_flight():
+    """The e4m3 tile GEMM fetches its weight bytes with a load written in assembly, so the compiler does not know that
+    the destination registers are pending until the wait that names them (s_waitcnt vmcnt(4)).  Inside the slab loops
+    nothing between such a load and that wait may read, copy or spill those registers."""
+    text = _assembly("ffn_fp8_tile.hip")
+    kernels = re.findall(r"\n(_ZN6moe355\w*fp8_tile_kernel\w*):[^\n]*\n(.*?)\n\s*s_endpgm", text, re.S)
+    assert len(kernels) == 2
+    for name, body in kernels:
+        lines = [x.strip() for x in body.split("\n") if x.strip() and not x.strip().startswith(";")]
+        labels = {x.split(":")[0]: i for i, x in enumerate(lines) if re.match(r"\.LBB\d+_\d+:", x)}
+        checked = 0
+        for i, x in enumerate(lines):
+            j = re.match(r"s_cbranch_\w+ (\.LBB\d+_\d+)", x)
+            if not (j and j.group(1) in labels and labels[j.group(1)] < i):
+                continue
+            loop = [y for y in lines[labels[j.group(1)]:i] if not re.match(r"\.LBB\d+_\d+:", y)]
+            if sum(y.startswith("v_mfma") for y in loop) < 32 or sum(y.startswith("s_barrier") for y in loop) != 2:
+                continue
+            n = len(loop)
+            for k, y in enumerate(loop):
+                m = re.match(r"global_load_dwordx4 v\[(\d+):(\d+)\], v\[\d+:\d+\], off", y)
+                if not m:
+                    continue
+                pending = set(range(int(m.group(1)), int(m.group(2)) + 1))
+                for step in range(1, n + 1):           # the wait may sit behind the loop's back edge
+                    z = loop[(k + step) % n]
+                    if z == "s_waitcnt vmcnt(4)":
+                        break
+                    assert not (_vregs(z) & pending), (name, y, z)
+                else:
+                    raise AssertionError("no wait for " + y)
+                checked += 1
+        assert checked >= 4, (name, checked)       # two loads per slab, two slabs per loop iteration

@@ -37,6 +37,60 @@ __device__ __forceinline__ void load8(const T16* p, float (&v)[8]) {
     v[6] = lo16(a.w, T16{}); v[7] = hi16(a.w, T16{});
 }
 
+// Folds the 64 per-lane partial sums of 16 independent sums at once.  At xor distance 32, 16, 8, 4 a lane keeps one
+// register of each pair and hands the other to its partner (halving the registers per step), then distances 2 and 1
+// on the one register left.  Each sum adds lane l to lane l ^ d for d = 32, 16, 8, 4, 2, 1 in that order: the result
+// has the bits of the plain butterfly.  Returns the sum of red[index] with index = fold16_index(lane), valid in the
+// lanes with (lane & 3) == 0.
+// The exchanges stay in the vector ALU: v_permlane32_swap / v_permlane16_swap trade the halves (the odd 16-lane rows)
+// of a register pair, which is the keep-one-hand-over-the-other step in one instruction; distances 8 .. 1 are DPP
+// moves (row rotate by 8; row shifts by 4 under bank masks; quad permutes).  Through the LDS crossbar (ds_bpermute)
+// the seventeen exchanges of a fold cost about as much as a quarter of the multiply-adds they follow.
+template <int CTRL, int BANKS = 0xF>
+__device__ __forceinline__ float dpp_from(float old, float v) {
+    return __uint_as_float(__builtin_amdgcn_update_dpp(__float_as_uint(old), __float_as_uint(v), CTRL, 0xF, BANKS, false));
+}
+__device__ __forceinline__ float lane_xor8(float v) { return dpp_from<0x128>(0.0f, v); }                    // row_ror:8
+__device__ __forceinline__ float lane_xor4(float v) { return dpp_from<0x114, 0xA>(dpp_from<0x104, 0x5>(0.0f, v), v); }   // row_shl:4 | row_shr:4
+__device__ __forceinline__ float lane_xor2(float v) { return dpp_from<0x4E>(0.0f, v); }                     // quad_perm [2,3,0,1]
+__device__ __forceinline__ float lane_xor1(float v) { return dpp_from<0xB1>(0.0f, v); }                     // quad_perm [1,0,3,2]
+
+__device__ __forceinline__ float fold16(float (&red)[16], int lane) {
+    typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {      // distance 32: lanes 0..31 keep red[2i], lanes 32..63 keep red[2i+1]
+        const u32x2_t r = __builtin_amdgcn_permlane32_swap(__float_as_uint(red[2 * i]), __float_as_uint(red[2 * i + 1]), false, false);
+        red[i] = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {      // distance 16: even 16-lane rows keep red[2i], odd rows red[2i+1]
+        const u32x2_t r = __builtin_amdgcn_permlane16_swap(__float_as_uint(red[2 * i]), __float_as_uint(red[2 * i + 1]), false, false);
+        red[i] = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    }
+    {
+        const bool hi = (lane & 8) != 0;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const float keep = hi ? red[2 * i + 1] : red[2 * i];
+            const float send = hi ? red[2 * i] : red[2 * i + 1];
+            red[i] = keep + lane_xor8(send);
+        }
+    }
+    {
+        const bool hi = (lane & 4) != 0;
+        const float keep = hi ? red[1] : red[0];
+        const float send = hi ? red[0] : red[1];
+        red[0] = keep + lane_xor4(send);
+    }
+    float sum = red[0];
+    sum = sum + lane_xor2(sum);
+    sum = sum + lane_xor1(sum);
+    return sum;
+}
+__device__ __forceinline__ int fold16_index(int lane) {
+    return ((lane >> 5) & 1) | (((lane >> 4) & 1) << 1) | (((lane >> 3) & 1) << 2) | (((lane >> 2) & 1) << 3);
+}
+
 // A wavefront keeps TPW token rows in registers (lane l owns the 8-element chunks l, l+64, ... of each row, as
 // fp32) and walks over its share of the experts: one 16-byte load of the expert's row per chunk feeds 8*TPW
 // fmafs; the 64 partial sums of 16 (token, expert) pairs are folded together (see the loop).  grid = (token groups of 4*TPW, expert chunks); NCH = chunks per lane = ceil(H / 512).
@@ -117,22 +171,8 @@ __global__ __launch_bounds__(256) void gate_logits_kernel(const T* __restrict__ 
                 }
             }
         }
-#pragma unroll
-        for (int step = 0; step < 4; ++step) {
-            const int off = 32 >> step, n = 16 >> step;
-            const bool hi = (lane & off) != 0;
-#pragma unroll
-            for (int i = 0; i < n / 2; ++i) {
-                const float keep = hi ? red[2 * i + 1] : red[2 * i];
-                const float send = hi ? red[2 * i] : red[2 * i + 1];
-                red[i] = keep + __shfl_xor(send, off, kWave);
-            }
-        }
-        float sum = red[0];
-        sum = sum + __shfl_xor(sum, 2, kWave);
-        sum = sum + __shfl_xor(sum, 1, kWave);
-        // the lane's register index: bit 0 came from lane bit 5, bit 1 from bit 4, bit 2 from bit 3, bit 3 from bit 2
-        const int r = ((lane >> 5) & 1) | (((lane >> 4) & 1) << 1) | (((lane >> 3) & 1) << 2) | (((lane >> 2) & 1) << 3);
+        const float sum = fold16(red, lane);
+        const int r = fold16_index(lane);
         const int e = eb + r / TPW, t = t0 + r % TPW;
         if ((lane & 3) == 0 && e < e1 && t < S) logits[(size_t)t * E + e] = gate_bias ? sum + gate_bias[e] : sum;
     }
@@ -193,32 +233,6 @@ __device__ __forceinline__ void widen8(const typename RawChunk<T>::type& r, floa
             v[2 * i + 1] = hi16(r[i], T{});
         }
     }
-}
-
-// Folds the 64 per-lane partial sums of 16 independent sums at once.  At xor distance 32, 16, 8, 4 a lane keeps one
-// register of each pair and hands the other to its partner (halving the registers per step), then distances 2 and 1
-// on the one register left.  Each sum adds lane l to lane l ^ d for d = 32, 16, 8, 4, 2, 1 in that order: the result
-// has the bits of the plain butterfly.  Returns the sum of red[index] with index = fold16_index(lane), valid in the
-// lanes with (lane & 3) == 0.
-__device__ __forceinline__ float fold16(float (&red)[16], int lane) {
-#pragma unroll
-    for (int step = 0; step < 4; ++step) {
-        const int off = 32 >> step, n = 16 >> step;
-        const bool hi = (lane & off) != 0;
-#pragma unroll
-        for (int i = 0; i < n / 2; ++i) {
-            const float keep = hi ? red[2 * i + 1] : red[2 * i];
-            const float send = hi ? red[2 * i] : red[2 * i + 1];
-            red[i] = keep + __shfl_xor(send, off, kWave);
-        }
-    }
-    float sum = red[0];
-    sum = sum + __shfl_xor(sum, 2, kWave);
-    sum = sum + __shfl_xor(sum, 1, kWave);
-    return sum;
-}
-__device__ __forceinline__ int fold16_index(int lane) {
-    return ((lane >> 5) & 1) | (((lane >> 4) & 1) << 1) | (((lane >> 3) & 1) << 2) | (((lane >> 2) & 1) << 3);
 }
 
 template <typename T, int TT, int TE, int WT, int WE>

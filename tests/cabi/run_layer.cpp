@@ -122,10 +122,32 @@ int main(int argc, char** argv) {
         fprintf(stderr, "short workspace was not refused\n");
         return 4;
     }
+    // the per-task trace of the queue kernel: a buffer of the caller's, one record per tile of the call that follows
+    void* trace = nullptr;
+    const size_t trace_bytes = moe_task_trace_bytes(1 << 14);
+    HIP_OK(hipMalloc(&trace, trace_bytes));
+    MOE_OK_OR_DIE(moe_set_task_trace(h, trace, trace_bytes));
     MOE_OK_OR_DIE(moe_forward(h, x, &w, out, &r, ws, ws_bytes, st));
     HIP_OK(hipStreamSynchronize(st));
     int64_t t0 = 0, t1 = 0;
     MOE_OK_OR_DIE(moe_get_task_counts(h, ws, st, &t0, &t1));
+    int64_t traced = 0;
+    int32_t mode = 0;
+    MOE_OK_OR_DIE(moe_get_ffn_mode(h, &mode));
+    {
+        std::vector<moe_task_record> rec(1 << 14);
+        MOE_OK_OR_DIE(moe_get_task_trace(h, st, rec.data(), (int64_t)rec.size(), &traced));
+        if (mode == MOE_FFN_PERSISTENT && traced != t0 + t1) {
+            fprintf(stderr, "trace holds %lld records for %lld tasks\n", (long long)traced, (long long)(t0 + t1));
+            return 6;
+        }
+        for (int64_t i = 0; i < traced; ++i)
+            if (rec[i].end_us < rec[i].start_us || rec[i].phase < 0 || rec[i].phase > 1) {
+                fprintf(stderr, "bad trace record %lld\n", (long long)i);
+                return 6;
+            }
+    }
+    MOE_OK_OR_DIE(moe_set_task_trace(h, nullptr, 0));
 
     std::vector<char> host((size_t)S * H * es);
     HIP_OK(hipMemcpy(host.data(), out, host.size(), hipMemcpyDeviceToHost));
@@ -139,7 +161,8 @@ int main(int argc, char** argv) {
     HIP_OK(hipMemcpy(counts.data(), r.expert_count, E * 4, hipMemcpyDeviceToHost));
     if (!write_file(dir + "expert_count.bin", counts.data(), E * 4)) return 5;
 
-    printf("ok tokens=%lld tasks=%lld+%lld version=%d\n", (long long)S, (long long)t0, (long long)t1, moe_version());
+    printf("ok tokens=%lld tasks=%lld+%lld traced=%lld version=%d\n", (long long)S, (long long)t0, (long long)t1,
+           (long long)traced, moe_version());
     moe_destroy(h);
     return 0;
 }

@@ -36,15 +36,15 @@ BF16_SOURCES = ("ffn_bf16.hip", "ffn_bf16_slab_steady.inc", "ffn_common.hpp", "r
 FP8_SOURCES = ("ffn_fp8.hip", "ffn_common.hpp", "route.hip")
 FP8_TILE_SOURCES = ("ffn_fp8_tile.hip", "ffn_common.hpp", "route.hip")
 MEASURED_TRAFFIC = {
-    "mixtral": {"bytes": 19.23e9, "sources": BF16_SOURCES, "kernel_digest": "c4350c29010d",
+    "mixtral": {"bytes": 19.48e9, "sources": BF16_SOURCES, "kernel_digest": "2192860045c2",
                 "profile": "profiles/ffn_persistent_kernel_bf16_mixtral_c3_hbm_traffic.txt"},
-    "mid": {"bytes": 0.808e9, "sources": BF16_SOURCES, "kernel_digest": "c4350c29010d",
+    "mid": {"bytes": 0.808e9, "sources": BF16_SOURCES, "kernel_digest": "2192860045c2",
             "profile": "profiles/ffn_persistent_kernel_bf16_mid_c2_hbm_traffic.txt"},
-    "finegrained": {"bytes": 3.353e9, "sources": BF16_SOURCES, "kernel_digest": "c4350c29010d",
+    "finegrained": {"bytes": 3.35e9, "sources": BF16_SOURCES, "kernel_digest": "2192860045c2",
                     "profile": "profiles/ffn_persistent_kernel_bf16_finegrained_c4_hbm_traffic.txt"},
-    "decode_fp8": {"bytes": 9.884e9, "sources": FP8_SOURCES, "kernel_digest": "ab362d972ea4",
+    "decode_fp8": {"bytes": 9.885e9, "sources": FP8_SOURCES, "kernel_digest": "ab362d972ea4",
                    "profile": "profiles/ffn_persistent_fp8_kernel_decode_c5_hbm_traffic.txt"},
-    "prefill_fp8": {"bytes": 26.82e9, "sources": FP8_TILE_SOURCES, "kernel_digest": "3aa597eaefd2",
+    "prefill_fp8": {"bytes": 26.83e9, "sources": FP8_TILE_SOURCES, "kernel_digest": "3aa597eaefd2",
                     "profile": "profiles/ffn_persistent_fp8_tile_kernel_prefill_fp8_hbm_traffic.txt"},
 }
 

@@ -1014,6 +1014,7 @@ __global__ __launch_bounds__(P::THREADS) void ffn_persistent_ring_kernel(FfnArgs
         const bool reserve = cur.last_id + kReserveMargin < ids;
         int rid = 0;
         if (reserve && wave == 0) rid = pop_async(&kernel_args_again().q->heads[cur.group]);
+        const long long traced_from = trace_clock(kernel_args_again().task_trace);   // the first loads left earlier, under the previous tile's end
         f32x4 acc[8][8];
         const bool active = ring_slabs<T>(rows, L, smem, acc);
 
@@ -1058,6 +1059,7 @@ __global__ __launch_bounds__(P::THREADS) void ffn_persistent_ring_kernel(FfnArgs
 #pragma unroll
             for (int i = 0; i < 8; ++i) token_loads(i);
         }
+        if (a.task_trace) trace_task(a.task_trace, a.task_trace_cap, ph, ex, mt, nt, rows, traced_from);
         if (ph == 0) signal_phase0_done(a.done0, mt);
         else if (a.arrive) combine_arrivals<ET>(combine_args(a), row0, a.mtiles[mt].rows, nt, nt * T::BN, T::BN, s_list);
         if (reserve && nid < ids && n_valid) {   // the reserved task is the next one

@@ -18,11 +18,14 @@ CASES = {
 }
 
 
-@pytest.mark.parametrize("name", sorted(CASES))
-def test_every_task_is_recorded_once_and_in_dependency_order(name):
+@pytest.mark.parametrize("name", sorted(CASES) + ["bf16_large_tile_early_start"])
+def test_every_task_is_recorded_once_and_in_dependency_order(name, monkeypatch):
     import torch
     import cuplayground_amd as moe
     assert torch.cuda.is_available(), "these tests need the MI355X"
+    if name.endswith("_early_start"):        # the queue loop that starts the next task under the current tile's end
+        monkeypatch.setenv("MOE355_QUEUE_EARLY", "1")
+        name = name[:-len("_early_start")]
     cfg = CASES[name]
     inp = ob.make_inputs(cfg, seed=13)
     want = ob.route(cfg, inp)

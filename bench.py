@@ -42,9 +42,9 @@ MEASURED_TRAFFIC = {
             "profile": "profiles/ffn_persistent_kernel_bf16_mid_c2_hbm_traffic.txt"},
     "finegrained": {"bytes": 3.35e9, "sources": BF16_SOURCES, "kernel_digest": "2192860045c2",
                     "profile": "profiles/ffn_persistent_kernel_bf16_finegrained_c4_hbm_traffic.txt"},
-    "decode_fp8": {"bytes": 9.885e9, "sources": FP8_SOURCES, "kernel_digest": "ab362d972ea4",
+    "decode_fp8": {"bytes": 9.884e9, "sources": FP8_SOURCES, "kernel_digest": "f8fa608ab58a",
                    "profile": "profiles/ffn_persistent_fp8_kernel_decode_c5_hbm_traffic.txt"},
-    "prefill_fp8": {"bytes": 26.83e9, "sources": FP8_TILE_SOURCES, "kernel_digest": "3aa597eaefd2",
+    "prefill_fp8": {"bytes": 27.06e9, "sources": FP8_TILE_SOURCES, "kernel_digest": "8f1a6919616f",
                     "profile": "profiles/ffn_persistent_fp8_tile_kernel_prefill_fp8_hbm_traffic.txt"},
 }
 

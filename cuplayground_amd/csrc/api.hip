@@ -32,12 +32,12 @@ hipError_t launch_gemm_dense_f32(const void*, const void*, const void*, void*, i
                                  hipStream_t);
 hipError_t launch_ffn_fp8(const FfnArgs&, int max_mtiles, int nnt0, int nnt1, int blocks, hipStream_t);
 int fp8_block_m();
-int fp8_block_n0();
+int fp8_block_n0(int swiglu);
 int fp8_block_n1();
 int ffn_persistent_occupancy_fp8();
 hipError_t launch_ffn_fp8_tile(const FfnArgs&, int max_mtiles, int nnt0, int nnt1, int blocks, hipStream_t);
 int fp8_tile_block_m();
-int fp8_tile_block_n0();
+int fp8_tile_block_n0(int swiglu);
 int fp8_tile_block_n1();
 int ffn_persistent_occupancy_fp8_tile();
 
@@ -72,9 +72,8 @@ int act_dtype_of(int torch_dtype) {
 
 int check_supported(const moe_config& c) {
     if (c.num_experts > kMaxExperts || c.expert_top_k > kMaxTopK) return MOE_ERR_UNSUPPORTED;
-    if (c.torch_dtype == MOE_DTYPE_FP8_E4M3_B128 &&
-        (c.hidden_size % 128 || c.intermediate_size % 128 || c.hidden_act != MOE_ACT_SWIGLU))
-        return MOE_ERR_UNSUPPORTED;
+    if (c.torch_dtype == MOE_DTYPE_FP8_E4M3_B128 && (c.hidden_size % 128 || c.intermediate_size % 128))
+        return MOE_ERR_UNSUPPORTED;     // one scale per 128 x 128 block of a weight matrix
     if (c.hidden_size > 16384) return MOE_ERR_UNSUPPORTED;   // the router keeps a token row in registers
     return MOE_OK;
 }
@@ -149,7 +148,7 @@ FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E) {
             if (v == 0 || v == 1) p.tile = v;
         }
         p.block_m = p.tile ? fp8_tile_block_m() : fp8_block_m();
-        p.nnt0 = ceil_div(I, p.tile ? fp8_tile_block_n0() : fp8_block_n0());
+        p.nnt0 = ceil_div(I, p.tile ? fp8_tile_block_n0(sw) : fp8_block_n0(sw));
         p.nnt1 = ceil_div(H, p.tile ? fp8_tile_block_n1() : fp8_block_n1());
     } else {
         p.tile = bf16_tile(A, E, H, I, sw);
@@ -543,7 +542,7 @@ int forward_on(moe_handle* h, const void* x, const moe_weights* w, void* out, co
     if (!w->gate_w || !w->w_up || !w->w_down) return MOE_ERR_BAD_ARGUMENT;
     if (sw != (w->w_gate != nullptr)) return MOE_ERR_BAD_ARGUMENT;
     if (!sw && w->b_gate) return MOE_ERR_BAD_ARGUMENT;
-    if (fp8 && (!w->s_up || !w->s_down || !w->s_gate)) return MOE_ERR_BAD_ARGUMENT;
+    if (fp8 && (!w->s_up || !w->s_down || sw != (w->s_gate != nullptr))) return MOE_ERR_BAD_ARGUMENT;
     if (!fp8 && (w->s_up || w->s_down || w->s_gate)) return MOE_ERR_BAD_ARGUMENT;
     int rc = check_ws(h, workspace, workspace_bytes);
     if (rc) return rc;

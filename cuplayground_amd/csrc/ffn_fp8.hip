@@ -6,7 +6,8 @@
 // (mma.cuh:59,108-111,415-427).
 //
 // This shape is decode-like: a handful of token rows per expert against tens of megabytes of weights, so
-// the kernel is a weight streamer.  A task is (expert, 16-token row block, chunk of weight rows):
+// the kernel is a weight streamer.  A task is (expert, 16-token row block, chunk of weight rows -- 64 gate + 64 up rows
+// per sub-tile of a SwiGLU up projection, 128 rows of one matrix otherwise):
 //   * v_mfma_f32_16x16x32_bf16 with the weights as the "A" operand (16 weight rows) and up to 16 token rows
 //     as "B"; e4m3 bytes are widened to bf16 in registers (exact) right before the MFMA;
 //   * each lane fetches 16 contiguous weight bytes per 64-wide k slab, so a wavefront load covers 64
@@ -67,6 +68,8 @@ struct Fp8Task {
     int64_t a_row0;
     uint16_t* c_base;           // h or y at the first row of the block
     int K, N, rows, c0, phase;
+    int act;        // up projection without SwiGLU: the activation of the epilogue (else MOE_ACT_NONE)
+    bool paired;    // up projection with SwiGLU: 64 gate rows + 64 up rows per sub-tile; otherwise 128 rows of one matrix
     bool publish;   // rows are read by other workgroups of the same launch
 };
 
@@ -85,7 +88,7 @@ __device__ __forceinline__ void fp8_tile(const Fp8Task& t, float* red) {
     for (int g = 0; g < QGROUPS; ++g) {
         int n;
         const uint8_t* base;
-        if (t.phase == 0) {
+        if (t.paired) {
             n = t.c0 + (g & 3) * 16 + idx;
             base = t.w[g >> 2];
         } else {
@@ -122,7 +125,7 @@ __device__ __forceinline__ void fp8_tile(const Fp8Task& t, float* red) {
                 part = __builtin_amdgcn_mfma_f32_16x16x32_bf16(widen8(wv[g][s].x, wv[g][s].y), xa[s][0].v, part, 0, 0, 0);
                 part = __builtin_amdgcn_mfma_f32_16x16x32_bf16(widen8(wv[g][s].z, wv[g][s].w), xa[s][1].v, part, 0, 0, 0);
             }
-            const float sc = (t.phase == 0 && g >= 4) ? sc1 : sc0;
+            const float sc = (t.paired && g >= 4) ? sc1 : sc0;
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[g][r] = __builtin_fmaf(sc, part[r], acc[g][r]);
         }
@@ -149,7 +152,7 @@ __device__ __forceinline__ void fp8_tile(const Fp8Task& t, float* red) {
         }
     if (idx >= t.rows) return;
     uint16_t* crow = t.c_base + (int64_t)idx * t.N;
-    if (t.phase == 0) {
+    if (t.paired) {
         const int col = t.c0 + wave * 16 + 4 * kg;
         float o[4];
 #pragma unroll
@@ -173,6 +176,7 @@ __device__ __forceinline__ void fp8_tile(const Fp8Task& t, float* red) {
             for (int r = 0; r < 4; ++r) {
                 o[r] = v[h][r];
                 if (t.bias[0]) o[r] = o[r] + bf16_bits_to_f32(t.bias[0][col + r]);
+                o[r] = act_apply(o[r], t.act);
             }
             uint2 st;
             st.x = pack2_bf16(o[0], o[1]);
@@ -190,17 +194,27 @@ __device__ __forceinline__ Fp8Task resolve_fp8(const FfnArgs& a, const Task& t, 
     const int kbH = a.H >> 7, kbI = a.I >> 7;
     p.phase = t.phase;
     p.rows = t.rows;
+    p.act = MOE_ACT_NONE;
+    p.paired = t.phase == 0 && a.act == MOE_ACT_SWIGLU;
     if (t.phase == 0) {
-        p.c0 = (t.ntile * QSUB + sub) * QN0;
+        p.c0 = (t.ntile * QSUB + sub) * (p.paired ? QN0 : QN1);
         p.K = a.H;
         p.N = a.I;
-        p.w[0] = (const uint8_t*)a.w_gate + t.expert * HI;
-        p.w[1] = (const uint8_t*)a.w_up + t.expert * HI;
         const int64_t srow = ((int64_t)t.expert * (a.I >> 7) + (p.c0 >> 7)) * kbH;
-        p.s[0] = a.s_gate + srow;
-        p.s[1] = a.s_up + srow;
-        p.bias[0] = a.b_gate ? (const uint16_t*)a.b_gate + (int64_t)t.expert * a.I : nullptr;
-        p.bias[1] = a.b_up ? (const uint16_t*)a.b_up + (int64_t)t.expert * a.I : nullptr;
+        if (p.paired) {
+            p.w[0] = (const uint8_t*)a.w_gate + t.expert * HI;
+            p.w[1] = (const uint8_t*)a.w_up + t.expert * HI;
+            p.s[0] = a.s_gate + srow;
+            p.s[1] = a.s_up + srow;
+            p.bias[0] = a.b_gate ? (const uint16_t*)a.b_gate + (int64_t)t.expert * a.I : nullptr;
+            p.bias[1] = a.b_up ? (const uint16_t*)a.b_up + (int64_t)t.expert * a.I : nullptr;
+        } else {
+            p.w[0] = p.w[1] = (const uint8_t*)a.w_up + t.expert * HI;
+            p.s[0] = p.s[1] = a.s_up + srow;
+            p.bias[0] = a.b_up ? (const uint16_t*)a.b_up + (int64_t)t.expert * a.I : nullptr;
+            p.bias[1] = nullptr;
+            p.act = a.act;
+        }
         p.a_base = (const uint16_t*)a.x;
         p.gather = a.token_indices + t.row0;
         p.a_row0 = 0;
@@ -267,7 +281,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 }  // namespace
 
 int fp8_block_m() { return QBM; }
-int fp8_block_n0() { return QN0 * QSUB; }
+int fp8_block_n0(int swiglu) { return (swiglu ? QN0 : QN1) * QSUB; }
 int fp8_block_n1() { return QN1 * QSUB1; }
 
 int ffn_persistent_occupancy_fp8() {

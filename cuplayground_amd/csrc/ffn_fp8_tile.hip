@@ -5,9 +5,10 @@
 // fp32 accumulation, one cast on store) for that operand pair, with the numerics of ffn_fp8.hip:
 //   y[n] = sum over 128-wide k blocks of scale[n/128][kb] * (fp32 dot product of that block).
 //
-// A task is (expert, 128-token row block, 128 weight rows): 64 gate + 64 up rows for the up projection (SwiGLU pairs
-// stay inside a lane), 128 rows of w_down for the down projection; so all weight rows of a wavefront's fragments lie
-// in one scale block and the scale of a k block is one scalar (two for the up projection).
+// A task is (expert, 128-token row block, 128 weight rows): 64 gate + 64 up rows for a SwiGLU up projection (the pairs
+// stay inside a lane), 128 rows of w_up for ReLU / GELU layers, 128 rows of w_down for the down projection; so all
+// weight rows of a wavefront's fragments lie in one scale block and the scale of a k block is one scalar (two for a
+// SwiGLU up projection).
 //   * four wavefronts of 64 x 64 outputs, v_mfma_f32_16x16x32_bf16, weights as the "A" operand;
 //   * K slabs of 64: token rows go from global memory straight into LDS (global_load ... lds) as 128-byte rows with
 //     xor-swizzled 16-byte chunks; weight bytes are fetched into registers two slabs ahead, widened to bf16 once per
@@ -52,6 +53,8 @@ struct TileTask {
     const uint16_t* bias[2];
     uint16_t* c_base;           // h or y at the first row of the block
     int K, N, rows, c0, phase;
+    int act;                    // up projection without SwiGLU: the activation of the epilogue (else MOE_ACT_NONE)
+    bool paired;                // up projection with SwiGLU: 64 gate + 64 up rows; otherwise 128 rows of one matrix
     bool publish;               // rows are read by other workgroups of the same launch
 };
 
@@ -96,7 +99,7 @@ __device__ __forceinline__ void tile_mainloop(const TileTask& p, unsigned char* 
         const int j = brow + i * 64;                              // row of the weight tile
         const uint8_t* base = p.w[0];
         int col;
-        if (p.phase == 0) {   // wavefront column w owns tile rows [64 w, 64 w + 64): 32 gate rows, then 32 up rows
+        if (p.paired) {       // wavefront column w owns tile rows [64 w, 64 w + 64): 32 gate rows, then 32 up rows
             const int w = j >> 6, jj = j & 63;
             col = p.c0 + w * 32 + (jj & 31);
             base = (jj >> 5) ? p.w[1] : p.w[0];
@@ -259,7 +262,7 @@ __device__ __forceinline__ void tile_epilogue(const TileTask& p, f32x4 (&acc)[PT
         const int m = wm * 16 * PTM + i * 16 + frow;
         if (m >= p.rows) continue;
         uint16_t* crow = p.c_base + (int64_t)m * p.N;
-        if (p.phase == 0) {
+        if (p.paired) {
 #pragma unroll
             for (int j = 0; j < PTN / 2; ++j) {
                 const int col = p.c0 + wn * 32 + j * 16 + 4 * fk;
@@ -284,6 +287,7 @@ __device__ __forceinline__ void tile_epilogue(const TileTask& p, f32x4 (&acc)[PT
                 for (int r = 0; r < 4; ++r) {
                     o[r] = acc[i][j][r];
                     if (p.bias[0]) o[r] = o[r] + bf16_bits_to_f32(p.bias[0][col + r]);
+                    o[r] = act_apply(o[r], p.act);
                 }
                 const uint32_t lo = pack2_bf16(o[0], o[1]), hi = pack2_bf16(o[2], o[3]);
                 if (p.publish) publish8(crow + col, lo, hi);
@@ -307,17 +311,27 @@ __device__ __forceinline__ TileTask resolve_tile(const FfnArgs& a, const Task& t
     const int kbH = a.H >> 7, kbI = a.I >> 7;
     p.phase = t.phase;
     p.rows = t.rows;
+    p.act = MOE_ACT_NONE;
+    p.paired = t.phase == 0 && a.act == MOE_ACT_SWIGLU;
     if (t.phase == 0) {
-        p.c0 = t.ntile * PN0;
+        p.c0 = t.ntile * (p.paired ? PN0 : PN1);
         p.K = a.H;
         p.N = a.I;
-        p.w[0] = (const uint8_t*)a.w_gate + t.expert * HI;
-        p.w[1] = (const uint8_t*)a.w_up + t.expert * HI;
         const int64_t srow = ((int64_t)t.expert * kbI + (p.c0 >> 7)) * kbH;
-        p.s[0] = a.s_gate + srow;
-        p.s[1] = a.s_up + srow;
-        p.bias[0] = a.b_gate ? (const uint16_t*)a.b_gate + (int64_t)t.expert * a.I : nullptr;
-        p.bias[1] = a.b_up ? (const uint16_t*)a.b_up + (int64_t)t.expert * a.I : nullptr;
+        if (p.paired) {
+            p.w[0] = (const uint8_t*)a.w_gate + t.expert * HI;
+            p.w[1] = (const uint8_t*)a.w_up + t.expert * HI;
+            p.s[0] = a.s_gate + srow;
+            p.s[1] = a.s_up + srow;
+            p.bias[0] = a.b_gate ? (const uint16_t*)a.b_gate + (int64_t)t.expert * a.I : nullptr;
+            p.bias[1] = a.b_up ? (const uint16_t*)a.b_up + (int64_t)t.expert * a.I : nullptr;
+        } else {
+            p.w[0] = p.w[1] = (const uint8_t*)a.w_up + t.expert * HI;
+            p.s[0] = p.s[1] = a.s_up + srow;
+            p.bias[0] = a.b_up ? (const uint16_t*)a.b_up + (int64_t)t.expert * a.I : nullptr;
+            p.bias[1] = nullptr;
+            p.act = a.act;
+        }
         p.a_base = (const uint16_t*)a.x;
         p.gather = a.token_indices + t.row0;
         p.a_row0 = 0;
@@ -368,7 +382,7 @@ __global__ __launch_bounds__(PTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
         const TileTask p = resolve_tile(a, t, t.phase == 0 || a.arrive);
         const long long started = trace_clock(a.task_trace);
         if (ok) fp8_gemm_tile(p, smem);
-        else poison_tile(p.c_base, p.rows, p.N, p.c0, t.phase ? PN1 : PN0, 2);
+        else poison_tile(p.c_base, p.rows, p.N, p.c0, PN1, 2);
         if (a.task_trace) trace_task(a.task_trace, a.task_trace_cap, t.phase, t.expert, t.mtile, t.ntile, t.rows, started);
         if (t.phase == 0) signal_phase0_done(a.done0, t.mtile);
         else if (a.arrive) combine_arrivals<bf16_s>(combine_args(a), t.row0, t.rows, t.ntile, p.c0, PN1, s_list);
@@ -384,7 +398,7 @@ hipError_t allow_lds(K kernel) {
 }  // namespace
 
 int fp8_tile_block_m() { return PBM; }
-int fp8_tile_block_n0() { return PN0; }
+int fp8_tile_block_n0(int swiglu) { return swiglu ? PN0 : PN1; }
 int fp8_tile_block_n1() { return PN1; }
 
 int ffn_persistent_occupancy_fp8_tile() {

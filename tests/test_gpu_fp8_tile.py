@@ -20,6 +20,11 @@ SHAPES = {
     # many experts just above the plan's threshold: every row block is a partial one (about 40 of 128 rows), top-1
     "many_partial_blocks": ob.Cfg(S=2000, H=256, I=256, E=48, k=1, act=ob.ACT_SWIGLU, dtype=ob.FP8, gate_fn=ob.GATE_SOFTMAX,
                                   norm_topk=0, drop=0),
+    # up projection without SwiGLU: 128 rows of w_up per tile, activation in the epilogue; with and without biases
+    "gelu_bias": ob.Cfg(S=900, H=256, I=384, E=5, k=2, act=ob.ACT_GELU, dtype=ob.FP8, gate_fn=ob.GATE_SOFTMAX, drop=1,
+                        capacity_factor=1.25),
+    "relu": ob.Cfg(S=640, H=384, I=128, E=3, k=1, act=ob.ACT_RELU, dtype=ob.FP8, gate_fn=ob.GATE_SIGMOID, norm_topk=0,
+                   drop=0),
     # fewer rows than one block everywhere (the tile forced onto a decode-sized layer)
     "tiny_rows": ob.Cfg(S=40, H=256, I=128, E=8, k=2, act=ob.ACT_SWIGLU, dtype=ob.FP8, gate_fn=ob.GATE_SIGMOID, drop=0),
 }

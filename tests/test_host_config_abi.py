@@ -109,6 +109,11 @@ def test_workspace_and_unsupported_shapes():
     # every dtype of the reference schema has a kernel: tf32 is stored and computed as fp32 (twice the bytes of bf16)
     assert moe.MoEConfig(**{**base, "torch_dtype": 3}).workspace_bytes() == small
     assert moe.MoEConfig(**{**base, "torch_dtype": 1}).workspace_bytes() == moe.MoEConfig(**{**base, "torch_dtype": 0}).workspace_bytes() > small
+    # e4m3 layers take every activation; their sizes are multiples of the 128 x 128 scale block
+    assert moe.MoEConfig(**{**base, "torch_dtype": 4}).workspace_bytes() > 0
+    with pytest.raises(moe.MoEError) as e:
+        moe.MoEConfig(**{**base, "torch_dtype": 4, "intermediate_size": 192}).workspace_bytes()
+    assert e.value.status == 2
     for patch in ({"num_experts": 1024}, {"expert_top_k": 17, "num_experts": 64}, {"hidden_size": 32768}):
         with pytest.raises(moe.MoEError) as e:
             moe.MoEConfig(**{**base, **patch}).workspace_bytes()

@@ -35,6 +35,7 @@ PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
 BF16_SOURCES = ("ffn_bf16.hip", "ffn_bf16_slab_steady.inc", "ffn_common.hpp", "route.hip")
 FP8_SOURCES = ("ffn_fp8.hip", "ffn_common.hpp", "route.hip")
 FP8_TILE_SOURCES = ("ffn_fp8_tile.hip", "ffn_common.hpp", "route.hip")
+WIDEN_SOURCES = BF16_SOURCES + ("quant.hip",)
 MEASURED_TRAFFIC = {
     "mixtral": {"bytes": 19.48e9, "sources": BF16_SOURCES, "kernel_digest": "2192860045c2",
                 "profile": "profiles/ffn_persistent_kernel_bf16_mixtral_c3_hbm_traffic.txt"},
@@ -44,8 +45,12 @@ MEASURED_TRAFFIC = {
                     "profile": "profiles/ffn_persistent_kernel_bf16_finegrained_c4_hbm_traffic.txt"},
     "decode_fp8": {"bytes": 9.884e9, "sources": FP8_SOURCES, "kernel_digest": "f8fa608ab58a",
                    "profile": "profiles/ffn_persistent_fp8_kernel_decode_c5_hbm_traffic.txt"},
-    "prefill_fp8": {"bytes": 27.06e9, "sources": FP8_TILE_SOURCES, "kernel_digest": "8f1a6919616f",
-                    "profile": "profiles/ffn_persistent_fp8_tile_kernel_prefill_fp8_hbm_traffic.txt"},
+    # the widening pass and the bf16 queue kernel together (what the layer's FFN stage launches by default) ...
+    "prefill_fp8": {"bytes": 24.82e9, "sources": WIDEN_SOURCES, "kernel_digest": "b11cdfccc263",
+                    "profile": "profiles/widen_plus_ffn_persistent_kernel_prefill_fp8_hbm_traffic.txt"},
+    # ... and the e4m3 tile GEMM on the same layer (MOE355_FP8_WIDEN=0)
+    "prefill_fp8/e4m3_tile": {"bytes": 26.98e9, "sources": FP8_TILE_SOURCES, "kernel_digest": "8f1a6919616f",
+                              "profile": "profiles/ffn_persistent_fp8_tile_kernel_prefill_fp8_hbm_traffic.txt"},
 }
 
 
@@ -123,6 +128,7 @@ def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False, balanced_
     ffn = stats(samples["ffn"][-steps:])
     queue = layer.ffn_mode == 2   # one launch of the task-queue kernel; otherwise one launch per projection
     fp8 = c.torch_dtype == api.DTYPE_FP8
+    widened = fp8 and layer.kernel_dtype != c.torch_dtype   # the FFN stage widens the weights, then runs the bf16 tiles
     if w.bound == "hbm" and fp8:
         active = int((cnt > 0).sum())
         nbytes = wl.fp8_ffn_bytes(c, active, kept)
@@ -134,14 +140,16 @@ def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False, balanced_
     else:
         roof = {"bound": "mfma", "achieved": flops / (ffn["mean"] * 1e-3) / 1e12,
                 "peak": PEAK_F32_TFLOPS if c.torch_dtype == api.DTYPE_F32 else PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                "kernel": (("ffn_persistent_fp8_tile_kernel" if queue else "ffn_tiled_fp8_tile_kernel x2") if fp8 else
+                "kernel": (("ffn_persistent_fp8_tile_kernel" if queue else "ffn_tiled_fp8_tile_kernel x2")
+                           if fp8 and not widened else
+                           ("widen_block128_kernel x%d + " % (3 if c.hidden_act == api.ACT_SWIGLU else 2) if widened else "") +
                            ("ffn_persistent_kernel" if queue else "ffn_tiled_kernel x2")), "algorithmic_flops": flops}
         roof["layer_frac"] = layer_flops / (ms_per_step * 1e-3) / 1e12 / roof["peak"]
     roof["frac"] = roof["achieved"] / roof["peak"]
     roof["kernel_ms"] = ffn["mean"]
     roof["kernel_ms_median"] = ffn["median"]
     roof["kernel_ms_min"] = ffn["min"]
-    t = MEASURED_TRAFFIC.get(name)
+    t = MEASURED_TRAFFIC.get(name + ("/e4m3_tile" if fp8 and w.bound == "mfma" and not widened else ""))
     digest = kernel_digest(t["sources"]) if t else None
     if queue and t and t["kernel_digest"] == digest:
         roof["traffic"] = t["bytes"]
@@ -285,6 +293,7 @@ def cpu_leg(name, dev, out, routing, seconds, seed):
     c = w.config
     S = c.tokens
     fp8 = c.torch_dtype == api.DTYPE_FP8
+    widened = fp8 and layer.kernel_dtype != c.torch_dtype   # the FFN stage widens the weights, then runs the bf16 tiles
     threads = os.cpu_count() or 1
     env = os.environ.get("OMP_NUM_THREADS")
     if env and env.isdigit():

@@ -16,6 +16,7 @@ from .api import (  # noqa: F401
     load_library,
     measured_peaks,
     quantize_block128,
+    dequantize_block128,
     transpose,
 )
 from . import api  # noqa: F401

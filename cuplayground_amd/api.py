@@ -22,11 +22,11 @@ STAGES = ("gate", "route", "ffn", "combine")
 
 EXPORTS = (
     "moe_config_default", "moe_config_from_json_string", "moe_config_from_json_file", "moe_config_validate",
-    "moe_config_tokens", "moe_config_capacity", "moe_create", "moe_destroy", "moe_get_arch", "moe_get_plan",
+    "moe_config_tokens", "moe_config_capacity", "moe_create", "moe_destroy", "moe_get_arch", "moe_get_plan", "moe_get_kernel_dtype",
     "moe_workspace_bytes",
     "moe_set_ffn_mode", "moe_get_ffn_mode", "moe_forward", "moe_forward_static", "moe_set_spin_limit", "moe_clear_stall", "moe_gate", "moe_router_stats", "moe_route", "moe_gemm_bias_act", "moe_combine",
     "moe_set_stage_timing", "moe_get_stage_ms", "moe_get_stage_samples", "moe_get_task_counts", "moe_get_queue_balance", "moe_task_trace_bytes", "moe_set_task_trace", "moe_get_task_trace", "moe_measure_mfma_tflops",
-    "moe_measure_hbm_read_gbs", "moe_quant_block128", "moe_backward_scratch_bytes", "moe_transpose", "moe_expert_gemm",
+    "moe_measure_hbm_read_gbs", "moe_quant_block128", "moe_dequant_block128", "moe_backward_scratch_bytes", "moe_transpose", "moe_expert_gemm",
     "moe_expert_wgrad", "moe_act_backward", "moe_bias_grad", "moe_combine_backward", "moe_last_hip_error", "moe_status_string",
     "moe_version",
 )
@@ -87,6 +87,7 @@ def load_library():
     L.moe_destroy.argtypes = [vp]
     L.moe_get_arch.argtypes = [vp, C.POINTER(_CArch)]
     L.moe_get_plan.argtypes = [vp, C.POINTER(i32), C.POINTER(i32), C.POINTER(i32)]
+    L.moe_get_kernel_dtype.argtypes = [vp, C.POINTER(i32)]
     L.moe_workspace_bytes.argtypes = [cfgp, C.POINTER(C.c_size_t)]
     L.moe_set_ffn_mode.argtypes = [vp, C.c_int]
     L.moe_get_ffn_mode.argtypes = [vp, C.POINTER(C.c_int32)]
@@ -110,6 +111,7 @@ def load_library():
     L.moe_set_task_trace.argtypes = [vp, vp, C.c_size_t]
     L.moe_get_task_trace.argtypes = [vp, vp, vp, C.c_int64, C.POINTER(C.c_int64)]
     L.moe_quant_block128.argtypes = [vp, C.c_int32, C.c_int64, C.c_int64, C.c_int64, vp, vp, vp]
+    L.moe_dequant_block128.argtypes = [vp, vp, C.c_int64, C.c_int64, C.c_int64, vp, vp]
     L.moe_measure_mfma_tflops.argtypes = [vp, C.c_size_t, vp, C.c_int, C.POINTER(C.c_float)]
     L.moe_measure_hbm_read_gbs.argtypes = [vp, C.c_size_t, vp, vp, C.POINTER(C.c_float)]
     L.moe_backward_scratch_bytes.argtypes = [cfgp, C.POINTER(C.c_size_t)]
@@ -257,6 +259,14 @@ class MoELayer:
         a, b, c = C.c_int32(0), C.c_int32(0), C.c_int32(0)
         _check(self.L.moe_get_plan(self._h, C.byref(a), C.byref(b), C.byref(c)))
         return dict(block_rows=a.value, col_tiles_up=b.value, col_tiles_down=c.value)
+
+    @property
+    def kernel_dtype(self) -> int:
+        """The dtype whose FFN kernels run: the layer's own, or DTYPE_BF16 for an e4m3 layer with so many rows per
+        expert that every call widens the weights into the workspace and runs the bf16 tiles."""
+        d = C.c_int32(0)
+        _check(self.L.moe_get_kernel_dtype(self._h, C.byref(d)))
+        return d.value
 
     def set_ffn_mode(self, mode: int):
         _check(self.L.moe_set_ffn_mode(self._h, mode))
@@ -509,6 +519,20 @@ def quantize_block128(w):
     _check(load_library().moe_quant_block128(_ptr(w), dtype, mats, N, K, _ptr(q), _ptr(s), _stream()),
            "moe_quant_block128")
     return q, s
+
+
+def dequantize_block128(q, s):
+    """bf16(e4m3(q) * scale of its 128x128 block), rounded once: what an e4m3 layer with many rows per expert runs its
+    bf16 tile GEMM on.  q: uint8 / float8_e4m3fn [..., N, K], s: fp32 [..., N/128, K/128]."""
+    import torch
+    N, K = q.shape[-2:]
+    mats = q.numel() // (N * K)
+    q = q.contiguous()
+    s = s.contiguous()
+    out = torch.empty(q.shape, dtype=torch.bfloat16, device=q.device)
+    _check(load_library().moe_dequant_block128(_ptr(q), _ptr(s), mats, N, K, _ptr(out), _stream()),
+           "moe_dequant_block128")
+    return out
 
 
 def gemm_bias_act(A, B, bias, act: int):

@@ -54,12 +54,13 @@ struct Derived {
     int64_t capacity;
     FfnPlan plan;
     int nblk;          // workgroups of the slot-assignment kernels
+    int wide_mats;     // weight matrices per expert (3 with SwiGLU, else 2)
     int max_mtiles;
 };
 
 struct WsLayout {
     size_t logits, topk_idx, topk_w, slot, pair_row, token_indices, expert_count, expert_offset, rank_local,
-        block_hist, mtiles, seg0, seg1, segq, qstate, done0, wg_clock, arrive, stats_prob, stats_cnt, h, y, total;
+        block_hist, mtiles, seg0, seg1, segq, qstate, done0, wg_clock, arrive, stats_prob, stats_cnt, h, y, wide, total;
 };
 
 // Storage type of activations (x, biases, h, y, out): the layer's own, except that tf32 -- fp32 storage with
@@ -94,6 +95,7 @@ int derive(const moe_config& c, Derived* d) {
     moe_config_capacity(&c, &d->capacity);
     if (d->capacity > d->A) d->capacity = d->A;
     d->plan = ffn_plan(c.torch_dtype, c.hidden_act, d->H, d->I, d->A, d->E);
+    d->wide_mats = c.hidden_act == MOE_ACT_SWIGLU ? 3 : 2;
     d->nblk = ceil_div(d->A, kRouteBlock);
     d->max_mtiles = ceil_div(d->A, d->plan.block_m) + d->E;
     return MOE_OK;
@@ -125,6 +127,8 @@ WsLayout layout(const Derived& d) {
     w.stats_cnt = take((size_t)kStatsBlocks * d.E * 4);
     w.h = take((size_t)d.A * d.I * d.act_bytes);
     w.y = take((size_t)d.A * d.H * d.act_bytes);
+    // bf16 copies of an e4m3 layer's expert weights (up, down, gate), rewritten by every call of such a plan
+    w.wide = take(d.plan.widen ? (size_t)d.wide_mats * d.E * d.I * d.H * 2 : 0);
     w.total = off;
     return w;
 }
@@ -134,7 +138,19 @@ WsLayout layout(const Derived& d) {
 FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E) {
     FfnPlan p;
     p.tile = 0;
+    p.kernel_dtype = dtype;
+    p.widen = false;
     const bool sw = act == MOE_ACT_SWIGLU;
+    if (dtype == MOE_DTYPE_FP8_E4M3_B128) {
+        // With this many rows per expert one more pass over the weights (e4m3 -> bf16 into the workspace) costs less
+        // than the e4m3 tile GEMM loses to the bf16 one.
+        p.widen = A / (E > 0 ? E : 1) >= kFp8WidenRowsPerExpert;
+        if (const char* env = getenv("MOE355_FP8_WIDEN")) {   // tuning knob
+            const int v = atoi(env);
+            if (v == 0 || v == 1) p.widen = v;
+        }
+        if (p.widen) p.kernel_dtype = dtype = MOE_DTYPE_BF16;
+    }
     if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32) {
         p.block_m = f32_block_m();
         p.nnt0 = sw ? ceil_div(I, f32_block_n() / 2) : ceil_div(I, f32_block_n());
@@ -342,7 +358,8 @@ int moe_create(const moe_config* cfg, moe_handle** out) {
     if (hipDeviceGetAttribute(&h->wall_clock_khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess || h->wall_clock_khz <= 0)
         h->wall_clock_khz = 100000;   // 100 MHz on gfx950
     snprintf(h->arch.name, sizeof h->arch.name, "%s", prop.gcnArchName);
-    int per_cu = ffn_persistent_blocks(cfg->torch_dtype, d.plan.tile, 1);
+    const int kdt = d.plan.kernel_dtype;
+    int per_cu = ffn_persistent_blocks(kdt, d.plan.tile, 1);
     if (const char* env = getenv("MOE355_BLOCKS_PER_CU")) {   // tuning knob: resident workgroups per CU
         const int v = atoi(env);
         if (v >= 1 && v <= 16) per_cu = v;
@@ -350,8 +367,8 @@ int moe_create(const moe_config* cfg, moe_handle** out) {
     h->arch.persistent_blocks = prop.multiProcessorCount * per_cu;
     // One task queue per XCD for the MFMA-bound bf16 tiles, whose operand tiles are then shared in that XCD's L2;
     // so does the e4m3 tile GEMM; the f32 path and the e4m3 weight streamer keep a single queue.
-    h->queue_groups = (cfg->torch_dtype == MOE_DTYPE_BF16 || cfg->torch_dtype == MOE_DTYPE_FP16 ||
-                       (cfg->torch_dtype == MOE_DTYPE_FP8_E4M3_B128 && d.plan.tile)) ? h->arch.xcds : 1;
+    h->queue_groups = (kdt == MOE_DTYPE_BF16 || kdt == MOE_DTYPE_FP16 ||
+                       (kdt == MOE_DTYPE_FP8_E4M3_B128 && d.plan.tile)) ? h->arch.xcds : 1;
     if (const char* env = getenv("MOE355_QUEUE_GROUPS")) {   // tuning knob; never more queues than XCDs
         const int v = atoi(env);
         if ((v == 1 || v == 2 || v == 4 || v == 8) && v <= h->arch.xcds) h->queue_groups = v;
@@ -361,7 +378,7 @@ int moe_create(const moe_config* cfg, moe_handle** out) {
     // of their weight rows (e4m3): two row blocks at a time, all of a queue's column tiles of those (measured on the
     // Mixtral shape with e4m3 weights: 6.57 ms against 6.96 with all row blocks of the expert at a time; 1: 6.62,
     // 4: 6.76, 8: 6.89).  The bf16 tiles are indifferent (within 1 %) and keep the plain order.
-    h->row_chunk = (cfg->torch_dtype == MOE_DTYPE_FP8_E4M3_B128 && d.plan.tile) ? 2 : 0;
+    h->row_chunk = (kdt == MOE_DTYPE_FP8_E4M3_B128 && d.plan.tile) ? 2 : 0;
     if (const char* env = getenv("MOE355_ROW_CHUNK")) {   // tuning knob
         const int v = atoi(env);
         if (v >= 0 && v <= 4096) h->row_chunk = v;
@@ -403,6 +420,12 @@ int moe_get_plan(const moe_handle* h, int32_t* block_rows, int32_t* col_tiles_up
     if (block_rows) *block_rows = h->d.plan.block_m;
     if (col_tiles_up) *col_tiles_up = h->d.plan.nnt0;
     if (col_tiles_down) *col_tiles_down = h->d.plan.nnt1;
+    return MOE_OK;
+}
+
+int moe_get_kernel_dtype(const moe_handle* h, int32_t* dtype) {
+    if (!h || !dtype) return MOE_ERR_BAD_ARGUMENT;
+    *dtype = h->d.plan.kernel_dtype;
     return MOE_OK;
 }
 
@@ -604,13 +627,29 @@ int forward_on(moe_handle* h, const void* x, const moe_weights* w, void* out, co
         fa.w_bytes = (uint32_t)((int64_t)d.I * d.H * es);
     }
     const int mode = resolved_ffn_mode(h);
-    if (fp8) {
+    const int kdt = d.plan.kernel_dtype;
+    if (d.plan.widen) {   // the layer's e4m3 weights become bf16 ones in the workspace; from here on it is a bf16 layer
+        const int64_t mat = (int64_t)d.I * d.H;
+        char* wide = at<char>(workspace, L.wide);
+        const void* src[3] = {w->w_up, w->w_down, w->w_gate};
+        const float* scl[3] = {w->s_up, w->s_down, w->s_gate};
+        const void** dst[3] = {&fa.w_up, &fa.w_down, &fa.w_gate};
+        for (int i = 0; i < d.wide_mats; ++i) {
+            void* o = wide + (size_t)i * d.E * mat * 2;
+            // w_up and w_gate are [E, I, H], w_down is [E, H, I]
+            e = launch_widen_block128(src[i], scl[i], o, d.E, i == 1 ? d.H : d.I, i == 1 ? d.I : d.H, st);
+            if (e != hipSuccess) return hip_fail(h, e);
+            *dst[i] = o;
+        }
+        fa.s_up = fa.s_gate = fa.s_down = nullptr;
+    }
+    if (kdt == MOE_DTYPE_FP8_E4M3_B128) {
         e = (d.plan.tile ? launch_ffn_fp8_tile : launch_ffn_fp8)(fa, d.max_mtiles, d.plan.nnt0, d.plan.nnt1,
                                                                  mode == MOE_FFN_PERSISTENT ? h->arch.persistent_blocks : 0, st);
     } else if (mode == MOE_FFN_PERSISTENT) {
-        e = launch_ffn_persistent(fa, c.torch_dtype, d.plan, h->arch.persistent_blocks, st);
+        e = launch_ffn_persistent(fa, kdt, d.plan, h->arch.persistent_blocks, st);
     } else {
-        e = launch_ffn_tiled(fa, c.torch_dtype, d.plan, d.max_mtiles, st);
+        e = launch_ffn_tiled(fa, kdt, d.plan, d.max_mtiles, st);
     }
     if (e != hipSuccess) return hip_fail(h, e);
     if ((e = mark(3)) != hipSuccess) return hip_fail(h, e);

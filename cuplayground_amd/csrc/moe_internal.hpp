@@ -50,6 +50,11 @@ constexpr int kMaxQueueGroups = 8;   // XCDs of a gfx950
 // (H 4096, I 14336, 8 experts and H 7168, I 2048, 64 experts): at 16 rows per expert the streamer is 18 % faster, at 32
 // the tile GEMM 13-17 %, at 128 it is 2.5 times and from 1024 on 3.3 times as fast.
 constexpr int kFp8TileRowsPerExpert = 32;
+// ... and from which widening the weights to bf16 in the workspace (one pass over them per call, 4.9 TB/s) and running
+// the bf16 tile GEMM replaces the e4m3 tile GEMM.  Measured, e4m3 tile time / this: H 4096, I 14336, 8 experts 1.01 at
+// 512 rows per expert, 1.08 at 768, 1.18 at 1024, 1.34 at 2048; H 7168, I 2048, 64 experts 0.95 at 512, 1.17 at 1024,
+// 1.30 at 2048; H = I = 2048, 16 experts 1.23 at 1024, 1.36 at 2048.
+constexpr int kFp8WidenRowsPerExpert = 768;
 struct QueueState {
     int32_t groups;        // queue groups (1 or the number of XCDs)
     int32_t total_tasks;   // tasks of both phases (holes not counted)
@@ -149,12 +154,16 @@ hipError_t launch_combine(const void* y_rows, const int32_t* pair_row, const flo
 
 // FFN stage.  block_m / block_n are the tile sizes the routing stage must be told about.
 struct FfnPlan {
+    int kernel_dtype;   // the dtype whose kernels run: the layer's, or bf16 for an e4m3 layer whose weights are widened
+    bool widen;         // e4m3 layer run as a bf16 layer on weights widened into the workspace by every call
     int tile;        // 16-bit layers: which tile the kernels are instantiated with (ffn_bf16.hip: bf16_tile)
     int block_m;
     int nnt0;        // column tiles of phase 0
     int nnt1;        // column tiles of phase 1
 };
 FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E);
+hipError_t launch_widen_block128(const void* q, const float* scales, void* out, int64_t matrices, int64_t N, int64_t K,
+                                 hipStream_t st);
 hipError_t launch_ffn_tiled(const FfnArgs& a, int dtype, const FfnPlan& p, int max_mtiles, hipStream_t st);
 hipError_t launch_ffn_persistent(const FfnArgs& a, int dtype, const FfnPlan& p, int blocks, hipStream_t st);
 int ffn_persistent_blocks(int dtype, int tile, int compute_units);

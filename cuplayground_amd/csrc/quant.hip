@@ -73,7 +73,50 @@ __global__ __launch_bounds__(256) void quant_block128_kernel(const T* __restrict
     }
 }
 
+// The inverse, for layers that run the 16-bit tile GEMM on e4m3 weights: out = bf16(e4m3(q) * scale of its block), round
+// to nearest even (the product of a 4-bit significand and an fp32 scale is rounded once, to 8 bits: 2^-9 relative,
+// a thirty-second of the e4m3 rounding step).  A lane widens 16 consecutive codes of one row (one scale block).
+__global__ __launch_bounds__(256) void widen_block128_kernel(const uint8_t* __restrict__ q, const float* __restrict__ scales,
+                                                             uint16_t* __restrict__ out, int64_t rows, int64_t N,
+                                                             int64_t K) {
+    const int64_t chunk = (int64_t)blockIdx.x * 256 + threadIdx.x;   // 16 codes each
+    const int64_t per_row = K / 16;
+    if (chunk >= rows * per_row) return;
+    const int64_t row = chunk / per_row, c0 = (chunk - row * per_row) * 16;
+    const int64_t mat = row / N, r = row - mat * N;
+    const float s = scales[(mat * (N / 128) + r / 128) * (K / 128) + c0 / 128];
+    const uint4 in = *reinterpret_cast<const uint4*>(q + row * K + c0);
+    const uint32_t w[4] = {in.x, in.y, in.z, in.w};
+    uint32_t o[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int hi = 0; hi < 2; ++hi) {
+            const auto f = hi ? __builtin_amdgcn_cvt_pk_f32_fp8(w[i], true) : __builtin_amdgcn_cvt_pk_f32_fp8(w[i], false);
+            uint32_t b[2];
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const uint32_t u = __float_as_uint(f[e] * s);
+                b[e] = (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+            }
+            o[2 * i + hi] = b[0] | (b[1] << 16);
+        }
+    }
+    uint4* dst = reinterpret_cast<uint4*>(out + row * K + c0);
+    dst[0] = make_uint4(o[0], o[1], o[2], o[3]);
+    dst[1] = make_uint4(o[4], o[5], o[6], o[7]);
+}
+
 }  // namespace
+
+hipError_t launch_widen_block128(const void* q, const float* scales, void* out, int64_t matrices, int64_t N, int64_t K,
+                                 hipStream_t st) {
+    const int64_t chunks = matrices * N * (K / 16);
+    widen_block128_kernel<<<(unsigned)((chunks + 255) / 256), 256, 0, st>>>((const uint8_t*)q, scales, (uint16_t*)out,
+                                                                             matrices * N, N, K);
+    return hipGetLastError();
+}
+
 }  // namespace moe355
 
 using namespace moe355;
@@ -90,4 +133,11 @@ extern "C" int moe_quant_block128(const void* w, int32_t src_dtype, int64_t matr
     else
         quant_block128_kernel<uint16_t><<<grid, 256, 0, st>>>((const uint16_t*)w, (uint8_t*)q, scales, N, K);
     return hipGetLastError() == hipSuccess ? MOE_OK : MOE_ERR_HIP;
+}
+
+extern "C" int moe_dequant_block128(const void* q, const float* scales, int64_t matrices, int64_t N, int64_t K, void* out,
+                                    void* stream) {
+    if (!q || !out || !scales || matrices < 1 || N < 128 || K < 128 || (N % 128) || (K % 128)) return MOE_ERR_BAD_ARGUMENT;
+    if (matrices * N * (K / 16) > (int64_t)0x7FFFFFFF * 256) return MOE_ERR_BAD_ARGUMENT;
+    return launch_widen_block128(q, scales, out, matrices, N, K, (hipStream_t)stream) == hipSuccess ? MOE_OK : MOE_ERR_HIP;
 }

@@ -105,6 +105,11 @@ int moe_get_arch(const moe_handle* h, moe_arch* out);
 /* The tiling the handle chose: rows per row block, and column tiles of the up(/gate) and of the down projection.
  * Task totals follow the reference's bound tilesM*tilesNx + tilesM*tilesN (scheduling.cuh:212-222) per expert. */
 int moe_get_plan(const moe_handle* h, int32_t* block_rows, int32_t* col_tiles_up, int32_t* col_tiles_down);
+/* The dtype whose FFN kernels the handle runs: cfg.torch_dtype, except MOE_DTYPE_BF16 for an e4m3 layer whose experts
+ * see so many rows (768 on average; MOE355_FP8_WIDEN = 0 / 1 overrides) that every moe_forward first widens the weights
+ * to bf16 in the workspace (moe_dequant_block128; moe_workspace_bytes then includes 2 bytes per weight) and runs
+ * the bf16 tiles on them.  The reference fixes its element types at compile time (processor/tiling.cuh:97-159). */
+int moe_get_kernel_dtype(const moe_handle* h, int32_t* dtype);
 int moe_workspace_bytes(const moe_config* cfg, size_t* bytes);
 
 typedef struct moe_weights {
@@ -262,6 +267,13 @@ int moe_measure_hbm_read_gbs(const void* src, size_t bytes, void* scratch, void*
  * `stream`.  No counterpart in the reference, whose dtypes stop at fp16 (aristos_config.schema.json:49-53). */
 int moe_quant_block128(const void* w, int32_t src_dtype, int64_t matrices, int64_t N, int64_t K, void* q,
                        float* scales, void* stream);
+
+/* The inverse: out[matrices,N,K] (bf16) = e4m3(q) * scale of its block, rounded to nearest even once.  moe_forward
+ * runs this on an e4m3 layer's weights, into its workspace, when the experts see enough rows for the bf16 tile GEMM
+ * plus this pass to beat the e4m3 kernels (see moe_workspace_bytes).  Asynchronous on `stream`.  No counterpart in
+ * the reference (same reason). */
+int moe_dequant_block128(const void* q, const float* scales, int64_t matrices, int64_t N, int64_t K, void* out,
+                         void* stream);
 
 /* ---- Backward building blocks (bf16 and fp16 layers) -------------------------------------------------------------
  * The reference declares a training knob (is_training, aristos_config.schema.json:20-23) that none of its code reads

@@ -18,8 +18,9 @@ def test_traffic_table_names_existing_profiles_and_sources():
     sys.path.insert(0, ROOT)
     import bench
     from cuplayground_amd import workloads as wl
-    assert set(bench.MEASURED_TRAFFIC) <= set(wl.WORKLOADS)
-    for name, t in bench.MEASURED_TRAFFIC.items():
+    assert {k.split("/")[0] for k in bench.MEASURED_TRAFFIC} <= set(wl.WORKLOADS)
+    for key, t in bench.MEASURED_TRAFFIC.items():
+        name = key.split("/")[0]       # "<workload>/<plan>": the same workload under a non-default plan
         assert os.path.isfile(os.path.join(ROOT, t["profile"])), t["profile"]
         for src in t["sources"]:
             assert os.path.isfile(os.path.join(ROOT, "cuplayground_amd", "csrc", src)), src

@@ -35,6 +35,7 @@ def _run(cfg, inp, mode, tile, monkeypatch, calls=1):
     import cuplayground_amd as moe
     assert torch.cuda.is_available(), "these tests need the MI355X"
     monkeypatch.setenv("MOE355_FP8_TILE", str(tile))
+    monkeypatch.setenv("MOE355_FP8_WIDEN", "0")
     layer = moe.MoELayer(product_config(cfg), ffn_mode=mode)
     assert layer.plan["block_rows"] == (128 if tile else 16)
     dev = upload_inputs(cfg, inp)
@@ -97,6 +98,7 @@ def test_prefill_sized_layer_on_a_stratified_sample(monkeypatch):
     import cuplayground_amd as moe
     from test_gpu_fullsize import stratified_tokens
     cfg = ob.Cfg(S=4096, H=2048, I=5632, E=8, k=2, act=ob.ACT_SWIGLU, dtype=ob.FP8, gate_fn=ob.GATE_SOFTMAX, drop=0)
+    monkeypatch.setenv("MOE355_FP8_WIDEN", "0")   # this many rows per expert would run the bf16 tile on widened weights
     inp = ob.make_inputs(cfg, seed=42)
     want = ob.route(cfg, inp)
     layer = moe.MoELayer(product_config(cfg), ffn_mode=FFN_PERSISTENT)

@@ -36,6 +36,7 @@ BF16_SOURCES = ("ffn_bf16.hip", "ffn_bf16_slab_steady.inc", "ffn_common.hpp", "r
 FP8_SOURCES = ("ffn_fp8.hip", "ffn_common.hpp", "route.hip")
 FP8_TILE_SOURCES = ("ffn_fp8_tile.hip", "ffn_common.hpp", "route.hip")
 WIDEN_SOURCES = BF16_SOURCES + ("quant.hip",)
+F32_TILE_SOURCES = ("ffn_f32_tile.hip", "ffn_common.hpp", "route.hip")
 MEASURED_TRAFFIC = {
     "mixtral": {"bytes": 19.48e9, "sources": BF16_SOURCES, "kernel_digest": "2192860045c2",
                 "profile": "profiles/ffn_persistent_kernel_bf16_mixtral_c3_hbm_traffic.txt"},
@@ -45,6 +46,8 @@ MEASURED_TRAFFIC = {
                     "profile": "profiles/ffn_persistent_kernel_bf16_finegrained_c4_hbm_traffic.txt"},
     "decode_fp8": {"bytes": 9.884e9, "sources": FP8_SOURCES, "kernel_digest": "f8fa608ab58a",
                    "profile": "profiles/ffn_persistent_fp8_kernel_decode_c5_hbm_traffic.txt"},
+    "reference_default": {"bytes": 2.646e9, "sources": F32_TILE_SOURCES, "kernel_digest": "4c8b49a5d3ae",
+                          "profile": "profiles/ffn_persistent_f32_tile_kernel_reference_default_hbm_traffic.txt"},
     # the widening pass and the bf16 queue kernel together (what the layer's FFN stage launches by default) ...
     "prefill_fp8": {"bytes": 24.82e9, "sources": WIDEN_SOURCES, "kernel_digest": "b11cdfccc263",
                     "profile": "profiles/widen_plus_ffn_persistent_kernel_prefill_fp8_hbm_traffic.txt"},
@@ -129,6 +132,8 @@ def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False, balanced_
     queue = layer.ffn_mode == 2   # one launch of the task-queue kernel; otherwise one launch per projection
     fp8 = c.torch_dtype == api.DTYPE_FP8
     widened = fp8 and layer.kernel_dtype != c.torch_dtype   # the FFN stage widens the weights, then runs the bf16 tiles
+    # fp32 layers: the matrix-core tile (128-row blocks) or the vector-ALU kernel (64-row blocks)
+    f32_kind = "" if c.torch_dtype != api.DTYPE_F32 else ("_f32_tile" if layer.plan["block_rows"] == 128 else "_f32")
     if w.bound == "hbm" and fp8:
         active = int((cnt > 0).sum())
         nbytes = wl.fp8_ffn_bytes(c, active, kept)
@@ -143,7 +148,8 @@ def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False, balanced_
                 "kernel": (("ffn_persistent_fp8_tile_kernel" if queue else "ffn_tiled_fp8_tile_kernel x2")
                            if fp8 and not widened else
                            ("widen_block128_kernel x%d + " % (3 if c.hidden_act == api.ACT_SWIGLU else 2) if widened else "") +
-                           ("ffn_persistent_kernel" if queue else "ffn_tiled_kernel x2")), "algorithmic_flops": flops}
+                           ("ffn_persistent%s_kernel" if queue else "ffn_tiled%s_kernel x2") % f32_kind),
+                "algorithmic_flops": flops}
         roof["layer_frac"] = layer_flops / (ms_per_step * 1e-3) / 1e12 / roof["peak"]
     roof["frac"] = roof["achieved"] / roof["peak"]
     roof["kernel_ms"] = ffn["mean"]
@@ -294,6 +300,8 @@ def cpu_leg(name, dev, out, routing, seconds, seed):
     S = c.tokens
     fp8 = c.torch_dtype == api.DTYPE_FP8
     widened = fp8 and layer.kernel_dtype != c.torch_dtype   # the FFN stage widens the weights, then runs the bf16 tiles
+    # fp32 layers: the matrix-core tile (128-row blocks) or the vector-ALU kernel (64-row blocks)
+    f32_kind = "" if c.torch_dtype != api.DTYPE_F32 else ("_f32_tile" if layer.plan["block_rows"] == 128 else "_f32")
     threads = os.cpu_count() or 1
     env = os.environ.get("OMP_NUM_THREADS")
     if env and env.isdigit():
@@ -384,7 +392,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="mixtral", choices=sorted(wl.WORKLOADS))
-    ap.add_argument("--extra", default="decode_fp8,mid,finegrained",
+    ap.add_argument("--extra", default="decode_fp8,mid,finegrained,reference_default,prefill_fp8",
                     help="comma-separated workloads measured besides the headline one (\"\" or none: skip)")
     ap.add_argument("--extra-steps", type=int, default=20)
     ap.add_argument("--ffn-mode", type=int, default=0, help="0 auto, 1 tiled (two launches), 2 persistent queue")

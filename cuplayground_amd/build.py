@@ -10,7 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmoe355.so")
 SOURCES = ["config.cpp", "api.hip", "gate.hip", "route.hip", "combine.hip", "ffn_bf16.hip", "ffn_f32.hip",
-           "ffn_fp8.hip", "ffn_fp8_tile.hip", "peaks.hip", "quant.hip", "backward.hip"]
+           "ffn_fp8.hip", "ffn_fp8_tile.hip", "ffn_f32_tile.hip", "peaks.hip", "quant.hip", "backward.hip"]
 # packed-fp32 VALU forms are disabled for every device code object of this library
 FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-x", "hip", "-Wall", "-Wno-unused-function",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

@@ -40,6 +40,11 @@ int fp8_tile_block_m();
 int fp8_tile_block_n0(int swiglu);
 int fp8_tile_block_n1();
 int ffn_persistent_occupancy_fp8_tile();
+hipError_t launch_ffn_f32_tile(const FfnArgs&, int max_mtiles, int nnt0, int nnt1, int blocks, hipStream_t);
+int f32_tile_block_m();
+int f32_tile_block_n0(int swiglu);
+int f32_tile_block_n1();
+int ffn_persistent_occupancy_f32_tile();
 
 namespace {
 
@@ -152,9 +157,24 @@ FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E) {
         if (p.widen) p.kernel_dtype = dtype = MOE_DTYPE_BF16;
     }
     if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32) {
-        p.block_m = f32_block_m();
-        p.nnt0 = sw ? ceil_div(I, f32_block_n() / 2) : ceil_div(I, f32_block_n());
-        p.nnt1 = ceil_div(H, f32_block_n());
+        // 0: 64 x 64 tiles on the vector ALUs (small and ragged layers); 1: 128 x 128 tiles on the matrix cores
+        // (from a full row block per expert on average, and enough 128 x 128 tiles to occupy the compute units twice over:
+        // below that the smaller tiles of the vector kernel spread the same work over more of the chip)
+        const int64_t tiles = (A / f32_tile_block_m()) * (ceil_div(I, f32_tile_block_n0(sw)) + ceil_div(H, f32_tile_block_n1()));
+        p.tile = H % 128 == 0 && I % 128 == 0 && A / (E > 0 ? E : 1) >= kF32TileRowsPerExpert && tiles >= kF32TileMinTiles ? 1 : 0;
+        if (const char* env = getenv("MOE355_F32_TILE")) {   // tuning knob
+            const int v = atoi(env);
+            if (v == 0 || (v == 1 && H % 128 == 0 && I % 128 == 0)) p.tile = v;
+        }
+        if (p.tile) {
+            p.block_m = f32_tile_block_m();
+            p.nnt0 = ceil_div(I, f32_tile_block_n0(sw));
+            p.nnt1 = ceil_div(H, f32_tile_block_n1());
+        } else {
+            p.block_m = f32_block_m();
+            p.nnt0 = sw ? ceil_div(I, f32_block_n() / 2) : ceil_div(I, f32_block_n());
+            p.nnt1 = ceil_div(H, f32_block_n());
+        }
     } else if (dtype == MOE_DTYPE_FP8_E4M3_B128) {
         // 0: weight streamer over 16-token row blocks (decode); 1: 128 x 128 tile GEMM once the experts see enough
         // rows for a weight tile to be reused from LDS instead of being fetched again per 16 rows
@@ -366,7 +386,8 @@ int moe_create(const moe_config* cfg, moe_handle** out) {
     }
     h->arch.persistent_blocks = prop.multiProcessorCount * per_cu;
     // One task queue per XCD for the MFMA-bound bf16 tiles, whose operand tiles are then shared in that XCD's L2;
-    // so does the e4m3 tile GEMM; the f32 path and the e4m3 weight streamer keep a single queue.
+    // so does the e4m3 tile GEMM; the fp32 kernels (the matrix-core tile measured 5 % faster on one queue than on eight)
+    // and the e4m3 weight streamer keep a single queue.
     h->queue_groups = (kdt == MOE_DTYPE_BF16 || kdt == MOE_DTYPE_FP16 ||
                        (kdt == MOE_DTYPE_FP8_E4M3_B128 && d.plan.tile)) ? h->arch.xcds : 1;
     if (const char* env = getenv("MOE355_QUEUE_GROUPS")) {   // tuning knob; never more queues than XCDs
@@ -929,17 +950,21 @@ int moe_combine(const void* y_rows, const int32_t* pair_row, const float* topk_w
 namespace moe355 {
 
 hipError_t launch_ffn_tiled(const FfnArgs& a, int dtype, const FfnPlan& p, int max_mtiles, hipStream_t st) {
-    if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32) return launch_ffn_tiled_f32(a, max_mtiles, p.nnt0, p.nnt1, st);
+    if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32)
+        return p.tile ? launch_ffn_f32_tile(a, max_mtiles, p.nnt0, p.nnt1, 0, st)
+                      : launch_ffn_tiled_f32(a, max_mtiles, p.nnt0, p.nnt1, st);
     return launch_ffn_tiled_bf16(a, p.tile, max_mtiles, p.nnt0, p.nnt1, st, dtype == MOE_DTYPE_FP16);
 }
 
 hipError_t launch_ffn_persistent(const FfnArgs& a, int dtype, const FfnPlan& p, int blocks, hipStream_t st) {
-    if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32) return launch_ffn_persistent_f32(a, blocks, st);
+    if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32)
+        return p.tile ? launch_ffn_f32_tile(a, 0, p.nnt0, p.nnt1, blocks, st) : launch_ffn_persistent_f32(a, blocks, st);
     return launch_ffn_persistent_bf16(a, p.tile, blocks, st, dtype == MOE_DTYPE_FP16);
 }
 
 int ffn_persistent_blocks(int dtype, int tile, int compute_units) {
-    if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32) return compute_units * 4;
+    if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32)
+        return compute_units * (tile ? ffn_persistent_occupancy_f32_tile() : 4);
     if (dtype == MOE_DTYPE_FP8_E4M3_B128)
         return compute_units * (tile ? ffn_persistent_occupancy_fp8_tile() : ffn_persistent_occupancy_fp8());
     return compute_units * ffn_persistent_occupancy_bf16(tile);

@@ -1,6 +1,6 @@
 // Expert FFN in fp32 (torch_dtype 0): the reference's tile GEMM contract, C = act(A.B^T + bias)
 // (mma.cuh:46-179; its only instantiated case is fp32 + ReLU, mma.cuh:378-384), on the vector ALUs.
-// fp32 layers are tiny and bandwidth bound, so this is a plain LDS-tiled FMA kernel: 64x64 output tile,
+// This is the kernel of small and ragged fp32 layers (large ones take ffn_f32_tile.hip): a plain LDS-tiled FMA kernel, 64x64 output tile,
 // 16-wide K slabs, 256 threads with a 4x4 register block each.  Task decoding, dispatch-by-gather and the
 // phase dependency protocol are shared with the bf16 path.
 #include "ffn_common.hpp"

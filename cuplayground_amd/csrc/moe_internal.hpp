@@ -55,6 +55,12 @@ constexpr int kFp8TileRowsPerExpert = 32;
 // 512 rows per expert, 1.08 at 768, 1.18 at 1024, 1.34 at 2048; H 7168, I 2048, 64 experts 0.95 at 512, 1.17 at 1024,
 // 1.30 at 2048; H = I = 2048, 16 experts 1.23 at 1024, 1.36 at 2048.
 constexpr int kFp8WidenRowsPerExpert = 768;
+// fp32 layers: average rows per expert and number of 128 x 128 tiles from which the matrix-core tile replaces the 64 x 64
+// vector-ALU one.  Measured FFN stage, vector / matrix: the reference's knob file (8192 rows, one expert, H 1024, I 4096)
+// 2.13 / 1.13 ms; 512 rows per expert, 16 experts, H 1024, I 2048, SwiGLU 1.81 / 1.00 ms; 64 rows per expert, 8 experts,
+// H 1024, I 4096 (320 tiles) 0.387 / 0.384 ms; 128 rows per expert, 8 experts, H 256, I 512 (48 tiles) 0.059 / 0.077 ms.
+constexpr int kF32TileRowsPerExpert = 128;
+constexpr int kF32TileMinTiles = 512;
 struct QueueState {
     int32_t groups;        // queue groups (1 or the number of XCDs)
     int32_t total_tasks;   // tasks of both phases (holes not counted)

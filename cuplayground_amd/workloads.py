@@ -8,8 +8,9 @@ aristos_config.schema.json:5-58):
   finegrained  S=16384 H=2048 I=1408  E=64  top-6, SwiGLU, bf16, cf 1.0, per-expert logit bias ~ Zipf(1.1) loads
   decode_fp8   S=64    H=7168 I=2048  E=256 top-8 sigmoid, SwiGLU, e4m3 weights with 128x128 block scales, bf16 tokens
 Tokens are N(0,1), gate and expert weights N(0,0.02), rounded once to their storage types.
-One more shape, not among the five, exercises the e4m3 tile GEMM that prefill-sized e4m3 layers take:
-  prefill_fp8  the mixtral shape with e4m3 weights and 128x128 block scales (bf16 tokens, bf16 MFMA arithmetic)
+Two more shapes, not among the five:
+  prefill_fp8        the mixtral shape with e4m3 weights and 128x128 block scales (bf16 tokens, bf16 MFMA arithmetic)
+  reference_default  the reference's own aristos_config.json: S=8192 H=1024 I=4096 E=1 top-1, ReLU, fp32
 """
 from __future__ import annotations
 
@@ -48,6 +49,8 @@ WORKLOADS = {
     "decode_fp8": Workload("C5", _cfg(64, 7168, 2048, 256, 8, api.ACT_SWIGLU, api.DTYPE_FP8, 1.0, 0,
                                       gate_fn=api.GATE_SIGMOID), bound="hbm"),
     "prefill_fp8": Workload("X1", _cfg(8192, 4096, 14336, 8, 2, api.ACT_SWIGLU, api.DTYPE_FP8, 2.0, 0)),
+    # the knob file the reference ships (aristos_config.json): one expert, fp32, ReLU, 4 x 2048 tokens
+    "reference_default": Workload("R0", _cfg(8192, 1024, 4096, 1, 1, api.ACT_RELU, api.DTYPE_F32, 1.0, 0, norm=0)),
 }
 
 

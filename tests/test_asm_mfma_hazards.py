@@ -102,7 +102,7 @@ def test_no_accumulator_access_behind_asm_mfma():
 
 
 @pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
-@pytest.mark.parametrize("source", ["ffn_bf16.hip", "ffn_f32.hip", "ffn_fp8.hip", "ffn_fp8_tile.hip"])
+@pytest.mark.parametrize("source", ["ffn_bf16.hip", "ffn_f32.hip", "ffn_f32_tile.hip", "ffn_fp8.hip", "ffn_fp8_tile.hip"])
 def test_phase0_results_are_complete_before_they_are_signalled(source):
     """The hand-off of the intermediate rows between workgroups: in signal_phase0_done every wavefront must wait for
     its own stores (s_waitcnt vmcnt(0)) before the workgroup barrier and the counter increment that publishes the
@@ -159,6 +159,41 @@ def test_fp8_tile_barriers_sit_behind_their_waits():
                     assert not [y for y in loop if y.startswith("scratch_")], (name, "spill in the slab loop")
                     slab_loops += 1
         assert slab_loops >= 2, name      # the full-block loop and the partial-block loops
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
+def test_f32_tile_barriers_sit_behind_their_waits():
+    """The fp32 tile GEMM (ffn_f32_tile.hip) fills both LDS stages with direct-to-LDS loads and meets once per slab at a
+    bare s_barrier behind s_waitcnt vmcnt(0) lgkmcnt(0): between that wait and the barrier the compiler may not have
+    placed an LDS access or a load, and each slab loop holds its 64 fp32 MFMAs, its 8 loads and no spill."""
+    text = _assembly("ffn_f32_tile.hip")
+    kernels = re.findall(r"\n(_ZN6moe355\w*f32_tile_kernel\w*):[^\n]*\n(.*?)\n\s*s_endpgm", text, re.S)
+    assert len(kernels) == 2
+    for name, body in kernels:
+        lines = [x.strip() for x in body.split("\n") if x.strip() and not x.strip().startswith(";")]
+        labels = {x.split(":")[0]: i for i, x in enumerate(lines) if re.match(r"\.LBB\d+_\d+:", x)}
+        # loops = label .. back-branch ranges; of nested ranges around the same MFMAs the innermost is the slab loop
+        loops = {}
+        for i, x in enumerate(lines):
+            j = re.match(r"s_c?branch\w* (\.LBB\d+_\d+)", x)
+            if not (j and j.group(1) in labels and labels[j.group(1)] < i):
+                continue
+            first = labels[j.group(1)]
+            mf = [k for k in range(first, i) if lines[k].startswith("v_mfma_f32_32x32x2_f32")]
+            if len(mf) == 64 and (mf[0] not in loops or i - first < len(loops[mf[0]])):
+                loops[mf[0]] = lines[first:i]
+        slab_loops = 0
+        for loop in loops.values():
+            bars = [k for k, y in enumerate(loop) if y.startswith("s_barrier")]
+            assert len(bars) == 1, (name, bars)
+            back = bars[0] - 1
+            while re.match(r"\.LBB\d+_\d+:", loop[back]) or loop[back].startswith(("s_or_b64 exec", "s_mov_b64 exec")):
+                back -= 1
+            assert loop[back] == "s_waitcnt vmcnt(0) lgkmcnt(0)", (name, loop[back - 2:bars[0] + 1])
+            assert not [y for y in loop if y.startswith("scratch_")], (name, "spill in the slab loop")
+            assert sum(y.startswith("global_load_lds_dwordx4") for y in loop) == 8, name
+            slab_loops += 1
+        assert slab_loops == 2, (name, slab_loops)      # the full-block and the partial-block loop
 
 
 def _vregs(text):

@@ -83,6 +83,8 @@ def test_route_drops_out_of_range_expert_ids(moe):
     ("fp8", ob.Cfg(S=64, H=256, I=256, E=8, k=2, act=ob.ACT_SWIGLU, dtype=ob.FP8, gate_fn=ob.GATE_SIGMOID, drop=0)),
     # enough rows per expert for the e4m3 tile GEMM instead of the weight streamer
     ("fp8_tile", ob.Cfg(S=600, H=256, I=256, E=4, k=2, act=ob.ACT_SWIGLU, dtype=ob.FP8, gate_fn=ob.GATE_SIGMOID, drop=0)),
+    # the fp32 matrix-core tile (forced: the layer is too small for the plan to pick it)
+    ("f32_tile", ob.Cfg(S=600, H=256, I=128, E=2, k=1, act=ob.ACT_SWIGLU, dtype=ob.F32, norm_topk=0, drop=0)),
 ])
 @pytest.mark.parametrize("fused_combine", ["0", "1"])
 def test_expired_dependency_wait_poisons_the_output_and_is_reported(moe, name, cfg, fused_combine, monkeypatch):
@@ -92,9 +94,11 @@ def test_expired_dependency_wait_poisons_the_output_and_is_reported(moe, name, c
     synchronisation of their own, until it is cleared; after that the handle computes correctly again."""
     import torch
     monkeypatch.setenv("MOE355_FUSED_COMBINE", fused_combine)   # the combine inside the FFN kernels must carry the NaNs too
+    monkeypatch.setenv("MOE355_F32_TILE", "1" if name == "f32_tile" else "0")
     inp = ob.make_inputs(cfg, seed=9)
     want = ob.forward(cfg, inp)
     layer = moe.MoELayer(product_config(cfg), ffn_mode=FFN_PERSISTENT)
+    assert name != "f32_tile" or layer.plan["block_rows"] == 128
     dev = upload_inputs(cfg, inp)
     layer.set_spin_limit(-1)
     out = layer.forward(dev["x"], dev)          # enqueues; the stall is not known yet

@@ -13,6 +13,7 @@ CASES = {
     "bf16_large_tile": ob.Cfg(S=2500, H=256, I=512, E=4, k=2, act=ob.ACT_SWIGLU, dtype=ob.BF16, drop=0),
     "bf16_small_tile": ob.Cfg(S=700, H=192, I=320, E=5, k=2, act=ob.ACT_GELU, dtype=ob.BF16, drop=1, capacity_factor=1.1),
     "f32": ob.Cfg(S=333, H=192, I=320, E=7, k=3, act=ob.ACT_SWIGLU, dtype=ob.F32, drop=1, capacity_factor=0.75),
+    "f32_tile": ob.Cfg(S=900, H=256, I=384, E=3, k=2, act=ob.ACT_GELU, dtype=ob.F32, drop=0),
     "fp8_streamer": ob.Cfg(S=64, H=512, I=256, E=32, k=8, act=ob.ACT_SWIGLU, dtype=ob.FP8, gate_fn=ob.GATE_SIGMOID, drop=0),
     "fp8_tile": ob.Cfg(S=1500, H=384, I=256, E=6, k=2, act=ob.ACT_SWIGLU, dtype=ob.FP8, gate_fn=ob.GATE_SIGMOID, drop=0),
 }
@@ -27,6 +28,7 @@ def test_every_task_is_recorded_once_and_in_dependency_order(name, monkeypatch):
         monkeypatch.setenv("MOE355_QUEUE_EARLY", "1")
         name = name[:-len("_early_start")]
     cfg = CASES[name]
+    monkeypatch.setenv("MOE355_F32_TILE", "1" if name == "f32_tile" else "0")
     inp = ob.make_inputs(cfg, seed=13)
     want = ob.route(cfg, inp)
     layer = moe.MoELayer(product_config(cfg), ffn_mode=FFN_PERSISTENT)

@@ -41,6 +41,9 @@ int fp8_tile_block_n0(int swiglu);
 int fp8_tile_block_n1();
 int ffn_persistent_occupancy_fp8_tile();
 hipError_t launch_ffn_f32_tile(const FfnArgs&, int max_mtiles, int nnt0, int nnt1, int blocks, hipStream_t);
+bool gemm_dense_f32_takes_tile(int64_t M, int64_t N, int64_t K);
+hipError_t launch_gemm_dense_f32_tile(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t, int,
+                                      hipStream_t);
 int f32_tile_block_m();
 int f32_tile_block_n0(int swiglu);
 int f32_tile_block_n1();
@@ -836,7 +839,7 @@ int moe_gemm_bias_act(const void* A, const void* B, const void* bias, void* C, i
     hipError_t e;
     if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32) {
         if (K % 16 || N % 2) return MOE_ERR_UNSUPPORTED;
-        e = launch_gemm_dense_f32(A, B, bias, C, M, N, K, act, (hipStream_t)stream);
+        e = launch_gemm_bias_act(A, B, bias, C, M, N, K, dtype, act, (hipStream_t)stream);
     } else if (dtype == MOE_DTYPE_BF16 || dtype == MOE_DTYPE_FP16) {
         if (K % 64 || N % 4) return MOE_ERR_UNSUPPORTED;
         e = launch_gemm_dense_bf16(A, B, bias, C, M, N, K, act, (hipStream_t)stream, dtype == MOE_DTYPE_FP16);
@@ -972,7 +975,14 @@ int ffn_persistent_blocks(int dtype, int tile, int compute_units) {
 
 hipError_t launch_gemm_bias_act(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N,
                                 int64_t K, int dtype, int act, hipStream_t st) {
-    if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32) return launch_gemm_dense_f32(A, B, bias, C, M, N, K, act, st);
+    if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32) {
+        bool tile = gemm_dense_f32_takes_tile(M, N, K);
+        if (const char* env = getenv("MOE355_F32_TILE")) {   // tuning knob: 0 keeps the vector-ALU kernel
+            if (atoi(env) == 0) tile = false;
+        }
+        return tile ? launch_gemm_dense_f32_tile(A, B, bias, C, M, N, K, act, st)
+                    : launch_gemm_dense_f32(A, B, bias, C, M, N, K, act, st);
+    }
     return launch_gemm_dense_bf16(A, B, bias, C, M, N, K, act, st, dtype == MOE_DTYPE_FP16);
 }
 

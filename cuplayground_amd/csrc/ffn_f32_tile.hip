@@ -281,6 +281,20 @@ __global__ __launch_bounds__(GTHREADS) void ffn_persistent_f32_tile_kernel(FfnAr
     queue_clock_stamp(a.wg_clock, 1);
 }
 
+// The same tile on dense operands (moe_gemm_bias_act): C[M,N] = act(A[M,K] . B[N,K]^T + bias), N % 128 = 0, K % 32 = 0.
+__global__ __launch_bounds__(GTHREADS) void gemm_dense_f32_tile_kernel(const float* A, const float* B, const float* bias,
+                                                                       float* C, int M, int N, int K, int act) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    TileTaskF p;
+    const int row0 = blockIdx.y * GBM;
+    p.a_base = A; p.gather = nullptr; p.a_row0 = row0;
+    p.w[0] = p.w[1] = B; p.bias[0] = bias; p.bias[1] = nullptr;
+    p.c_base = C + (int64_t)row0 * N;
+    p.K = K; p.N = N; p.rows = min(GBM, M - row0); p.c0 = blockIdx.x * GN1; p.act = act;
+    p.paired = false; p.publish = false;
+    f32_gemm_tile(p, smem);
+}
+
 template <class K>
 hipError_t allow_lds(K kernel) {
     return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, GLDS);
@@ -299,6 +313,21 @@ int ffn_persistent_occupancy_f32_tile() {
                                                      GTHREADS, GLDS) != hipSuccess || n < 1)
         n = 1;
     return n;
+}
+
+bool gemm_dense_f32_takes_tile(int64_t M, int64_t N, int64_t K) {
+    // full tiles only, and enough of them to occupy the chip (the 64 x 64 vector-ALU tiles spread small products wider)
+    return N % GBN == 0 && K % GBK == 0 && M >= GBM && (M / GBM) * (N / GBN) >= 256;
+}
+
+hipError_t launch_gemm_dense_f32_tile(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N,
+                                      int64_t K, int act, hipStream_t st) {
+    hipError_t e = allow_lds(&gemm_dense_f32_tile_kernel);
+    if (e != hipSuccess) return e;
+    const dim3 grid((unsigned)(N / GBN), (unsigned)((M + GBM - 1) / GBM));
+    gemm_dense_f32_tile_kernel<<<grid, GTHREADS, GLDS, st>>>((const float*)A, (const float*)B, (const float*)bias, (float*)C,
+                                                             (int)M, (int)N, (int)K, act);
+    return hipGetLastError();
 }
 
 hipError_t launch_ffn_f32_tile(const FfnArgs& a, int max_mtiles, int nnt0, int nnt1, int blocks, hipStream_t st) {

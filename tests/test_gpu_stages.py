@@ -43,7 +43,9 @@ def test_gemm_reference_driver_known_answer(moe, dtype):
 
 
 @pytest.mark.parametrize("act", [ob.ACT_RELU, ob.ACT_GELU, ob.ACT_NONE])
-@pytest.mark.parametrize("dtype,M,N,K", [(ob.F32, 100, 66, 48), (ob.F32, 64, 128, 256), (ob.BF16, 300, 200, 192),
+@pytest.mark.parametrize("dtype,M,N,K", [(ob.F32, 100, 66, 48), (ob.F32, 64, 128, 256),
+                                         (ob.F32, 2100, 2048, 160),     # 17 x 16 tiles of 128 x 128: the matrix-core tile, ragged last block
+                                         (ob.BF16, 300, 200, 192),
                                          (ob.BF16, 128, 128, 64), (ob.BF16, 1, 4, 64), (ob.BF16, 129, 260, 1024),
                                          (ob.F16, 300, 200, 192), (ob.F16, 129, 260, 1024), (ob.F16, 1100, 1024, 256)])
 def test_gemm_vs_oracle(moe, dtype, M, N, K, act):

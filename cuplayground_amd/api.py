@@ -419,7 +419,7 @@ class MoELayer:
                                 _ptr(self.workspace), self.workspace_bytes, _stream()), "moe_route")
         return r
 
-    # ---- backward building blocks (bf16 / fp16 layers) ----
+    # ---- backward building blocks (fp32, bf16 and fp16 layers) ----
     def backward_scratch(self):
         """Device scratch for expert_gemm / expert_wgrad, allocated on first use and kept with the layer."""
         import torch

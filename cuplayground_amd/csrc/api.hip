@@ -854,8 +854,8 @@ int moe_backward_scratch_bytes(const moe_config* cfg, size_t* bytes) {
     Derived d;
     const int rc = derive(*cfg, &d);
     if (rc) return rc;
-    if (d.act_dtype != MOE_DTYPE_BF16 && d.act_dtype != MOE_DTYPE_FP16) return MOE_ERR_UNSUPPORTED;
-    *bytes = backward_scratch_bytes(d.A, d.E, d.H, d.I);
+    if (cfg->torch_dtype == MOE_DTYPE_FP8_E4M3_B128) return MOE_ERR_UNSUPPORTED;
+    *bytes = backward_scratch_bytes(d.A, d.E, d.H, d.I, (int)d.act_bytes);
     return MOE_OK;
 }
 
@@ -869,11 +869,10 @@ int moe_transpose(const void* src, void* dst, int64_t batch, int64_t rows, int64
 
 namespace {
 int check_backward_call(const moe_handle* h, int32_t N, int32_t K, const void* scratch, size_t scratch_bytes) {
-    if (h->d.act_dtype != MOE_DTYPE_BF16 && h->d.act_dtype != MOE_DTYPE_FP16) return MOE_ERR_UNSUPPORTED;
     if (h->cfg.torch_dtype == MOE_DTYPE_FP8_E4M3_B128) return MOE_ERR_UNSUPPORTED;
     const bool dims_ok = (N == h->d.H && K == h->d.I) || (N == h->d.I && K == h->d.H);
     if (!dims_ok) return MOE_ERR_BAD_ARGUMENT;      // (N, K) is a projection of this layer, one way or the other
-    if (!scratch || ((uintptr_t)scratch % kAlign) || scratch_bytes < backward_scratch_bytes(h->d.A, h->d.E, h->d.H, h->d.I))
+    if (!scratch || ((uintptr_t)scratch % kAlign) || scratch_bytes < backward_scratch_bytes(h->d.A, h->d.E, h->d.H, h->d.I, (int)h->d.act_bytes))
         return MOE_ERR_WORKSPACE;
     return MOE_OK;
 }
@@ -887,7 +886,7 @@ int moe_expert_gemm(moe_handle* h, const void* a_rows, const void* w, const void
     const int rc = check_backward_call(h, N, K, scratch, scratch_bytes);
     if (rc) return rc;
     const hipError_t e = launch_expert_gemm(a_rows, w, bias, expert_count, expert_offset, h->d.A, h->d.E, N, K, act,
-                                            h->d.act_dtype == MOE_DTYPE_FP16, out_rows, scratch, (hipStream_t)stream);
+                                            h->d.act_dtype, out_rows, scratch, (hipStream_t)stream);
     return e == hipSuccess ? MOE_OK : hip_fail(h, e);
 }
 
@@ -898,13 +897,13 @@ int moe_expert_wgrad(moe_handle* h, const void* dy_rows, const void* a_rows, con
     const int rc = check_backward_call(h, N, K, scratch, scratch_bytes);
     if (rc) return rc;
     const hipError_t e = launch_expert_wgrad(dy_rows, a_rows, expert_count, expert_offset, h->d.A, h->d.E, N, K,
-                                             h->d.act_dtype == MOE_DTYPE_FP16, dw, scratch, (hipStream_t)stream);
+                                             h->d.act_dtype, dw, scratch, (hipStream_t)stream);
     return e == hipSuccess ? MOE_OK : hip_fail(h, e);
 }
 
 namespace {
 bool backward_dtype(const moe_handle* h) {
-    return h->cfg.torch_dtype == MOE_DTYPE_BF16 || h->cfg.torch_dtype == MOE_DTYPE_FP16;
+    return h->cfg.torch_dtype != MOE_DTYPE_FP8_E4M3_B128;
 }
 }  // namespace
 
@@ -916,7 +915,7 @@ int moe_act_backward(moe_handle* h, const void* dh_rows, const void* u_rows, con
     if (sw != (g_rows != nullptr) || sw != (dg_rows != nullptr)) return MOE_ERR_BAD_ARGUMENT;
     if (rows > h->d.A) return MOE_ERR_BAD_ARGUMENT;
     const hipError_t e = launch_act_backward(dh_rows, u_rows, g_rows, rows * h->d.I, h->cfg.hidden_act,
-                                             h->cfg.torch_dtype == MOE_DTYPE_FP16, du_rows, dg_rows, (hipStream_t)stream);
+                                             h->d.act_dtype, du_rows, dg_rows, (hipStream_t)stream);
     return e == hipSuccess ? MOE_OK : hip_fail(h, e);
 }
 
@@ -926,7 +925,7 @@ int moe_bias_grad(moe_handle* h, const void* dy_rows, const int32_t* expert_coun
     if (!backward_dtype(h)) return MOE_ERR_UNSUPPORTED;
     if (N != h->d.H && N != h->d.I) return MOE_ERR_BAD_ARGUMENT;
     const hipError_t e = launch_bias_grad(dy_rows, expert_count, expert_offset, h->d.E, N,
-                                          h->cfg.torch_dtype == MOE_DTYPE_FP16, db, (hipStream_t)stream);
+                                          h->d.act_dtype, db, (hipStream_t)stream);
     return e == hipSuccess ? MOE_OK : hip_fail(h, e);
 }
 
@@ -935,7 +934,7 @@ int moe_combine_backward(moe_handle* h, const void* dout, const void* y_rows, co
     if (!h || !dout || !y_rows || !pair_row || !topk_w || !dy_rows || !dw) return MOE_ERR_BAD_ARGUMENT;
     if (!backward_dtype(h)) return MOE_ERR_UNSUPPORTED;
     const hipError_t e = launch_combine_backward(dout, y_rows, pair_row, topk_w, h->d.S, h->d.k, h->d.H,
-                                                 h->cfg.torch_dtype == MOE_DTYPE_FP16, dy_rows, dw, (hipStream_t)stream);
+                                                 h->d.act_dtype, dy_rows, dw, (hipStream_t)stream);
     return e == hipSuccess ? MOE_OK : hip_fail(h, e);
 }
 

@@ -21,6 +21,17 @@ hipError_t launch_grouped_gemm_16(const void* a_rows, const void* w, const void*
 hipError_t launch_wgrad_16(const void* dyT, const void* aT, void* dw, const int32_t* poff, int E, int N, int K,
                            int64_t ld, bool f16, hipStream_t st);
 
+hipError_t launch_grouped_gemm_f32(const void* a_rows, const void* w, const void* bias, void* out, const MTile* mtiles,
+                                   const int32_t* num_mtiles, int max_mtiles, int N, int K, int act, hipStream_t st);
+hipError_t launch_wgrad_f32(const void* dyT, const void* aT, void* dw, const int32_t* poff, int E, int N, int K, int64_t ld,
+                            hipStream_t st);
+bool grouped_gemm_f32_takes_tile(int64_t A, int N, int K);
+hipError_t launch_grouped_gemm_f32_tile(const void* a_rows, const void* w, const void* bias, void* out, const MTile* mtiles,
+                                        const int32_t* num_mtiles, int max_mtiles, int N, int K, int act, hipStream_t st);
+bool wgrad_f32_takes_tile(int E, int N, int K);
+hipError_t launch_wgrad_f32_tile(const void* dyT, const void* aT, void* dw, const int32_t* poff, int E, int N, int K,
+                                 int64_t ld, hipStream_t st);
+
 namespace {
 
 constexpr int kWindowAlign = 128;   // columns an expert's window of a transposed operand is padded to
@@ -171,11 +182,42 @@ __global__ __launch_bounds__(256) void transpose_rows_padded_kernel(const uint16
     }
 }
 
-// ---- elementwise and reduction steps of a backward pass (16-bit layers) ----
-template <class T16> __device__ __forceinline__ float ld16(const uint16_t* p, size_t i);
+// The same for 4-byte elements (fp32 layers): any C.  grid = (ld / 64, ceil(C / 64)).
+__global__ __launch_bounds__(256) void transpose_rows_padded32_kernel(const uint32_t* __restrict__ rows, int C,
+                                                                      const int32_t* __restrict__ count,
+                                                                      const int32_t* __restrict__ offset,
+                                                                      const int32_t* __restrict__ poff, int E, int64_t ld,
+                                                                      uint32_t* __restrict__ dst) {
+    __shared__ uint32_t tile[64][65];
+    const int p0 = blockIdx.x * 64;
+    if (p0 >= poff[E]) return;                 // behind the last window: never read
+    int lo = 0, hi = E - 1;
+    while (lo < hi) {                          // last expert whose window starts at or before p0 (empty windows skipped)
+        const int mid = (lo + hi + 1) >> 1;
+        if (poff[mid] <= p0) lo = mid; else hi = mid - 1;
+    }
+    const int e = lo, s0 = p0 - poff[e], n = count[e], off = offset[e];
+    const int c0 = blockIdx.y * 64;
+    for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+        const int r = i >> 6, c = i & 63;
+        tile[r][c] = (s0 + r < n && c0 + c < C) ? rows[(size_t)(off + s0 + r) * C + c0 + c] : 0u;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+        const int c = i >> 6, r = i & 63;
+        if (c0 + c < C) dst[(size_t)(c0 + c) * ld + p0 + r] = tile[r][c];
+    }
+}
+
+// ---- elementwise and reduction steps of a backward pass ----
+struct f32_s {};
+template <class T> struct RawOf { typedef uint16_t type; };
+template <> struct RawOf<f32_s> { typedef float type; };
+template <class T16> __device__ __forceinline__ float ld16(const typename RawOf<T16>::type* p, size_t i);
 template <> __device__ __forceinline__ float ld16<bf16_s>(const uint16_t* p, size_t i) { return __uint_as_float((uint32_t)p[i] << 16); }
 template <> __device__ __forceinline__ float ld16<f16_s>(const uint16_t* p, size_t i) { return (float)__builtin_bit_cast(_Float16, p[i]); }
-template <class T16> __device__ __forceinline__ uint16_t st16(float v);
+template <> __device__ __forceinline__ float ld16<f32_s>(const float* p, size_t i) { return p[i]; }
+template <class T16> __device__ __forceinline__ typename RawOf<T16>::type st16(float v);
 template <> __device__ __forceinline__ uint16_t st16<bf16_s>(float v) {
     typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
     typedef float f32x2_t __attribute__((ext_vector_type(2)));
@@ -183,12 +225,13 @@ template <> __device__ __forceinline__ uint16_t st16<bf16_s>(float v) {
     return (uint16_t)(__builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2_t)) & 0xFFFFu);
 }
 template <> __device__ __forceinline__ uint16_t st16<f16_s>(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
+template <> __device__ __forceinline__ float st16<f32_s>(float v) { return v; }
 
 // du = dh * act'(u); SwiGLU (h = silu(g) u): du = dh silu(g), dg = dh u s (1 + g (1 - s)), s = sigmoid(g).
-template <class T16>
-__global__ __launch_bounds__(256) void act_backward_kernel(const uint16_t* __restrict__ dh, const uint16_t* __restrict__ u,
-                                                           const uint16_t* __restrict__ g, size_t n, int act,
-                                                           uint16_t* __restrict__ du, uint16_t* __restrict__ dg) {
+template <class T16, class RAW = typename RawOf<T16>::type>
+__global__ __launch_bounds__(256) void act_backward_kernel(const RAW* __restrict__ dh, const RAW* __restrict__ u,
+                                                           const RAW* __restrict__ g, size_t n, int act,
+                                                           RAW* __restrict__ du, RAW* __restrict__ dg) {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
         const float d = ld16<T16>(dh, i), uv = ld16<T16>(u, i);
         if (act == MOE_ACT_SWIGLU) {
@@ -208,9 +251,9 @@ __global__ __launch_bounds__(256) void act_backward_kernel(const uint16_t* __res
 
 // db[e, n] = sum over expert e's rows, ascending, of dy[r, n]: one thread per column, so the order is fixed.
 // grid = (ceil(N / 256), E).
-template <class T16>
-__global__ __launch_bounds__(256) void bias_grad_kernel(const uint16_t* __restrict__ dy, const int32_t* __restrict__ count,
-                                                        const int32_t* __restrict__ offset, int N, uint16_t* __restrict__ db) {
+template <class T16, class RAW = typename RawOf<T16>::type>
+__global__ __launch_bounds__(256) void bias_grad_kernel(const RAW* __restrict__ dy, const int32_t* __restrict__ count,
+                                                        const int32_t* __restrict__ offset, int N, RAW* __restrict__ db) {
     const int n = blockIdx.x * 256 + threadIdx.x, e = blockIdx.y;
     if (n >= N) return;
     const int r0 = offset[e], r1 = r0 + max(count[e], 0);
@@ -220,11 +263,11 @@ __global__ __launch_bounds__(256) void bias_grad_kernel(const uint16_t* __restri
 }
 
 // One workgroup per token: dy[row(t,r), :] = w[t,r] * dout[t, :]; dw[t,r] = <dout[t, :], y[row(t,r), :]>.
-template <class T16>
-__global__ __launch_bounds__(256) void combine_backward_kernel(const uint16_t* __restrict__ dout, const uint16_t* __restrict__ y,
+template <class T16, class RAW = typename RawOf<T16>::type>
+__global__ __launch_bounds__(256) void combine_backward_kernel(const RAW* __restrict__ dout, const RAW* __restrict__ y,
                                                                const int32_t* __restrict__ pair_row,
                                                                const float* __restrict__ topk_w, int k, int H,
-                                                               uint16_t* __restrict__ dy, float* __restrict__ dw) {
+                                                               RAW* __restrict__ dy, float* __restrict__ dw) {
     __shared__ float part[4];
     const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     for (int r = 0; r < k; ++r) {
@@ -253,9 +296,9 @@ size_t align256(size_t v) { return (v + 255) / 256 * 256; }
 
 int64_t wgrad_ld(int64_t A, int E) { return (A + (int64_t)kWindowAlign * E + 127) / 128 * 128; }
 
-size_t backward_scratch_bytes(int64_t A, int E, int H, int I) {
-    const size_t tables = align256(sizeof(int32_t)) + align256((size_t)(A / 128 + E + 1) * sizeof(MTile)) + align256((size_t)(E + 1) * 4);
-    const size_t operands = align256((size_t)H * wgrad_ld(A, E) * 2) + align256((size_t)I * wgrad_ld(A, E) * 2);
+size_t backward_scratch_bytes(int64_t A, int E, int H, int I, int elem_bytes) {
+    const size_t tables = align256(sizeof(int32_t)) + align256((size_t)(A / 64 + E + 1) * sizeof(MTile)) + align256((size_t)(E + 1) * 4);
+    const size_t operands = align256((size_t)H * wgrad_ld(A, E) * elem_bytes) + align256((size_t)I * wgrad_ld(A, E) * elem_bytes);
     return tables + operands;
 }
 
@@ -270,10 +313,46 @@ hipError_t launch_transpose(const void* src, void* dst, int64_t batch, int64_t r
     return hipGetLastError();
 }
 
+namespace {
+// The table region at the head of the scratch buffer: the number of row blocks, the row blocks (64 rows is the
+// smallest block any kernel here uses), the window offsets.
+struct ScratchTables {
+    int32_t* num_mtiles;
+    MTile* mtiles;
+    int32_t* poff;
+    char* operands;
+};
+ScratchTables scratch_tables(void* scratch, int64_t A, int E) {
+    char* s = static_cast<char*>(scratch);
+    ScratchTables t;
+    t.num_mtiles = reinterpret_cast<int32_t*>(s);
+    t.mtiles = reinterpret_cast<MTile*>(s + align256(sizeof(int32_t)));
+    const size_t tables = align256(sizeof(int32_t)) + align256((size_t)(A / 64 + E + 1) * sizeof(MTile));
+    t.poff = reinterpret_cast<int32_t*>(s + tables);
+    t.operands = s + tables + align256((size_t)(E + 1) * 4);
+    return t;
+}
+}  // namespace
+
 // out_rows[r,:] = act(a_rows[r,:] . w[e(r)]^T + bias[e(r)]); scratch holds the row-block table.
+// dtype: the storage type of every operand (MOE_DTYPE_F32, _BF16 or _FP16).
 hipError_t launch_expert_gemm(const void* a_rows, const void* w, const void* bias, const int32_t* count,
-                              const int32_t* offset, int64_t A, int E, int N, int K, int act, bool f16, void* out_rows,
+                              const int32_t* offset, int64_t A, int E, int N, int K, int act, int dtype, void* out_rows,
                               void* scratch, hipStream_t st) {
+    const ScratchTables t = scratch_tables(scratch, A, E);
+    if (dtype == MOE_DTYPE_F32) {
+        bool mfma = grouped_gemm_f32_takes_tile(A, N, K);
+        if (const char* env = getenv("MOE355_F32_TILE")) {   // tuning knob: 0 keeps the vector-ALU kernel
+            if (atoi(env) == 0) mfma = false;
+        }
+        const int block_m = mfma ? 128 : 64;
+        const int max_mtiles = (int)(A / block_m + E);
+        backward_tables_kernel<<<1, kMaxExperts, 0, st>>>(count, offset, E, block_m, t.mtiles, t.num_mtiles, nullptr);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        return (mfma ? launch_grouped_gemm_f32_tile : launch_grouped_gemm_f32)(a_rows, w, bias, out_rows, t.mtiles,
+                                                                               t.num_mtiles, max_mtiles, N, K, act, st);
+    }
     int tile = grouped_gemm_takes_large_tile(A, E, N, K) ? 1 : 0;     // 1: 256 x 256, 0: 128 x 128
     if (const char* env = getenv("MOE355_GROUPED_TILE")) {             // tuning knob; 2: 128 x 256 (hand-ordered)
         const int v = atoi(env);
@@ -282,55 +361,66 @@ hipError_t launch_expert_gemm(const void* a_rows, const void* w, const void* bia
         if (v == 0) tile = 0;
     }
     const int block_m = tile == 1 ? 256 : 128;
-    char* s = static_cast<char*>(scratch);
-    int32_t* num_mtiles = reinterpret_cast<int32_t*>(s);
-    MTile* mtiles = reinterpret_cast<MTile*>(s + align256(sizeof(int32_t)));
     const int max_mtiles = (int)(A / block_m + E);
-    backward_tables_kernel<<<1, kMaxExperts, 0, st>>>(count, offset, E, block_m, mtiles, num_mtiles, nullptr);
+    backward_tables_kernel<<<1, kMaxExperts, 0, st>>>(count, offset, E, block_m, t.mtiles, t.num_mtiles, nullptr);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    return launch_grouped_gemm_16(a_rows, w, bias, out_rows, mtiles, num_mtiles, count, max_mtiles, tile, A, N, K, act, f16, st);
+    return launch_grouped_gemm_16(a_rows, w, bias, out_rows, t.mtiles, t.num_mtiles, count, max_mtiles, tile, A, N, K, act,
+                                  dtype == MOE_DTYPE_FP16, st);
 }
 
 // dw[e] [N,K] = dy_e^T . a_e; scratch holds the window offsets and the two transposed operands.
 hipError_t launch_expert_wgrad(const void* dy_rows, const void* a_rows, const int32_t* count, const int32_t* offset,
-                               int64_t A, int E, int N, int K, bool f16, void* dw, void* scratch, hipStream_t st) {
-    char* s = static_cast<char*>(scratch);
-    const size_t tables = align256(sizeof(int32_t)) + align256((size_t)(A / 128 + E + 1) * sizeof(MTile));
-    int32_t* poff = reinterpret_cast<int32_t*>(s + tables);
+                               int64_t A, int E, int N, int K, int dtype, void* dw, void* scratch, hipStream_t st) {
+    const ScratchTables t = scratch_tables(scratch, A, E);
     const int64_t ld = wgrad_ld(A, E);
-    uint16_t* dyT = reinterpret_cast<uint16_t*>(s + tables + align256((size_t)(E + 1) * 4));
-    uint16_t* aT = reinterpret_cast<uint16_t*>(reinterpret_cast<char*>(dyT) + align256((size_t)N * ld * 2));
-    backward_tables_kernel<<<1, kMaxExperts, 0, st>>>(count, offset, E, 128, nullptr, nullptr, poff);
+    const size_t eb = dtype == MOE_DTYPE_F32 ? 4 : 2;
+    void* dyT = t.operands;
+    void* aT = t.operands + align256((size_t)N * ld * eb);
+    backward_tables_kernel<<<1, kMaxExperts, 0, st>>>(count, offset, E, 128, nullptr, nullptr, t.poff);
     const dim3 g1((unsigned)(ld / 64), (unsigned)((N + 63) / 64)), g2((unsigned)(ld / 64), (unsigned)((K + 63) / 64));
-    transpose_rows_padded_kernel<<<g1, 256, 0, st>>>((const uint16_t*)dy_rows, N, count, offset, poff, E, ld, dyT);
-    transpose_rows_padded_kernel<<<g2, 256, 0, st>>>((const uint16_t*)a_rows, K, count, offset, poff, E, ld, aT);
+    if (dtype == MOE_DTYPE_F32) {
+        transpose_rows_padded32_kernel<<<g1, 256, 0, st>>>((const uint32_t*)dy_rows, N, count, offset, t.poff, E, ld, (uint32_t*)dyT);
+        transpose_rows_padded32_kernel<<<g2, 256, 0, st>>>((const uint32_t*)a_rows, K, count, offset, t.poff, E, ld, (uint32_t*)aT);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        bool mfma = wgrad_f32_takes_tile(E, N, K);
+        if (const char* env = getenv("MOE355_F32_TILE")) {   // tuning knob: 0 keeps the vector-ALU kernel
+            if (atoi(env) == 0) mfma = false;
+        }
+        return (mfma ? launch_wgrad_f32_tile : launch_wgrad_f32)(dyT, aT, dw, t.poff, E, N, K, ld, st);
+    }
+    transpose_rows_padded_kernel<<<g1, 256, 0, st>>>((const uint16_t*)dy_rows, N, count, offset, t.poff, E, ld, (uint16_t*)dyT);
+    transpose_rows_padded_kernel<<<g2, 256, 0, st>>>((const uint16_t*)a_rows, K, count, offset, t.poff, E, ld, (uint16_t*)aT);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    return launch_wgrad_16(dyT, aT, dw, poff, E, N, K, ld, f16, st);
+    return launch_wgrad_16(dyT, aT, dw, t.poff, E, N, K, ld, dtype == MOE_DTYPE_FP16, st);
 }
 
-hipError_t launch_act_backward(const void* dh, const void* u, const void* g, int64_t n, int act, bool f16, void* du,
+hipError_t launch_act_backward(const void* dh, const void* u, const void* g, int64_t n, int act, int dtype, void* du,
                                void* dg, hipStream_t st) {
     if (n <= 0) return hipSuccess;
     const int grid = (int)std::min<int64_t>((n + 255) / 256, 65536);
-    if (f16) act_backward_kernel<f16_s><<<grid, 256, 0, st>>>((const uint16_t*)dh, (const uint16_t*)u, (const uint16_t*)g, (size_t)n, act, (uint16_t*)du, (uint16_t*)dg);
+    if (dtype == MOE_DTYPE_F32) act_backward_kernel<f32_s><<<grid, 256, 0, st>>>((const float*)dh, (const float*)u, (const float*)g, (size_t)n, act, (float*)du, (float*)dg);
+    else if (dtype == MOE_DTYPE_FP16) act_backward_kernel<f16_s><<<grid, 256, 0, st>>>((const uint16_t*)dh, (const uint16_t*)u, (const uint16_t*)g, (size_t)n, act, (uint16_t*)du, (uint16_t*)dg);
     else act_backward_kernel<bf16_s><<<grid, 256, 0, st>>>((const uint16_t*)dh, (const uint16_t*)u, (const uint16_t*)g, (size_t)n, act, (uint16_t*)du, (uint16_t*)dg);
     return hipGetLastError();
 }
 
-hipError_t launch_bias_grad(const void* dy, const int32_t* count, const int32_t* offset, int E, int N, bool f16, void* db,
+hipError_t launch_bias_grad(const void* dy, const int32_t* count, const int32_t* offset, int E, int N, int dtype, void* db,
                             hipStream_t st) {
     const dim3 grid((unsigned)((N + 255) / 256), (unsigned)E);
-    if (f16) bias_grad_kernel<f16_s><<<grid, 256, 0, st>>>((const uint16_t*)dy, count, offset, N, (uint16_t*)db);
+    if (dtype == MOE_DTYPE_F32) bias_grad_kernel<f32_s><<<grid, 256, 0, st>>>((const float*)dy, count, offset, N, (float*)db);
+    else if (dtype == MOE_DTYPE_FP16) bias_grad_kernel<f16_s><<<grid, 256, 0, st>>>((const uint16_t*)dy, count, offset, N, (uint16_t*)db);
     else bias_grad_kernel<bf16_s><<<grid, 256, 0, st>>>((const uint16_t*)dy, count, offset, N, (uint16_t*)db);
     return hipGetLastError();
 }
 
 hipError_t launch_combine_backward(const void* dout, const void* y, const int32_t* pair_row, const float* topk_w, int S,
-                                   int k, int H, bool f16, void* dy, float* dw, hipStream_t st) {
+                                   int k, int H, int dtype, void* dy, float* dw, hipStream_t st) {
     if (S <= 0) return hipSuccess;
-    if (f16) combine_backward_kernel<f16_s><<<S, 256, 0, st>>>((const uint16_t*)dout, (const uint16_t*)y, pair_row, topk_w, k, H, (uint16_t*)dy, dw);
+    if (dtype == MOE_DTYPE_F32) combine_backward_kernel<f32_s><<<S, 256, 0, st>>>((const float*)dout, (const float*)y, pair_row, topk_w, k, H, (float*)dy, dw);
+    else if (dtype == MOE_DTYPE_FP16) combine_backward_kernel<f16_s><<<S, 256, 0, st>>>((const uint16_t*)dout, (const uint16_t*)y, pair_row, topk_w, k, H, (uint16_t*)dy, dw);
     else combine_backward_kernel<bf16_s><<<S, 256, 0, st>>>((const uint16_t*)dout, (const uint16_t*)y, pair_row, topk_w, k, H, (uint16_t*)dy, dw);
     return hipGetLastError();
 }

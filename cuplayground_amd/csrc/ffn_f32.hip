@@ -15,6 +15,7 @@ struct TaskPtrsF {
     const int32_t* gather;
     int64_t a_row0;
     int a_ld;
+    int b_ld;          // row pitch of b0 / b1 (K, except for windows of a wider matrix)
     const float* b0;
     const float* b1;
     const float* bias0;
@@ -43,7 +44,7 @@ __device__ __forceinline__ void gemm_tile_f32(const TaskPtrsF& p, float (*As)[FB
         col = p.n0 + lrow;
     }
     if (col >= p.N) col = p.N - 1;
-    const float* b_src = bbase + (int64_t)col * p.K + lk;
+    const float* b_src = bbase + (int64_t)col * p.b_ld + lk;
 
     float acc[4][4];
 #pragma unroll
@@ -111,6 +112,7 @@ __device__ __forceinline__ TaskPtrsF resolve_f32(const FfnArgs& a, const Task& t
         p.gather = a.token_indices + t.row0;
         p.a_row0 = 0;
         p.a_ld = a.H;
+        p.b_ld = a.H;
         p.b0 = (const float*)a.w_up + t.expert * HI;
         p.b1 = sw ? (const float*)a.w_gate + t.expert * HI : nullptr;
         p.bias0 = a.b_up ? (const float*)a.b_up + (int64_t)t.expert * a.I : nullptr;
@@ -127,6 +129,7 @@ __device__ __forceinline__ TaskPtrsF resolve_f32(const FfnArgs& a, const Task& t
         p.gather = nullptr;
         p.a_row0 = t.row0;
         p.a_ld = a.I;
+        p.b_ld = a.I;
         p.b0 = (const float*)a.w_down + t.expert * HI;
         p.b1 = nullptr;
         p.bias0 = a.b_down ? (const float*)a.b_down + (int64_t)t.expert * a.H : nullptr;
@@ -188,10 +191,46 @@ __global__ __launch_bounds__(256) void gemm_dense_f32_kernel(const float* A, con
     __shared__ __align__(16) float Bs[FBK][FBN + FPAD];
     TaskPtrsF p;
     const int row0 = blockIdx.y * FBM;
-    p.a_base = A; p.gather = nullptr; p.a_row0 = row0; p.a_ld = K;
+    p.a_base = A; p.gather = nullptr; p.a_row0 = row0; p.a_ld = K; p.b_ld = K;
     p.b0 = B; p.b1 = nullptr; p.bias0 = bias; p.bias1 = nullptr;
     p.c_base = C + (int64_t)row0 * N;
     p.N = N; p.K = K; p.rows = min(FBM, M - row0); p.n0 = blockIdx.x * FBN; p.act = act; p.swiglu = false; p.publish = false;
+    gemm_tile_f32(p, As, Bs);
+}
+
+// Grouped product over packed expert-major rows (backward.hip): out[r,:] = act(a_rows[r,:] . w[e(r)]^T + bias[e(r)]),
+// one workgroup per (row block of 64 from `mtiles`, 64 output columns).
+__global__ __launch_bounds__(256) void grouped_gemm_f32_kernel(const float* a_rows, const float* w, const float* bias,
+                                                               float* out, const MTile* mtiles, const int32_t* num_mtiles,
+                                                               int nnt, int N, int K, int act) {
+    __shared__ __align__(16) float As[FBK][FBM + FPAD];
+    __shared__ __align__(16) float Bs[FBK][FBN + FPAD];
+    const int mt = blockIdx.x / nnt, nt = blockIdx.x % nnt;
+    if (mt >= *num_mtiles) return;
+    const MTile m = mtiles[mt];
+    TaskPtrsF p;
+    p.a_base = a_rows; p.gather = nullptr; p.a_row0 = m.row0; p.a_ld = K; p.b_ld = K;
+    p.b0 = w + (int64_t)m.expert * N * K; p.b1 = nullptr;
+    p.bias0 = bias ? bias + (int64_t)m.expert * N : nullptr; p.bias1 = nullptr;
+    p.c_base = out + (int64_t)m.row0 * N;
+    p.N = N; p.K = K; p.rows = m.rows; p.n0 = nt * FBN; p.act = act; p.swiglu = false; p.publish = false;
+    gemm_tile_f32(p, As, Bs);
+}
+
+// Weight gradient of one expert: dw[e] [N,K] = dyT[:, window e] . aT[:, window e]^T, the windows being the expert's
+// packed rows as columns of the transposed operands (zero padded to a multiple of 128, pitch ld).
+// grid = (ceil(K / 64), ceil(N / 64), E).
+__global__ __launch_bounds__(256) void wgrad_f32_kernel(const float* dyT, const float* aT, float* dw, const int32_t* poff,
+                                                        int N, int K, int64_t ld) {
+    __shared__ __align__(16) float As[FBK][FBM + FPAD];
+    __shared__ __align__(16) float Bs[FBK][FBN + FPAD];
+    const int e = blockIdx.z, row0 = blockIdx.y * FBM;
+    TaskPtrsF p;
+    p.a_base = dyT + poff[e]; p.gather = nullptr; p.a_row0 = row0; p.a_ld = (int)ld; p.b_ld = (int)ld;
+    p.b0 = aT + poff[e]; p.b1 = nullptr; p.bias0 = nullptr; p.bias1 = nullptr;
+    p.c_base = dw + (int64_t)e * N * K + (int64_t)row0 * K;
+    p.N = K; p.K = poff[e + 1] - poff[e]; p.rows = min(FBM, N - row0); p.n0 = blockIdx.x * FBN; p.act = MOE_ACT_NONE;
+    p.swiglu = false; p.publish = false;
     gemm_tile_f32(p, As, Bs);
 }
 
@@ -216,6 +255,22 @@ hipError_t launch_gemm_dense_f32(const void* A, const void* B, const void* bias,
     const dim3 grid((unsigned)((N + FBN - 1) / FBN), (unsigned)((M + FBM - 1) / FBM));
     gemm_dense_f32_kernel<<<grid, 256, 0, st>>>((const float*)A, (const float*)B, (const float*)bias, (float*)C,
                                                 (int)M, (int)N, (int)K, act);
+    return hipGetLastError();
+}
+
+hipError_t launch_grouped_gemm_f32(const void* a_rows, const void* w, const void* bias, void* out, const MTile* mtiles,
+                                   const int32_t* num_mtiles, int max_mtiles, int N, int K, int act, hipStream_t st) {
+    const int nnt = (N + FBN - 1) / FBN;
+    grouped_gemm_f32_kernel<<<(unsigned)max_mtiles * nnt, 256, 0, st>>>((const float*)a_rows, (const float*)w,
+                                                                        (const float*)bias, (float*)out, mtiles,
+                                                                        num_mtiles, nnt, N, K, act);
+    return hipGetLastError();
+}
+
+hipError_t launch_wgrad_f32(const void* dyT, const void* aT, void* dw, const int32_t* poff, int E, int N, int K, int64_t ld,
+                            hipStream_t st) {
+    const dim3 grid((unsigned)((K + FBN - 1) / FBN), (unsigned)((N + FBM - 1) / FBM), (unsigned)E);
+    wgrad_f32_kernel<<<grid, 256, 0, st>>>((const float*)dyT, (const float*)aT, (float*)dw, poff, N, K, ld);
     return hipGetLastError();
 }
 

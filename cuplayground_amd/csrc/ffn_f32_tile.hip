@@ -44,6 +44,7 @@ struct TileTaskF {
     const float* bias[2];
     float* c_base;              // h or y at the first row of the block
     int K, N, rows, c0;
+    int a_ld, b_ld;             // row pitch of the operands in elements (K, except for windows of a wider matrix)
     int act;                    // activation of the epilogue (MOE_ACT_NONE for SwiGLU pairs and the down projection)
     bool paired;
     bool publish;               // rows are read by other workgroups of the same launch
@@ -65,7 +66,7 @@ __device__ __forceinline__ void tile_mainloop_f32(const TileTaskF& p, unsigned c
         int r = prow + i * 32;
         if (r >= p.rows) r = 0;                                   // padding rows re-read row 0; never stored
         const int64_t src_row = p.gather ? (int64_t)p.gather[r] : p.a_row0 + r;
-        a_src[i] = p.a_base + src_row * p.K + chunk * 4;
+        a_src[i] = p.a_base + src_row * p.a_ld + chunk * 4;
         const int j = prow + i * 32;                              // row of the weight tile
         const float* base = p.w[0];
         int col;
@@ -76,7 +77,7 @@ __device__ __forceinline__ void tile_mainloop_f32(const TileTaskF& p, unsigned c
         } else {
             col = p.c0 + j;
         }
-        b_src[i] = base + (int64_t)col * p.K + chunk * 4;
+        b_src[i] = base + (int64_t)col * p.b_ld + chunk * 4;
     }
     const int wrow = __builtin_amdgcn_readfirstlane(prow & ~7);
     auto issue = [&](int kt) {
@@ -131,10 +132,10 @@ __device__ __forceinline__ void tile_mainloop_f32(const TileTaskF& p, unsigned c
         asm volatile("" ::: "memory");
     };
 
+    const int nk = p.K / GBK;               // 0 for the empty window of an expert without rows (weight gradient)
     __syncthreads();                        // the previous task may still be reading the stages
-    issue(0);
+    if (nk > 0) issue(0);
     end_slab();
-    const int nk = p.K / GBK;
     for (int kt = 0; kt < nk; ++kt) {
         // slab kt sits in stage kt & 1; the other stage is free: every wavefront is past the barrier that ended slab kt - 1
         if (kt + 1 < nk) issue(kt + 1);
@@ -214,7 +215,7 @@ __device__ __forceinline__ TileTaskF resolve_tile_f32(const FfnArgs& a, const Ta
     p.bias[1] = nullptr;
     if (t.phase == 0) {
         p.c0 = t.ntile * (p.paired ? GN0 : GN1);
-        p.K = a.H;
+        p.K = p.a_ld = p.b_ld = a.H;
         p.N = a.I;
         if (p.paired) {
             p.w[0] = (const float*)a.w_gate + t.expert * HI;
@@ -232,7 +233,7 @@ __device__ __forceinline__ TileTaskF resolve_tile_f32(const FfnArgs& a, const Ta
         p.c_base = (float*)a.h + (int64_t)t.row0 * a.I;
     } else {
         p.c0 = t.ntile * GN1;
-        p.K = a.I;
+        p.K = p.a_ld = p.b_ld = a.I;
         p.N = a.H;
         p.w[0] = p.w[1] = (const float*)a.w_down + t.expert * HI;
         p.bias[0] = a.b_down ? (const float*)a.b_down + (int64_t)t.expert * a.H : nullptr;
@@ -290,8 +291,44 @@ __global__ __launch_bounds__(GTHREADS) void gemm_dense_f32_tile_kernel(const flo
     p.a_base = A; p.gather = nullptr; p.a_row0 = row0;
     p.w[0] = p.w[1] = B; p.bias[0] = bias; p.bias[1] = nullptr;
     p.c_base = C + (int64_t)row0 * N;
-    p.K = K; p.N = N; p.rows = min(GBM, M - row0); p.c0 = blockIdx.x * GN1; p.act = act;
+    p.K = p.a_ld = p.b_ld = K; p.N = N; p.rows = min(GBM, M - row0); p.c0 = blockIdx.x * GN1; p.act = act;
     p.paired = false; p.publish = false;
+    f32_gemm_tile(p, smem);
+}
+
+// Grouped product over packed expert-major rows (backward.hip): out[r,:] = act(a_rows[r,:] . w[e(r)]^T + bias[e(r)]),
+// one workgroup per (row block of 128 from `mtiles`, 128 output columns).  N % 128 = 0, K % 32 = 0.
+__global__ __launch_bounds__(GTHREADS) void grouped_gemm_f32_tile_kernel(const float* a_rows, const float* w,
+                                                                         const float* bias, float* out, const MTile* mtiles,
+                                                                         const int32_t* num_mtiles, int nnt, int N, int K,
+                                                                         int act) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int mt = blockIdx.x / nnt, nt = blockIdx.x % nnt;
+    if (mt >= *num_mtiles) return;
+    const MTile m = mtiles[mt];
+    TileTaskF p;
+    p.a_base = a_rows; p.gather = nullptr; p.a_row0 = m.row0;
+    p.w[0] = p.w[1] = w + (int64_t)m.expert * N * K;
+    p.bias[0] = bias ? bias + (int64_t)m.expert * N : nullptr; p.bias[1] = nullptr;
+    p.c_base = out + (int64_t)m.row0 * N;
+    p.K = p.a_ld = p.b_ld = K; p.N = N; p.rows = m.rows; p.c0 = nt * GN1; p.act = act;
+    p.paired = false; p.publish = false;
+    f32_gemm_tile(p, smem);
+}
+
+// Weight gradient of one expert: dw[e] [N,K] = dyT[:, window e] . aT[:, window e]^T over the expert's zero-padded
+// window of packed rows (a multiple of 128 columns of the transposed operands, pitch ld).  K % 128 = 0.
+// grid = (K / 128, ceil(N / 128), E).
+__global__ __launch_bounds__(GTHREADS) void wgrad_f32_tile_kernel(const float* dyT, const float* aT, float* dw,
+                                                                  const int32_t* poff, int N, int K, int64_t ld) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int e = blockIdx.z, row0 = blockIdx.y * GBM;
+    TileTaskF p;
+    p.a_base = dyT + poff[e]; p.gather = nullptr; p.a_row0 = row0;
+    p.w[0] = p.w[1] = aT + poff[e]; p.bias[0] = p.bias[1] = nullptr;
+    p.c_base = dw + (int64_t)e * N * K + (int64_t)row0 * K;
+    p.K = poff[e + 1] - poff[e]; p.a_ld = p.b_ld = (int)ld; p.N = K; p.rows = min(GBM, N - row0); p.c0 = blockIdx.x * GN1;
+    p.act = MOE_ACT_NONE; p.paired = false; p.publish = false;
     f32_gemm_tile(p, smem);
 }
 
@@ -327,6 +364,31 @@ hipError_t launch_gemm_dense_f32_tile(const void* A, const void* B, const void* 
     const dim3 grid((unsigned)(N / GBN), (unsigned)((M + GBM - 1) / GBM));
     gemm_dense_f32_tile_kernel<<<grid, GTHREADS, GLDS, st>>>((const float*)A, (const float*)B, (const float*)bias, (float*)C,
                                                              (int)M, (int)N, (int)K, act);
+    return hipGetLastError();
+}
+
+bool grouped_gemm_f32_takes_tile(int64_t A, int N, int K) {
+    return N % GBN == 0 && K % GBK == 0 && (A / GBM) * (N / GBN) >= 256;
+}
+
+hipError_t launch_grouped_gemm_f32_tile(const void* a_rows, const void* w, const void* bias, void* out, const MTile* mtiles,
+                                        const int32_t* num_mtiles, int max_mtiles, int N, int K, int act, hipStream_t st) {
+    hipError_t e = allow_lds(&grouped_gemm_f32_tile_kernel);
+    if (e != hipSuccess) return e;
+    const int nnt = N / GBN;
+    grouped_gemm_f32_tile_kernel<<<(unsigned)max_mtiles * nnt, GTHREADS, GLDS, st>>>(
+        (const float*)a_rows, (const float*)w, (const float*)bias, (float*)out, mtiles, num_mtiles, nnt, N, K, act);
+    return hipGetLastError();
+}
+
+bool wgrad_f32_takes_tile(int E, int N, int K) { return K % GBN == 0 && (int64_t)E * (N / GBM) * (K / GBN) >= 128; }
+
+hipError_t launch_wgrad_f32_tile(const void* dyT, const void* aT, void* dw, const int32_t* poff, int E, int N, int K,
+                                 int64_t ld, hipStream_t st) {
+    hipError_t e = allow_lds(&wgrad_f32_tile_kernel);
+    if (e != hipSuccess) return e;
+    const dim3 grid((unsigned)(K / GBN), (unsigned)((N + GBM - 1) / GBM), (unsigned)E);
+    wgrad_f32_tile_kernel<<<grid, GTHREADS, GLDS, st>>>((const float*)dyT, (const float*)aT, (float*)dw, poff, N, K, ld);
     return hipGetLastError();
 }
 

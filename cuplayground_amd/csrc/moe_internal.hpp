@@ -175,21 +175,21 @@ hipError_t launch_ffn_persistent(const FfnArgs& a, int dtype, const FfnPlan& p, 
 int ffn_persistent_blocks(int dtype, int tile, int compute_units);
 
 // ---- backward building blocks (csrc/backward.hip) ----
-size_t backward_scratch_bytes(int64_t A, int E, int H, int I);
+size_t backward_scratch_bytes(int64_t A, int E, int H, int I, int elem_bytes);
 hipError_t launch_transpose(const void* src, void* dst, int64_t batch, int64_t rows, int64_t cols, int elem_bytes,
                             hipStream_t st);
 hipError_t launch_expert_gemm(const void* a_rows, const void* w, const void* bias, const int32_t* count,
-                              const int32_t* offset, int64_t A, int E, int N, int K, int act, bool f16, void* out_rows,
+                              const int32_t* offset, int64_t A, int E, int N, int K, int act, int dtype, void* out_rows,
                               void* scratch, hipStream_t st);
 hipError_t launch_expert_wgrad(const void* dy_rows, const void* a_rows, const int32_t* count, const int32_t* offset,
-                               int64_t A, int E, int N, int K, bool f16, void* dw, void* scratch, hipStream_t st);
+                               int64_t A, int E, int N, int K, int dtype, void* dw, void* scratch, hipStream_t st);
 
-hipError_t launch_act_backward(const void* dh, const void* u, const void* g, int64_t n, int act, bool f16, void* du,
+hipError_t launch_act_backward(const void* dh, const void* u, const void* g, int64_t n, int act, int dtype, void* du,
                                void* dg, hipStream_t st);
-hipError_t launch_bias_grad(const void* dy, const int32_t* count, const int32_t* offset, int E, int N, bool f16, void* db,
+hipError_t launch_bias_grad(const void* dy, const int32_t* count, const int32_t* offset, int E, int N, int dtype, void* db,
                             hipStream_t st);
 hipError_t launch_combine_backward(const void* dout, const void* y, const int32_t* pair_row, const float* topk_w, int S,
-                                   int k, int H, bool f16, void* dy, float* dw, hipStream_t st);
+                                   int k, int H, int dtype, void* dy, float* dw, hipStream_t st);
 
 hipError_t launch_gemm_bias_act(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N,
                                 int64_t K, int dtype, int act, hipStream_t st);

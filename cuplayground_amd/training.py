@@ -1,4 +1,4 @@
-"""A trainable MoE layer over the backward building blocks of libmoe355 (bf16 / fp16 layers).
+"""A trainable MoE layer over the backward building blocks of libmoe355 (fp32, tf32, bf16 and fp16 layers).
 
 The reference declares a training knob (`is_training`, aristos_config.schema.json:20-23) that none of its code reads.
 Here it has a consumer: `MoE355Train` runs the expert projections through `moe_expert_gemm` and gets their gradients
@@ -47,8 +47,8 @@ class MoE355Train(torch.nn.Module):
 
     def __init__(self, cfg: api.MoEConfig, init_std: float = 0.02, seed: int = 0):
         super().__init__()
-        if cfg.torch_dtype not in (api.DTYPE_BF16, api.DTYPE_FP16):
-            raise ValueError("the backward building blocks exist for bf16 and fp16 layers")
+        if cfg.torch_dtype == api.DTYPE_FP8:
+            raise ValueError("the backward building blocks exist for fp32, tf32, bf16 and fp16 layers, not for e4m3 weights")
         self.cfg = cfg
         self.layer = api.MoELayer(cfg)
         dt = self.layer.act_dtype

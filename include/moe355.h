@@ -275,7 +275,7 @@ int moe_quant_block128(const void* w, int32_t src_dtype, int64_t matrices, int64
 int moe_dequant_block128(const void* q, const float* scales, int64_t matrices, int64_t N, int64_t K, void* out,
                          void* stream);
 
-/* ---- Backward building blocks (bf16 and fp16 layers) -------------------------------------------------------------
+/* ---- Backward building blocks (fp32, tf32, bf16 and fp16 layers; e4m3 layers: MOE_ERR_UNSUPPORTED) ------------------
  * The reference declares a training knob (is_training, aristos_config.schema.json:20-23) that none of its code reads
  * and has no backward pass; these entry points are what a training step needs beyond the forward stages above.  All
  * of them work on packed expert-major rows as moe_route lays them out: rows [expert_offset[e], expert_offset[e] +
@@ -289,7 +289,7 @@ int moe_dequant_block128(const void* q, const float* scales, int64_t matrices, i
  * moe_expert_gemm: out_rows[r,:] = act(a_rows[r,:K] . w[e(r)]^T + bias[e(r)]) for every kept row r, w [E,N,K], bias
  *   [E,N] or null, act RELU / GELU / NONE; the grouped product of the forward FFN as a stage of its own.
  * moe_expert_wgrad: dw[e] [N,K] = sum over the rows r of expert e of dy_rows[r,:N]^T a_rows[r,:K]; an expert with no
- *   rows gets zeros.  dw is written in the layer's 16-bit type. */
+ *   rows gets zeros.  dw is written in the layer's storage type (fp32, bf16 or fp16), like every operand here. */
 int moe_backward_scratch_bytes(const moe_config* cfg, size_t* bytes);
 int moe_transpose(const void* src, void* dst, int64_t batch, int64_t rows, int64_t cols, int32_t elem_bytes,
                   void* stream);
@@ -305,7 +305,7 @@ int moe_expert_wgrad(moe_handle* h, const void* dy_rows, const void* a_rows, con
  *   with s = sigmoid(g).  u_rows / g_rows are the projections before the activation (moe_expert_gemm with
  *   MOE_ACT_NONE); g_rows and dg_rows are given exactly when the layer is SwiGLU.
  * moe_bias_grad: db[e, n] = sum over expert e's rows, in ascending row order, of dy_rows[r, n], stored in the layer's
- *   16-bit type like the bias it belongs to; N is H or I, db is [E, N].
+ *   storage type like the bias it belongs to; N is H or I, db is [E, N].
  * moe_combine_backward: the adjoint of moe_combine: dy_rows[pair_row[t,r], :] = topk_w[t,r] * dout[t, :] and
  *   dw[t,r] = <dout[t, :], y_rows[pair_row[t,r], :]> (0 for a dropped pair); rows of dy_rows that no pair maps to are
  *   left untouched. */

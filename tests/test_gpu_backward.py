@@ -7,7 +7,7 @@ from oracle import binding as ob
 from helpers import OUT_TOL, from_device, max_rel_err, product_config, to_device
 
 pytestmark = pytest.mark.gpu
-KIND = {ob.BF16: "bf16", ob.F16: "f16"}
+KIND = {ob.BF16: "bf16", ob.F16: "f16", ob.F32: "f32"}
 
 
 @pytest.fixture(scope="module")
@@ -54,7 +54,7 @@ CASES = [  # S, H, I, E, k, capacity factor, router skew
 ]
 
 
-@pytest.mark.parametrize("dtype", [ob.BF16, ob.F16])
+@pytest.mark.parametrize("dtype", [ob.BF16, ob.F16, ob.F32])
 @pytest.mark.parametrize("case", CASES)
 def test_expert_gemm_vs_oracle(moe, case, dtype):
     S, H, I, E, k, cf, skew = case
@@ -71,6 +71,35 @@ def test_expert_gemm_vs_oracle(moe, case, dtype):
         kept = int(count.sum())
         assert max_rel_err(got[:kept], want[:kept]) <= OUT_TOL[dtype]
         assert not got[kept:].any()            # rows of no expert are not written (the output started as zeros)
+
+
+def test_fp32_products_on_the_matrix_core_tile_and_on_the_vector_tile(moe, monkeypatch):
+    """fp32 layers: the grouped product and the weight gradient of a shape that takes the 128 x 128 matrix-core tile,
+    and the same calls held on the 64 x 64 vector-ALU tile (MOE355_F32_TILE=0).  Both within the fp32 tolerance of the
+    oracle; their sums run in different orders, so the results are not the same bits -- which shows both ran."""
+    S, H, I, E, k, cf, skew = CASES[2]
+    dtype = ob.F32
+    cfg, rng, count, offset = routed_case(S, H, I, E, k, dtype, seed=79, cf=cf, skew=0.3)
+    layer = moe.MoELayer(product_config(cfg))
+    a, dy, w, bias = operands(rng, S * k, E, I, H, dtype)
+    want = ob.expert_gemm(a, w, bias, count, offset, dtype, ob.ACT_GELU)
+    want_dw = ob.expert_wgrad(dy, a, count, offset, dtype)
+    kept = int(count.sum())
+    dev = [to_device(v, "f32") for v in (a, dy, w, bias)] + [to_device(count, "i32"), to_device(offset, "i32")]
+    outs, grads = {}, {}
+    for knob in ("0", None):
+        if knob is None:
+            monkeypatch.delenv("MOE355_F32_TILE")
+        else:
+            monkeypatch.setenv("MOE355_F32_TILE", knob)
+        outs[knob] = from_device(layer.expert_gemm(dev[0], dev[2], dev[3], dev[4], dev[5], ob.ACT_GELU))
+        grads[knob] = from_device(layer.expert_wgrad(dev[1], dev[0], dev[4], dev[5]))
+        assert max_rel_err(outs[knob][:kept], want[:kept]) <= OUT_TOL[dtype]
+        for e in range(E):
+            if count[e] > 0:
+                assert max_rel_err(grads[knob][e], want_dw[e]) <= OUT_TOL[dtype], e
+    assert not np.array_equal(outs["0"][:kept], outs[None][:kept])
+    assert not np.array_equal(grads["0"], grads[None])
 
 
 @pytest.mark.parametrize("dtype", [ob.BF16, ob.F16])
@@ -95,7 +124,7 @@ def test_grouped_product_tiles_agree(moe, dtype, monkeypatch):
     assert np.array_equal(outs["1"], outs["2"])
 
 
-@pytest.mark.parametrize("dtype", [ob.BF16, ob.F16])
+@pytest.mark.parametrize("dtype", [ob.BF16, ob.F16, ob.F32])
 @pytest.mark.parametrize("case", CASES)
 def test_data_gradient_is_the_grouped_product_with_the_transposed_weight(moe, case, dtype):
     """dX = dY . W: the oracle works on numpy's transpose, the product on moe_transpose's."""
@@ -113,7 +142,7 @@ def test_data_gradient_is_the_grouped_product_with_the_transposed_weight(moe, ca
     assert max_rel_err(ob.to_f32(from_device(got), dtype)[:kept], want[:kept]) <= OUT_TOL[dtype]
 
 
-@pytest.mark.parametrize("dtype", [ob.BF16, ob.F16])
+@pytest.mark.parametrize("dtype", [ob.BF16, ob.F16, ob.F32])
 @pytest.mark.parametrize("case", CASES)
 def test_weight_gradient_vs_oracle(moe, case, dtype):
     S, H, I, E, k, cf, skew = case
@@ -151,11 +180,11 @@ def test_empty_experts_and_second_call_reuse_scratch(moe):
 
 def test_unsupported_layers_and_bad_arguments_are_refused(moe):
     import torch
-    cfg = ob.Cfg(S=128, H=128, I=256, E=4, k=1, dtype=ob.F32, act=ob.ACT_RELU, drop=0)
+    cfg = ob.Cfg(S=128, H=128, I=256, E=4, k=1, dtype=ob.FP8, act=ob.ACT_RELU, drop=0)
     layer = moe.MoELayer(product_config(cfg))
     with pytest.raises(moe.MoEError) as e:
         layer.backward_scratch()
-    assert e.value.status == 2                    # fp32 layers have no backward kernels
+    assert e.value.status == 2                    # e4m3 layers have no backward kernels
     cfg = ob.Cfg(S=128, H=128, I=256, E=4, k=1, dtype=ob.BF16, act=ob.ACT_RELU, drop=0)
     layer = moe.MoELayer(product_config(cfg))
     z = torch.zeros(128, 192, dtype=torch.bfloat16, device="cuda")
@@ -166,7 +195,7 @@ def test_unsupported_layers_and_bad_arguments_are_refused(moe):
     assert e.value.status == 4
 
 
-@pytest.mark.parametrize("dtype", [ob.BF16, ob.F16])
+@pytest.mark.parametrize("dtype", [ob.BF16, ob.F16, ob.F32])
 @pytest.mark.parametrize("act", [ob.ACT_RELU, ob.ACT_GELU, ob.ACT_SWIGLU])
 def test_activation_backward_vs_oracle(moe, act, dtype):
     cfg = ob.Cfg(S=300, H=128, I=320, E=4, k=2, dtype=dtype, act=act, drop=0)
@@ -189,7 +218,7 @@ def test_activation_backward_vs_oracle(moe, act, dtype):
         assert dg is None
 
 
-@pytest.mark.parametrize("dtype", [ob.BF16, ob.F16])
+@pytest.mark.parametrize("dtype", [ob.BF16, ob.F16, ob.F32])
 def test_bias_gradient_is_bit_exact(moe, dtype):
     """One thread per column adds the rows in ascending order, as the oracle does: the same fp32 sums, bit for bit."""
     S, H, I, E, k, cf, skew = CASES[1]
@@ -202,7 +231,7 @@ def test_bias_gradient_is_bit_exact(moe, dtype):
         assert np.array_equal(got, ob.bias_grad(dy, count, offset, dtype))
 
 
-@pytest.mark.parametrize("dtype", [ob.BF16, ob.F16])
+@pytest.mark.parametrize("dtype", [ob.BF16, ob.F16, ob.F32])
 def test_combine_backward_vs_oracle(moe, dtype):
     cfg = ob.Cfg(S=257, H=320, I=128, E=5, k=3, dtype=dtype, act=ob.ACT_RELU, drop=1, capacity_factor=0.8)
     rng = np.random.default_rng(41)
@@ -216,7 +245,7 @@ def test_combine_backward_vs_oracle(moe, dtype):
     dout = ob.from_f32(rng.standard_normal((cfg.S, cfg.H)).astype(np.float32), dtype)
     want_dy, want_dw = ob.combine_backward(dout, y, r["pair_row"], w, dtype)
     dy, dw = layer.combine_backward(to_device(dout, kind), to_device(y, kind), to_device(r["pair_row"], "i32"), to_device(w, "f32"))
-    if dtype == ob.BF16:
+    if dtype in (ob.BF16, ob.F32):
         assert np.array_equal(from_device(dy), want_dy)        # one multiplication and one rounding per element
     else:   # fp16: the compiler multiplies and narrows in one mixed-precision instruction (one rounding), the oracle
         # rounds the fp32 product first; on near-ties they differ by one fp16 ulp

@@ -157,7 +157,8 @@ int moe_forward(moe_handle* h, const void* x, const moe_weights* w, void* out, c
  * the library is loaded until the process ends) instead of from the caller.  It has no counterpart in the reference,
  * whose drivers allocate one arena per run (mma.cuh:385-391).  Calls no hipMalloc / hipFree or any other allocating
  * routine.  Returns MOE_ERR_WORKSPACE when moe_workspace_bytes(config) exceeds the array (decode-sized and small
- * prefill layers fit; the Mixtral-shape intermediate does not).  Every call on a GPU uses that GPU's one array: calls
+ * prefill layers fit; the Mixtral-shape intermediate does not; the bf16 weight copies of an e4m3 layer on the widening
+ * plan count, see moe_get_kernel_dtype).  Every call on a GPU uses that GPU's one array: calls
  * that overlap in time on one GPU (two streams, two threads, two handles) race; calls in sequence on one stream are
  * safe, each call re-initialises what it needs.
  */

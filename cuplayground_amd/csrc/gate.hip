@@ -334,6 +334,115 @@ hipError_t launch_gate_tiled(const void* x, const void* gate_w, const float* gat
     }
 }
 
+// ---- third logits kernel: the same sums on the matrix cores (16-bit layers, H a multiple of 512) ----
+//
+// v_mfma_f32_16x16x1_4b_f32 is four independent 16 x 16 outer products with k = 1: D_b[i][j] = C_b[i][j] + A_b[i] B_b[j],
+// one multiply-add per element -- and the product of two bf16 (or fp16) values is exact in fp32, so each element sees
+// exactly the fmaf the kernels above perform, at the full fp32 rate of the matrix pipe (twice the unpacked vector rate)
+// with the widening running beside it on the vector ALU.  A pair of wavefronts owns 16 tokens x 16 experts.  Block b of
+// accumulator g carries partial sum p = 4 g + b of every pair of the tile: lane 16 b + i loads the 16-byte chunk
+// p + 64 j of token row i (and of expert row i) -- the chunk partial sum p takes in step j, i.e. elements
+// 32 (16 j + g) + 8 b onwards -- and its 8 elements go through 8 MFMAs in ascending k.  The even g belong to one
+// wavefront of the pair and the odd g to the other (8 accumulators = 128 registers each, so two wavefronts fit a
+// SIMD and one's loads and widening hide behind the other's MFMAs).  The 32 partial sums a wavefront holds of a pair
+// sit in one lane (accumulator g, register 4 b + r: token 4 (lane / 16) + r, expert lane % 16): p is folded with
+// p + 32, 16 and 8 (g with g + 8, 4, 2) in the lane, with p + 4 (g with g + 1) across the two wavefronts through LDS,
+// then with p + 2 and p + 1 (b) in the lane again -- the pairings of fold16, so the logits are bit-identical.
+typedef float gate_f32x16 __attribute__((ext_vector_type(16)));
+
+template <typename T>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gate_mfma_kernel(const T* __restrict__ x, const T* __restrict__ gate_w,
+                                                        const float* __restrict__ gate_bias, float* __restrict__ logits,
+                                                        int S, int H, int E) {
+    typedef typename RawChunk<T>::type raw_t;
+    __shared__ float s_odd[2][16][64];          // [pair][4 b + r][lane]: the odd wavefront's sums over its g
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int pair = wave >> 1, odd = wave & 1;
+    const int b = lane >> 4, i = lane & 15;
+    const int t0 = blockIdx.x * 16, e0 = (blockIdx.y * 2 + pair) * 16;
+    const bool live = e0 < E;                   // an expert tile past the last one: nothing to do, but meet the barrier
+    gate_f32x16 acc[8];
+#pragma unroll
+    for (int g = 0; g < 8; ++g)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[g][v] = 0.f;
+    if (live) {
+        // this wavefront's chunks: g = 2 gg + odd
+        const T* xrow = x + (size_t)min(t0 + i, S - 1) * H + 8 * b + 32 * odd;
+        const T* wrow = gate_w + (size_t)min(e0 + i, E - 1) * H + 8 * b + 32 * odd;
+        raw_t xn[8], wn[8];
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+            xn[g] = *reinterpret_cast<const raw_t*>(xrow + 64 * g);
+            wn[g] = *reinterpret_cast<const raw_t*>(wrow + 64 * g);
+        }
+        const int nstep = H / 512;
+        for (int j = 0; j < nstep; ++j) {
+            const bool more = j + 1 < nstep;
+            const T* xnext = xrow + 512 * (j + 1);
+            const T* wnext = wrow + 512 * (j + 1);
+#pragma unroll
+            for (int g = 0; g < 8; g += 2) {    // two accumulators at a time: consecutive MFMAs are independent
+                float xv[2][8], wv[2][8];
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    widen8<T>(xn[g + h], xv[h]);
+                    widen8<T>(wn[g + h], wv[h]);
+                    if (more) {
+                        xn[g + h] = *reinterpret_cast<const raw_t*>(xnext + 64 * (g + h));
+                        wn[g + h] = *reinterpret_cast<const raw_t*>(wnext + 64 * (g + h));
+                    }
+                }
+#pragma unroll
+                for (int v = 0; v < 8; ++v)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h)
+                        acc[g + h] = __builtin_amdgcn_mfma_f32_16x16x1f32(xv[h][v], wv[h][v], acc[g + h], 0, 0, 0);
+            }
+        }
+    }
+    // acc[gg] holds g = 2 gg + odd: g + 8, g + 4, g + 2 are gg + 4, gg + 2, gg + 1
+    float u[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        const float s0 = acc[0][v] + acc[4][v], s1 = acc[1][v] + acc[5][v], s2 = acc[2][v] + acc[6][v],
+                    s3 = acc[3][v] + acc[7][v];                                        // p with p + 32
+        u[v] = (s0 + s2) + (s1 + s3);                                                  // ... p + 16, then p + 8
+    }
+    if (odd) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s_odd[pair][v][lane] = u[v];
+    }
+    __syncthreads();
+    if (odd || !live) return;
+    const int e = e0 + i;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        float q[4];
+#pragma unroll
+        for (int bb = 0; bb < 4; ++bb) q[bb] = u[4 * bb + r] + s_odd[pair][4 * bb + r][lane];     // ... p + 4
+        const float sum = (q[0] + q[2]) + (q[1] + q[3]);                                           // ... p + 2, p + 1
+        const int t = t0 + 4 * b + r;
+        if (t < S && e < E) logits[(size_t)t * E + e] = gate_bias ? sum + gate_bias[e] : sum;
+    }
+}
+
+// The matrix-core kernel takes 16-bit layers whose rows split into full steps of 512 elements, when the experts fill
+// most of its 16 columns and there are enough 16 x 16 tiles for every SIMD of the chip to get several.
+template <typename T>
+bool launch_gate_mfma(const void* x, const void* gate_w, const float* gate_bias, float* logits, int S, int H, int E,
+                      hipStream_t st, hipError_t* err) {
+    if (H % 512 != 0) return false;
+    const int et = (E + 15) / 16;
+    bool use = et * 16 * 3 <= E * 4 && (int64_t)((S + 15) / 16) * et >= 2048;
+    if (const char* env = getenv("MOE355_GATE_MFMA")) use = atoi(env) != 0;   // tuning knob
+    if (!use) return false;
+    const dim3 grid((S + 15) / 16, (et + 1) / 2);
+    gate_mfma_kernel<T><<<grid, 256, 0, st>>>((const T*)x, (const T*)gate_w, gate_bias, logits, S, H, E);
+    *err = hipGetLastError();
+    return true;
+}
+
 // One wavefront per token.
 __global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ logits, int S, int E, int k, int gate_fn,
                                                    int norm, int32_t* __restrict__ topk_idx,
@@ -444,6 +553,12 @@ hipError_t launch_gate_logits(const void* x, const void* gate_w, const float* ga
                               int E, int act_dtype, hipStream_t st) {
     // Many experts on many tokens: the first kernel (token rows in registers, experts streamed) reads least per sum.
     // Everything else -- few experts, or decode-sized batches -- goes to the register-tiled kernel.
+    if (act_dtype != MOE_DTYPE_F32) {
+        hipError_t e = hipSuccess;
+        const bool taken = act_dtype == MOE_DTYPE_FP16 ? launch_gate_mfma<f16_s>(x, gate_w, gate_bias, logits, S, H, E, st, &e)
+                                                       : launch_gate_mfma<bf16_s>(x, gate_w, gate_bias, logits, S, H, E, st, &e);
+        if (taken) return e;
+    }
     bool rows_in_registers = E >= 32 && (int64_t)S * E >= ((int64_t)1 << 19);
     if (const char* env = getenv("MOE355_GATE_KERNEL")) rows_in_registers = atoi(env) == 1;   // tuning knob
     if (rows_in_registers) {

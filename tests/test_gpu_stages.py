@@ -153,11 +153,17 @@ GATE_CASES = [
     ob.Cfg(S=300, H=1536, I=64, E=40, k=4, dtype=ob.F16),
     ob.Cfg(S=20000, H=512, I=64, E=32, k=2, dtype=ob.F16),     # many pairs: the kernel that keeps token rows in registers
     ob.Cfg(S=50, H=128, I=64, E=5, k=2, dtype=ob.TF32),
+    ob.Cfg(S=77, H=512, I=64, E=5, k=2, dtype=ob.BF16, zipf_bias=True),      # ragged token and expert tiles of the matrix-core kernel
+    ob.Cfg(S=4100, H=1024, I=64, E=8, k=2, dtype=ob.F16),                     # its 16-token x 8-expert arrangement
 ]
 
 
+# mfma: the logits kernel on the matrix cores forced on / off (it takes 16-bit layers with H % 512 = 0 only; elsewhere
+# the knob changes nothing) -- every kernel must produce the oracle's bit patterns
+@pytest.mark.parametrize("mfma", ["0", "1"], ids=["valu", "mfma"])
 @pytest.mark.parametrize("cfg", GATE_CASES, ids=lambda c: "S%d_H%d_E%d_k%d_d%d" % (c.S, c.H, c.E, c.k, c.dtype))
-def test_gate_vs_oracle(moe, cfg):
+def test_gate_vs_oracle(moe, cfg, mfma, monkeypatch):
+    monkeypatch.setenv("MOE355_GATE_MFMA", mfma)
     inp = ob.make_inputs(cfg, seed=7, router_only=True)
     want = ob.route(cfg, inp)
     layer = moe.MoELayer(product_config(cfg))

@@ -444,13 +444,14 @@ bool launch_gate_mfma(const void* x, const void* gate_w, const float* gate_bias,
 }
 
 // One wavefront per token.
+template <int J>
 __global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ logits, int S, int E, int k, int gate_fn,
                                                    int norm, int32_t* __restrict__ topk_idx,
                                                    float* __restrict__ topk_w) {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int t = blockIdx.x * 4 + wave;
     if (t >= S) return;
-    topk_one_token(logits, t, E, k, gate_fn, norm, topk_idx, topk_w, lane);
+    topk_one_token<J>(logits, t, E, k, gate_fn, norm, topk_idx, topk_w, lane);
 }
 
 // Router statistics for a load-balancing loss.  Block b, wavefront w takes tokens (4b + w) + 4*gridDim.x*i; a lane
@@ -573,7 +574,11 @@ hipError_t launch_gate_logits(const void* x, const void* gate_w, const float* ga
 
 hipError_t launch_topk(const float* logits, int S, int E, int k, int gate_fn, int norm, int32_t* topk_idx,
                        float* topk_w, hipStream_t st) {
-    topk_kernel<<<(S + 3) / 4, 256, 0, st>>>(logits, S, E, k, gate_fn, norm, topk_idx, topk_w);
+    const unsigned grid = (unsigned)((S + 3) / 4);
+    if (E <= 64) topk_kernel<1><<<grid, 256, 0, st>>>(logits, S, E, k, gate_fn, norm, topk_idx, topk_w);
+    else if (E <= 128) topk_kernel<2><<<grid, 256, 0, st>>>(logits, S, E, k, gate_fn, norm, topk_idx, topk_w);
+    else if (E <= 256) topk_kernel<4><<<grid, 256, 0, st>>>(logits, S, E, k, gate_fn, norm, topk_idx, topk_w);
+    else topk_kernel<kMaxExperts / kWave><<<grid, 256, 0, st>>>(logits, S, E, k, gate_fn, norm, topk_idx, topk_w);
     return hipGetLastError();
 }
 

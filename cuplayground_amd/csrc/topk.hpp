@@ -44,14 +44,16 @@ __device__ __forceinline__ Cand wave_best(Cand c) {
     return best;
 }
 
-// Lane l keeps the logits of experts l, l+64, ... (at most 8) in registers.  Called by all 64 lanes of a wavefront.
+// Lane l keeps the logits of experts l, l+64, ... (J of them; J * 64 >= E) in registers.  Called by all 64 lanes of a
+// wavefront.  J is a template parameter so that layers with up to 64 experts do not walk eight slots per step.
 // The selection is total: a NaN logit ranks as -inf (behind every number, ties to the lower index), so a token row
 // that overflowed still gets k distinct, valid experts; its weights are computed from the logits as they are and
 // come out NaN, which is what reaches the output of that token and of no other.
+template <int J>
 __device__ __forceinline__ void topk_one_token(const float* __restrict__ logits, int t, int E, int k, int gate_fn,
                                                int norm, int32_t* __restrict__ topk_idx, float* __restrict__ topk_w,
                                                int lane) {
-    constexpr int J = kMaxExperts / kWave;
+    static_assert(J >= 1 && J <= kMaxExperts / kWave, "slots per lane");
     float v[J];
     unsigned avail = 0;
 #pragma unroll
@@ -82,7 +84,8 @@ __device__ __forceinline__ void topk_one_token(const float* __restrict__ logits,
         float mine = v[0];
 #pragma unroll
         for (int j = 1; j < J; ++j) mine = (c.i >> 6) == j ? v[j] : mine;
-        const float cv = __shfl(mine, c.i & (kWave - 1), kWave);
+        // c comes out of wave_best through scalar registers: the winner's lane is uniform, so a lane read, not a shuffle
+        const float cv = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(mine), c.i & (kWave - 1)));
         if (lane == r) { my_l = cv; my_i = c.i; }
         if (r == 0) top_l = cv;
     }

@@ -33,6 +33,7 @@ def _cases(n=36, seed=2024):
                      MOE355_QUEUE_EARLY=str(int(rng.integers(0, 2))), MOE355_FUSED_COMBINE=str(int(rng.integers(0, 2))))
         knobs["MOE355_ROW_CHUNK"] = str(i % 4)      # order of the tasks inside a queue segment (0: plain; drawn outside the seeded stream)
         knobs["MOE355_FP8_TILE"] = str(i // 5 % 2)  # e4m3 layers: weight streamer or tile GEMM
+        knobs["MOE355_GATE_MFMA"] = str(i // 2 % 2)   # 16-bit layers with H % 512 = 0: logits on the vector ALU or on the matrix cores
         knobs["MOE355_F32_TILE"] = str(i // 5 % 2)   # fp32 layers: vector-ALU kernel or (shape permitting) the matrix-core tile
         knobs["MOE355_FP8_WIDEN"] = str(i // 10 % 2)  # ... or the bf16 tiles on weights widened in the workspace
         out.append(pytest.param(cfg, knobs, int(rng.integers(1, 3)), bool(rng.integers(0, 2)), id="case%02d" % i))

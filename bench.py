@@ -120,6 +120,31 @@ def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False, balanced_
     step_ms = [a.elapsed_time(b) for a, b in ev]
     ms_per_step_events = (t3 - t2) * 1e3 / steps
 
+    # the same `steps` calls once more as replays of a HIP graph holding one forward call: what a serving loop that
+    # captures the layer pays per step (launch-bound shapes gain; the others show that capture costs nothing)
+    graph_ms = graph_err = None
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            layer.forward(dev["x"], dev, out=out)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            layer.forward(dev["x"], dev, out=out)
+        for _ in range(warmup):
+            graph.replay()
+        torch.cuda.synchronize()
+        t4 = time.perf_counter()
+        for _ in range(steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        graph_ms = (time.perf_counter() - t4) * 1e3 / steps
+        del graph
+    except Exception as e:        # reported, never fatal: the figures above do not depend on it
+        graph_err = "%s: %s" % (type(e).__name__, e)
+
     routing = layer.new_routing()                 # one extra, untimed call fetches the routing result
     layer.forward(dev["x"], dev, out=out, routing=routing)
     torch.cuda.synchronize()
@@ -166,7 +191,8 @@ def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False, balanced_
             else "no counter run for this kernel"
     res = {
         "workload": w.describe(), "tokens_per_s": c.tokens / (ms_per_step * 1e-3), "ms_per_step": ms_per_step,
-        "ms_per_step_with_events": ms_per_step_events, "step_ms": stats(step_ms), "steps": steps, "warmup": warmup,
+        "ms_per_step_with_events": ms_per_step_events, "ms_per_step_graph_replay": graph_ms if graph_err is None else graph_err,
+        "step_ms": stats(step_ms), "steps": steps, "warmup": warmup,
         "tflops": layer_flops / (ms_per_step * 1e-3) / 1e12,
         "stage_ms": {k: round(v, 4) for k, v in stage_mean.items() if k != "calls"},
         "stage_ms_median": {k: round(statistics.median(v[-steps:]), 4) for k, v in samples.items()},
@@ -464,6 +490,8 @@ def main():
         "warmup": args.warmup, "ms_per_step": res["ms_per_step"],
         # a second pass over the same steps carries the hipEvents behind step_ms, stage_ms and roofline.kernel_ms
         "ms_per_step_with_events": res["ms_per_step_with_events"], "step_ms": res["step_ms"],
+        # the same steps as replays of a HIP graph that holds one forward call
+        "ms_per_step_graph_replay": res["ms_per_step_graph_replay"],
         "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": dtype[main_w.config.torch_dtype], "data": "synthetic",
         "config": {"workload": res["workload"], "ffn_mode": res["ffn_mode"], "block_rows": res["block_rows"],

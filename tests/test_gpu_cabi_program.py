@@ -15,6 +15,10 @@ PROGRAM = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cabi", "run_
 CASES = {
     "bf16_swiglu": ob.Cfg(S=384, H=256, I=384, E=8, k=2, act=ob.ACT_SWIGLU, dtype=ob.BF16, drop=1, capacity_factor=1.0),
     "f32_gelu": ob.Cfg(S=128, H=128, I=256, E=4, k=1, act=ob.ACT_GELU, dtype=ob.F32, norm_topk=0, drop=0),
+    # the knob values of the reference's own aristos_config.json at one of its four micro-batches: fp32, one expert,
+    # ReLU, H 1024, I 4096 -- the plan that runs the fp32 matrix-core tile
+    "f32_reference_knobs": ob.Cfg(S=2048, H=1024, I=4096, E=1, k=1, act=ob.ACT_RELU, dtype=ob.F32, norm_topk=0, drop=0,
+                                  capacity_factor=1.0),
 }
 
 

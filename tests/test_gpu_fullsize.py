@@ -12,8 +12,14 @@ from helpers import OUT_TOL, from_device, max_rel_err, product_config, upload_in
 
 pytestmark = pytest.mark.gpu
 FFN_TILED, FFN_PERSISTENT = 1, 2
-RANDOM_TOKENS = {"C2": 512, "C3": 256, "C4": 512, "C5": 64}   # C5: all of its tokens
+RANDOM_TOKENS = {"C2": 512, "C3": 256, "C4": 512, "C5": 64, "R0": 256, "X1": 128}   # C5: all of its tokens
 MAX_STRATA_EXPERTS = 32
+# Two more full-size layers beside the five measured configurations: the knob file the reference ships
+# (aristos_config.json: fp32, 4 x 2048 tokens, one expert, ReLU -- the fp32 matrix-core tile), and the Mixtral shape
+# with e4m3 weights (the plan that widens the weights to bf16 in the workspace).
+FULL_SIZE = dict(ob.BASELINE)
+FULL_SIZE["R0"] = ob.Cfg(S=8192, H=1024, I=4096, E=1, k=1, act=ob.ACT_RELU, dtype=ob.F32, norm_topk=0, drop=0)
+FULL_SIZE["X1"] = ob.BASELINE["C3"].scaled(dtype=ob.FP8)
 
 
 def stratified_tokens(cfg, want, block_rows, seed=7):
@@ -40,17 +46,21 @@ def stratified_tokens(cfg, want, block_rows, seed=7):
     return chosen, strata, np.random.default_rng(seed)
 
 
-@pytest.mark.parametrize("name", ["C2", "C3", "C4", "C5"])
+@pytest.mark.parametrize("name", ["C2", "C3", "C4", "C5", "R0", "X1"])
 def test_baseline_config_full_size(name, monkeypatch):
     import torch
     import cuplayground_amd as moe
     assert torch.cuda.is_available()
-    cfg = ob.BASELINE[name]
+    cfg = FULL_SIZE[name]
     print("config", name, cfg, flush=True)
     inp = ob.make_inputs(cfg, seed=42)
     want = ob.route(cfg, inp)
     layer = moe.MoELayer(product_config(cfg), ffn_mode=FFN_PERSISTENT)
     dev = upload_inputs(cfg, inp)
+    if name == "R0":
+        assert layer.plan["block_rows"] == 128             # the matrix-core tile, not the 64-row vector one
+    if name == "X1":
+        assert layer.kernel_dtype == ob.BF16               # widened weights, bf16 kernels
     routing = layer.new_routing()
     out = layer.forward(dev["x"], dev, routing=routing)
     torch.cuda.synchronize()

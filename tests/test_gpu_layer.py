@@ -303,14 +303,31 @@ def test_two_handles_on_two_streams_from_two_threads(moe):
         layers[i].close()
 
 
+GRAPH_CASES = {
+    "bf16": (None, {}),
+    # an e4m3 layer on the widening plan (three more launches per call, the workspace copy rewritten by every replay)
+    "e4m3_widened": (ob.Cfg(S=600, H=256, I=384, E=4, k=2, act=ob.ACT_SWIGLU, dtype=ob.FP8, gate_fn=ob.GATE_SIGMOID, drop=0),
+                     {"MOE355_FP8_WIDEN": "1"}),
+    # an fp32 layer on the matrix-core tile, and a 16-bit one whose logits come from the matrix-core gate kernel
+    "f32_tile": (ob.Cfg(S=500, H=256, I=256, E=2, k=1, act=ob.ACT_GELU, dtype=ob.F32, norm_topk=0, drop=0),
+                 {"MOE355_F32_TILE": "1"}),
+    "f16_gate_mfma": (ob.Cfg(S=300, H=512, I=128, E=20, k=3, act=ob.ACT_RELU, dtype=ob.F16, drop=1, capacity_factor=1.0),
+                      {"MOE355_GATE_MFMA": "1"}),
+}
+
+
 @pytest.mark.parametrize("mode", [FFN_TILED, FFN_PERSISTENT], ids=["tiled", "persistent"])
-def test_forward_under_graph_capture(moe, mode):
+@pytest.mark.parametrize("case", sorted(GRAPH_CASES))
+def test_forward_under_graph_capture(moe, mode, case, monkeypatch):
     """moe_forward only enqueues kernels: it can be captured into a HIP graph.  The graph is replayed several times
     with eager work and synchronisations in between, on changing inputs, and every replay is checked against the
     eager result for the same input."""
     import torch
-    cfg = RAGGED["bf16_swiglu_bias_dropless"]
-    inp = ob.make_inputs(cfg, seed=13, with_bias=True)
+    cfg, env = GRAPH_CASES[case]
+    cfg = cfg or RAGGED["bf16_swiglu_bias_dropless"]
+    for k_, v_ in env.items():
+        monkeypatch.setenv(k_, v_)
+    inp = ob.make_inputs(cfg, seed=13, with_bias=case == "bf16")
     layer = moe.MoELayer(product_config(cfg), ffn_mode=mode)
     dev = upload_inputs(cfg, inp)
     x = dev["x"].clone()

@@ -317,7 +317,11 @@ int resolved_ffn_mode(const moe_handle* h) {
     const int64_t hit = d.A < d.E ? d.A : d.E;
     if (row_blocks < hit) row_blocks = hit;
     const int64_t est_tasks = row_blocks * (d.plan.nnt0 + d.plan.nnt1);
-    return est_tasks >= 2 * (int64_t)h->arch.persistent_blocks ? MOE_FFN_PERSISTENT : MOE_FFN_TILED;
+    // The queue pays off from a couple of tasks per resident workgroup on.  The fp32 matrix-core tile has long tasks
+    // (a down-projection tile of the reference's knob file takes half a millisecond) and needs twice that to balance:
+    // 4096 tokens of that file, 2.6 tasks per workgroup, take 0.79 ms on the queue and 0.60 ms as two launches.
+    const bool f32_tile = (d.plan.kernel_dtype == MOE_DTYPE_F32 || d.plan.kernel_dtype == MOE_DTYPE_TF32) && d.plan.tile;
+    return est_tasks >= (f32_tile ? 4 : 2) * (int64_t)h->arch.persistent_blocks ? MOE_FFN_PERSISTENT : MOE_FFN_TILED;
 }
 
 }  // namespace

@@ -322,9 +322,11 @@ int resolved_ffn_mode(const moe_handle* h) {
     // 4096 tokens of that file, 2.6 tasks per workgroup, take 0.79 ms on the queue and 0.60 ms as two launches.
     const bool f32_tile = (d.plan.kernel_dtype == MOE_DTYPE_F32 || d.plan.kernel_dtype == MOE_DTYPE_TF32) && d.plan.tile;
     // With a single expert the queue has no second expert's up projection to run beside the down projection: it is the
-    // two launches plus dependency waits and written-through intermediate rows (the knob file itself: 1.13 ms against
-    // 1.03-1.10 ms as two launches).
-    if (f32_tile && d.E == 1) return MOE_FFN_TILED;
+    // two launches plus dependency waits and written-through intermediate rows (the reference's knob file: 1.13 ms
+    // against 1.03-1.10 ms as two launches; the same file in bf16 0.183 against 0.170 ms; the Mixtral dimensions with one
+    // expert: no difference).
+    const bool tile16 = d.plan.kernel_dtype == MOE_DTYPE_BF16 || d.plan.kernel_dtype == MOE_DTYPE_FP16;
+    if ((f32_tile || tile16) && d.E == 1) return MOE_FFN_TILED;
     return est_tasks >= (f32_tile ? 4 : 2) * (int64_t)h->arch.persistent_blocks ? MOE_FFN_PERSISTENT : MOE_FFN_TILED;
 }
 

@@ -314,9 +314,38 @@ def task_trace_summary(layer, dev, out):
                     "down-projection task's dependency wait lies in its gap, not in its duration"}
 
 
-def cpu_leg(name, dev, out, routing, seconds, seed):
+def host_cores():
+    """(threads to use, physical cores of this host): physical cores are the distinct (package, core) pairs of
+    /proc/cpuinfo; the thread count is that, capped by OMP_NUM_THREADS (a GPU box hands a job its share of the host)."""
+    phys = set()
+    try:
+        pkg = core = None
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("physical id"):
+                    pkg = line.split(":")[1].strip()
+                elif line.startswith("core id"):
+                    core = line.split(":")[1].strip()
+                elif not line.strip():
+                    if core is not None:
+                        phys.add((pkg, core))
+                    pkg = core = None
+        if core is not None:
+            phys.add((pkg, core))
+    except OSError:
+        pass
+    physical = len(phys) or (os.cpu_count() or 1)
+    threads = physical
+    env = os.environ.get("OMP_NUM_THREADS")
+    if env and env.isdigit() and int(env) >= 1:
+        threads = min(threads, int(env))
+    return threads, physical
+
+
+def cpu_leg(name, dev, out, routing, seconds, seed, oracle_share=0.5):
     """The CPU baseline (libtorch layer, then the oracle) on a bounded token sample, and the parity spot check of the
-    GPU output against the oracle on the same sample.  The only part of this script that touches oracle/."""
+    GPU output against the oracle on the same sample.  The only part of this script that touches oracle/.
+    `seconds` bounds the libtorch sample; the oracle gets `oracle_share` of that."""
     import numpy as np
     import torch
     from cuplayground_amd import api, workloads as wl
@@ -327,32 +356,23 @@ def cpu_leg(name, dev, out, routing, seconds, seed):
     c = w.config
     S = c.tokens
     fp8 = c.torch_dtype == api.DTYPE_FP8
-    widened = fp8 and layer.kernel_dtype != c.torch_dtype   # the FFN stage widens the weights, then runs the bf16 tiles
-    # fp32 layers: the matrix-core tile (128-row blocks) or the vector-ALU kernel (64-row blocks)
-    f32_kind = "" if c.torch_dtype != api.DTYPE_F32 else ("_f32_tile" if layer.plan["block_rows"] == 128 else "_f32")
-    threads = os.cpu_count() or 1
-    env = os.environ.get("OMP_NUM_THREADS")
-    if env and env.isdigit():
-        threads = int(env)
+    threads, physical = host_cores()
     torch.set_num_threads(threads)
     rng = np.random.default_rng(seed)
     order = rng.permutation(S)
 
     # ---- libtorch CPU layer: weights widened once (bf16 -> fp32; e4m3 -> bf16) outside the timed region ----
-    host = {k: v.cpu() for k, v in dev.items()}
+    mats = [n for n in ("w_up", "w_gate", "w_down") if n in dev]
+    host = {k: v.cpu() for k, v in dev.items() if not (fp8 and (k in mats or k.startswith("s_")))}
     if fp8:
-        def deq(q, s):
-            wq = q.view(torch.float8_e4m3fn).to(torch.float32)
-            E, N, K = wq.shape
-            wq = wq.view(E, N // 128, 128, K // 128, 128) * s.view(E, N // 128, 1, K // 128, 1)
-            return wq.view(E, N, K).to(torch.bfloat16)
-        cw = {n: deq(host[n], host["s_" + n[2:]]) for n in ("w_up", "w_gate", "w_down")}
+        # the library's own inverse of the block quantiser, on the GPU (exact: bf16(e4m3 * scale)), then one copy down
+        cw = {n: api.dequantize_block128(dev[n], dev["s_" + n[2:]]).cpu() for n in mats}
         prep = "e4m3 weights dequantised to bf16 once outside the timed region, bf16 linear"
     elif c.torch_dtype == api.DTYPE_BF16:
-        cw = {n: host[n].float() for n in ("w_up", "w_gate", "w_down") if n in host}
+        cw = {n: host[n].float() for n in mats}
         prep = "bf16 storage, weights widened to fp32 once outside the timed region, fp32 matmul"
     else:
-        cw = {n: host[n] for n in ("w_up", "w_gate", "w_down") if n in host}
+        cw = {n: host[n] for n in mats}
         prep = "fp32"
 
     def run_torch(tokens):
@@ -369,9 +389,10 @@ def cpu_leg(name, dev, out, routing, seconds, seed):
     dt0, _, _ = run_torch(order[:n0])
     n = int(min(S, max(n0, seconds * n0 / max(dt0, 1e-6))))
     dt, o_cpu, idx_cpu = run_torch(order[:n])
-    libtorch = {"value": n / dt, "unit": "tokens/s", "cores": threads, "kind": "port", "engine": "libtorch",
+    libtorch = {"value": n / dt, "unit": "tokens/s", "cores": threads, "host_physical_cores": physical,
+                "kind": "port", "engine": "libtorch",
                 "sample": "%d of %d tokens through the whole layer in libtorch CPU ops (linear, softmax/sigmoid, topk, "
-                          "stable sort, index_select, per-expert linear/act/linear, index_add; %s), %.1f s on %d threads"
+                          "stable sort, index_select, per-expert linear/act/linear, index_add; %s), %.2f s on %d threads"
                           % (n, S, prep, dt, threads)}
     # the same tokens on the GPU: rows agree where the CPU router picked the same experts (its fp32 sum runs in
     # another order, so near-ties may differ) and no capacity drop depends on the rest of the batch
@@ -382,7 +403,7 @@ def cpu_leg(name, dev, out, routing, seconds, seed):
         r = o_cpu.float().numpy()[same]
         libtorch["max_rel_err_gpu_vs_libtorch"] = float(np.abs(g - r).max() / max(np.abs(r).max(), 1e-30))
         libtorch["tokens_with_same_routing"] = int(same.sum())
-    del cw
+    del cw, host
 
     # ---- the CPU oracle on (a part of) the same sample + parity of the GPU output ----
     ocfg = ob.Cfg(S=S, H=c.hidden_size, I=c.intermediate_size, E=c.num_experts, k=c.expert_top_k, act=c.hidden_act,
@@ -395,7 +416,7 @@ def cpu_leg(name, dev, out, routing, seconds, seed):
     t = time.perf_counter()
     rows = ob.forward_tokens(ocfg, hostnp, r["topk_idx"], r["topk_w"], r["slot"], tok[:m0])
     d0 = time.perf_counter() - t
-    extra = int(min(S - m0, max(0, 0.5 * seconds / max(d0 / m0, 1e-9) - m0)))
+    extra = int(min(S - m0, max(0, oracle_share * seconds / max(d0 / m0, 1e-9) - m0)))
     if extra > 0:
         t = time.perf_counter()
         rows2 = ob.forward_tokens(ocfg, hostnp, r["topk_idx"], r["topk_w"], r["slot"], tok[m0:m0 + extra])
@@ -403,7 +424,7 @@ def cpu_leg(name, dev, out, routing, seconds, seed):
         rows = np.concatenate([rows, rows2])
         m0 += extra
     oracle = {"value": m0 / d0, "unit": "tokens/s", "cores": ob.num_threads(), "kind": "port", "engine": "oracle (C11 + OpenMP)",
-              "sample": "%d of %d tokens through the oracle's expert FFN + combine (routing taken as given), %.1f s"
+              "sample": "%d of %d tokens through the oracle's expert FFN + combine (routing taken as given), %.2f s"
                         % (m0, S, d0)}
     got = out[torch.from_numpy(tok[:m0].astype(np.int64)).cuda()].float().cpu().numpy()
     ref = ob.to_f32(rows, ocfg.act_dtype)
@@ -425,6 +446,8 @@ def main():
     ap.add_argument("--extra-steps", type=int, default=20)
     ap.add_argument("--ffn-mode", type=int, default=0, help="0 auto, 1 tiled (two launches), 2 persistent queue")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample (0 = skip)")
+    ap.add_argument("--extra-cpu-seconds", type=float, default=1.5,
+                    help="target CPU time of the baseline sample of each --extra workload (0 = skip)")
     ap.add_argument("--seed", type=int, default=42)
     ap.add_argument("--balanced-routing", action="store_true",
                     help="experiment: replace the router's inputs so that every expert receives exactly S*k/E rows "
@@ -480,6 +503,9 @@ def main():
             print("bench.py: unknown workload %r in --extra" % name, file=sys.stderr)
             sys.exit(2)
         r, l2, d2, o2, rt2 = measure(name, args.extra_steps, args.warmup, args.seed, args.ffn_mode)
+        if args.extra_cpu_seconds > 0:      # every workload has its CPU baseline beside it, on a smaller sample
+            r["cpu_baseline"], r["cpu_baseline_oracle"], r["parity"] = cpu_leg(name, d2, o2, rt2, args.extra_cpu_seconds,
+                                                                                args.seed)
         l2.close()
         del l2, d2, o2, rt2
         torch.cuda.empty_cache()

@@ -65,7 +65,12 @@ def _undefined_names(path):
                 names.add(n.name)
         return names
 
-    module_names = bound_in(tree) | set(dir(builtins))
+    module_names = set(dir(builtins))
+    for stmt in tree.body:        # module level only: what a function binds is not visible to its neighbours
+        if isinstance(stmt, (ast.FunctionDef, ast.AsyncFunctionDef, ast.ClassDef)):
+            module_names.add(stmt.name)
+        else:
+            module_names |= bound_in(stmt)
     missing = []
     for fn in [n for n in tree.body if isinstance(n, (ast.FunctionDef, ast.AsyncFunctionDef))]:
         local = bound_in(fn)      # nested functions included: a superset of what any inner scope can see

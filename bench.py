@@ -73,7 +73,7 @@ def stats(samples):
             "min": round(min(samples), 5), "n": len(samples)}
 
 
-def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False, balanced_routing=False):
+def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False, balanced_routing=False, options=None):
     """Runs one workload; returns (result dict, layer, device operands, output tensor, routing tensors)."""
     import torch
     import cuplayground_amd as moe
@@ -81,7 +81,7 @@ def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False, balanced_
 
     w = wl.WORKLOADS[name]
     c = w.config
-    layer = moe.MoELayer(c, ffn_mode=ffn_mode)
+    layer = moe.MoELayer(c, ffn_mode=ffn_mode, options=options)
     dev = wl.make_device_inputs(w, seed)
     if balanced_routing:
         wl.balance_routing(c, dev)
@@ -200,6 +200,7 @@ def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False, balanced_
         "stage_ms_median": {k: round(statistics.median(v[-steps:]), 4) for k, v in samples.items()},
         "ffn_mode": layer.ffn_mode, "block_rows": layer.plan["block_rows"],
         "persistent_blocks": layer.arch["persistent_blocks"], "kept_assignments": kept, "tile_tasks": [tasks0, tasks1],
+        "options": layer.options,
         # row blocks the FFN ran against the row blocks its rows would fill (the rest is padding of ragged last blocks)
         "row_blocks": int(sum((int(n) + layer.plan["block_rows"] - 1) // layer.plan["block_rows"] for n in cnt)),
         "row_blocks_full": round(kept / layer.plan["block_rows"], 2),
@@ -448,6 +449,10 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample (0 = skip)")
     ap.add_argument("--extra-cpu-seconds", type=float, default=1.5,
                     help="target CPU time of the baseline sample of each --extra workload (0 = skip)")
+    ap.add_argument("--option", action="append", default=[], metavar="FIELD=VALUE",
+                    help="a tuning option of the handle by its moe_options field name (repeatable), e.g. --option "
+                         "combine=0 --option tail_split=1; applies to every workload measured; without any, handles are "
+                         "created by moe_create (library defaults, MOE355_* environment variables honoured)")
     ap.add_argument("--seed", type=int, default=42)
     ap.add_argument("--balanced-routing", action="store_true",
                     help="experiment: replace the router's inputs so that every expert receives exactly S*k/E rows "
@@ -473,8 +478,14 @@ def main():
     torch.cuda.set_device(0)
     moe.load_library()
     main_w = wl.WORKLOADS[args.workload]
+    options = None
+    if args.option:
+        options = {}
+        for kv in args.option:
+            key, _, val = kv.partition("=")
+            options[key.strip()] = int(val)
     res, layer, dev, out, routing = measure(args.workload, args.steps, args.warmup, args.seed, args.ffn_mode,
-                                            args.calibrate_copy, args.balanced_routing)
+                                            args.calibrate_copy, args.balanced_routing, options)
     arch = layer.arch
     # ceilings measured on this box in this run (the published peaks assume the maximum clock)
     peaks = moe.measured_peaks()
@@ -502,7 +513,7 @@ def main():
         if name not in wl.WORKLOADS:
             print("bench.py: unknown workload %r in --extra" % name, file=sys.stderr)
             sys.exit(2)
-        r, l2, d2, o2, rt2 = measure(name, args.extra_steps, args.warmup, args.seed, args.ffn_mode)
+        r, l2, d2, o2, rt2 = measure(name, args.extra_steps, args.warmup, args.seed, args.ffn_mode, options=options)
         if args.extra_cpu_seconds > 0:      # every workload has its CPU baseline beside it, on a smaller sample
             r["cpu_baseline"], r["cpu_baseline_oracle"], r["parity"] = cpu_leg(name, d2, o2, rt2, args.extra_cpu_seconds,
                                                                                 args.seed)

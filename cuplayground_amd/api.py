@@ -23,7 +23,8 @@ STAGES = ("gate", "route", "ffn", "combine")
 EXPORTS = (
     "moe_config_default", "moe_config_from_json_string", "moe_config_from_json_file", "moe_config_validate",
     "moe_config_tokens", "moe_config_capacity", "moe_create", "moe_destroy", "moe_get_arch", "moe_get_plan", "moe_get_kernel_dtype",
-    "moe_workspace_bytes",
+    "moe_workspace_bytes", "moe_options_default", "moe_options_from_env", "moe_create_with_options",
+    "moe_workspace_bytes_with_options", "moe_get_options", "moe_get_workspace_bytes", "moe_get_stall", "moe_gemm_bias_act_tile",
     "moe_set_ffn_mode", "moe_get_ffn_mode", "moe_forward", "moe_forward_static", "moe_set_spin_limit", "moe_clear_stall", "moe_gate", "moe_router_stats", "moe_route", "moe_gemm_bias_act", "moe_combine",
     "moe_set_stage_timing", "moe_get_stage_ms", "moe_get_stage_samples", "moe_get_task_counts", "moe_get_queue_balance", "moe_task_trace_bytes", "moe_set_task_trace", "moe_get_task_trace", "moe_measure_mfma_tflops",
     "moe_measure_hbm_read_gbs", "moe_quant_block128", "moe_dequant_block128", "moe_backward_scratch_bytes", "moe_transpose", "moe_expert_gemm",
@@ -43,6 +44,31 @@ class _CConfig(C.Structure):
     _fields_ = [("capacity_factor", C.c_double)] + [(n, C.c_int32) for n in (
         "drop_tokens", "expert_top_k", "is_training", "hidden_act", "hidden_size", "intermediate_size", "micro_batch",
         "num_experts", "sequence_len", "torch_dtype", "gate_fn", "norm_topk_prob")]
+
+
+OPTION_FIELDS = ("tile16", "block_rows", "f32_tile", "fp8_tile", "fp8_widen", "queue_groups", "queue_lag", "queue_early",
+                 "row_chunk", "blocks_per_cu", "combine", "gate_kernel", "gate_mfma", "gate_tile", "gate_fused_topk",
+                 "grouped_tile", "tail_split", "fp8_mfma")
+OPT_AUTO = -1
+COMBINE_SEPARATE, COMBINE_ARRIVALS, COMBINE_QUEUE = 0, 1, 2
+
+
+class _COptions(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in OPTION_FIELDS] + [("reserved", C.c_int32 * 8)]
+
+
+def make_options(options: dict | None = None, from_env: bool = False) -> _COptions:
+    """moe_options with every field AUTO, then (from_env) the MOE355_* variables, then `options` (field name -> int)."""
+    L = load_library()
+    o = _COptions()
+    _check(L.moe_options_default(C.byref(o)))
+    if from_env:
+        _check(L.moe_options_from_env(C.byref(o)))
+    for k, v in (options or {}).items():
+        if k not in OPTION_FIELDS:
+            raise KeyError("unknown option %r (known: %s)" % (k, ", ".join(OPTION_FIELDS)))
+        setattr(o, k, int(v))
+    return o
 
 
 class _CArch(C.Structure):
@@ -89,6 +115,15 @@ def load_library():
     L.moe_get_plan.argtypes = [vp, C.POINTER(i32), C.POINTER(i32), C.POINTER(i32)]
     L.moe_get_kernel_dtype.argtypes = [vp, C.POINTER(i32)]
     L.moe_workspace_bytes.argtypes = [cfgp, C.POINTER(C.c_size_t)]
+    optp = C.POINTER(_COptions)
+    L.moe_options_default.argtypes = [optp]
+    L.moe_options_from_env.argtypes = [optp]
+    L.moe_create_with_options.argtypes = [cfgp, optp, C.POINTER(vp)]
+    L.moe_workspace_bytes_with_options.argtypes = [cfgp, optp, C.POINTER(C.c_size_t)]
+    L.moe_get_options.argtypes = [vp, optp]
+    L.moe_get_workspace_bytes.argtypes = [vp, C.POINTER(C.c_size_t)]
+    L.moe_get_stall.argtypes = [vp, C.POINTER(i32)]
+    L.moe_gemm_bias_act_tile.argtypes = [vp, vp, vp, vp, i64, i64, i64, i32, i32, i32, vp]
     L.moe_set_ffn_mode.argtypes = [vp, C.c_int]
     L.moe_get_ffn_mode.argtypes = [vp, C.POINTER(C.c_int32)]
     L.moe_forward.argtypes = [vp, vp, C.POINTER(_CWeights), vp, C.POINTER(_CRouting), vp, C.c_size_t, vp]
@@ -219,14 +254,23 @@ class MoELayer:
     WEIGHT_KEYS = ("gate_w", "gate_bias", "w_up", "w_gate", "w_down", "b_up", "b_gate", "b_down", "s_up", "s_gate",
                    "s_down")
 
-    def __init__(self, cfg: MoEConfig, ffn_mode: int = FFN_AUTO, allocate_workspace: bool = True):
+    def __init__(self, cfg: MoEConfig, ffn_mode: int = FFN_AUTO, allocate_workspace: bool = True,
+                 options: dict | None = None):
+        """options: tuning options by field name of moe_options (e.g. {"tile16": 1, "combine": 2}); None creates the
+        handle with moe_create, i.e. library defaults overridden by MOE355_* environment variables."""
         import torch
         self.cfg = cfg
         self.L = load_library()
         self._h = C.c_void_p()
         c = cfg.to_c()
-        _check(self.L.moe_create(C.byref(c), C.byref(self._h)), "moe_create")
-        self.workspace_bytes = cfg.workspace_bytes()
+        if options is None:
+            _check(self.L.moe_create(C.byref(c), C.byref(self._h)), "moe_create")
+        else:
+            o = make_options(options)
+            _check(self.L.moe_create_with_options(C.byref(c), C.byref(o), C.byref(self._h)), "moe_create_with_options")
+        n = C.c_size_t(0)
+        _check(self.L.moe_get_workspace_bytes(self._h, C.byref(n)), "moe_get_workspace_bytes")
+        self.workspace_bytes = n.value
         # allocate_workspace=False: for callers that only use forward(static_workspace=True)
         self.workspace = (torch.empty(self.workspace_bytes, dtype=torch.uint8, device="cuda")
                           if allocate_workspace else None)
@@ -268,6 +312,19 @@ class MoELayer:
         _check(self.L.moe_get_kernel_dtype(self._h, C.byref(d)))
         return d.value
 
+    @property
+    def options(self) -> dict:
+        """The options in force, every AUTO the library could resolve at creation replaced by its choice."""
+        o = _COptions()
+        _check(self.L.moe_get_options(self._h, C.byref(o)))
+        return {n: getattr(o, n) for n in OPTION_FIELDS}
+
+    @property
+    def stalled(self) -> bool:
+        v = C.c_int32(0)
+        _check(self.L.moe_get_stall(self._h, C.byref(v)))
+        return bool(v.value)
+
     def set_ffn_mode(self, mode: int):
         _check(self.L.moe_set_ffn_mode(self._h, mode))
 
@@ -304,6 +361,8 @@ class MoELayer:
         return out
 
     def task_counts(self):
+        """(up-projection tasks, down-projection tasks) of the last forward; without a workspace of its own the layer
+        reads the library's static array (the last forward(static_workspace=True))."""
         a, b = C.c_int64(0), C.c_int64(0)
         _check(self.L.moe_get_task_counts(self._h, _ptr(self.workspace), _stream(), C.byref(a), C.byref(b)))
         return a.value, b.value
@@ -535,15 +594,16 @@ def dequantize_block128(q, s):
     return out
 
 
-def gemm_bias_act(A, B, bias, act: int):
-    """C = act(A.B^T + bias): the reference tile GEMM contract (mma.cuh:46-179) on dense operands."""
+def gemm_bias_act(A, B, bias, act: int, tile: int = OPT_AUTO):
+    """C = act(A.B^T + bias): the reference tile GEMM contract (mma.cuh:46-179) on dense operands.
+    tile: OPT_AUTO, or the tile of moe_gemm_bias_act_tile."""
     import torch
     M, K = A.shape
     N = B.shape[0]
     dtype = {torch.float32: DTYPE_F32, torch.bfloat16: DTYPE_BF16, torch.float16: DTYPE_FP16}[A.dtype]
     Cm = torch.empty(M, N, dtype=A.dtype, device=A.device)
-    _check(load_library().moe_gemm_bias_act(_ptr(A), _ptr(B), _ptr(bias), _ptr(Cm), M, N, K, dtype, act, _stream()),
-           "moe_gemm_bias_act")
+    _check(load_library().moe_gemm_bias_act_tile(_ptr(A), _ptr(B), _ptr(bias), _ptr(Cm), M, N, K, dtype, act, tile,
+                                                 _stream()), "moe_gemm_bias_act_tile")
     return Cm
 
 

@@ -15,17 +15,17 @@
 namespace moe355 {
 
 // per-dtype pieces defined next to their kernels
-int bf16_tile(int64_t pairs, int experts, int H, int I, int swiglu);
+int bf16_tile(int64_t pairs, int experts, int H, int I, int swiglu, int opt_block_rows, int opt_tile);
 int bf16_block_m(int tile);
 int bf16_block_n0(int tile);
 int bf16_block_n1(int tile);
 int f32_block_m();
 int f32_block_n();
 hipError_t launch_ffn_tiled_bf16(const FfnArgs&, int tile, int max_mtiles, int nnt0, int nnt1, hipStream_t, bool f16);
-hipError_t launch_ffn_persistent_bf16(const FfnArgs&, int tile, int blocks, hipStream_t, bool f16);
+hipError_t launch_ffn_persistent_bf16(const FfnArgs&, int tile, int blocks, bool early, hipStream_t, bool f16);
 int ffn_persistent_occupancy_bf16(int tile);
 hipError_t launch_gemm_dense_bf16(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t, int,
-                                  hipStream_t, bool f16);
+                                  int opt_tile, hipStream_t, bool f16);
 hipError_t launch_ffn_tiled_f32(const FfnArgs&, int max_mtiles, int nnt0, int nnt1, hipStream_t);
 hipError_t launch_ffn_persistent_f32(const FfnArgs&, int blocks, hipStream_t);
 hipError_t launch_gemm_dense_f32(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t, int,
@@ -87,7 +87,7 @@ int check_supported(const moe_config& c) {
     return MOE_OK;
 }
 
-int derive(const moe_config& c, Derived* d) {
+int derive(const moe_config& c, const moe_options& o, Derived* d) {
     int rc = moe_config_validate(&c, nullptr, 0);
     if (rc) return rc;
     rc = check_supported(c);
@@ -102,7 +102,7 @@ int derive(const moe_config& c, Derived* d) {
     d->act_bytes = d->act_dtype == MOE_DTYPE_F32 ? 4 : 2;
     moe_config_capacity(&c, &d->capacity);
     if (d->capacity > d->A) d->capacity = d->A;
-    d->plan = ffn_plan(c.torch_dtype, c.hidden_act, d->H, d->I, d->A, d->E);
+    d->plan = ffn_plan(c.torch_dtype, c.hidden_act, d->H, d->I, d->A, d->E, o);
     d->wide_mats = c.hidden_act == MOE_ACT_SWIGLU ? 3 : 2;
     d->nblk = ceil_div(d->A, kRouteBlock);
     d->max_mtiles = ceil_div(d->A, d->plan.block_m) + d->E;
@@ -143,7 +143,7 @@ WsLayout layout(const Derived& d) {
 
 }  // namespace
 
-FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E) {
+FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E, const moe_options& o) {
     FfnPlan p;
     p.tile = 0;
     p.kernel_dtype = dtype;
@@ -153,10 +153,7 @@ FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E) {
         // With this many rows per expert one more pass over the weights (e4m3 -> bf16 into the workspace) costs less
         // than the e4m3 tile GEMM loses to the bf16 one.
         p.widen = A / (E > 0 ? E : 1) >= kFp8WidenRowsPerExpert;
-        if (const char* env = getenv("MOE355_FP8_WIDEN")) {   // tuning knob
-            const int v = atoi(env);
-            if (v == 0 || v == 1) p.widen = v;
-        }
+        if (o.fp8_widen != MOE_OPT_AUTO) p.widen = o.fp8_widen != 0;
         if (p.widen) p.kernel_dtype = dtype = MOE_DTYPE_BF16;
     }
     if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32) {
@@ -165,10 +162,7 @@ FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E) {
         // below that the smaller tiles of the vector kernel spread the same work over more of the chip)
         const int64_t tiles = (A / f32_tile_block_m()) * (ceil_div(I, f32_tile_block_n0(sw)) + ceil_div(H, f32_tile_block_n1()));
         p.tile = H % 128 == 0 && I % 128 == 0 && A / (E > 0 ? E : 1) >= kF32TileRowsPerExpert && tiles >= kF32TileMinTiles ? 1 : 0;
-        if (const char* env = getenv("MOE355_F32_TILE")) {   // tuning knob
-            const int v = atoi(env);
-            if (v == 0 || (v == 1 && H % 128 == 0 && I % 128 == 0)) p.tile = v;
-        }
+        if (o.f32_tile == 0 || (o.f32_tile == 1 && H % 128 == 0 && I % 128 == 0)) p.tile = o.f32_tile;
         if (p.tile) {
             p.block_m = f32_tile_block_m();
             p.nnt0 = ceil_div(I, f32_tile_block_n0(sw));
@@ -182,15 +176,12 @@ FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E) {
         // 0: weight streamer over 16-token row blocks (decode); 1: 128 x 128 tile GEMM once the experts see enough
         // rows for a weight tile to be reused from LDS instead of being fetched again per 16 rows
         p.tile = A / (E > 0 ? E : 1) >= kFp8TileRowsPerExpert ? 1 : 0;
-        if (const char* env = getenv("MOE355_FP8_TILE")) {   // tuning knob
-            const int v = atoi(env);
-            if (v == 0 || v == 1) p.tile = v;
-        }
+        if (o.fp8_tile != MOE_OPT_AUTO) p.tile = o.fp8_tile;
         p.block_m = p.tile ? fp8_tile_block_m() : fp8_block_m();
         p.nnt0 = ceil_div(I, p.tile ? fp8_tile_block_n0(sw) : fp8_block_n0(sw));
         p.nnt1 = ceil_div(H, p.tile ? fp8_tile_block_n1() : fp8_block_n1());
     } else {
-        p.tile = bf16_tile(A, E, H, I, sw);
+        p.tile = bf16_tile(A, E, H, I, sw, o.block_rows, o.tile16);
         p.block_m = bf16_block_m(p.tile);
         p.nnt0 = sw ? ceil_div(I, bf16_block_n0(p.tile) / 2) : ceil_div(I, bf16_block_n0(p.tile));
         p.nnt1 = ceil_div(H, bf16_block_n1(p.tile));
@@ -210,12 +201,14 @@ struct moe_handle {
     Derived d;
     WsLayout ws;
     moe_arch arch;
+    moe_options opt;       // the options in force, every AUTO resolved (moe_get_options)
     int ffn_mode;
     int queue_groups;      // task queues of the FFN stage: one per XCD, or 1
+    int queue_lag;         // experts of up-projection work between an expert's two projections in the queue
     int row_chunk;         // task order inside a queue segment (FfnArgs::row_chunk)
     int64_t* task_trace;   // the caller's device buffer for per-task records of the queue kernel, or null
     int task_trace_cap;    // records it holds
-    bool fused_combine;    // the FFN kernels combine a token when its last expert row arrives (no combine launch)
+    int combine_mode;      // 0: a launch of its own, 1: arrival counters inside the FFN kernels, 2: tasks of the FFN queue
     int wall_clock_khz;    // rate of the constant clock the queue kernels stamp their entry and exit with
     int spin_limit;        // polls a dependency wait of the queue kernel makes before it gives up
     int32_t* stall_host;   // pinned host word the queue kernel sets when such a wait expired (never cleared by a kernel)
@@ -283,7 +276,7 @@ RouteArgs route_args(const moe_handle* h, void* ws) {
     a.seg_queue = at<Segment>(ws, w.segq);
     a.q = at<QueueState>(ws, w.qstate);
     a.done0 = at<int32_t>(ws, w.done0);
-    a.arrive = h->fused_combine ? at<int32_t>(ws, w.arrive) : nullptr;
+    a.arrive = h->combine_mode == 1 ? at<int32_t>(ws, w.arrive) : nullptr;
     a.task_trace = h->task_trace;
     a.S = d.S; a.k = d.k; a.E = d.E; a.A = d.A; a.nblk = d.nblk;
     a.drop = h->cfg.drop_tokens;
@@ -292,17 +285,7 @@ RouteArgs route_args(const moe_handle* h, void* ws) {
     a.nnt0 = d.plan.nnt0;
     a.nnt1 = d.plan.nnt1;
     a.max_mtiles = d.max_mtiles;
-    // phase-0 tasks an average expert contributes; enough experts of them to cover four tasks per workgroup
-    const int64_t avg_mt = d.A / ((int64_t)d.E * d.plan.block_m) > 0 ? d.A / ((int64_t)d.E * d.plan.block_m) : 1;
-    const int64_t per_expert = avg_mt * d.plan.nnt0;
-    int64_t lag = (4 * (int64_t)h->arch.persistent_blocks + per_expert - 1) / per_expert;
-    if (lag < 1) lag = 1;
-    if (const char* env = getenv("MOE355_QUEUE_LAG")) {   // tuning knob: experts of phase-0 work between phases
-        const int v = atoi(env);
-        if (v >= 1) lag = v;
-    }
-    if (lag > d.E) lag = d.E;
-    a.lag = (int)lag;
+    a.lag = h->queue_lag;
     a.groups = h->queue_groups;
     return a;
 }
@@ -334,20 +317,107 @@ int resolved_ffn_mode(const moe_handle* h) {
 
 extern "C" {
 
-int moe_workspace_bytes(const moe_config* cfg, size_t* bytes) {
-    if (!cfg || !bytes) return MOE_ERR_BAD_ARGUMENT;
+// ---- options ----
+namespace {
+struct OptField {
+    const char* name;            // field name; the environment variable is MOE355_ + upper case
+    int32_t moe_options::*ptr;
+    int lo, hi;                  // domain (besides MOE_OPT_AUTO)
+    bool pow2;                   // only powers of two
+};
+const OptField kOptFields[] = {
+    {"tile16", &moe_options::tile16, 0, 3, false},
+    {"block_rows", &moe_options::block_rows, 128, 256, true},
+    {"f32_tile", &moe_options::f32_tile, 0, 1, false},
+    {"fp8_tile", &moe_options::fp8_tile, 0, 1, false},
+    {"fp8_widen", &moe_options::fp8_widen, 0, 1, false},
+    {"queue_groups", &moe_options::queue_groups, 1, kMaxQueueGroups, true},
+    {"queue_lag", &moe_options::queue_lag, 1, kMaxExperts, false},
+    {"queue_early", &moe_options::queue_early, 0, 1, false},
+    {"row_chunk", &moe_options::row_chunk, 0, 4096, false},
+    {"blocks_per_cu", &moe_options::blocks_per_cu, 1, 16, false},
+    {"combine", &moe_options::combine, 0, 2, false},
+    {"gate_kernel", &moe_options::gate_kernel, 0, 1, false},
+    {"gate_mfma", &moe_options::gate_mfma, 0, 1, false},
+    {"gate_tile", &moe_options::gate_tile, 0, 2, false},
+    {"gate_fused_topk", &moe_options::gate_fused_topk, 0, 1, false},
+    {"grouped_tile", &moe_options::grouped_tile, 0, 2, false},
+    {"tail_split", &moe_options::tail_split, 1, 4, true},
+    {"fp8_mfma", &moe_options::fp8_mfma, 0, 1, false},
+};
+bool opt_in_domain(const OptField& f, int v) {
+    if (v == MOE_OPT_AUTO) return true;
+    if (v < f.lo || v > f.hi) return false;
+    return !f.pow2 || (v & (v - 1)) == 0;
+}
+int check_options(const moe_options& o) {
+    for (const OptField& f : kOptFields)
+        if (!opt_in_domain(f, o.*(f.ptr))) return MOE_ERR_BAD_ARGUMENT;
+    for (int32_t r : o.reserved)
+        if (r != MOE_OPT_AUTO) return MOE_ERR_BAD_ARGUMENT;
+    return MOE_OK;
+}
+// The options of the entry points that take none: defaults, then the environment.
+moe_options ambient_options() {
+    moe_options o;
+    moe_options_default(&o);
+    moe_options_from_env(&o);
+    return o;
+}
+}  // namespace
+
+int moe_options_default(moe_options* opt) {
+    if (!opt) return MOE_ERR_BAD_ARGUMENT;
+    for (const OptField& f : kOptFields) opt->*(f.ptr) = MOE_OPT_AUTO;
+    for (int32_t& r : opt->reserved) r = MOE_OPT_AUTO;
+    return MOE_OK;
+}
+
+int moe_options_from_env(moe_options* opt) {
+    if (!opt) return MOE_ERR_BAD_ARGUMENT;
+    for (const OptField& f : kOptFields) {
+        char var[64] = "MOE355_";
+        size_t n = strlen(var);
+        for (const char* c = f.name; *c && n + 1 < sizeof var; ++c) var[n++] = (char)(*c >= 'a' && *c <= 'z' ? *c - 32 : *c);
+        var[n] = 0;
+        const char* env = getenv(var);
+        if (!env || !*env) continue;
+        char* endp = nullptr;
+        const long v = strtol(env, &endp, 10);
+        if (endp == env || *endp) continue;                       // not a number: ignored
+        if (v >= INT32_MIN && v <= INT32_MAX && opt_in_domain(f, (int)v)) opt->*(f.ptr) = (int32_t)v;
+    }
+    return MOE_OK;
+}
+
+int moe_workspace_bytes_with_options(const moe_config* cfg, const moe_options* opt, size_t* bytes) {
+    if (!cfg || !bytes || !opt) return MOE_ERR_BAD_ARGUMENT;
+    int rc = check_options(*opt);
+    if (rc) return rc;
     Derived d;
-    const int rc = derive(*cfg, &d);
+    rc = derive(*cfg, *opt, &d);
     if (rc) return rc;
     *bytes = layout(d).total;
     return MOE_OK;
 }
 
+int moe_workspace_bytes(const moe_config* cfg, size_t* bytes) {
+    const moe_options o = ambient_options();
+    return moe_workspace_bytes_with_options(cfg, &o, bytes);
+}
+
 int moe_create(const moe_config* cfg, moe_handle** out) {
-    if (!cfg || !out) return MOE_ERR_BAD_ARGUMENT;
+    const moe_options o = ambient_options();
+    return moe_create_with_options(cfg, &o, out);
+}
+
+int moe_create_with_options(const moe_config* cfg, const moe_options* opt, moe_handle** out) {
+    if (!cfg || !out || !opt) return MOE_ERR_BAD_ARGUMENT;
     *out = nullptr;
+    int rc = check_options(*opt);
+    if (rc) return rc;
     Derived d;
-    int rc = derive(*cfg, &d);
+    rc = derive(*cfg, *opt, &d);
     if (rc) return rc;
     int ndev = 0;
     if (hipGetDeviceCount(&ndev) != hipSuccess || ndev < 1) return MOE_ERR_NO_DEVICE;
@@ -361,15 +431,8 @@ int moe_create(const moe_config* cfg, moe_handle** out) {
     h->cfg = *cfg;
     h->d = d;
     h->ws = layout(d);
+    h->opt = *opt;
     h->ffn_mode = MOE_FFN_AUTO;
-    {   // opt-in: 1 = the FFN kernels combine a token when its last expert row is stored, no combine launch.
-        // Bit-identical and measured slower on every shape (Mixtral shape +2.9 % per step, 16 experts of 512 rows
-        // +14 %, 64 small experts +18 %, decode +0.9 %): the workgroup that completes a token holds a whole compute
-        // unit while it gathers k rows at memory latency, where the separate launch does the same gather with the
-        // whole chip's occupancy in 8-38 us.
-        const char* env = getenv("MOE355_FUSED_COMBINE");
-        h->fused_combine = env && atoi(env) == 1;
-    }
     h->timing = 0;
     h->ev_valid = false;
     h->ev_calls = 0;
@@ -392,31 +455,36 @@ int moe_create(const moe_config* cfg, moe_handle** out) {
         h->wall_clock_khz = 100000;   // 100 MHz on gfx950
     snprintf(h->arch.name, sizeof h->arch.name, "%s", prop.gcnArchName);
     const int kdt = d.plan.kernel_dtype;
+    const bool tile16 = kdt == MOE_DTYPE_BF16 || kdt == MOE_DTYPE_FP16;
     int per_cu = ffn_persistent_blocks(kdt, d.plan.tile, 1);
-    if (const char* env = getenv("MOE355_BLOCKS_PER_CU")) {   // tuning knob: resident workgroups per CU
-        const int v = atoi(env);
-        if (v >= 1 && v <= 16) per_cu = v;
-    }
+    if (opt->blocks_per_cu != MOE_OPT_AUTO) per_cu = opt->blocks_per_cu;    // resident workgroups per CU
     h->arch.persistent_blocks = prop.multiProcessorCount * per_cu;
     // One task queue per XCD for the MFMA-bound bf16 tiles, whose operand tiles are then shared in that XCD's L2;
     // so does the e4m3 tile GEMM; the fp32 kernels (the matrix-core tile measured 5 % faster on one queue than on eight)
     // and the e4m3 weight streamer keep a single queue.
-    h->queue_groups = (kdt == MOE_DTYPE_BF16 || kdt == MOE_DTYPE_FP16 ||
-                       (kdt == MOE_DTYPE_FP8_E4M3_B128 && d.plan.tile)) ? h->arch.xcds : 1;
-    if (const char* env = getenv("MOE355_QUEUE_GROUPS")) {   // tuning knob; never more queues than XCDs
-        const int v = atoi(env);
-        if ((v == 1 || v == 2 || v == 4 || v == 8) && v <= h->arch.xcds) h->queue_groups = v;
-    }
+    h->queue_groups = (tile16 || (kdt == MOE_DTYPE_FP8_E4M3_B128 && d.plan.tile)) ? h->arch.xcds : 1;
+    if (opt->queue_groups != MOE_OPT_AUTO && opt->queue_groups <= h->arch.xcds) h->queue_groups = opt->queue_groups;   // never more queues than XCDs
     if (h->queue_groups > h->arch.persistent_blocks) h->queue_groups = 1;   // every queue needs a home workgroup
     // The e4m3 tile GEMM holds 64 workgroups per XCD on 128 x 128 tiles whose token rows (bf16) take twice the L2 space
     // of their weight rows (e4m3): two row blocks at a time, all of a queue's column tiles of those (measured on the
     // Mixtral shape with e4m3 weights: 6.57 ms against 6.96 with all row blocks of the expert at a time; 1: 6.62,
     // 4: 6.76, 8: 6.89).  The bf16 tiles are indifferent (within 1 %) and keep the plain order.
     h->row_chunk = (kdt == MOE_DTYPE_FP8_E4M3_B128 && d.plan.tile) ? 2 : 0;
-    if (const char* env = getenv("MOE355_ROW_CHUNK")) {   // tuning knob
-        const int v = atoi(env);
-        if (v >= 0 && v <= 4096) h->row_chunk = v;
+    if (opt->row_chunk != MOE_OPT_AUTO) h->row_chunk = opt->row_chunk;
+    {   // phase-0 tasks an average expert contributes; enough experts of them to cover four tasks per workgroup
+        const int64_t avg_mt = d.A / ((int64_t)d.E * d.plan.block_m) > 0 ? d.A / ((int64_t)d.E * d.plan.block_m) : 1;
+        const int64_t per_expert = avg_mt * d.plan.nnt0;
+        int64_t lag = (4 * (int64_t)h->arch.persistent_blocks + per_expert - 1) / per_expert;
+        if (lag < 1) lag = 1;
+        if (opt->queue_lag != MOE_OPT_AUTO) lag = opt->queue_lag;
+        if (lag > d.E) lag = d.E;
+        h->queue_lag = (int)lag;
     }
+    // Combine: a launch of its own unless asked otherwise.  Inside the FFN kernels by arrival counters it is bit-identical
+    // and measured slower on every shape (Mixtral shape +2.9 % per step, 16 experts of 512 rows +14 %, 64 small experts
+    // +18 %, decode +0.9 %): the workgroup that completes a token holds a whole compute unit while it gathers k rows
+    // at memory latency, where the separate launch does the same gather with the whole chip's occupancy in 8-38 us.
+    h->combine_mode = opt->combine == MOE_OPT_AUTO ? 0 : opt->combine;
     h->spin_limit = kDefaultSpinLimit;
     h->task_trace = nullptr;
     h->task_trace_cap = 0;
@@ -428,8 +496,32 @@ int moe_create(const moe_config* cfg, moe_handle** out) {
         h->stall_host = static_cast<int32_t*>(p);
         *h->stall_host = 0;
     }
+    // what moe_get_options reports: the values in force
+    h->opt.tile16 = tile16 ? d.plan.tile : MOE_OPT_AUTO;
+    h->opt.block_rows = tile16 ? d.plan.block_m : MOE_OPT_AUTO;
+    h->opt.f32_tile = (kdt == MOE_DTYPE_F32 || kdt == MOE_DTYPE_TF32) ? d.plan.tile : MOE_OPT_AUTO;
+    h->opt.fp8_tile = kdt == MOE_DTYPE_FP8_E4M3_B128 ? d.plan.tile : MOE_OPT_AUTO;
+    h->opt.fp8_widen = cfg->torch_dtype == MOE_DTYPE_FP8_E4M3_B128 ? (int)d.plan.widen : MOE_OPT_AUTO;
+    h->opt.queue_groups = h->queue_groups;
+    h->opt.queue_lag = h->queue_lag;
+    h->opt.queue_early = opt->queue_early == 1 && tile16 && d.plan.tile == 1 ? 1 : 0;
+    h->opt.row_chunk = h->row_chunk;
+    h->opt.blocks_per_cu = per_cu;
+    h->opt.combine = h->combine_mode;
     resolve_static_scratch(dev);
     *out = h;
+    return MOE_OK;
+}
+
+int moe_get_options(const moe_handle* h, moe_options* opt) {
+    if (!h || !opt) return MOE_ERR_BAD_ARGUMENT;
+    *opt = h->opt;
+    return MOE_OK;
+}
+
+int moe_get_workspace_bytes(const moe_handle* h, size_t* bytes) {
+    if (!h || !bytes) return MOE_ERR_BAD_ARGUMENT;
+    *bytes = h->ws.total;
     return MOE_OK;
 }
 
@@ -536,7 +628,7 @@ int moe_gate(moe_handle* h, const void* x, const void* gate_w, const float* gate
     hipStream_t st = (hipStream_t)stream;
     const Derived& d = h->d;
     float* lg = logits ? logits : at<float>(workspace, h->ws.logits);
-    hipError_t e = launch_gate_logits(x, gate_w, gate_bias, lg, d.S, d.H, d.E, d.act_dtype, st);
+    hipError_t e = launch_gate_logits(x, gate_w, gate_bias, lg, d.S, d.H, d.E, d.act_dtype, h->opt, st);
     if (e != hipSuccess) return hip_fail(h, e);
     e = launch_topk(lg, d.S, d.E, d.k, h->cfg.gate_fn, h->cfg.norm_topk_prob, topk_idx, topk_w, st);
     if (e != hipSuccess) return hip_fail(h, e);
@@ -593,6 +685,10 @@ int forward_on(moe_handle* h, const void* x, const moe_weights* w, void* out, co
     if (!h || !x || !w || !out) return MOE_ERR_BAD_ARGUMENT;
     // a dependency wait of an earlier call expired: that call's output was poisoned; say so until the caller clears it
     if (*(volatile int32_t*)h->stall_host) return MOE_ERR_QUEUE_STALL;
+    {   // the handle's grid size, queue count and (static) workspace belong to the device it was created on
+        int dev = -1;
+        if (hipGetDevice(&dev) != hipSuccess || dev != h->arch.device) return MOE_ERR_BAD_ARGUMENT;
+    }
     const moe_config& c = h->cfg;
     const bool sw = c.hidden_act == MOE_ACT_SWIGLU;
     const bool fp8 = c.torch_dtype == MOE_DTYPE_FP8_E4M3_B128;
@@ -616,7 +712,7 @@ int forward_on(moe_handle* h, const void* x, const moe_weights* w, void* out, co
     float* logits = at<float>(workspace, L.logits);
     int32_t* topk_idx = at<int32_t>(workspace, L.topk_idx);
     float* topk_w = at<float>(workspace, L.topk_w);
-    e = launch_gate_logits(x, w->gate_w, w->gate_bias, logits, d.S, d.H, d.E, d.act_dtype, st);
+    e = launch_gate_logits(x, w->gate_w, w->gate_bias, logits, d.S, d.H, d.E, d.act_dtype, h->opt, st);
     if (e != hipSuccess) return hip_fail(h, e);
     e = launch_topk(logits, d.S, d.E, d.k, c.gate_fn, c.norm_topk_prob, topk_idx, topk_w, st);
     if (e != hipSuccess) return hip_fail(h, e);
@@ -681,7 +777,7 @@ int forward_on(moe_handle* h, const void* x, const moe_weights* w, void* out, co
         e = (d.plan.tile ? launch_ffn_fp8_tile : launch_ffn_fp8)(fa, d.max_mtiles, d.plan.nnt0, d.plan.nnt1,
                                                                  mode == MOE_FFN_PERSISTENT ? h->arch.persistent_blocks : 0, st);
     } else if (mode == MOE_FFN_PERSISTENT) {
-        e = launch_ffn_persistent(fa, kdt, d.plan, h->arch.persistent_blocks, st);
+        e = launch_ffn_persistent(fa, kdt, d.plan, h->arch.persistent_blocks, h->opt.queue_early == 1, st);
     } else {
         e = launch_ffn_tiled(fa, kdt, d.plan, d.max_mtiles, st);
     }
@@ -745,29 +841,51 @@ int moe_clear_stall(moe_handle* h) {
     return MOE_OK;
 }
 
+int moe_get_stall(const moe_handle* h, int32_t* stalled) {
+    if (!h || !stalled) return MOE_ERR_BAD_ARGUMENT;
+    *stalled = *(volatile int32_t*)h->stall_host != 0;
+    return MOE_OK;
+}
+
+namespace {
+// The workspace a getter reads: the caller's, or (null) this device's static array, as moe_forward_static used it.
+const char* getter_workspace(const moe_handle* h, const void* workspace) {
+    if (workspace) return static_cast<const char*>(workspace);
+    const int dev = h->arch.device;
+    if (dev < 0 || dev >= kMaxDevices || !g_scratch_done[dev]) return nullptr;
+    return static_cast<const char*>(g_scratch_ptr[dev]);
+}
+}  // namespace
+
 int moe_get_task_counts(moe_handle* h, const void* workspace, void* stream, int64_t* gemm0_tasks,
                         int64_t* gemm1_tasks) {
-    if (!h || !workspace) return MOE_ERR_BAD_ARGUMENT;
+    if (!h) return MOE_ERR_BAD_ARGUMENT;
+    const char* ws = getter_workspace(h, workspace);
+    if (!ws) return MOE_ERR_WORKSPACE;
     QueueState q;
     hipStream_t st = (hipStream_t)stream;
-    hipError_t e = hipMemcpyAsync(&q, static_cast<const char*>(workspace) + h->ws.qstate, sizeof q,
+    hipError_t e = hipMemcpyAsync(&q, ws + h->ws.qstate, sizeof q,
                                   hipMemcpyDeviceToHost, st);
     if (e != hipSuccess) return hip_fail(h, e);
     e = hipStreamSynchronize(st);
     if (e != hipSuccess) return hip_fail(h, e);
     if (gemm0_tasks) *gemm0_tasks = q.tasks_phase0;
     if (gemm1_tasks) *gemm1_tasks = q.tasks_phase1;
-    return (q.stall || *(volatile int32_t*)h->stall_host) ? MOE_ERR_QUEUE_STALL : MOE_OK;
+    // the handle's word is the one that is sticky and that moe_clear_stall clears; the workspace word only says what the
+    // last call on that workspace did
+    return *(volatile int32_t*)h->stall_host ? MOE_ERR_QUEUE_STALL : MOE_OK;
 }
 
 int moe_get_queue_balance(moe_handle* h, const void* workspace, void* stream, int32_t* workgroups, float* span_us,
                           float* mean_active_us, float* mean_tail_idle_us) {
-    if (!h || !workspace) return MOE_ERR_BAD_ARGUMENT;
+    if (!h) return MOE_ERR_BAD_ARGUMENT;
+    const char* ws = getter_workspace(h, workspace);
+    if (!ws) return MOE_ERR_WORKSPACE;
     if (resolved_ffn_mode(h) != MOE_FFN_PERSISTENT) return MOE_ERR_UNSUPPORTED;
     const int n = std::min(h->arch.persistent_blocks, kMaxQueueWorkgroups);
     std::vector<int64_t> t((size_t)2 * n);
     hipStream_t st = (hipStream_t)stream;
-    hipError_t e = hipMemcpyAsync(t.data(), static_cast<const char*>(workspace) + h->ws.wg_clock, t.size() * 8,
+    hipError_t e = hipMemcpyAsync(t.data(), ws + h->ws.wg_clock, t.size() * 8,
                                   hipMemcpyDeviceToHost, st);
     if (e != hipSuccess) return hip_fail(h, e);
     e = hipStreamSynchronize(st);
@@ -841,28 +959,36 @@ int moe_get_task_trace(moe_handle* h, void* stream, moe_task_record* out, int64_
     return MOE_OK;
 }
 
-int moe_gemm_bias_act(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N, int64_t K,
-                      int32_t dtype, int32_t act, void* stream) {
+int moe_gemm_bias_act_tile(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N, int64_t K,
+                           int32_t dtype, int32_t act, int32_t tile, void* stream) {
     if (!A || !B || !C || M < 1 || N < 1 || K < 1) return MOE_ERR_BAD_ARGUMENT;
     if (act != MOE_ACT_RELU && act != MOE_ACT_GELU && act != MOE_ACT_NONE) return MOE_ERR_BAD_ARGUMENT;
+    if (tile != MOE_OPT_AUTO && (tile < 0 || tile > 2)) return MOE_ERR_BAD_ARGUMENT;
     if (M > INT32_MAX / 2 || N > INT32_MAX / 2 || K > INT32_MAX / 2) return MOE_ERR_UNSUPPORTED;
     hipError_t e;
     if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32) {
-        if (K % 16 || N % 2) return MOE_ERR_UNSUPPORTED;
-        e = launch_gemm_bias_act(A, B, bias, C, M, N, K, dtype, act, (hipStream_t)stream);
+        if (K % 16 || N % 2 || tile == 2) return MOE_ERR_UNSUPPORTED;
+        e = launch_gemm_bias_act(A, B, bias, C, M, N, K, dtype, act, tile, (hipStream_t)stream);
     } else if (dtype == MOE_DTYPE_BF16 || dtype == MOE_DTYPE_FP16) {
         if (K % 64 || N % 4) return MOE_ERR_UNSUPPORTED;
-        e = launch_gemm_dense_bf16(A, B, bias, C, M, N, K, act, (hipStream_t)stream, dtype == MOE_DTYPE_FP16);
+        e = launch_gemm_dense_bf16(A, B, bias, C, M, N, K, act, tile, (hipStream_t)stream, dtype == MOE_DTYPE_FP16);
     } else {
         return MOE_ERR_UNSUPPORTED;
     }
     return e == hipSuccess ? MOE_OK : MOE_ERR_HIP;
 }
 
+int moe_gemm_bias_act(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N, int64_t K,
+                      int32_t dtype, int32_t act, void* stream) {
+    return moe_gemm_bias_act_tile(A, B, bias, C, M, N, K, dtype, act, MOE_OPT_AUTO, stream);
+}
+
 int moe_backward_scratch_bytes(const moe_config* cfg, size_t* bytes) {
     if (!cfg || !bytes) return MOE_ERR_BAD_ARGUMENT;
     Derived d;
-    const int rc = derive(*cfg, &d);
+    moe_options o;
+    moe_options_default(&o);                    // the scratch depends on the shape only
+    const int rc = derive(*cfg, o, &d);
     if (rc) return rc;
     if (cfg->torch_dtype == MOE_DTYPE_FP8_E4M3_B128) return MOE_ERR_UNSUPPORTED;
     *bytes = backward_scratch_bytes(d.A, d.E, d.H, d.I, (int)d.act_bytes);
@@ -896,7 +1022,7 @@ int moe_expert_gemm(moe_handle* h, const void* a_rows, const void* w, const void
     const int rc = check_backward_call(h, N, K, scratch, scratch_bytes);
     if (rc) return rc;
     const hipError_t e = launch_expert_gemm(a_rows, w, bias, expert_count, expert_offset, h->d.A, h->d.E, N, K, act,
-                                            h->d.act_dtype, out_rows, scratch, (hipStream_t)stream);
+                                            h->d.act_dtype, h->opt, out_rows, scratch, (hipStream_t)stream);
     return e == hipSuccess ? MOE_OK : hip_fail(h, e);
 }
 
@@ -907,7 +1033,7 @@ int moe_expert_wgrad(moe_handle* h, const void* dy_rows, const void* a_rows, con
     const int rc = check_backward_call(h, N, K, scratch, scratch_bytes);
     if (rc) return rc;
     const hipError_t e = launch_expert_wgrad(dy_rows, a_rows, expert_count, expert_offset, h->d.A, h->d.E, N, K,
-                                             h->d.act_dtype, dw, scratch, (hipStream_t)stream);
+                                             h->d.act_dtype, h->opt, dw, scratch, (hipStream_t)stream);
     return e == hipSuccess ? MOE_OK : hip_fail(h, e);
 }
 
@@ -968,10 +1094,10 @@ hipError_t launch_ffn_tiled(const FfnArgs& a, int dtype, const FfnPlan& p, int m
     return launch_ffn_tiled_bf16(a, p.tile, max_mtiles, p.nnt0, p.nnt1, st, dtype == MOE_DTYPE_FP16);
 }
 
-hipError_t launch_ffn_persistent(const FfnArgs& a, int dtype, const FfnPlan& p, int blocks, hipStream_t st) {
+hipError_t launch_ffn_persistent(const FfnArgs& a, int dtype, const FfnPlan& p, int blocks, bool early, hipStream_t st) {
     if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32)
         return p.tile ? launch_ffn_f32_tile(a, 0, p.nnt0, p.nnt1, blocks, st) : launch_ffn_persistent_f32(a, blocks, st);
-    return launch_ffn_persistent_bf16(a, p.tile, blocks, st, dtype == MOE_DTYPE_FP16);
+    return launch_ffn_persistent_bf16(a, p.tile, blocks, early, st, dtype == MOE_DTYPE_FP16);
 }
 
 int ffn_persistent_blocks(int dtype, int tile, int compute_units) {
@@ -983,16 +1109,14 @@ int ffn_persistent_blocks(int dtype, int tile, int compute_units) {
 }
 
 hipError_t launch_gemm_bias_act(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N,
-                                int64_t K, int dtype, int act, hipStream_t st) {
+                                int64_t K, int dtype, int act, int opt_tile, hipStream_t st) {
     if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32) {
         bool tile = gemm_dense_f32_takes_tile(M, N, K);
-        if (const char* env = getenv("MOE355_F32_TILE")) {   // tuning knob: 0 keeps the vector-ALU kernel
-            if (atoi(env) == 0) tile = false;
-        }
+        if (opt_tile == 0) tile = false;     // asked to keep the vector-ALU kernel
         return tile ? launch_gemm_dense_f32_tile(A, B, bias, C, M, N, K, act, st)
                     : launch_gemm_dense_f32(A, B, bias, C, M, N, K, act, st);
     }
-    return launch_gemm_dense_bf16(A, B, bias, C, M, N, K, act, st, dtype == MOE_DTYPE_FP16);
+    return launch_gemm_dense_bf16(A, B, bias, C, M, N, K, act, opt_tile, st, dtype == MOE_DTYPE_FP16);
 }
 
 }  // namespace moe355

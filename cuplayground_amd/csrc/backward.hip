@@ -337,14 +337,12 @@ ScratchTables scratch_tables(void* scratch, int64_t A, int E) {
 // out_rows[r,:] = act(a_rows[r,:] . w[e(r)]^T + bias[e(r)]); scratch holds the row-block table.
 // dtype: the storage type of every operand (MOE_DTYPE_F32, _BF16 or _FP16).
 hipError_t launch_expert_gemm(const void* a_rows, const void* w, const void* bias, const int32_t* count,
-                              const int32_t* offset, int64_t A, int E, int N, int K, int act, int dtype, void* out_rows,
-                              void* scratch, hipStream_t st) {
+                              const int32_t* offset, int64_t A, int E, int N, int K, int act, int dtype,
+                              const moe_options& opt, void* out_rows, void* scratch, hipStream_t st) {
     const ScratchTables t = scratch_tables(scratch, A, E);
     if (dtype == MOE_DTYPE_F32) {
         bool mfma = grouped_gemm_f32_takes_tile(A, N, K);
-        if (const char* env = getenv("MOE355_F32_TILE")) {   // tuning knob: 0 keeps the vector-ALU kernel
-            if (atoi(env) == 0) mfma = false;
-        }
+        if (opt.f32_tile == 0) mfma = false;   // option: keep the vector-ALU kernel
         const int block_m = mfma ? 128 : 64;
         const int max_mtiles = (int)(A / block_m + E);
         backward_tables_kernel<<<1, kMaxExperts, 0, st>>>(count, offset, E, block_m, t.mtiles, t.num_mtiles, nullptr);
@@ -354,8 +352,8 @@ hipError_t launch_expert_gemm(const void* a_rows, const void* w, const void* bia
                                                                                t.num_mtiles, max_mtiles, N, K, act, st);
     }
     int tile = grouped_gemm_takes_large_tile(A, E, N, K) ? 1 : 0;     // 1: 256 x 256, 0: 128 x 128
-    if (const char* env = getenv("MOE355_GROUPED_TILE")) {             // tuning knob; 2: 128 x 256 (hand-ordered)
-        const int v = atoi(env);
+    if (opt.grouped_tile != MOE_OPT_AUTO) {                            // option; 2: 128 x 256 (hand-ordered)
+        const int v = opt.grouped_tile;
         const int64_t lim = (int64_t)1 << 32;
         if ((v == 1 || v == 2) && N % 256 == 0 && K % 128 == 0 && A * K * 2 < lim && (int64_t)N * K * 2 < lim) tile = v;
         if (v == 0) tile = 0;
@@ -371,7 +369,8 @@ hipError_t launch_expert_gemm(const void* a_rows, const void* w, const void* bia
 
 // dw[e] [N,K] = dy_e^T . a_e; scratch holds the window offsets and the two transposed operands.
 hipError_t launch_expert_wgrad(const void* dy_rows, const void* a_rows, const int32_t* count, const int32_t* offset,
-                               int64_t A, int E, int N, int K, int dtype, void* dw, void* scratch, hipStream_t st) {
+                               int64_t A, int E, int N, int K, int dtype, const moe_options& opt, void* dw, void* scratch,
+                               hipStream_t st) {
     const ScratchTables t = scratch_tables(scratch, A, E);
     const int64_t ld = wgrad_ld(A, E);
     const size_t eb = dtype == MOE_DTYPE_F32 ? 4 : 2;
@@ -385,9 +384,7 @@ hipError_t launch_expert_wgrad(const void* dy_rows, const void* a_rows, const in
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
         bool mfma = wgrad_f32_takes_tile(E, N, K);
-        if (const char* env = getenv("MOE355_F32_TILE")) {   // tuning knob: 0 keeps the vector-ALU kernel
-            if (atoi(env) == 0) mfma = false;
-        }
+        if (opt.f32_tile == 0) mfma = false;   // option: keep the vector-ALU kernel
         return (mfma ? launch_wgrad_f32_tile : launch_wgrad_f32)(dyT, aT, dw, t.poff, E, N, K, ld, st);
     }
     transpose_rows_padded_kernel<<<g1, 256, 0, st>>>((const uint16_t*)dy_rows, N, count, offset, t.poff, E, ld, (uint16_t*)dyT);

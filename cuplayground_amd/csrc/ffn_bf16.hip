@@ -17,7 +17,6 @@
 // slab loop ordered by hand (gemm_tile_ring) and an epilogue staged through LDS; chosen when experts see many rows
 // and every tile of the layer meets that loop's conditions (large_tile_ok).  "Small": 128 x 128 tiles, four
 // wavefronts of 64 x 64, compiler-scheduled loop (mainloop_generic), general epilogue; takes everything else.
-#include <cstdlib>
 #include <type_traits>
 
 #include "ffn_common.hpp"
@@ -1214,12 +1213,11 @@ hipError_t launch_tiled(const FfnArgs& a, int max_mtiles, int nnt0, int nnt1, hi
 }
 
 template <class P>
-hipError_t launch_persistent(const FfnArgs& a, int blocks, hipStream_t st) {
+hipError_t launch_persistent(const FfnArgs& a, int blocks, bool early, hipStream_t st) {
     if constexpr (P::T0::RING && !P::MIXED) {
-        // tuning knob: 1 = the queue loop that starts the next task under the end of the current one (measured: no
+        // option queue_early: the queue loop that starts the next task under the end of the current one (measured: no
         // faster on the Mixtral shape, 2-3 % slower on short tiles; kept for machines where the balance differs)
-        const char* env = getenv("MOE355_QUEUE_EARLY");
-        if (env && atoi(env) == 1) {
+        if (early) {
             hipError_t e = allow_lds(&ffn_persistent_ring_kernel<P>, P::LDS_BYTES);
             if (e != hipSuccess) return e;
             ffn_persistent_ring_kernel<P><<<blocks, P::THREADS, P::LDS_BYTES, st>>>(a);
@@ -1268,17 +1266,11 @@ static bool large_tile_ok(int64_t pairs, int H, int I, bool swiglu) {
 // such a task runs through K faster than the full blocks that share its weight tile, drops out of their lockstep
 // and fetches its weights past the L2 on its own, with half the time per slab to hide that latency in (with a
 // routing that leaves no partial blocks both kernels take the same time).
-int bf16_tile(int64_t pairs, int experts, int H, int I, int swiglu) {
+int bf16_tile(int64_t pairs, int experts, int H, int I, int swiglu, int opt_block_rows, int opt_tile) {
     if (!large_tile_ok(pairs, H, I, swiglu != 0)) return 0;
     const int up_columns = swiglu ? 2 * I : I;
-    if (const char* env = getenv("MOE355_BLOCK_ROWS")) {   // tuning knob: force the row-block height ...
-        const int v = atoi(env);
-        if (v == 128 || v == 256) return v == 256 ? 1 : 0;
-    }
-    if (const char* env = getenv("MOE355_TILE")) {         // ... or the tile
-        const int v = atoi(env);
-        if (v >= 0 && v <= 3) return v;
-    }
+    if (opt_block_rows == 128 || opt_block_rows == 256) return opt_block_rows == 256 ? 1 : 0;   // option block_rows ...
+    if (opt_tile >= 0 && opt_tile <= 3) return opt_tile;                                        // ... or tile16
     const int64_t per_expert = pairs / (experts > 0 ? experts : 1);
     if (per_expert < 256) return 0;
     const int64_t tasks = (pairs / 256) * ((up_columns + Tile256::BN - 1) / Tile256::BN);
@@ -1305,7 +1297,7 @@ template <class P> struct RunTiled {
     static hipError_t run(const FfnArgs& a, int max_mtiles, int nnt0, int nnt1, hipStream_t st) { return launch_tiled<P>(a, max_mtiles, nnt0, nnt1, st); }
 };
 template <class P> struct RunPersistent {
-    static hipError_t run(const FfnArgs& a, int blocks, hipStream_t st) { return launch_persistent<P>(a, blocks, st); }
+    static hipError_t run(const FfnArgs& a, int blocks, bool early, hipStream_t st) { return launch_persistent<P>(a, blocks, early, st); }
 };
 template <class P> struct RunOccupancy {
     static int run() { return occupancy<P>(); }
@@ -1316,8 +1308,8 @@ hipError_t launch_ffn_tiled_bf16(const FfnArgs& a, int tile, int max_mtiles, int
     return for_plan<RunTiled>(tile, f16, a, max_mtiles, nnt0, nnt1, st);
 }
 
-hipError_t launch_ffn_persistent_bf16(const FfnArgs& a, int tile, int blocks, hipStream_t st, bool f16) {
-    return for_plan<RunPersistent>(tile, f16, a, blocks, st);
+hipError_t launch_ffn_persistent_bf16(const FfnArgs& a, int tile, int blocks, bool early, hipStream_t st, bool f16) {
+    return for_plan<RunPersistent>(tile, f16, a, blocks, early, st);
 }
 
 int ffn_persistent_occupancy_bf16(int tile) { return for_plan<RunOccupancy>(tile, false); }
@@ -1335,11 +1327,12 @@ static hipError_t launch_dense(const void* A, const void* B, const void* bias, v
 }
 
 hipError_t launch_gemm_dense_bf16(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N,
-                                  int64_t K, int act, hipStream_t st, bool f16) {
+                                  int64_t K, int act, int opt_tile, hipStream_t st, bool f16) {
     const int64_t lim = (int64_t)1 << 32;
     const bool large = M >= 1024 && N >= 1024 && N % 256 == 0 && K % 128 == 0 && M * K * 2 < lim && N * K * 2 < lim;
-    if (const char* env = getenv("MOE355_DENSE_TILE")) {   // tuning knob: 1 = 256 x 256, 2 = 128 x 256 (shapes they accept only)
-        const int v = atoi(env);
+    {   // the tile asked for: 1 = 256 x 256, 2 = 128 x 256 (shapes they accept only), 0 = 128 x 128
+        const int v = opt_tile;
+        if (v == 0) return f16 ? launch_dense<SmallPlanH::T0>(A, B, bias, C, M, N, K, act, st) : launch_dense<SmallPlan::T0>(A, B, bias, C, M, N, K, act, st);
         if ((v == 1 || v == 2) && N % 256 == 0 && K % 128 == 0 && M * K * 2 < lim && N * K * 2 < lim) {
             if (v == 1) return f16 ? launch_dense<Tile256H>(A, B, bias, C, M, N, K, act, st) : launch_dense<Tile256>(A, B, bias, C, M, N, K, act, st);
             return f16 ? launch_dense<Tile128x256H>(A, B, bias, C, M, N, K, act, st) : launch_dense<Tile128x256>(A, B, bias, C, M, N, K, act, st);

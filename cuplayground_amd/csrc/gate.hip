@@ -317,10 +317,10 @@ hipError_t launch_gate_tile(const void* x, const void* gate_w, const float* gate
 // the experts fit one wavefront's tile.
 template <typename T>
 hipError_t launch_gate_tiled(const void* x, const void* gate_w, const float* gate_bias, float* logits, int S, int H,
-                             int E, hipStream_t st) {
+                             int E, int opt_tile, hipStream_t st) {
     const int64_t pairs = (int64_t)S * E;
     int variant = pairs >= 32768 ? 0 : 1;
-    if (const char* env = getenv("MOE355_GATE_TILE")) variant = atoi(env);   // tuning knob
+    if (opt_tile >= 0 && opt_tile <= 2) variant = opt_tile;
     switch (variant) {
         case 0:
             return E <= 8 ? launch_gate_tile<T, 4, 8, 4, 1>(x, gate_w, gate_bias, logits, S, H, E, st)
@@ -431,11 +431,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // most of its 16 columns and there are enough 16 x 16 tiles for every SIMD of the chip to get several.
 template <typename T>
 bool launch_gate_mfma(const void* x, const void* gate_w, const float* gate_bias, float* logits, int S, int H, int E,
-                      hipStream_t st, hipError_t* err) {
+                      int opt_mfma, hipStream_t st, hipError_t* err) {
     if (H % 512 != 0) return false;
     const int et = (E + 15) / 16;
     bool use = et * 16 * 3 <= E * 4 && (int64_t)((S + 15) / 16) * et >= 2048;
-    if (const char* env = getenv("MOE355_GATE_MFMA")) use = atoi(env) != 0;   // tuning knob
+    if (opt_mfma != MOE_OPT_AUTO) use = opt_mfma != 0;
     if (!use) return false;
     const dim3 grid((S + 15) / 16, (et + 1) / 2);
     gate_mfma_kernel<T><<<grid, 256, 0, st>>>((const T*)x, (const T*)gate_w, gate_bias, logits, S, H, E);
@@ -551,25 +551,25 @@ hipError_t launch_router_stats(const float* logits, const int32_t* topk_idx, int
 }
 
 hipError_t launch_gate_logits(const void* x, const void* gate_w, const float* gate_bias, float* logits, int S, int H,
-                              int E, int act_dtype, hipStream_t st) {
+                              int E, int act_dtype, const moe_options& opt, hipStream_t st) {
     // Many experts on many tokens: the first kernel (token rows in registers, experts streamed) reads least per sum.
     // Everything else -- few experts, or decode-sized batches -- goes to the register-tiled kernel.
     if (act_dtype != MOE_DTYPE_F32) {
         hipError_t e = hipSuccess;
-        const bool taken = act_dtype == MOE_DTYPE_FP16 ? launch_gate_mfma<f16_s>(x, gate_w, gate_bias, logits, S, H, E, st, &e)
-                                                       : launch_gate_mfma<bf16_s>(x, gate_w, gate_bias, logits, S, H, E, st, &e);
+        const bool taken = act_dtype == MOE_DTYPE_FP16 ? launch_gate_mfma<f16_s>(x, gate_w, gate_bias, logits, S, H, E, opt.gate_mfma, st, &e)
+                                                       : launch_gate_mfma<bf16_s>(x, gate_w, gate_bias, logits, S, H, E, opt.gate_mfma, st, &e);
         if (taken) return e;
     }
     bool rows_in_registers = E >= 32 && (int64_t)S * E >= ((int64_t)1 << 19);
-    if (const char* env = getenv("MOE355_GATE_KERNEL")) rows_in_registers = atoi(env) == 1;   // tuning knob
+    if (opt.gate_kernel != MOE_OPT_AUTO) rows_in_registers = opt.gate_kernel == 1;
     if (rows_in_registers) {
         if (act_dtype == MOE_DTYPE_F32) return launch_gate_typed<float>(x, gate_w, gate_bias, logits, S, H, E, st);
         if (act_dtype == MOE_DTYPE_FP16) return launch_gate_typed<f16_s>(x, gate_w, gate_bias, logits, S, H, E, st);
         return launch_gate_typed<bf16_s>(x, gate_w, gate_bias, logits, S, H, E, st);
     }
-    if (act_dtype == MOE_DTYPE_F32) return launch_gate_tiled<float>(x, gate_w, gate_bias, logits, S, H, E, st);
-    if (act_dtype == MOE_DTYPE_FP16) return launch_gate_tiled<f16_s>(x, gate_w, gate_bias, logits, S, H, E, st);
-    return launch_gate_tiled<bf16_s>(x, gate_w, gate_bias, logits, S, H, E, st);
+    if (act_dtype == MOE_DTYPE_F32) return launch_gate_tiled<float>(x, gate_w, gate_bias, logits, S, H, E, opt.gate_tile, st);
+    if (act_dtype == MOE_DTYPE_FP16) return launch_gate_tiled<f16_s>(x, gate_w, gate_bias, logits, S, H, E, opt.gate_tile, st);
+    return launch_gate_tiled<bf16_s>(x, gate_w, gate_bias, logits, S, H, E, opt.gate_tile, st);
 }
 
 hipError_t launch_topk(const float* logits, int S, int E, int k, int gate_fn, int norm, int32_t* topk_idx,

@@ -148,8 +148,9 @@ struct RouteArgs {
 };
 
 // ---- launchers (defined next to their kernels) ----
+// gate_kernel / gate_mfma / gate_tile: the handle's options of those names (MOE_OPT_AUTO: chosen from the shape)
 hipError_t launch_gate_logits(const void* x, const void* gate_w, const float* gate_bias, float* logits, int S, int H,
-                              int E, int act_dtype, hipStream_t st);
+                              int E, int act_dtype, const moe_options& opt, hipStream_t st);
 hipError_t launch_topk(const float* logits, int S, int E, int k, int gate_fn, int norm, int32_t* topk_idx,
                        float* topk_w, hipStream_t st);
 constexpr int kStatsBlocks = 64;   // per-block partials of the router statistics kept in the workspace
@@ -169,11 +170,11 @@ struct FfnPlan {
     int nnt0;        // column tiles of phase 0
     int nnt1;        // column tiles of phase 1
 };
-FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E);
+FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E, const moe_options& o);
 hipError_t launch_widen_block128(const void* q, const float* scales, void* out, int64_t matrices, int64_t N, int64_t K,
                                  hipStream_t st);
 hipError_t launch_ffn_tiled(const FfnArgs& a, int dtype, const FfnPlan& p, int max_mtiles, hipStream_t st);
-hipError_t launch_ffn_persistent(const FfnArgs& a, int dtype, const FfnPlan& p, int blocks, hipStream_t st);
+hipError_t launch_ffn_persistent(const FfnArgs& a, int dtype, const FfnPlan& p, int blocks, bool early, hipStream_t st);
 int ffn_persistent_blocks(int dtype, int tile, int compute_units);
 
 // ---- backward building blocks (csrc/backward.hip) ----
@@ -181,10 +182,11 @@ size_t backward_scratch_bytes(int64_t A, int E, int H, int I, int elem_bytes);
 hipError_t launch_transpose(const void* src, void* dst, int64_t batch, int64_t rows, int64_t cols, int elem_bytes,
                             hipStream_t st);
 hipError_t launch_expert_gemm(const void* a_rows, const void* w, const void* bias, const int32_t* count,
-                              const int32_t* offset, int64_t A, int E, int N, int K, int act, int dtype, void* out_rows,
-                              void* scratch, hipStream_t st);
+                              const int32_t* offset, int64_t A, int E, int N, int K, int act, int dtype,
+                              const moe_options& opt, void* out_rows, void* scratch, hipStream_t st);
 hipError_t launch_expert_wgrad(const void* dy_rows, const void* a_rows, const int32_t* count, const int32_t* offset,
-                               int64_t A, int E, int N, int K, int dtype, void* dw, void* scratch, hipStream_t st);
+                               int64_t A, int E, int N, int K, int dtype, const moe_options& opt, void* dw, void* scratch,
+                               hipStream_t st);
 
 hipError_t launch_act_backward(const void* dh, const void* u, const void* g, int64_t n, int act, int dtype, void* du,
                                void* dg, hipStream_t st);
@@ -193,7 +195,8 @@ hipError_t launch_bias_grad(const void* dy, const int32_t* count, const int32_t*
 hipError_t launch_combine_backward(const void* dout, const void* y, const int32_t* pair_row, const float* topk_w, int S,
                                    int k, int H, int dtype, void* dy, float* dw, hipStream_t st);
 
+// tile: MOE_OPT_AUTO, or the tile asked for (moe_gemm_bias_act_tile)
 hipError_t launch_gemm_bias_act(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N,
-                                int64_t K, int dtype, int act, hipStream_t st);
+                                int64_t K, int dtype, int act, int tile, hipStream_t st);
 
 }  // namespace moe355

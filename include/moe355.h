@@ -99,6 +99,66 @@ typedef struct moe_arch {
 
 typedef struct moe_handle moe_handle;
 
+/*
+ * Tuning options of a handle: which tile, which kernel, which schedule -- everything the library would otherwise choose
+ * from the layer's shape.  The reference has one knob surface, the JSON file turned into compile definitions
+ * (CMakeLists.txt:204-216), and chooses tiles and schedulers at compile time (processor/tiling.cuh:97-159,
+ * scheduling.cuh:170-200 against warpScheduler.cuh:167-265); these are the same choices as run-time values of a handle.
+ * Every field is MOE_OPT_AUTO (the library chooses) or one of the values named beside it; a value outside its domain
+ * makes moe_create_with_options return MOE_ERR_BAD_ARGUMENT, a value the layer's shape cannot take (the 256-row tile on
+ * a layer with H % 256 != 0, say) falls back to the library's choice.  Results never depend on these options beyond
+ * what is said here: schedules and tiles of one dtype agree bit for bit except where a field says otherwise.
+ * Options are fixed when the handle is created; two handles of one process may differ in every one of them.
+ */
+#define MOE_OPT_AUTO (-1)
+typedef struct moe_options {
+    int32_t tile16;          /* bf16 / fp16 layers: 0 = 128x128 tile, 1 = 256x256 (hand-ordered), 2 = 128x256 (hand-ordered),
+                                3 = 256x256 with the 128x256 tile for row blocks of at most 128 rows */
+    int32_t block_rows;      /* bf16 / fp16 layers: 128 or 256 rows per row block (a coarser way to say tile16 = 0 / 1) */
+    int32_t f32_tile;        /* fp32 / tf32 layers: 0 = 64x64 vector-ALU tile, 1 = 128x128 matrix-core tile; also read by the
+                                backward entry points of an fp32 handle (there 1 means "where the shape allows") */
+    int32_t fp8_tile;        /* e4m3 layers: 0 = weight streamer (decode), 1 = 128x128 tile GEMM */
+    int32_t fp8_widen;       /* e4m3 layers: 1 = run the bf16 tiles on bf16 copies of the weights (widened into the workspace
+                                by every call, or taken from moe_prepare_weights), 0 = never */
+    int32_t queue_groups;    /* task queues of the FFN stage: 1, 2, 4 or 8 (never more than the device has XCDs) */
+    int32_t queue_lag;       /* experts of up-projection work queued between an expert's two projections, >= 1 */
+    int32_t queue_early;     /* 1 = the queue loop that starts the next task under the current one's epilogue (256x256 tile) */
+    int32_t row_chunk;       /* order of the tasks of one expert and projection: 0 = row blocks fastest, R > 0 = R row
+                                blocks at a time */
+    int32_t blocks_per_cu;   /* resident workgroups per compute unit of the queue kernels, 1..16 */
+    int32_t combine;         /* 0 = a launch of its own behind the FFN stage; 1 = inside the FFN kernels, by the workgroup
+                                whose tile completes a token (arrival counters); 2 = as tasks of the FFN queue, taken by
+                                workgroups that find no GEMM task left (task-queue mode only; the rest of the tokens is
+                                combined by a short launch behind it).  All three give the same bits. */
+    int32_t gate_kernel;     /* logits kernel: 0 = register-tiled, 1 = token rows in registers */
+    int32_t gate_mfma;       /* 1 = the logits on the matrix cores where the shape allows (16-bit layers, H % 512 == 0), 0 = never */
+    int32_t gate_tile;       /* register-tiled logits kernel: 0 = 4x8 pairs per wavefront, 1 = 4x4, 2 = 2x8 */
+    int32_t gate_fused_topk; /* 1 = top-k inside the logits kernel where one exists for the shape (no logits round trip
+                                through memory unless the caller asks for them), 0 = always a launch of its own */
+    int32_t grouped_tile;    /* moe_expert_gemm on a 16-bit handle: 0 = 128x128, 1 = 256x256, 2 = 128x256 */
+    int32_t tail_split;      /* 16-bit layers on the 256x256 tile, task-queue mode: the down-projection tiles of the last
+                                queue segments run as this many partial sums over the intermediate dimension (1 = whole
+                                tiles, 2 or 4).  Changes the order of the fp32 sum of those tiles (within the layer's
+                                tolerance, deterministic); the two-launch mode then splits the same tiles the same way. */
+    int32_t fp8_mfma;        /* e4m3 layers on the tile GEMM: 1 = tokens quantised to e4m3 per (row, 128-wide k block) and
+                                the products taken by the fp8 matrix instructions; 0 = bf16 tokens, weights widened.  Not
+                                bit-compatible with 0: see moe_get_kernel_dtype. */
+    int32_t reserved[8];     /* must be MOE_OPT_AUTO */
+} moe_options;
+/* Every field MOE_OPT_AUTO. */
+int moe_options_default(moe_options* opt);
+/* Overrides the fields of *opt for which a MOE355_<FIELD> environment variable (upper-case field name) is set to a value
+ * of the field's domain.  This is the only place the library reads its environment, and it is never called from
+ * moe_forward or any other per-step entry point: moe_create and moe_workspace_bytes (the entry points without an options
+ * argument) call it once on defaults; moe_create_with_options and moe_workspace_bytes_with_options never do. */
+int moe_options_from_env(moe_options* opt);
+int moe_create_with_options(const moe_config* cfg, const moe_options* opt, moe_handle** out);
+int moe_workspace_bytes_with_options(const moe_config* cfg, const moe_options* opt, size_t* bytes);
+/* The options the handle runs with, every AUTO resolved to the value in force; and the workspace it needs -- the value to
+ * trust when options and environment may have changed between moe_workspace_bytes and moe_create. */
+int moe_get_options(const moe_handle* h, moe_options* opt);
+int moe_get_workspace_bytes(const moe_handle* h, size_t* bytes);
+
 int moe_create(const moe_config* cfg, moe_handle** out);
 int moe_destroy(moe_handle* h);
 int moe_get_arch(const moe_handle* h, moe_arch* out);
@@ -154,9 +214,8 @@ int moe_forward(moe_handle* h, const void* x, const moe_weights* w, void* out, c
  * moe_forward for callers that cannot allocate device memory at all -- code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc: the same layer, same kernels and same results, with the workspace taken
  * from an array that is part of the library's device code (MOE355_STATIC_WORKSPACE_BYTES per GPU, held from the moment
- * the library is loaded until the process ends) instead of from the caller.  It has no counterpart in the reference,
- * whose drivers allocate one arena per run (mma.cuh:385-391).  Calls no hipMalloc / hipFree or any other allocating
- * routine.  Returns MOE_ERR_WORKSPACE when moe_workspace_bytes(config) exceeds the array (decode-sized and small
+ * the library is loaded until the process ends) instead of from the caller.  It has no counterpart in the reference;
+ * it is for callers that cannot allocate.  Calls no hipMalloc / hipFree or any other allocating routine.  Returns MOE_ERR_WORKSPACE when moe_workspace_bytes(config) exceeds the array (decode-sized and small
  * prefill layers fit; the Mixtral-shape intermediate does not; the bf16 weight copies of an e4m3 layer on the widening
  * plan count, see moe_get_kernel_dtype).  Every call on a GPU uses that GPU's one array: calls
  * that overlap in time on one GPU (two streams, two threads, two handles) race; calls in sequence on one stream are
@@ -190,6 +249,12 @@ int moe_route(moe_handle* h, const int32_t* topk_idx, int32_t* slot, int32_t* ex
  * dtype is MOE_DTYPE_F32 (TF32 is taken as F32), MOE_DTYPE_BF16 or MOE_DTYPE_FP16; act is RELU, GELU or NONE; bias [N] may be NULL. */
 int moe_gemm_bias_act(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N, int64_t K,
                       int32_t dtype, int32_t act, void* stream);
+/* The same with the tile named (the reference fixes its tile at compile time, processor/tiling.cuh:273-323): MOE_OPT_AUTO,
+ * or for bf16 / fp16 0 = 128x128, 1 = 256x256, 2 = 128x256 (1 and 2 need N % 256 == 0 and K % 128 == 0, else the library's
+ * choice runs), for fp32 0 = the vector-ALU tile, 1 = the matrix-core tile where the shape allows.  Same results as
+ * moe_gemm_bias_act to the bit for the 16-bit tiles. */
+int moe_gemm_bias_act_tile(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N, int64_t K,
+                           int32_t dtype, int32_t act, int32_t tile, void* stream);
 
 /* out[t,:] = sum_r w[t,r] * y[pair_row[t,r],:]  (fp32, ascending r, one rounding); pair_row < 0 skipped.
  * With k = 1 and unit weights this is the reference's CombineMode::single row scatter
@@ -215,6 +280,7 @@ int moe_get_stage_samples(moe_handle* h, int stage, float* ms, int32_t capacity,
  * the queue kernel: span_us = first entry to last exit, mean_active_us = mean of (exit - entry), mean_tail_idle_us =
  * mean of (last exit - own exit), i.e. the time a workgroup had nothing left to pop while others still worked.
  * Synchronises `stream`.  No counterpart in the reference, whose scheduler keeps no statistics. */
+/* (Here and in moe_get_task_counts, workspace = NULL means this device's static array, i.e. the last moe_forward_static.) */
 int moe_get_queue_balance(moe_handle* h, const void* workspace, void* stream, int32_t* workgroups, float* span_us,
                           float* mean_active_us, float* mean_tail_idle_us);
 /* Per-task trace of the task-queue FFN kernel: with a trace buffer set, every task of a moe_forward on this handle
@@ -247,11 +313,15 @@ int moe_get_task_counts(moe_handle* h, const void* workspace, void* stream, int6
  * warpScheduler.cuh:339).  When one expires, the kernel does not compute on unfinished rows: it fills the affected
  * output tile with NaN (which the combine carries into the affected rows of `out`), sets the stall word of the
  * workspace and a host-visible word of the handle, and every kernel still exits normally.  From then on moe_forward /
- * moe_forward_static / moe_get_task_counts on that handle return MOE_ERR_QUEUE_STALL (checked on the host, without
- * synchronising) until moe_clear_stall.  moe_set_spin_limit sets the number of polls before a wait gives up
+ * moe_forward_static / moe_get_task_counts on that handle return MOE_ERR_QUEUE_STALL (the handle's word, checked on the
+ * host without synchronising) until moe_clear_stall.  moe_set_spin_limit sets the number of polls before a wait gives up
  * (0 = the default, about 2^24; negative = every wait expires at once, which exercises this path from the host). */
 int moe_set_spin_limit(moe_handle* h, int32_t polls);
 int moe_clear_stall(moe_handle* h);
+/* Whether the handle's stall word is set: one read of host memory, no synchronisation.  A HIP graph that holds a captured
+ * moe_forward runs no host code of this library when it is replayed, so a stall during a replay is reported by nothing
+ * until the next eager call on the handle: callers that replay graphs poll this behind their own synchronisation. */
+int moe_get_stall(const moe_handle* h, int32_t* stalled);
 
 /* Ceilings measured on the current device, to be quoted beside the published peaks: bf16 MFMA issue rate with no
  * memory traffic (scratch: >= 2 MiB of device memory, overwritten; random_operands = 0: all-zero operands, the

@@ -73,14 +73,14 @@ def test_expert_gemm_vs_oracle(moe, case, dtype):
         assert not got[kept:].any()            # rows of no expert are not written (the output started as zeros)
 
 
-def test_fp32_products_on_the_matrix_core_tile_and_on_the_vector_tile(moe, monkeypatch):
+def test_fp32_products_on_the_matrix_core_tile_and_on_the_vector_tile(moe):
     """fp32 layers: the grouped product and the weight gradient of a shape that takes the 128 x 128 matrix-core tile,
-    and the same calls held on the 64 x 64 vector-ALU tile (MOE355_F32_TILE=0).  Both within the fp32 tolerance of the
+    and the same calls held on the 64 x 64 vector-ALU tile (a handle created with the option f32_tile = 0).  Both within the fp32 tolerance of the
     oracle; their sums run in different orders, so the results are not the same bits -- which shows both ran."""
     S, H, I, E, k, cf, skew = CASES[2]
     dtype = ob.F32
     cfg, rng, count, offset = routed_case(S, H, I, E, k, dtype, seed=79, cf=cf, skew=0.3)
-    layer = moe.MoELayer(product_config(cfg))
+    layers = {"0": moe.MoELayer(product_config(cfg), options={"f32_tile": 0}), None: moe.MoELayer(product_config(cfg), options={})}
     a, dy, w, bias = operands(rng, S * k, E, I, H, dtype)
     want = ob.expert_gemm(a, w, bias, count, offset, dtype, ob.ACT_GELU)
     want_dw = ob.expert_wgrad(dy, a, count, offset, dtype)
@@ -88,10 +88,7 @@ def test_fp32_products_on_the_matrix_core_tile_and_on_the_vector_tile(moe, monke
     dev = [to_device(v, "f32") for v in (a, dy, w, bias)] + [to_device(count, "i32"), to_device(offset, "i32")]
     outs, grads = {}, {}
     for knob in ("0", None):
-        if knob is None:
-            monkeypatch.delenv("MOE355_F32_TILE")
-        else:
-            monkeypatch.setenv("MOE355_F32_TILE", knob)
+        layer = layers[knob]
         outs[knob] = from_device(layer.expert_gemm(dev[0], dev[2], dev[3], dev[4], dev[5], ob.ACT_GELU))
         grads[knob] = from_device(layer.expert_wgrad(dev[1], dev[0], dev[4], dev[5]))
         assert max_rel_err(outs[knob][:kept], want[:kept]) <= OUT_TOL[dtype]
@@ -103,19 +100,18 @@ def test_fp32_products_on_the_matrix_core_tile_and_on_the_vector_tile(moe, monke
 
 
 @pytest.mark.parametrize("dtype", [ob.BF16, ob.F16])
-def test_grouped_product_tiles_agree(moe, dtype, monkeypatch):
-    """The 128 x 128, 256 x 256 and 128 x 256 tiles forced on one grouped product (MOE355_GROUPED_TILE): the two
+def test_grouped_product_tiles_agree(moe, dtype):
+    """The 128 x 128, 256 x 256 and 128 x 256 tiles forced on one grouped product (option grouped_tile): the two
     hand-ordered ones accumulate every output element with the same MFMA sequence and must agree bit for bit; the
     compiler-ordered 128 x 128 tile only within the tolerance."""
     S, H, I, E, k, cf, skew = CASES[2]
     cfg, rng, count, offset = routed_case(S, H, I, E, k, dtype, seed=77, cf=cf, skew=0.3)
-    layer = moe.MoELayer(product_config(cfg))
     kind = KIND[dtype]
     a, _, w, bias = operands(rng, S * k, E, I, H, dtype)
     want = ob.to_f32(ob.expert_gemm(a, w, bias, count, offset, dtype, ob.ACT_GELU), dtype)
     outs = {}
     for tile in ("0", "1", "2"):
-        monkeypatch.setenv("MOE355_GROUPED_TILE", tile)
+        layer = moe.MoELayer(product_config(cfg), options={"grouped_tile": int(tile)})
         got = layer.expert_gemm(to_device(a, kind), to_device(w, kind), to_device(bias, kind), to_device(count, "i32"),
                                 to_device(offset, "i32"), ob.ACT_GELU)
         outs[tile] = from_device(got)

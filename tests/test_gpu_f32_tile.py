@@ -24,12 +24,11 @@ SHAPES = {
 }
 
 
-def _run(cfg, inp, mode, tile, monkeypatch, calls=1):
+def _run(cfg, inp, mode, tile, calls=1, combine=0):
     import torch
     import cuplayground_amd as moe
     assert torch.cuda.is_available(), "these tests need the MI355X"
-    monkeypatch.setenv("MOE355_F32_TILE", str(tile))
-    layer = moe.MoELayer(product_config(cfg), ffn_mode=mode)
+    layer = moe.MoELayer(product_config(cfg), ffn_mode=mode, options={"f32_tile": tile, "combine": combine})
     assert layer.plan["block_rows"] == (128 if tile else 64)
     dev = upload_inputs(cfg, inp)
     routing = layer.new_routing()
@@ -46,39 +45,38 @@ def _run(cfg, inp, mode, tile, monkeypatch, calls=1):
 
 @pytest.mark.parametrize("mode", [FFN_TILED, FFN_PERSISTENT], ids=["tiled", "persistent"])
 @pytest.mark.parametrize("name", sorted(SHAPES))
-def test_tile_vs_oracle_and_vector_kernel(name, mode, monkeypatch):
+def test_tile_vs_oracle_and_vector_kernel(name, mode):
     cfg = SHAPES[name]
     inp = ob.make_inputs(cfg, seed=23, with_bias="bias" in name)
     want = ob.forward(cfg, inp)
     ref = ob.to_f32(want["out"], cfg.act_dtype)
-    got = _run(cfg, inp, mode, 1, monkeypatch, calls=2)
+    got = _run(cfg, inp, mode, 1, calls=2)
     check_routing(got, want)
     assert not np.isnan(got["out"]).any()
     assert max_rel_err(got["out"], ref) <= OUT_TOL[ob.F32]
     assert not got["out"][(want["slot"] < 0).all(axis=1)].any()
-    vec = _run(cfg, inp, mode, 0, monkeypatch)      # the same fp32 sums in another order
+    vec = _run(cfg, inp, mode, 0)      # the same fp32 sums in another order
     assert max_rel_err(got["out"], vec["out"]) <= OUT_TOL[ob.F32]
 
 
 @pytest.mark.parametrize("name", sorted(SHAPES))
-def test_tile_schedules_agree_bit_for_bit(name, monkeypatch):
+def test_tile_schedules_agree_bit_for_bit(name):
     cfg = SHAPES[name]
     inp = ob.make_inputs(cfg, seed=31, with_bias="bias" in name)
-    a = _run(cfg, inp, FFN_TILED, 1, monkeypatch)
-    b = _run(cfg, inp, FFN_PERSISTENT, 1, monkeypatch)
+    a = _run(cfg, inp, FFN_TILED, 1)
+    b = _run(cfg, inp, FFN_PERSISTENT, 1)
     assert np.array_equal(a["out"], b["out"])
-    monkeypatch.setenv("MOE355_FUSED_COMBINE", "1")
-    c = _run(cfg, inp, FFN_PERSISTENT, 1, monkeypatch)
-    assert np.array_equal(a["out"], c["out"])
+    for combine in (1, 2):      # inside the FFN kernels: by arrival counters, as tasks of the queue
+        c = _run(cfg, inp, FFN_PERSISTENT, 1, combine=combine)
+        assert np.array_equal(a["out"], c["out"]), combine
 
 
-def test_plan_follows_rows_per_expert_and_shape(monkeypatch):
+def test_plan_follows_rows_per_expert_and_shape():
     import cuplayground_amd as moe
-    monkeypatch.delenv("MOE355_F32_TILE", raising=False)
-    small = moe.MoELayer(product_config(ob.BASELINE["C1"]))                # 16 rows per expert
-    few_tiles = moe.MoELayer(product_config(ob.Cfg(S=1024, H=256, I=512, E=8, k=1, act=ob.ACT_GELU, dtype=ob.F32)))
-    ragged = moe.MoELayer(product_config(ob.Cfg(S=8192, H=960, I=4096, E=1, k=1, act=ob.ACT_RELU, dtype=ob.F32)))
-    big = moe.MoELayer(product_config(ob.Cfg(S=8192, H=1024, I=4096, E=1, k=1, act=ob.ACT_RELU, dtype=ob.F32)))
+    small = moe.MoELayer(product_config(ob.BASELINE["C1"]), options={})                # 16 rows per expert
+    few_tiles = moe.MoELayer(product_config(ob.Cfg(S=1024, H=256, I=512, E=8, k=1, act=ob.ACT_GELU, dtype=ob.F32)), options={})
+    ragged = moe.MoELayer(product_config(ob.Cfg(S=8192, H=960, I=4096, E=1, k=1, act=ob.ACT_RELU, dtype=ob.F32)), options={})
+    big = moe.MoELayer(product_config(ob.Cfg(S=8192, H=1024, I=4096, E=1, k=1, act=ob.ACT_RELU, dtype=ob.F32)), options={})
     assert [l.plan["block_rows"] for l in (small, few_tiles, ragged, big)] == [64, 64, 64, 128]
     assert big.plan["col_tiles_up"] == 4096 // 128 and big.plan["col_tiles_down"] == 1024 // 128
     for l in (small, few_tiles, ragged, big):

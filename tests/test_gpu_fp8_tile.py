@@ -30,13 +30,12 @@ SHAPES = {
 }
 
 
-def _run(cfg, inp, mode, tile, monkeypatch, calls=1):
+def _run(cfg, inp, mode, tile, calls=1, combine=0):
     import torch
     import cuplayground_amd as moe
     assert torch.cuda.is_available(), "these tests need the MI355X"
-    monkeypatch.setenv("MOE355_FP8_TILE", str(tile))
-    monkeypatch.setenv("MOE355_FP8_WIDEN", "0")
-    layer = moe.MoELayer(product_config(cfg), ffn_mode=mode)
+    layer = moe.MoELayer(product_config(cfg), ffn_mode=mode,
+                         options={"fp8_tile": tile, "fp8_widen": 0, "fp8_mfma": 0, "combine": combine})
     assert layer.plan["block_rows"] == (128 if tile else 16)
     dev = upload_inputs(cfg, inp)
     routing = layer.new_routing()
@@ -53,44 +52,44 @@ def _run(cfg, inp, mode, tile, monkeypatch, calls=1):
 
 @pytest.mark.parametrize("mode", [FFN_TILED, FFN_PERSISTENT], ids=["tiled", "persistent"])
 @pytest.mark.parametrize("name", sorted(SHAPES))
-def test_tile_gemm_vs_oracle_and_streamer(name, mode, monkeypatch):
+def test_tile_gemm_vs_oracle_and_streamer(name, mode):
     cfg = SHAPES[name]
     inp = ob.make_inputs(cfg, seed=29, with_bias="bias" in name)
     want = ob.forward(cfg, inp)
     ref = ob.to_f32(want["out"], cfg.act_dtype)
-    got = _run(cfg, inp, mode, 1, monkeypatch, calls=2)
+    got = _run(cfg, inp, mode, 1, calls=2)
     check_routing(got, want)
     assert not np.isnan(got["out"]).any()
     assert max_rel_err(got["out"], ref) <= OUT_TOL[ob.FP8]
     assert not got["out"][(want["slot"] < 0).all(axis=1)].any()
     # the streamer computes the same block-scaled sums in another order: both round h and y to bf16 once
-    stream = _run(cfg, inp, mode, 0, monkeypatch)
+    stream = _run(cfg, inp, mode, 0)
     assert max_rel_err(got["out"], stream["out"]) <= 1e-2
 
 
 @pytest.mark.parametrize("name", sorted(SHAPES))
-def test_tile_gemm_schedules_agree_bit_for_bit(name, monkeypatch):
+def test_tile_gemm_schedules_agree_bit_for_bit(name):
     cfg = SHAPES[name]
     inp = ob.make_inputs(cfg, seed=31, with_bias="bias" in name)
-    a = _run(cfg, inp, FFN_TILED, 1, monkeypatch)
-    b = _run(cfg, inp, FFN_PERSISTENT, 1, monkeypatch)
+    a = _run(cfg, inp, FFN_TILED, 1)
+    b = _run(cfg, inp, FFN_PERSISTENT, 1)
     assert np.array_equal(a["out"], b["out"])
-    monkeypatch.setenv("MOE355_FUSED_COMBINE", "1")
-    c = _run(cfg, inp, FFN_PERSISTENT, 1, monkeypatch)
-    assert np.array_equal(a["out"], c["out"])
+    for combine in (1, 2):      # inside the FFN kernels: by arrival counters, as tasks of the queue
+        c = _run(cfg, inp, FFN_PERSISTENT, 1, combine=combine)
+        assert np.array_equal(a["out"], c["out"]), combine
 
 
 def test_plan_follows_rows_per_expert():
     """Decode-sized layers keep the weight streamer, prefill-sized ones take the tile."""
     import cuplayground_amd as moe
-    small = moe.MoELayer(product_config(ob.Cfg(S=64, H=256, I=256, E=32, k=8, act=ob.ACT_SWIGLU, dtype=ob.FP8)))
-    big = moe.MoELayer(product_config(ob.Cfg(S=2048, H=256, I=256, E=8, k=2, act=ob.ACT_SWIGLU, dtype=ob.FP8)))
+    small = moe.MoELayer(product_config(ob.Cfg(S=64, H=256, I=256, E=32, k=8, act=ob.ACT_SWIGLU, dtype=ob.FP8)), options={})
+    big = moe.MoELayer(product_config(ob.Cfg(S=2048, H=256, I=256, E=8, k=2, act=ob.ACT_SWIGLU, dtype=ob.FP8)), options={})
     assert small.plan["block_rows"] == 16 and big.plan["block_rows"] == 128
     assert big.plan["col_tiles_up"] == 256 // 64 and big.plan["col_tiles_down"] == 256 // 128
     small.close(); big.close()
 
 
-def test_prefill_sized_layer_on_a_stratified_sample(monkeypatch):
+def test_prefill_sized_layer_on_a_stratified_sample():
     """A layer big enough to fill the queue kernel several times over (8 experts of about 1024 rows, 72 row blocks x
     104 column tiles): routing in full, the output on each expert's first row, tail block and block boundaries plus
     random tokens, and the two schedules bit for bit."""
@@ -98,10 +97,10 @@ def test_prefill_sized_layer_on_a_stratified_sample(monkeypatch):
     import cuplayground_amd as moe
     from test_gpu_fullsize import stratified_tokens
     cfg = ob.Cfg(S=4096, H=2048, I=5632, E=8, k=2, act=ob.ACT_SWIGLU, dtype=ob.FP8, gate_fn=ob.GATE_SOFTMAX, drop=0)
-    monkeypatch.setenv("MOE355_FP8_WIDEN", "0")   # this many rows per expert would run the bf16 tile on widened weights
     inp = ob.make_inputs(cfg, seed=42)
     want = ob.route(cfg, inp)
-    layer = moe.MoELayer(product_config(cfg), ffn_mode=FFN_PERSISTENT)
+    # fp8_widen 0: this many rows per expert would run the bf16 tile on widened weights
+    layer = moe.MoELayer(product_config(cfg), ffn_mode=FFN_PERSISTENT, options={"fp8_widen": 0, "fp8_mfma": 0})
     assert layer.plan["block_rows"] == 128
     dev = upload_inputs(cfg, inp)
     routing = layer.new_routing()

@@ -19,12 +19,11 @@ SHAPES = {
 }
 
 
-def _forward(cfg, dev, mode, monkeypatch, widen):
+def _forward(cfg, dev, mode, widen):
     import torch
     import cuplayground_amd as moe
-    if widen is not None:
-        monkeypatch.setenv("MOE355_FP8_WIDEN", str(widen))
-    layer = moe.MoELayer(product_config(cfg), ffn_mode=mode)
+    layer = moe.MoELayer(product_config(cfg), ffn_mode=mode,
+                         options={} if widen is None else {"fp8_widen": widen, "fp8_mfma": 0})
     routing = layer.new_routing()
     out = torch.full((cfg.S, cfg.H), float("nan"), dtype=layer.act_dtype, device="cuda")
     for _ in range(2):   # the workspace copy of the weights is rewritten by every call
@@ -55,18 +54,18 @@ def test_widening_is_the_oracle_decode_rounded_once():
 
 @pytest.mark.parametrize("mode", [FFN_TILED, FFN_PERSISTENT], ids=["tiled", "persistent"])
 @pytest.mark.parametrize("name", sorted(SHAPES))
-def test_widened_layer(name, mode, monkeypatch):
+def test_widened_layer(name, mode):
     import cuplayground_amd as moe
     cfg = SHAPES[name]
     inp = ob.make_inputs(cfg, seed=37, with_bias="bias" in name)
     want = ob.forward(cfg, inp)
     dev = upload_inputs(cfg, inp)
-    got = _forward(cfg, dev, mode, monkeypatch, 1)
+    got = _forward(cfg, dev, mode, 1)
     check_routing(got, want)
     assert max_rel_err(got["out"], ob.to_f32(want["out"], cfg.act_dtype)) <= OUT_TOL[ob.FP8]
     assert not got["out"][(want["slot"] < 0).all(axis=1)].any()
     # the e4m3 tile GEMM scales fp32 partial sums instead of rounding scaled weights to bf16
-    tile = _forward(cfg, dev, mode, monkeypatch, 0)
+    tile = _forward(cfg, dev, mode, 0)
     assert max_rel_err(got["out"], tile["out"]) <= 1e-2
     assert got["workspace_bytes"] - tile["workspace_bytes"] >= (3 if cfg.act == ob.ACT_SWIGLU else 2) * cfg.E * cfg.H * cfg.I * 2
     # a bf16 layer handed the widened weights computes exactly the same thing
@@ -75,15 +74,14 @@ def test_widened_layer(name, mode, monkeypatch):
         if "w_" + n in dev:
             wide["w_" + n] = moe.dequantize_block128(dev["w_" + n], dev["s_" + n])
             del wide["s_" + n]
-    bf = _forward(cfg.scaled(dtype=ob.BF16), wide, mode, monkeypatch, None)
+    bf = _forward(cfg.scaled(dtype=ob.BF16), wide, mode, None)
     assert np.array_equal(got["bits"], bf["bits"])
 
 
-def test_plan_widens_from_a_thousand_rows_per_expert(monkeypatch):
+def test_plan_widens_from_a_thousand_rows_per_expert():
     import cuplayground_amd as moe
-    monkeypatch.delenv("MOE355_FP8_WIDEN", raising=False)
-    mid = moe.MoELayer(product_config(ob.Cfg(S=1024, H=256, I=256, E=4, k=2, act=ob.ACT_SWIGLU, dtype=ob.FP8)))
-    big = moe.MoELayer(product_config(ob.Cfg(S=2048, H=256, I=256, E=4, k=2, act=ob.ACT_SWIGLU, dtype=ob.FP8)))
+    mid = moe.MoELayer(product_config(ob.Cfg(S=1024, H=256, I=256, E=4, k=2, act=ob.ACT_SWIGLU, dtype=ob.FP8)), options={})
+    big = moe.MoELayer(product_config(ob.Cfg(S=2048, H=256, I=256, E=4, k=2, act=ob.ACT_SWIGLU, dtype=ob.FP8)), options={})
     assert mid.plan["block_rows"] == 128
     # the workspace grows by the bf16 copies of the three weight matrices, not only by the rows of twice the tokens
     rows = 2 * (2048 - 1024) * (256 + 256) * 2

@@ -47,7 +47,7 @@ def stratified_tokens(cfg, want, block_rows, seed=7):
 
 
 @pytest.mark.parametrize("name", ["C2", "C3", "C4", "C5", "R0", "X1"])
-def test_baseline_config_full_size(name, monkeypatch):
+def test_baseline_config_full_size(name):
     import torch
     import cuplayground_amd as moe
     assert torch.cuda.is_available()
@@ -101,14 +101,13 @@ def test_baseline_config_full_size(name, monkeypatch):
     out2 = layer.forward(dev["x"], dev)
     assert torch.equal(out, out2)
     # and so must the queue loop with the early start of the next task (an opt-in schedule of the 256-row tile)
-    layer.set_ffn_mode(FFN_PERSISTENT)
-    monkeypatch.setenv("MOE355_QUEUE_EARLY", "1")
-    out3 = layer.forward(dev["x"], dev)
-    torch.cuda.synchronize()
-    monkeypatch.delenv("MOE355_QUEUE_EARLY")
-    layer.task_counts()
-    assert torch.equal(out, out3)
     layer.close()
+    early = moe.MoELayer(product_config(cfg), ffn_mode=FFN_PERSISTENT, options={"queue_early": 1})
+    out3 = early.forward(dev["x"], dev)
+    torch.cuda.synchronize()
+    early.task_counts()
+    assert torch.equal(out, out3)
+    early.close()
 
 
 @pytest.mark.parametrize("S,H,I,k,rows", [(100000, 256, 8192, 2, 256), (140000, 256, 8192, 2, 128), (300000, 4096, 256, 1, 256)],

@@ -23,9 +23,10 @@ def moe():
     return cuplayground_amd
 
 
-def run_layer(moe, cfg, inp, mode):
+def run_layer(moe, cfg, inp, mode, options=None):
+    """options: a dict of moe_options fields; None = the handle moe_create makes (library defaults)."""
     import torch
-    layer = moe.MoELayer(product_config(cfg), ffn_mode=mode)
+    layer = moe.MoELayer(product_config(cfg), ffn_mode=mode, options=options)
     dev = upload_inputs(cfg, inp)
     routing = layer.new_routing()
     out = layer.forward(dev["x"], dev, routing=routing)
@@ -186,18 +187,17 @@ LARGE_TILE = {
 
 
 @pytest.mark.parametrize("name", sorted(LARGE_TILE))
-def test_large_tile_and_queue_groups(moe, name, monkeypatch):
+def test_large_tile_and_queue_groups(moe, name):
     """The 256-row tile forced on small layers, in both FFN modes and with 1, 2 and 8 task queues: every run must
     reproduce the first bit for bit (the schedule only reorders independent tiles) and match the oracle."""
     cfg = LARGE_TILE[name]
     inp = ob.make_inputs(cfg, seed=5, with_bias="bias" in name)
     want = ob.forward(cfg, inp)
-    monkeypatch.setenv("MOE355_BLOCK_ROWS", "256")
     first = None
-    for groups in ("1", "2", "8"):
-        monkeypatch.setenv("MOE355_QUEUE_GROUPS", groups)
+    for groups in (1, 2, 8):
+        opts = {"block_rows": 256, "queue_groups": groups}
         for mode in (FFN_TILED, FFN_PERSISTENT):
-            got = run_layer(moe, cfg, inp, mode)
+            got = run_layer(moe, cfg, inp, mode, opts)
             check_routing(got, want)
             eligible = cfg.H % 256 == 0 and cfg.I % (128 if cfg.act == ob.ACT_SWIGLU else 256) == 0
             assert got["plan"]["block_rows"] == (256 if eligible else 128)     # the cases cover both tiles
@@ -207,9 +207,7 @@ def test_large_tile_and_queue_groups(moe, name, monkeypatch):
             else:
                 assert np.array_equal(got["out"], first), (groups, mode)
         # the queue loop that starts the next task under the end of the current one (same tiles, other timing)
-        monkeypatch.setenv("MOE355_QUEUE_EARLY", "1")
-        got = run_layer(moe, cfg, inp, FFN_PERSISTENT)
-        monkeypatch.delenv("MOE355_QUEUE_EARLY")
+        got = run_layer(moe, cfg, inp, FFN_PERSISTENT, dict(opts, queue_early=1))
         check_routing(got, want)
         assert np.array_equal(got["out"], first), ("early", groups)
 
@@ -217,18 +215,19 @@ def test_large_tile_and_queue_groups(moe, name, monkeypatch):
 @pytest.mark.parametrize("name", ["bf16_gelu_ragged", "bf16_swiglu_skew", "f32_swiglu_ragged", "fp8_many_rows_bias",
                                   "fp16_swiglu_skew_bias", "tf32_gelu_ragged", "capacity_one", "many_experts_bias",
                                   "all_experts_selected", "one_token"])
-def test_combine_inside_the_ffn_kernels_changes_no_bit(moe, name, monkeypatch):
-    """With MOE355_FUSED_COMBINE=1 a token is combined by the FFN workgroup that stores its last expert row; by default
-    the combine is a launch of its own behind the FFN stage.  Same function, same rank order: the outputs must be
-    identical in every bit, in both FFN modes, including the all-zero rows of tokens that lost every pair to the
-    capacity limit, and over repeated calls on one handle (the arrival counters are cleared by every call)."""
+@pytest.mark.parametrize("combine", [1, 2], ids=["arrival_counters", "queue_tasks"])
+def test_combine_inside_the_ffn_kernels_changes_no_bit(moe, name, combine):
+    """Option combine = 1: a token is combined by the FFN workgroup that stores its last expert row; 2: by workgroups of
+    the queue kernel that find no GEMM task left (the rest by a short launch behind it); 0: a launch of its own behind
+    the FFN stage.  Same function, same rank order: the outputs must be identical in every bit, in both FFN modes,
+    including the all-zero rows of tokens that lost every pair to the capacity limit, and over repeated calls on one
+    handle (the counters are cleared by every call)."""
     import torch
     cfg = RAGGED[name]
     inp = ob.make_inputs(cfg, seed=3, with_bias="bias" in name)
-    separate = run_layer(moe, cfg, inp, FFN_TILED)["out"]
-    monkeypatch.setenv("MOE355_FUSED_COMBINE", "1")
+    separate = run_layer(moe, cfg, inp, FFN_TILED, {"combine": 0})["out"]
     for mode in (FFN_TILED, FFN_PERSISTENT):
-        layer = moe.MoELayer(product_config(cfg), ffn_mode=mode)
+        layer = moe.MoELayer(product_config(cfg), ffn_mode=mode, options={"combine": combine})
         dev = upload_inputs(cfg, inp)
         for call in range(3):
             out = torch.full((cfg.S, cfg.H), float("nan"), dtype=layer.act_dtype, device="cuda")   # nothing may be left unwritten
@@ -241,18 +240,17 @@ def test_combine_inside_the_ffn_kernels_changes_no_bit(moe, name, monkeypatch):
 
 @pytest.mark.parametrize("name", sorted(n for n, c in LARGE_TILE.items()
                                         if c.H % 256 == 0 and c.I % (128 if c.act == ob.ACT_SWIGLU else 256) == 0))
-def test_half_height_tile(moe, name, monkeypatch):
-    """The 128 x 256 tile as the tile of the whole layer (MOE355_TILE=2) and as the tile of the short last row blocks
+def test_half_height_tile(moe, name):
+    """The 128 x 256 tile as the tile of the whole layer (option tile16 = 2) and as the tile of the short last row blocks
     only (3): every output element is accumulated by the same MFMA sequence over K as in the 256 x 256 tile, so all
     three must agree bit for bit, in both FFN modes, and match the oracle."""
     cfg = LARGE_TILE[name]
     inp = ob.make_inputs(cfg, seed=5, with_bias="bias" in name)
     want = ob.forward(cfg, inp)
     first = None
-    for tile, rows in (("1", 256), ("2", 128), ("3", 256)):
-        monkeypatch.setenv("MOE355_TILE", tile)
+    for tile, rows in ((1, 256), (2, 128), (3, 256)):
         for mode in (FFN_TILED, FFN_PERSISTENT):
-            got = run_layer(moe, cfg, inp, mode)
+            got = run_layer(moe, cfg, inp, mode, {"tile16": tile})
             check_routing(got, want)
             assert got["plan"]["block_rows"] == rows
             if first is None:
@@ -307,28 +305,26 @@ GRAPH_CASES = {
     "bf16": (None, {}),
     # an e4m3 layer on the widening plan (three more launches per call, the workspace copy rewritten by every replay)
     "e4m3_widened": (ob.Cfg(S=600, H=256, I=384, E=4, k=2, act=ob.ACT_SWIGLU, dtype=ob.FP8, gate_fn=ob.GATE_SIGMOID, drop=0),
-                     {"MOE355_FP8_WIDEN": "1"}),
+                     {"fp8_widen": 1}),
     # an fp32 layer on the matrix-core tile, and a 16-bit one whose logits come from the matrix-core gate kernel
     "f32_tile": (ob.Cfg(S=500, H=256, I=256, E=2, k=1, act=ob.ACT_GELU, dtype=ob.F32, norm_topk=0, drop=0),
-                 {"MOE355_F32_TILE": "1"}),
+                 {"f32_tile": 1}),
     "f16_gate_mfma": (ob.Cfg(S=300, H=512, I=128, E=20, k=3, act=ob.ACT_RELU, dtype=ob.F16, drop=1, capacity_factor=1.0),
-                      {"MOE355_GATE_MFMA": "1"}),
+                      {"gate_mfma": 1}),
 }
 
 
 @pytest.mark.parametrize("mode", [FFN_TILED, FFN_PERSISTENT], ids=["tiled", "persistent"])
 @pytest.mark.parametrize("case", sorted(GRAPH_CASES))
-def test_forward_under_graph_capture(moe, mode, case, monkeypatch):
+def test_forward_under_graph_capture(moe, mode, case):
     """moe_forward only enqueues kernels: it can be captured into a HIP graph.  The graph is replayed several times
     with eager work and synchronisations in between, on changing inputs, and every replay is checked against the
     eager result for the same input."""
     import torch
-    cfg, env = GRAPH_CASES[case]
+    cfg, options = GRAPH_CASES[case]
     cfg = cfg or RAGGED["bf16_swiglu_bias_dropless"]
-    for k_, v_ in env.items():
-        monkeypatch.setenv(k_, v_)
     inp = ob.make_inputs(cfg, seed=13, with_bias=case == "bf16")
-    layer = moe.MoELayer(product_config(cfg), ffn_mode=mode)
+    layer = moe.MoELayer(product_config(cfg), ffn_mode=mode, options=options)
     dev = upload_inputs(cfg, inp)
     x = dev["x"].clone()
     out = torch.empty_like(x)

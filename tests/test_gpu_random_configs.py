@@ -29,27 +29,30 @@ def _cases(n=36, seed=2024):
         cfg = ob.Cfg(S=S, H=H, I=I, E=E, k=k, act=act, dtype=dtype, drop=drop,
                      capacity_factor=float(rng.choice([0.5, 1.0, 1.5])), norm_topk=int(k > 1),
                      gate_fn=ob.GATE_SIGMOID if dtype == ob.FP8 else int(rng.integers(0, 2)), zipf_bias=bool(i % 3 == 0))
-        knobs = dict(MOE355_TILE=str(int(rng.integers(0, 4))), MOE355_QUEUE_GROUPS=str(int(rng.choice([1, 2, 8]))),
-                     MOE355_QUEUE_EARLY=str(int(rng.integers(0, 2))), MOE355_FUSED_COMBINE=str(int(rng.integers(0, 2))))
-        knobs["MOE355_ROW_CHUNK"] = str(i % 4)      # order of the tasks inside a queue segment (0: plain; drawn outside the seeded stream)
-        knobs["MOE355_FP8_TILE"] = str(i // 5 % 2)  # e4m3 layers: weight streamer or tile GEMM
-        knobs["MOE355_GATE_MFMA"] = str(i // 2 % 2)   # 16-bit layers with H % 512 = 0: logits on the vector ALU or on the matrix cores
-        knobs["MOE355_F32_TILE"] = str(i // 5 % 2)   # fp32 layers: vector-ALU kernel or (shape permitting) the matrix-core tile
-        knobs["MOE355_FP8_WIDEN"] = str(i // 10 % 2)  # ... or the bf16 tiles on weights widened in the workspace
+        knobs = dict(tile16=int(rng.integers(0, 4)), queue_groups=int(rng.choice([1, 2, 8])),
+                     queue_early=int(rng.integers(0, 2)), combine=int(rng.integers(0, 2)))
+        if knobs["combine"] and i % 3 == 2:
+            knobs["combine"] = 2              # the combine as tasks of the FFN queue instead of by arrival counters
+        knobs["row_chunk"] = i % 4            # order of the tasks inside a queue segment (0: plain; drawn outside the seeded stream)
+        knobs["fp8_tile"] = i // 5 % 2        # e4m3 layers: weight streamer or tile GEMM
+        knobs["gate_mfma"] = i // 2 % 2       # 16-bit layers with H % 512 = 0: logits on the vector ALU or on the matrix cores
+        knobs["f32_tile"] = i // 5 % 2        # fp32 layers: vector-ALU kernel or (shape permitting) the matrix-core tile
+        knobs["fp8_widen"] = i // 10 % 2      # ... or the bf16 tiles on weights widened in the workspace
+        knobs["fp8_mfma"] = 0                 # bf16 tokens: the arithmetic the oracle's layer restates
+        knobs["gate_fused_topk"] = i // 3 % 2 # top-k inside the logits kernel or as a launch of its own
+        knobs["tail_split"] = (1, 2, 4)[i // 4 % 3]   # down-projection tiles of the last queue segments as partial sums
         out.append(pytest.param(cfg, knobs, int(rng.integers(1, 3)), bool(rng.integers(0, 2)), id="case%02d" % i))
     return out
 
 
 @pytest.mark.parametrize("cfg,knobs,mode,with_bias", _cases())
-def test_random_shape_and_knobs_vs_oracle(cfg, knobs, mode, with_bias, monkeypatch):
+def test_random_shape_and_knobs_vs_oracle(cfg, knobs, mode, with_bias):
     import torch
     import cuplayground_amd as moe
     assert torch.cuda.is_available(), "these tests need the MI355X"
-    for k, v in knobs.items():
-        monkeypatch.setenv(k, v)
     inp = ob.make_inputs(cfg, seed=17, with_bias=with_bias)
     want = ob.forward(cfg, inp)
-    layer = moe.MoELayer(product_config(cfg), ffn_mode=mode)
+    layer = moe.MoELayer(product_config(cfg), ffn_mode=mode, options=knobs)
     dev = upload_inputs(cfg, inp)
     routing = layer.new_routing()
     out = torch.full((cfg.S, cfg.H), float("nan"), dtype=layer.act_dtype, device="cuda")

@@ -86,18 +86,18 @@ def test_route_drops_out_of_range_expert_ids(moe):
     # the fp32 matrix-core tile (forced: the layer is too small for the plan to pick it)
     ("f32_tile", ob.Cfg(S=600, H=256, I=128, E=2, k=1, act=ob.ACT_SWIGLU, dtype=ob.F32, norm_topk=0, drop=0)),
 ])
-@pytest.mark.parametrize("fused_combine", ["0", "1"])
-def test_expired_dependency_wait_poisons_the_output_and_is_reported(moe, name, cfg, fused_combine, monkeypatch):
+@pytest.mark.parametrize("combine", [0, 1, 2], ids=["combine_launch", "combine_arrivals", "combine_queue"])
+def test_expired_dependency_wait_poisons_the_output_and_is_reported(moe, name, cfg, combine):
     """The queue kernel's bounded wait is made to give up from the host (spin limit < 0: every wait expires without
     polling).  Every kernel exits normally; no down-projection tile computes on unfinished rows -- its output is NaN,
     so every routed token's output is NaN; the stall is reported by the next calls on the handle without a
     synchronisation of their own, until it is cleared; after that the handle computes correctly again."""
     import torch
-    monkeypatch.setenv("MOE355_FUSED_COMBINE", fused_combine)   # the combine inside the FFN kernels must carry the NaNs too
-    monkeypatch.setenv("MOE355_F32_TILE", "1" if name == "f32_tile" else "0")
     inp = ob.make_inputs(cfg, seed=9)
     want = ob.forward(cfg, inp)
-    layer = moe.MoELayer(product_config(cfg), ffn_mode=FFN_PERSISTENT)
+    # the combine inside the FFN kernels must carry the NaNs too
+    layer = moe.MoELayer(product_config(cfg), ffn_mode=FFN_PERSISTENT,
+                         options={"combine": combine, "f32_tile": 1 if name == "f32_tile" else 0})
     assert name != "f32_tile" or layer.plan["block_rows"] == 128
     dev = upload_inputs(cfg, inp)
     layer.set_spin_limit(-1)

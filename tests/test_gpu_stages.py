@@ -67,8 +67,8 @@ def test_gemm_vs_oracle(moe, dtype, M, N, K, act):
 
 @pytest.mark.parametrize("dtype", [ob.BF16, ob.F16])
 @pytest.mark.parametrize("M,N,K", [(70, 512, 256), (128, 256, 128), (300, 768, 384)])
-def test_gemm_hand_ordered_tiles_agree(moe, dtype, M, N, K, monkeypatch):
-    """The 256 x 256 and the 128 x 256 hand-ordered tiles forced on a plain GEMM (MOE355_DENSE_TILE): same MFMA
+def test_gemm_hand_ordered_tiles_agree(moe, dtype, M, N, K):
+    """The 256 x 256 and the 128 x 256 hand-ordered tiles forced on a plain GEMM (moe_gemm_bias_act_tile): same MFMA
     sequence over K per output element, so bit-identical to each other, and within tolerance of the oracle."""
     rng = np.random.default_rng(M + N + K)
     kind = KIND[dtype]
@@ -77,9 +77,8 @@ def test_gemm_hand_ordered_tiles_agree(moe, dtype, M, N, K, monkeypatch):
     bias = ob.from_f32(rng.standard_normal(N).astype(np.float32), dtype)
     want = ob.to_f32(ob.gemm_bias_act(A, B, bias, dtype, ob.ACT_GELU), dtype)
     outs = []
-    for tile in ("1", "2"):
-        monkeypatch.setenv("MOE355_DENSE_TILE", tile)
-        outs.append(from_device(moe.gemm_bias_act(to_device(A, kind), to_device(B, kind), to_device(bias, kind), ob.ACT_GELU)))
+    for tile in (1, 2):
+        outs.append(from_device(moe.gemm_bias_act(to_device(A, kind), to_device(B, kind), to_device(bias, kind), ob.ACT_GELU, tile=tile)))
     assert np.array_equal(outs[0], outs[1])
     tol = {ob.BF16: 1e-2, ob.F16: 1.25e-3}[dtype]
     assert np.abs(ob.to_f32(outs[1], dtype) - want).max() <= tol * np.abs(want).max()
@@ -160,13 +159,12 @@ GATE_CASES = [
 
 # mfma: the logits kernel on the matrix cores forced on / off (it takes 16-bit layers with H % 512 = 0 only; elsewhere
 # the knob changes nothing) -- every kernel must produce the oracle's bit patterns
-@pytest.mark.parametrize("mfma", ["0", "1"], ids=["valu", "mfma"])
+@pytest.mark.parametrize("mfma", [0, 1], ids=["valu", "mfma"])
 @pytest.mark.parametrize("cfg", GATE_CASES, ids=lambda c: "S%d_H%d_E%d_k%d_d%d" % (c.S, c.H, c.E, c.k, c.dtype))
-def test_gate_vs_oracle(moe, cfg, mfma, monkeypatch):
-    monkeypatch.setenv("MOE355_GATE_MFMA", mfma)
+def test_gate_vs_oracle(moe, cfg, mfma):
     inp = ob.make_inputs(cfg, seed=7, router_only=True)
     want = ob.route(cfg, inp)
-    layer = moe.MoELayer(product_config(cfg))
+    layer = moe.MoELayer(product_config(cfg), options={"gate_mfma": mfma})
     dev = upload_inputs(cfg, inp)
     idx, w, logits = layer.gate(dev["x"], dev["gate_w"], dev.get("gate_bias"), want_logits=True)
     assert np.array_equal(bits(from_device(logits)), bits(want["logits"]))      # fp32 bit patterns

@@ -20,18 +20,19 @@ CASES = {
 
 
 @pytest.mark.parametrize("name", sorted(CASES) + ["bf16_large_tile_early_start"])
-def test_every_task_is_recorded_once_and_in_dependency_order(name, monkeypatch):
+def test_every_task_is_recorded_once_and_in_dependency_order(name):
     import torch
     import cuplayground_amd as moe
     assert torch.cuda.is_available(), "these tests need the MI355X"
+    options = {}
     if name.endswith("_early_start"):        # the queue loop that starts the next task under the current tile's end
-        monkeypatch.setenv("MOE355_QUEUE_EARLY", "1")
+        options["queue_early"] = 1
         name = name[:-len("_early_start")]
     cfg = CASES[name]
-    monkeypatch.setenv("MOE355_F32_TILE", "1" if name == "f32_tile" else "0")
+    options["f32_tile"] = 1 if name == "f32_tile" else 0
     inp = ob.make_inputs(cfg, seed=13)
     want = ob.route(cfg, inp)
-    layer = moe.MoELayer(product_config(cfg), ffn_mode=FFN_PERSISTENT)
+    layer = moe.MoELayer(product_config(cfg), ffn_mode=FFN_PERSISTENT, options=options)
     dev = upload_inputs(cfg, inp)
     plan = layer.plan
     layer.enable_task_trace(1 << 14)

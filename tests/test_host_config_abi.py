@@ -123,11 +123,58 @@ def test_workspace_and_unsupported_shapes():
     assert e.value.status == 1
 
 
+def test_options_default_env_and_domains(monkeypatch):
+    """moe_options: defaults are all AUTO; the environment is read by moe_options_from_env only (and by the entry points
+    that take no options), values outside a field's domain are ignored there and refused by the *_with_options entries;
+    the workspace follows the options, not the environment, when options are given."""
+    import ctypes as C
+    from cuplayground_amd import api
+    L = moe.load_library()
+    o = api.make_options()
+    assert all(getattr(o, n) == api.OPT_AUTO for n in api.OPTION_FIELDS) and all(v == api.OPT_AUTO for v in o.reserved)
+    for name in api.OPTION_FIELDS:
+        monkeypatch.delenv("MOE355_" + name.upper(), raising=False)
+    monkeypatch.setenv("MOE355_FP8_WIDEN", "1")
+    monkeypatch.setenv("MOE355_QUEUE_GROUPS", "3")       # not a power of two: ignored
+    monkeypatch.setenv("MOE355_TILE16", "x")             # not a number: ignored
+    monkeypatch.setenv("MOE355_COMBINE", "2")
+    e = api.make_options(from_env=True)
+    assert (e.fp8_widen, e.queue_groups, e.tile16, e.combine) == (1, api.OPT_AUTO, api.OPT_AUTO, 2)
+    cfg = moe.MoEConfig(capacity_factor=1.0, drop_tokens=0, expert_top_k=2, hidden_act=2, hidden_size=256,
+                        intermediate_size=256, micro_batch=1, num_experts=4, sequence_len=256, torch_dtype=4)
+    c = cfg.to_c()
+
+    def ws(opts):
+        n = C.c_size_t(0)
+        rc = L.moe_workspace_bytes_with_options(C.byref(c), C.byref(api.make_options(opts)), C.byref(n))
+        return rc, n.value
+
+    rc0, plain = ws({"fp8_widen": 0})
+    rc1, wide = ws({"fp8_widen": 1})
+    assert rc0 == 0 and rc1 == 0 and wide - plain >= 3 * 4 * 256 * 256 * 2    # the bf16 copies of three weight matrices
+    assert cfg.workspace_bytes() == wide                   # no options argument: MOE355_FP8_WIDEN=1 from the environment
+    monkeypatch.delenv("MOE355_FP8_WIDEN")
+    assert cfg.workspace_bytes() == ws({})[1] == plain     # 128 rows per expert: below the widening threshold
+    for bad in ({"tile16": 4}, {"queue_groups": 3}, {"block_rows": 200}, {"combine": 3}, {"tail_split": 3},
+                {"blocks_per_cu": 0}, {"fp8_tile": -2}):
+        assert ws(bad)[0] == 4, bad
+    r = api.make_options()
+    r.reserved[3] = 0
+    n = C.c_size_t(0)
+    assert L.moe_workspace_bytes_with_options(C.byref(c), C.byref(r), C.byref(n)) == 4
+    with pytest.raises(KeyError):
+        api.make_options({"no_such_option": 1})
+
+
 def test_null_arguments_are_errors_not_crashes():
     L = moe.load_library()
     assert L.moe_config_default(None) == 4
     assert L.moe_workspace_bytes(None, None) == 4
     assert L.moe_create(None, None) == 4
+    assert L.moe_create_with_options(None, None, None) == 4
+    assert L.moe_options_default(None) == 4 and L.moe_options_from_env(None) == 4
+    assert L.moe_get_options(None, None) == 4 and L.moe_get_workspace_bytes(None, None) == 4
+    assert L.moe_get_stall(None, None) == 4
     assert L.moe_destroy(None) == 0
     assert L.moe_forward(None, None, None, None, None, None, 0, None) == 4
     assert L.moe_gemm_bias_act(None, None, None, None, 1, 1, 1, 0, 0, None) == 4

@@ -25,6 +25,7 @@ EXPORTS = (
     "moe_config_tokens", "moe_config_capacity", "moe_create", "moe_destroy", "moe_get_arch", "moe_get_plan", "moe_get_kernel_dtype",
     "moe_workspace_bytes", "moe_options_default", "moe_options_from_env", "moe_create_with_options",
     "moe_workspace_bytes_with_options", "moe_get_options", "moe_get_workspace_bytes", "moe_get_stall", "moe_gemm_bias_act_tile",
+    "moe_prepared_bytes", "moe_prepare_weights",
     "moe_set_ffn_mode", "moe_get_ffn_mode", "moe_forward", "moe_forward_static", "moe_set_spin_limit", "moe_clear_stall", "moe_gate", "moe_router_stats", "moe_route", "moe_gemm_bias_act", "moe_combine",
     "moe_set_stage_timing", "moe_get_stage_ms", "moe_get_stage_samples", "moe_get_task_counts", "moe_get_queue_balance", "moe_task_trace_bytes", "moe_set_task_trace", "moe_get_task_trace", "moe_measure_mfma_tflops",
     "moe_measure_hbm_read_gbs", "moe_quant_block128", "moe_dequant_block128", "moe_backward_scratch_bytes", "moe_transpose", "moe_expert_gemm",
@@ -48,13 +49,13 @@ class _CConfig(C.Structure):
 
 OPTION_FIELDS = ("tile16", "block_rows", "f32_tile", "fp8_tile", "fp8_widen", "queue_groups", "queue_lag", "queue_early",
                  "row_chunk", "blocks_per_cu", "combine", "gate_kernel", "gate_mfma", "gate_tile", "gate_fused_topk",
-                 "grouped_tile", "tail_split", "fp8_mfma")
+                 "grouped_tile", "tail_split", "fp8_mfma", "prepared_weights")
 OPT_AUTO = -1
 COMBINE_SEPARATE, COMBINE_ARRIVALS, COMBINE_QUEUE = 0, 1, 2
 
 
 class _COptions(C.Structure):
-    _fields_ = [(n, C.c_int32) for n in OPTION_FIELDS] + [("reserved", C.c_int32 * 8)]
+    _fields_ = [(n, C.c_int32) for n in OPTION_FIELDS] + [("reserved", C.c_int32 * 7)]
 
 
 def make_options(options: dict | None = None, from_env: bool = False) -> _COptions:
@@ -78,7 +79,7 @@ class _CArch(C.Structure):
 
 class _CWeights(C.Structure):
     _fields_ = [(n, C.c_void_p) for n in ("gate_w", "gate_bias", "w_up", "w_gate", "w_down", "b_up", "b_gate",
-                                          "b_down", "s_up", "s_gate", "s_down")]
+                                          "b_down", "s_up", "s_gate", "s_down", "prepared")]
 
 
 class _CRouting(C.Structure):
@@ -123,6 +124,8 @@ def load_library():
     L.moe_get_options.argtypes = [vp, optp]
     L.moe_get_workspace_bytes.argtypes = [vp, C.POINTER(C.c_size_t)]
     L.moe_get_stall.argtypes = [vp, C.POINTER(i32)]
+    L.moe_prepared_bytes.argtypes = [vp, C.POINTER(C.c_size_t)]
+    L.moe_prepare_weights.argtypes = [vp, C.POINTER(_CWeights), vp, C.c_size_t, vp]
     L.moe_gemm_bias_act_tile.argtypes = [vp, vp, vp, vp, i64, i64, i64, i32, i32, i32, vp]
     L.moe_set_ffn_mode.argtypes = [vp, C.c_int]
     L.moe_get_ffn_mode.argtypes = [vp, C.POINTER(C.c_int32)]
@@ -252,7 +255,7 @@ class MoELayer:
     """One MoE layer shape bound to the current GPU: a `moe_handle` and its workspace."""
 
     WEIGHT_KEYS = ("gate_w", "gate_bias", "w_up", "w_gate", "w_down", "b_up", "b_gate", "b_down", "s_up", "s_gate",
-                   "s_down")
+                   "s_down", "prepared")
 
     def __init__(self, cfg: MoEConfig, ffn_mode: int = FFN_AUTO, allocate_workspace: bool = True,
                  options: dict | None = None):
@@ -405,6 +408,28 @@ class MoELayer:
             t = weights.get(n)
             setattr(w, n, None if t is None else t.data_ptr())
         return w
+
+    @property
+    def prepared_bytes(self) -> int:
+        """Bytes moe_prepare_weights writes for this handle's plan (0: the plan reads the weights as they are)."""
+        n = C.c_size_t(0)
+        _check(self.L.moe_prepared_bytes(self._h, C.byref(n)), "moe_prepared_bytes")
+        return n.value
+
+    def prepare_weights(self, weights: dict, out=None):
+        """The kernel-ready form of `weights` for this handle (a uint8 tensor to pass on as weights["prepared"]), or
+        None when the plan prepares nothing.  `out`: a tensor of prepared_bytes bytes to write into (e.g. one loaded
+        from a file's worth of storage); allocated when not given."""
+        import torch
+        n = self.prepared_bytes
+        if n == 0:
+            return None
+        if out is None:
+            out = torch.empty(n, dtype=torch.uint8, device="cuda")
+        w = self._weights(weights)
+        _check(self.L.moe_prepare_weights(self._h, C.byref(w), _ptr(out), out.numel() * out.element_size(), _stream()),
+               "moe_prepare_weights")
+        return out
 
     def new_routing(self) -> dict:
         import torch

@@ -56,6 +56,7 @@ size_t align_up(size_t v) { return (v + kAlign - 1) / kAlign * kAlign; }
 int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
 
 struct Derived {
+    bool wide_in_workspace;   // the widened weight copies live in the workspace (false: the caller brings prepared ones)
     int S, H, I, E, k, A;
     int act_dtype;     // MOE_DTYPE_F32, MOE_DTYPE_BF16 or MOE_DTYPE_FP16
     size_t act_bytes;
@@ -68,7 +69,8 @@ struct Derived {
 
 struct WsLayout {
     size_t logits, topk_idx, topk_w, slot, pair_row, token_indices, expert_count, expert_offset, rank_local,
-        block_hist, mtiles, seg0, seg1, segq, qstate, done0, wg_clock, arrive, stats_prob, stats_cnt, h, y, wide, total;
+        block_hist, mtiles, seg0, seg1, segq, qstate, cstate, done0, done1, pair_mt, wg_clock, arrive, stats_prob, stats_cnt, h, y,
+        wide, total;
 };
 
 // Storage type of activations (x, biases, h, y, out): the layer's own, except that tf32 -- fp32 storage with
@@ -104,6 +106,7 @@ int derive(const moe_config& c, const moe_options& o, Derived* d) {
     if (d->capacity > d->A) d->capacity = d->A;
     d->plan = ffn_plan(c.torch_dtype, c.hidden_act, d->H, d->I, d->A, d->E, o);
     d->wide_mats = c.hidden_act == MOE_ACT_SWIGLU ? 3 : 2;
+    d->wide_in_workspace = d->plan.widen && o.prepared_weights != 1;
     d->nblk = ceil_div(d->A, kRouteBlock);
     d->max_mtiles = ceil_div(d->A, d->plan.block_m) + d->E;
     return MOE_OK;
@@ -128,7 +131,10 @@ WsLayout layout(const Derived& d) {
     w.seg1 = take((size_t)d.E * sizeof(Segment));
     w.segq = take((size_t)2 * d.E * sizeof(Segment));
     w.qstate = take(sizeof(QueueState));
+    w.cstate = take(sizeof(CombineState));
     w.done0 = take((size_t)d.max_mtiles * 4);
+    w.done1 = take((size_t)d.max_mtiles * 4);
+    w.pair_mt = take((size_t)d.A * 4);
     w.wg_clock = take((size_t)kMaxQueueWorkgroups * 2 * sizeof(int64_t));
     w.arrive = take((size_t)d.S * d.plan.nnt1 * 4);
     w.stats_prob = take((size_t)kStatsBlocks * d.E * 8);
@@ -136,7 +142,7 @@ WsLayout layout(const Derived& d) {
     w.h = take((size_t)d.A * d.I * d.act_bytes);
     w.y = take((size_t)d.A * d.H * d.act_bytes);
     // bf16 copies of an e4m3 layer's expert weights (up, down, gate), rewritten by every call of such a plan
-    w.wide = take(d.plan.widen ? (size_t)d.wide_mats * d.E * d.I * d.H * 2 : 0);
+    w.wide = take(d.wide_in_workspace ? (size_t)d.wide_mats * d.E * d.I * d.H * 2 : 0);
     w.total = off;
     return w;
 }
@@ -258,10 +264,12 @@ int check_ws(const moe_handle* h, const void* ws, size_t bytes) {
 template <typename T>
 T* at(void* ws, size_t off) { return reinterpret_cast<T*>(static_cast<char*>(ws) + off); }
 
+int resolved_ffn_mode(const moe_handle* h);
+
 RouteArgs route_args(const moe_handle* h, void* ws) {
     const Derived& d = h->d;
     const WsLayout& w = h->ws;
-    RouteArgs a;
+    RouteArgs a{};
     a.topk_idx = at<int32_t>(ws, w.topk_idx);
     a.rank_local = at<int32_t>(ws, w.rank_local);
     a.block_hist = at<int32_t>(ws, w.block_hist);
@@ -276,7 +284,15 @@ RouteArgs route_args(const moe_handle* h, void* ws) {
     a.seg_queue = at<Segment>(ws, w.segq);
     a.q = at<QueueState>(ws, w.qstate);
     a.done0 = at<int32_t>(ws, w.done0);
-    a.arrive = h->combine_mode == 1 ? at<int32_t>(ws, w.arrive) : nullptr;
+    // arrival counters [S, nnt1] of the combine inside the FFN kernels, or the flags [S * slices] of the combine tasks of
+    // the queue (a slice is at least 1024 columns, a column tile at most 256: the flags fit the same array); the latter
+    // exist in task-queue mode only
+    const bool queue_combine = h->combine_mode == 2 && resolved_ffn_mode(h) == MOE_FFN_PERSISTENT;
+    a.arrive = (h->combine_mode == 1 || queue_combine) ? at<int32_t>(ws, w.arrive) : nullptr;
+    a.arrive_n = d.S * d.plan.nnt1;
+    a.done1 = queue_combine ? at<int32_t>(ws, w.done1) : nullptr;
+    a.pair_mt = queue_combine ? at<int32_t>(ws, w.pair_mt) : nullptr;
+    a.cs = queue_combine ? at<CombineState>(ws, w.cstate) : nullptr;
     a.task_trace = h->task_trace;
     a.S = d.S; a.k = d.k; a.E = d.E; a.A = d.A; a.nblk = d.nblk;
     a.drop = h->cfg.drop_tokens;
@@ -344,6 +360,7 @@ const OptField kOptFields[] = {
     {"grouped_tile", &moe_options::grouped_tile, 0, 2, false},
     {"tail_split", &moe_options::tail_split, 1, 4, true},
     {"fp8_mfma", &moe_options::fp8_mfma, 0, 1, false},
+    {"prepared_weights", &moe_options::prepared_weights, 0, 1, false},
 };
 bool opt_in_domain(const OptField& f, int v) {
     if (v == MOE_OPT_AUTO) return true;
@@ -508,6 +525,7 @@ int moe_create_with_options(const moe_config* cfg, const moe_options* opt, moe_h
     h->opt.row_chunk = h->row_chunk;
     h->opt.blocks_per_cu = per_cu;
     h->opt.combine = h->combine_mode;
+    h->opt.prepared_weights = d.plan.widen && !d.wide_in_workspace ? 1 : 0;
     resolve_static_scratch(dev);
     *out = h;
     return MOE_OK;
@@ -628,9 +646,8 @@ int moe_gate(moe_handle* h, const void* x, const void* gate_w, const float* gate
     hipStream_t st = (hipStream_t)stream;
     const Derived& d = h->d;
     float* lg = logits ? logits : at<float>(workspace, h->ws.logits);
-    hipError_t e = launch_gate_logits(x, gate_w, gate_bias, lg, d.S, d.H, d.E, d.act_dtype, h->opt, st);
-    if (e != hipSuccess) return hip_fail(h, e);
-    e = launch_topk(lg, d.S, d.E, d.k, h->cfg.gate_fn, h->cfg.norm_topk_prob, topk_idx, topk_w, st);
+    const hipError_t e = launch_gate(x, gate_w, gate_bias, lg, logits != nullptr, d.S, d.H, d.E, d.k, h->cfg.gate_fn,
+                                     h->cfg.norm_topk_prob, topk_idx, topk_w, d.act_dtype, h->opt, st);
     if (e != hipSuccess) return hip_fail(h, e);
     return MOE_OK;
 }
@@ -679,6 +696,20 @@ int moe_route(moe_handle* h, const int32_t* topk_idx, int32_t* slot, int32_t* ex
 
 namespace {
 
+// The bf16 copies of an e4m3 layer's expert weights: [up | down | gate], each [E, N, K].
+hipError_t widen_weights(const Derived& d, const moe_weights* w, char* wide, hipStream_t st) {
+    const int64_t mat = (int64_t)d.I * d.H;
+    const void* src[3] = {w->w_up, w->w_down, w->w_gate};
+    const float* scl[3] = {w->s_up, w->s_down, w->s_gate};
+    for (int i = 0; i < d.wide_mats; ++i) {
+        // w_up and w_gate are [E, I, H], w_down is [E, H, I]
+        const hipError_t e = launch_widen_block128(src[i], scl[i], wide + (size_t)i * d.E * mat * 2, d.E, i == 1 ? d.H : d.I,
+                                                   i == 1 ? d.I : d.H, st);
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
 // The whole layer on a workspace that has passed check_ws (the caller's, or this device's static array).
 int forward_on(moe_handle* h, const void* x, const moe_weights* w, void* out, const moe_routing_out* routing,
                void* workspace, size_t workspace_bytes, void* stream) {
@@ -697,6 +728,8 @@ int forward_on(moe_handle* h, const void* x, const moe_weights* w, void* out, co
     if (!sw && w->b_gate) return MOE_ERR_BAD_ARGUMENT;
     if (fp8 && (!w->s_up || !w->s_down || sw != (w->s_gate != nullptr))) return MOE_ERR_BAD_ARGUMENT;
     if (!fp8 && (w->s_up || w->s_down || w->s_gate)) return MOE_ERR_BAD_ARGUMENT;
+    if (w->prepared && (!h->d.plan.widen || ((uintptr_t)w->prepared % kAlign))) return MOE_ERR_BAD_ARGUMENT;   // nothing to prepare on this plan
+    if (!w->prepared && h->d.plan.widen && !h->d.wide_in_workspace) return MOE_ERR_BAD_ARGUMENT;   // promised at moe_create
     int rc = check_ws(h, workspace, workspace_bytes);
     if (rc) return rc;
     hipStream_t st = (hipStream_t)stream;
@@ -712,9 +745,8 @@ int forward_on(moe_handle* h, const void* x, const moe_weights* w, void* out, co
     float* logits = at<float>(workspace, L.logits);
     int32_t* topk_idx = at<int32_t>(workspace, L.topk_idx);
     float* topk_w = at<float>(workspace, L.topk_w);
-    e = launch_gate_logits(x, w->gate_w, w->gate_bias, logits, d.S, d.H, d.E, d.act_dtype, h->opt, st);
-    if (e != hipSuccess) return hip_fail(h, e);
-    e = launch_topk(logits, d.S, d.E, d.k, c.gate_fn, c.norm_topk_prob, topk_idx, topk_w, st);
+    e = launch_gate(x, w->gate_w, w->gate_bias, logits, false, d.S, d.H, d.E, d.k, c.gate_fn, c.norm_topk_prob, topk_idx,
+                    topk_w, d.act_dtype, h->opt, st);
     if (e != hipSuccess) return hip_fail(h, e);
     if ((e = mark(1)) != hipSuccess) return hip_fail(h, e);
     // ---- slots, capacity, task tables ----
@@ -723,7 +755,7 @@ int forward_on(moe_handle* h, const void* x, const moe_weights* w, void* out, co
     if (e != hipSuccess) return hip_fail(h, e);
     if ((e = mark(2)) != hipSuccess) return hip_fail(h, e);
     // ---- expert FFN ----
-    FfnArgs fa;
+    FfnArgs fa{};        // every field starts null / zero: a member nobody sets must not reach a kernel as stack garbage
     fa.x = x;
     fa.token_indices = ra.token_indices;
     fa.w_up = w->w_up; fa.w_gate = w->w_gate; fa.w_down = w->w_down;
@@ -742,7 +774,11 @@ int forward_on(moe_handle* h, const void* x, const moe_weights* w, void* out, co
     fa.host_stall = h->stall_host;
     fa.wg_clock = at<int64_t>(workspace, L.wg_clock);
     fa.row_chunk = h->row_chunk;
-    fa.arrive = ra.arrive;
+    fa.arrive = ra.done1 ? nullptr : ra.arrive;
+    fa.done1 = ra.done1;
+    fa.pair_mt = ra.pair_mt;
+    fa.combined = ra.done1 ? ra.arrive : nullptr;
+    fa.cs = ra.cs;
     fa.task_trace = h->task_trace;
     fa.task_trace_cap = h->task_trace_cap;
     fa.pair_row = ra.pair_row;
@@ -758,19 +794,15 @@ int forward_on(moe_handle* h, const void* x, const moe_weights* w, void* out, co
     }
     const int mode = resolved_ffn_mode(h);
     const int kdt = d.plan.kernel_dtype;
-    if (d.plan.widen) {   // the layer's e4m3 weights become bf16 ones in the workspace; from here on it is a bf16 layer
-        const int64_t mat = (int64_t)d.I * d.H;
-        char* wide = at<char>(workspace, L.wide);
-        const void* src[3] = {w->w_up, w->w_down, w->w_gate};
-        const float* scl[3] = {w->s_up, w->s_down, w->s_gate};
-        const void** dst[3] = {&fa.w_up, &fa.w_down, &fa.w_gate};
-        for (int i = 0; i < d.wide_mats; ++i) {
-            void* o = wide + (size_t)i * d.E * mat * 2;
-            // w_up and w_gate are [E, I, H], w_down is [E, H, I]
-            e = launch_widen_block128(src[i], scl[i], o, d.E, i == 1 ? d.H : d.I, i == 1 ? d.I : d.H, st);
+    if (d.plan.widen) {   // the layer's e4m3 weights become bf16 ones; from here on it is a bf16 layer
+        // made once by moe_prepare_weights, or by this call in the workspace
+        char* wide = w->prepared ? static_cast<char*>(const_cast<void*>(w->prepared)) : at<char>(workspace, L.wide);
+        if (!w->prepared) {
+            e = widen_weights(d, w, wide, st);
             if (e != hipSuccess) return hip_fail(h, e);
-            *dst[i] = o;
         }
+        const void** dst[3] = {&fa.w_up, &fa.w_down, &fa.w_gate};
+        for (int i = 0; i < d.wide_mats; ++i) *dst[i] = wide + (size_t)i * d.E * d.I * d.H * 2;
         fa.s_up = fa.s_gate = fa.s_down = nullptr;
     }
     if (kdt == MOE_DTYPE_FP8_E4M3_B128) {
@@ -784,8 +816,8 @@ int forward_on(moe_handle* h, const void* x, const moe_weights* w, void* out, co
     if (e != hipSuccess) return hip_fail(h, e);
     if ((e = mark(3)) != hipSuccess) return hip_fail(h, e);
     // ---- combine (already done inside the FFN kernels unless that is switched off) ----
-    if (!fa.arrive) {
-        e = launch_combine(fa.y, ra.pair_row, topk_w, d.S, d.k, d.H, d.act_dtype, out, st);
+    if (!fa.arrive) {   // everything, or what the combine tasks of the queue kernel have left
+        e = launch_combine(fa.y, ra.pair_row, topk_w, d.S, d.k, d.H, d.act_dtype, out, fa.combined, st);
         if (e != hipSuccess) return hip_fail(h, e);
     }
     if ((e = mark(4)) != hipSuccess) return hip_fail(h, e);
@@ -827,6 +859,25 @@ int moe_forward_static(moe_handle* h, const void* x, const moe_weights* w, void*
     if (dev < 0 || dev >= kMaxDevices || !g_scratch_done[dev]) return MOE_ERR_NO_DEVICE;
     if (!g_scratch_ptr[dev]) return hip_fail(h, g_scratch_err[dev]);
     return forward_on(h, x, w, out, routing, g_scratch_ptr[dev], kStaticScratchBytes, stream);
+}
+
+int moe_prepared_bytes(const moe_handle* h, size_t* bytes) {
+    if (!h || !bytes) return MOE_ERR_BAD_ARGUMENT;
+    *bytes = h->d.plan.widen ? (size_t)h->d.wide_mats * h->d.E * h->d.I * h->d.H * 2 : 0;
+    return MOE_OK;
+}
+
+int moe_prepare_weights(moe_handle* h, const moe_weights* w, void* prepared, size_t prepared_bytes, void* stream) {
+    if (!h || !w) return MOE_ERR_BAD_ARGUMENT;
+    size_t need = 0;
+    moe_prepared_bytes(h, &need);
+    if (need == 0) return MOE_OK;                       // this plan reads the weights as they are
+    if (!prepared || ((uintptr_t)prepared % kAlign) || prepared_bytes < need) return MOE_ERR_WORKSPACE;
+    const bool sw = h->cfg.hidden_act == MOE_ACT_SWIGLU;
+    if (!w->w_up || !w->w_down || !w->s_up || !w->s_down || sw != (w->w_gate != nullptr) || sw != (w->s_gate != nullptr))
+        return MOE_ERR_BAD_ARGUMENT;
+    const hipError_t e = widen_weights(h->d, w, static_cast<char*>(prepared), (hipStream_t)stream);
+    return e == hipSuccess ? MOE_OK : hip_fail(h, e);
 }
 
 int moe_set_spin_limit(moe_handle* h, int32_t polls) {
@@ -1079,7 +1130,7 @@ int moe_combine(const void* y_rows, const int32_t* pair_row, const float* topk_w
     if (!y_rows || !pair_row || !topk_w || !out || S < 0 || k < 1 || H < 1) return MOE_ERR_BAD_ARGUMENT;
     if (act_dtype != MOE_DTYPE_F32 && act_dtype != MOE_DTYPE_BF16 && act_dtype != MOE_DTYPE_FP16) return MOE_ERR_UNSUPPORTED;
     if (H % (act_dtype == MOE_DTYPE_F32 ? 4 : 8)) return MOE_ERR_UNSUPPORTED;
-    const hipError_t e = launch_combine(y_rows, pair_row, topk_w, S, k, H, act_dtype, out, (hipStream_t)stream);
+    const hipError_t e = launch_combine(y_rows, pair_row, topk_w, S, k, H, act_dtype, out, nullptr, (hipStream_t)stream);
     return e == hipSuccess ? MOE_OK : MOE_ERR_HIP;
 }
 

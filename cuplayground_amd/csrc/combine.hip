@@ -17,8 +17,9 @@ template <typename T16>
 __global__ __launch_bounds__(256) void combine_16_kernel(const uint16_t* __restrict__ y,
                                                          const int32_t* __restrict__ pair_row,
                                                          const float* __restrict__ topk_w, int k, int H,
-                                                         uint16_t* __restrict__ out) {
+                                                         uint16_t* __restrict__ out, const int32_t* __restrict__ taken) {
     const int t = blockIdx.x;
+    if (taken && taken[(size_t)blockIdx.y * gridDim.x + t]) return;   // combined inside the FFN queue kernel
     const int c = (blockIdx.y * 256 + threadIdx.x) * 8;
     if (c >= H) return;
     combine_token_16<T16, false>(y, pair_row, topk_w, t, k, H, c, out);
@@ -27,8 +28,9 @@ __global__ __launch_bounds__(256) void combine_16_kernel(const uint16_t* __restr
 __global__ __launch_bounds__(256) void combine_f32_kernel(const float* __restrict__ y,
                                                           const int32_t* __restrict__ pair_row,
                                                           const float* __restrict__ topk_w, int k, int H,
-                                                          float* __restrict__ out) {
+                                                          float* __restrict__ out, const int32_t* __restrict__ taken) {
     const int t = blockIdx.x;
+    if (taken && taken[(size_t)blockIdx.y * gridDim.x + t]) return;   // combined inside the FFN queue kernel
     const int c = (blockIdx.y * 256 + threadIdx.x) * 4;
     if (c >= H) return;
     combine_token_f32<false>(y, pair_row, topk_w, t, k, H, c, out);
@@ -37,17 +39,17 @@ __global__ __launch_bounds__(256) void combine_f32_kernel(const float* __restric
 }  // namespace
 
 hipError_t launch_combine(const void* y_rows, const int32_t* pair_row, const float* topk_w, int S, int k, int H,
-                          int act_dtype, void* out, hipStream_t st) {
+                          int act_dtype, void* out, const int32_t* taken, hipStream_t st) {
     if (S <= 0) return hipSuccess;
     if (act_dtype == MOE_DTYPE_F32) {
         const dim3 grid(S, (H + 256 * 4 - 1) / (256 * 4));
-        combine_f32_kernel<<<grid, 256, 0, st>>>((const float*)y_rows, pair_row, topk_w, k, H, (float*)out);
+        combine_f32_kernel<<<grid, 256, 0, st>>>((const float*)y_rows, pair_row, topk_w, k, H, (float*)out, taken);
     } else {
         const dim3 grid(S, (H + 256 * 8 - 1) / (256 * 8));
         if (act_dtype == MOE_DTYPE_FP16)
-            combine_16_kernel<f16_s><<<grid, 256, 0, st>>>((const uint16_t*)y_rows, pair_row, topk_w, k, H, (uint16_t*)out);
+            combine_16_kernel<f16_s><<<grid, 256, 0, st>>>((const uint16_t*)y_rows, pair_row, topk_w, k, H, (uint16_t*)out, taken);
         else
-            combine_16_kernel<bf16_s><<<grid, 256, 0, st>>>((const uint16_t*)y_rows, pair_row, topk_w, k, H, (uint16_t*)out);
+            combine_16_kernel<bf16_s><<<grid, 256, 0, st>>>((const uint16_t*)y_rows, pair_row, topk_w, k, H, (uint16_t*)out, taken);
     }
     return hipGetLastError();
 }

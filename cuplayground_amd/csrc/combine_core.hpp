@@ -122,4 +122,91 @@ __device__ __forceinline__ void combine_token_f32(const float* __restrict__ y, c
     *reinterpret_cast<uint4*>(out + (size_t)t * H + c) = o;
 }
 
+// ---- U tokens at a time, for the combine that runs as tasks of the FFN queue kernels (ffn_common.hpp: combine_while_idle) ----
+// A queue kernel keeps one to three workgroups per compute unit, so nothing but the code itself puts memory requests in
+// flight: the rows of up to U tokens (R ranks each) are requested together and waited for once.  Per token the
+// arithmetic is that of combine_token_16 / combine_token_f32 above, statement for statement -- acc = acc + w * y in
+// ascending rank order, one rounding -- so where and how many at a time a token is combined cannot change a bit.
+// All loads are agent-scope (the rows were written earlier in this launch, possibly on another XCD).
+template <class ET> struct CmbElem;      // ET: bf16_s, f16_s or float
+template <> struct CmbElem<bf16_s> { static constexpr int N = 8; };
+template <> struct CmbElem<f16_s> { static constexpr int N = 8; };
+template <> struct CmbElem<float> { static constexpr int N = 4; };
+
+template <class ET>
+__device__ __forceinline__ void cmb_accumulate(float (&acc)[CmbElem<ET>::N], float w, const uint32_t (&u)[4]) {
+    if constexpr (CmbElem<ET>::N == 4) {
+        acc[0] = acc[0] + w * __uint_as_float(u[0]);
+        acc[1] = acc[1] + w * __uint_as_float(u[1]);
+        acc[2] = acc[2] + w * __uint_as_float(u[2]);
+        acc[3] = acc[3] + w * __uint_as_float(u[3]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            acc[2 * i] = acc[2 * i] + w * cmb_lo(u[i], ET{});
+            acc[2 * i + 1] = acc[2 * i + 1] + w * cmb_hi(u[i], ET{});
+        }
+    }
+}
+
+// tok[u] (u < n <= U): the tokens; c: this thread's first column (CmbElem<ET>::N consecutive columns, c < H).  The ranks
+// are taken R at a time (U x R rows in flight).
+template <class ET, int U, int R>
+__device__ __forceinline__ void combine_tokens_fresh(const void* __restrict__ y, const int32_t* __restrict__ pair_row,
+                                                     const float* __restrict__ topk_w, const int (&tok)[U], int n, int k,
+                                                     int H, int c, void* __restrict__ out) {
+    typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+    constexpr int N = CmbElem<ET>::N;
+    constexpr int EB = 16 / N;                 // bytes per element
+    float acc[U][N];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int i = 0; i < N; ++i) acc[u][i] = 0.0f;
+    for (int r0 = 0; r0 < k; r0 += R) {
+        bool on[U][R];
+        float w[U][R];
+        u32x4_t v[U][R];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int j = 0; j < R; ++j) {
+                const int row = (u < n && r0 + j < k) ? pair_row[(size_t)tok[u] * k + r0 + j] : -1;
+                on[u][j] = row >= 0;
+                w[u][j] = on[u][j] ? topk_w[(size_t)tok[u] * k + r0 + j] : 0.0f;
+                const char* p = static_cast<const char*>(y) + ((size_t)(on[u][j] ? row : 0) * H + c) * EB;
+                v[u][j] = u32x4_t{0u, 0u, 0u, 0u};
+                // tied to the register it fills: a lane that skips the load keeps its zeros
+                if (on[u][j]) asm volatile("global_load_dwordx4 %0, %1, off sc1" : "+v"(v[u][j]) : "v"(p) : "memory");
+            }
+        // one wait for everything in flight; every destination register is named so that no use can move above it
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int j = 0; j < R; ++j) asm volatile("s_waitcnt vmcnt(0)" : "+v"(v[u][j])::"memory");
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int j = 0; j < R; ++j) {
+                if (!on[u][j]) continue;
+                const uint32_t q[4] = {v[u][j][0], v[u][j][1], v[u][j][2], v[u][j][3]};
+                cmb_accumulate<ET>(acc[u], w[u][j], q);
+            }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        if (u >= n) continue;
+        uint4 o;
+        if constexpr (N == 4) {
+            o = uint4{__float_as_uint(acc[u][0]), __float_as_uint(acc[u][1]), __float_as_uint(acc[u][2]), __float_as_uint(acc[u][3])};
+        } else {
+            o.x = cmb_pack2(acc[u][0], acc[u][1], ET{});
+            o.y = cmb_pack2(acc[u][2], acc[u][3], ET{});
+            o.z = cmb_pack2(acc[u][4], acc[u][5], ET{});
+            o.w = cmb_pack2(acc[u][6], acc[u][7], ET{});
+        }
+        *reinterpret_cast<uint4*>(static_cast<char*>(out) + ((size_t)tok[u] * H + c) * EB) = o;
+    }
+}
+
 }  // namespace moe355

@@ -916,6 +916,7 @@ __global__ __launch_bounds__(P::THREADS) void ffn_persistent_kernel(FfnArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ int s_task, s_ok;
     __shared__ int s_list[1 + P::T0::BM];
+    static_assert(1 + P::T0::BM >= kCombineLds, "s_list doubles as the scratch of the combine tasks");
     using ET = typename std::conditional<P::T0::F16, f16_s, bf16_s>::type;
     queue_kernel_entry();
     queue_clock_stamp(kernel_args_again().wg_clock, 0);
@@ -933,13 +934,14 @@ __global__ __launch_bounds__(P::THREADS) void ffn_persistent_kernel(FfnArgs a) {
             t.rows = 0;
         }
         const long long started = trace_clock(kernel_args_again().task_trace);
-        plan_tile<P>(a, t, t.phase == 0 || a.arrive, smem);
+        plan_tile<P>(a, t, t.phase == 0 || publish_y(a), smem);
         if (kernel_args_again().task_trace)
             trace_task(kernel_args_again().task_trace, kernel_args_again().task_trace_cap, t.phase, t.expert, t.mtile, t.ntile, t.rows, started);
         if (t.phase == 0) signal_phase0_done(a.done0, t.mtile);
-        else if (a.arrive)   // the row count from the table: a tile whose wait expired runs with none, and still arrives
-            combine_arrivals<ET>(combine_args(kernel_args_again()), t.row0, a.mtiles[t.mtile].rows, t.ntile, t.ntile * P::T1::BN, P::T1::BN, s_list);
+        else                 // the row count from the table: a tile whose wait expired runs with none, and still arrives
+            after_down_tile<ET>(kernel_args_again(), t.row0, a.mtiles[t.mtile].rows, t.mtile, t.ntile, t.ntile * P::T1::BN, P::T1::BN, s_list);
     }
+    if (kernel_args_again().combined) combine_while_idle<ET>(sweep_args(kernel_args_again()), &s_task, s_list);
     queue_clock_stamp(kernel_args_again().wg_clock, 1);
 }
 
@@ -1053,14 +1055,14 @@ __global__ __launch_bounds__(P::THREADS) void ffn_persistent_ring_kernel(FfnArgs
             }
         };
         if (active) {
-            epilogue_full_n<T>(resolve<T>(a, as_task(), ph == 0 || a.arrive), smem, acc, token_loads);
+            epilogue_full_n<T>(resolve<T>(a, as_task(), ph == 0 || publish_y(a)), smem, acc, token_loads);
         } else {
 #pragma unroll
             for (int i = 0; i < 8; ++i) token_loads(i);
         }
         if (a.task_trace) trace_task(a.task_trace, a.task_trace_cap, ph, ex, mt, nt, rows, traced_from);
         if (ph == 0) signal_phase0_done(a.done0, mt);
-        else if (a.arrive) combine_arrivals<ET>(combine_args(a), row0, a.mtiles[mt].rows, nt, nt * T::BN, T::BN, s_list);
+        else after_down_tile<ET>(a, row0, a.mtiles[mt].rows, mt, nt, nt * T::BN, T::BN, s_list);
         if (reserve && nid < ids && n_valid) {   // the reserved task is the next one
             ph = n_ph; ex = n_ex; mt = n_mt; nt = n_nt; row0 = n_row0; rows = n_rows;
             cur.last_id = nid;
@@ -1074,6 +1076,7 @@ __global__ __launch_bounds__(P::THREADS) void ffn_persistent_ring_kernel(FfnArgs
         have = pop_blocking();
         if (have) start_cold();
     }
+    if (kernel_args_again().combined) combine_while_idle<ET>(sweep_args(kernel_args_again()), &s_task, s_list);
     queue_clock_stamp(kernel_args_again().wg_clock, 1);
 }
 

@@ -316,6 +316,146 @@ __device__ __forceinline__ void zero_unrouted_rows(const FfnArgs& a, int elem_by
     }
 }
 
+// ---- Combine as tasks of the queue ----
+// The third way to run the combine (moe_options::combine = 2), the one that keeps it off the critical path where the
+// routing allows: a workgroup that finds every GEMM queue empty does not leave the kernel; as long as other workgroups
+// are still busy with their last tiles -- the idle tail of a task-queue launch -- it combines the tokens that are
+// already complete.  The reference's processor likewise applies the combine on chip as part of its task loop
+// (combine.cuh:105-188, overlap.cuh:94-153), there with unordered atomic adds.  Here:
+//   * every finished down-projection tile adds one to done1[row block] behind its written-through stores (the
+//     signal_phase0_done protocol on a second counter array); pair_mt[token, rank] names the row block of a pair;
+//   * a unit is (token, slice): the columns one pass of the workgroup covers (blockDim.x threads x 16 bytes); a combine
+//     task is kCombineChunk consecutive tokens of one slice; every workgroup walks the tasks in a stride of its own
+//     (no shared counter: hundreds of idle workgroups on one atomic hold up the queue pops of the busy ones, as does
+//     anything in the queue state's cache line -- the combine state has its own): the units whose token is complete
+//     (every kept pair's row block has done1 == nnt1) and that nobody has taken yet are claimed in combined[] and
+//     combined, the others are left alone, and a workgroup that finds nothing backs off before it looks again;
+//   * nobody ever waits: when the last down-projection tile is finished (cs->down_done == q->tasks_phase1; every one of
+//     them has been popped by then, so each is running on a workgroup that needs nothing from this one) everybody
+//     leaves, and the combine launch behind the kernel takes the units whose flag is still clear -- at the occupancy and cache
+//     hit rate of a kernel of its own, which a queue kernel with one to three workgroups per compute unit cannot match
+//     (measured: a blocking second sweep inside the kernel cost 47 to 140 us more than it saved).
+// Same arithmetic as the combine kernel (combine_core.hpp), so not a bit changes.
+constexpr int kCombineChunk = 16;      // tokens per combine task (one lane each checks readiness)
+constexpr int kCombineLds = kCombineChunk + 4;   // ints of LDS the combine tasks need
+
+// What the combine tasks need of FfnArgs, small enough to travel in registers: a function that is not inlined and takes
+// the whole argument block by reference makes the kernel copy it to scratch memory first.
+struct SweepArgs {
+    const QueueState* q;
+    CombineState* cs;
+    const int32_t* pair_mt;
+    const int32_t* done1;
+    int32_t* combined;
+    const int32_t* pair_row;
+    const float* topk_w;
+    const void* y;
+    void* out;
+    int64_t* task_trace;
+    int32_t task_trace_cap;
+    int32_t S, k, H, nnt1;
+};
+__device__ __forceinline__ SweepArgs sweep_args(const FfnArgs& a) {
+    return SweepArgs{a.q, a.cs, a.pair_mt, a.done1, a.combined, a.pair_row, a.topk_w, a.y, a.out, a.task_trace, a.task_trace_cap,
+                     a.S, a.k, a.H, a.nnt1};
+}
+
+// U tokens x R ranks: the rows a thread has in flight together.  s_lds: kCombineLds ints -- [0, 16) the tokens to
+// combine, [16] their number, [17] finished down-projection tiles.
+template <class ET, int U, int R>
+__device__ __forceinline__ void combine_while_idle_body(const SweepArgs a, int* s_task, int* s_lds) {
+    constexpr int N = CmbElem<ET>::N;
+    const int cols = (int)blockDim.x * N;                 // columns of a slice
+    const int nslice = (a.H + cols - 1) / cols;
+    const int per_slice = (a.S + kCombineChunk - 1) / kCombineChunk;   // tasks per slice
+    const int nchunks = per_slice * nslice;
+    const int tid = threadIdx.x;
+    const int down_tasks = a.q->tasks_phase1;
+    int backoff = 0;
+    unsigned c = blockIdx.x % (unsigned)nchunks;
+    const unsigned stride = gridDim.x % (unsigned)nchunks;
+    for (int polls = 0; polls < (1 << 22); ++polls) {     // bounded like every loop here that looks at other workgroups' progress
+        if (tid == 0) s_lds[kCombineChunk + 1] = __hip_atomic_load(&a.cs->down_done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        const int done = __builtin_amdgcn_readfirstlane(s_lds[kCombineChunk + 1]);
+        __syncthreads();
+        if (done >= down_tasks) break;                    // every GEMM task is done: the launch behind us takes the rest
+        const long long started = trace_clock(a.task_trace);
+        const int slice = (int)c / per_slice, t0 = ((int)c - slice * per_slice) * kCombineChunk;
+        if (tid < kWave) {                                // the first wavefront, whole: lane i looks at token t0 + i
+            const int t = t0 + tid;
+            bool take = false;
+            if (tid < kCombineChunk && t < a.S) {
+                int32_t* flag = a.combined + (size_t)slice * a.S + t;
+                if (!__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) {
+                    take = true;
+                    for (int j = 0; j < a.k && take; ++j) {
+                        const int mt = a.pair_mt[(size_t)t * a.k + j];
+                        if (mt >= 0 && __hip_atomic_load(a.done1 + mt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < a.nnt1) take = false;
+                    }
+                    // complete: ours if nobody was faster
+                    if (take) take = __hip_atomic_exchange(flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0;
+                }
+            }
+            const unsigned long long go = __ballot(take);
+            if (take) s_lds[__popcll(go & ((1ull << tid) - 1ull))] = t;
+            if (tid == 0) s_lds[kCombineChunk] = __popcll(go);
+        }
+        __syncthreads();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");   // keeps the rows' loads behind the barrier
+        const int n = s_lds[kCombineChunk];
+        const int col = slice * cols + tid * N;
+        for (int g = 0; g < n; g += U) {                  // uniform: every thread reads the same list
+            int tok[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) tok[u] = g + u < n ? s_lds[g + u] : 0;
+            if (col < a.H) combine_tokens_fresh<ET, U, R>(a.y, a.pair_row, a.topk_w, tok, min(U, n - g), a.k, a.H, col, a.out);
+        }
+        if (n > 0) {
+            backoff = 0;
+            if (a.task_trace) trace_task(a.task_trace, a.task_trace_cap, 2, slice, (int)c, n, n, started);
+        } else {                                          // nothing complete here: look again later, and later still
+            backoff = min(backoff + 1, 2);                // (the kernel ends when the last sleeper has woken up: keep it short)
+            for (int i = 0; i < backoff; ++i) __builtin_amdgcn_s_sleep(127);   // 127 x 64 cycles, about 3.5 us
+        }
+        c += stride + 1;                                  // (stride + 1 and nchunks need not be coprime: every task is
+        if (c >= (unsigned)nchunks) c -= (unsigned)nchunks;   // some workgroup's, and the launch behind takes the rest)
+        if (c >= (unsigned)nchunks) c %= (unsigned)nchunks;
+    }
+}
+
+// The forms the kernels call.  The kernels that keep one workgroup per compute unit (the 16-bit tiles) have registers to
+// spare and nothing but the code itself to keep requests in flight: 32 rows at a time (16 tokens with up to 2 ranks, 8
+// with up to 4, 4 with more), in a function of its own so that the slab loop's register allocation never sees it.  The
+// kernels that keep two to four workgroups per compute unit get their overlap from that: two tokens at a time, inlined --
+// a function that is not inlined is compiled without regard to the occupancy its callers were written for, and a
+// kernel's register count is the larger of its own and its callees'.
+template <class ET>
+__device__ __noinline__ void combine_while_idle(const SweepArgs a, int* s_task, int* s_lds) {
+    if (a.k <= 2) combine_while_idle_body<ET, 16, 2>(a, s_task, s_lds);
+    else if (a.k <= 4) combine_while_idle_body<ET, 8, 4>(a, s_task, s_lds);
+    else combine_while_idle_body<ET, 4, 8>(a, s_task, s_lds);
+}
+template <class ET>
+__device__ __forceinline__ void combine_while_idle_narrow(const SweepArgs& a, int* s_task, int* s_lds) {
+    combine_while_idle_body<ET, 2, 4>(a, s_task, s_lds);
+}
+
+// What follows a stored down-projection tile: nothing (separate combine launch), the arrival counters, or the row
+// block's counter of finished tiles for the combine tasks of the queue.
+template <class ET>
+__device__ __forceinline__ void after_down_tile(const FfnArgs& a, int row0, int rows, int mtile, int ntile, int n0, int ncols,
+                                                int* s_list) {
+    if (a.arrive) {
+        combine_arrivals<ET>(combine_args(a), row0, rows, ntile, n0, ncols, s_list);
+    } else if (a.combined) {
+        signal_phase0_done(a.done1, mtile);
+        if (threadIdx.x == 0) __hip_atomic_fetch_add(&a.cs->down_done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+// Rows of y must be written through when another workgroup of the same launch will read them.
+__device__ __forceinline__ bool publish_y(const FfnArgs& a) { return a.arrive != nullptr || a.combined != nullptr; }
+
 // Workgroups of a tiled launch: every group's id space, holes included.
 inline int tiled_grid(int max_mtiles, int nnt, int groups) { return groups * max_mtiles * ((nnt + groups - 1) / groups); }
 

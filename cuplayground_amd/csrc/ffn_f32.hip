@@ -162,6 +162,7 @@ __global__ __launch_bounds__(256) void ffn_persistent_f32_kernel(FfnArgs a) {
     __shared__ __align__(16) float As[FBK][FBM + FPAD];
     __shared__ __align__(16) float Bs[FBK][FBN + FPAD];
     __shared__ int s_task, s_ok;
+    __shared__ int s_cmb[kCombineLds];
     __shared__ int s_list[1 + FBM];
     queue_kernel_entry();
     queue_clock_stamp(a.wg_clock, 0);
@@ -174,14 +175,15 @@ __global__ __launch_bounds__(256) void ffn_persistent_f32_kernel(FfnArgs a) {
     while (next_task(a, cur, &s_task, ids, nseg, nnt0, t)) {
         int ok = 1;
         if (t.phase == 1) ok = wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q, a.host_stall, &s_ok);
-        const TaskPtrsF p = resolve_f32(a, t, t.phase == 0 || a.arrive);
+        const TaskPtrsF p = resolve_f32(a, t, t.phase == 0 || publish_y(a));
         const long long started = trace_clock(a.task_trace);
         if (ok) gemm_tile_f32(p, As, Bs);
         else poison_tile(p.c_base, p.rows, p.N, p.n0, FBN, 4);
         if (a.task_trace) trace_task(a.task_trace, a.task_trace_cap, t.phase, t.expert, t.mtile, t.ntile, t.rows, started);
         if (t.phase == 0) signal_phase0_done(a.done0, t.mtile);
-        else if (a.arrive) combine_arrivals<float>(combine_args(a), t.row0, t.rows, t.ntile, p.n0, FBN, s_list);
+        else after_down_tile<float>(a, t.row0, t.rows, t.mtile, t.ntile, p.n0, FBN, s_list);
     }
+    if (a.combined) combine_while_idle_narrow<float>(sweep_args(a), &s_task, s_cmb);
     queue_clock_stamp(a.wg_clock, 1);
 }
 

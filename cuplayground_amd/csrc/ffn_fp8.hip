@@ -252,6 +252,7 @@ __global__ __launch_bounds__(256) void ffn_tiled_fp8_kernel(FfnArgs a, int phase
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void ffn_persistent_fp8_kernel(FfnArgs a) {
     __shared__ float red[QWAVES * QGROUPS * 4 * 64];
     __shared__ int s_task, s_ok;
+    __shared__ int s_cmb[kCombineLds];
     __shared__ int s_list[1 + QBM];
     queue_kernel_entry();
     queue_clock_stamp(a.wg_clock, 0);
@@ -266,15 +267,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         if (t.phase == 1) ok = wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q, a.host_stall, &s_ok);
         const long long started = trace_clock(a.task_trace);
         for (int sub = 0; sub < (t.phase ? QSUB1 : QSUB); ++sub) {
-            const Fp8Task p = resolve_fp8(a, t, sub, t.phase == 0 || a.arrive);
+            const Fp8Task p = resolve_fp8(a, t, sub, t.phase == 0 || publish_y(a));
             if (p.c0 >= p.N) continue;
             if (ok) fp8_tile(p, red);
             else poison_tile(p.c_base, p.rows, p.N, p.c0, QN1, 2);
         }
         if (a.task_trace) trace_task(a.task_trace, a.task_trace_cap, t.phase, t.expert, t.mtile, t.ntile, t.rows, started);
         if (t.phase == 0) signal_phase0_done(a.done0, t.mtile);
-        else if (a.arrive) combine_arrivals<bf16_s>(combine_args(a), t.row0, t.rows, t.ntile, t.ntile * QSUB1 * QN1, QSUB1 * QN1, s_list);
+        else after_down_tile<bf16_s>(a, t.row0, t.rows, t.mtile, t.ntile, t.ntile * QSUB1 * QN1, QSUB1 * QN1, s_list);
     }
+    if (a.combined) combine_while_idle_narrow<bf16_s>(sweep_args(a), &s_task, s_cmb);
     queue_clock_stamp(a.wg_clock, 1);
 }
 

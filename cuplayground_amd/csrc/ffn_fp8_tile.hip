@@ -367,6 +367,7 @@ __global__ __launch_bounds__(PTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
 __global__ __launch_bounds__(PTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void ffn_persistent_fp8_tile_kernel(FfnArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ int s_task, s_ok;
+    __shared__ int s_cmb[kCombineLds];
     __shared__ int s_list[1 + PBM];
     queue_kernel_entry();
     queue_clock_stamp(a.wg_clock, 0);
@@ -379,14 +380,15 @@ __global__ __launch_bounds__(PTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
     while (next_task(a, cur, &s_task, ids, nseg, nnt0, t)) {
         int ok = 1;
         if (t.phase == 1) ok = wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q, a.host_stall, &s_ok);
-        const TileTask p = resolve_tile(a, t, t.phase == 0 || a.arrive);
+        const TileTask p = resolve_tile(a, t, t.phase == 0 || publish_y(a));
         const long long started = trace_clock(a.task_trace);
         if (ok) fp8_gemm_tile(p, smem);
         else poison_tile(p.c_base, p.rows, p.N, p.c0, PN1, 2);
         if (a.task_trace) trace_task(a.task_trace, a.task_trace_cap, t.phase, t.expert, t.mtile, t.ntile, t.rows, started);
         if (t.phase == 0) signal_phase0_done(a.done0, t.mtile);
-        else if (a.arrive) combine_arrivals<bf16_s>(combine_args(a), t.row0, t.rows, t.ntile, p.c0, PN1, s_list);
+        else after_down_tile<bf16_s>(a, t.row0, t.rows, t.mtile, t.ntile, p.c0, PN1, s_list);
     }
+    if (a.combined) combine_while_idle_narrow<bf16_s>(sweep_args(a), &s_task, s_cmb);
     queue_clock_stamp(a.wg_clock, 1);
 }
 

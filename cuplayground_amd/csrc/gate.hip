@@ -235,80 +235,114 @@ __device__ __forceinline__ void widen8(const typename RawChunk<T>::type& r, floa
     }
 }
 
-template <typename T, int TT, int TE, int WT, int WE>
+// The token's top-k selection right behind its sums (FUSE): when the workgroup's WE x TE expert columns cover every
+// expert, the logits of its WT x TT tokens meet in LDS and each wavefront selects for its share of the tokens with the
+// very function the stand-alone top-k kernel runs -- one launch less, and the logits go to memory only when the caller
+// asked for them (`logits` may then be null).
+struct GateTopk {
+    int32_t* idx;       // [S, k]
+    float* w;           // [S, k]
+    int k, gate_fn, norm;
+};
+
+template <typename T, int TT, int TE, int WT, int WE, bool FUSE>
 __global__ __launch_bounds__(WT * WE * 64) void gate_tile_kernel(const T* __restrict__ x, const T* __restrict__ gate_w,
                                                                  const float* __restrict__ gate_bias,
-                                                                 float* __restrict__ logits, int S, int H, int E) {
+                                                                 float* __restrict__ logits, int S, int H, int E,
+                                                                 GateTopk tk) {
     static_assert((TT * TE) % 16 == 0 && 16 % TT == 0, "sums are folded sixteen at a time: TT tokens x 16/TT experts");
     typedef typename RawChunk<T>::type raw_t;
+    constexpr int ECOLS = WE * TE;                        // expert columns of a workgroup
+    __shared__ float s_log[FUSE ? WT * TT * ECOLS : 1];   // [token of the workgroup][expert]
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int t0 = (blockIdx.x * WT + wave / WE) * TT, e0 = (blockIdx.y * WE + wave % WE) * TE;
-    if (t0 >= S || e0 >= E) return;
-    const int nchunk = H >> 3, nstep = (nchunk + kWave - 1) / kWave;
-    const T* xrow[TT];
-    const T* wrow[TE];
+    const bool live = t0 < S && e0 < E;
+    if (!FUSE && !live) return;
+    if (live) {
+        const int nchunk = H >> 3, nstep = (nchunk + kWave - 1) / kWave;
+        const T* xrow[TT];
+        const T* wrow[TE];
 #pragma unroll
-    for (int q = 0; q < TT; ++q) xrow[q] = x + (size_t)min(t0 + q, S - 1) * H + lane * 8;    // rows past the end are
+        for (int q = 0; q < TT; ++q) xrow[q] = x + (size_t)min(t0 + q, S - 1) * H + lane * 8;    // rows past the end are
 #pragma unroll
-    for (int g = 0; g < TE; ++g) wrow[g] = gate_w + (size_t)min(e0 + g, E - 1) * H + lane * 8;   // computed, not stored
-    float acc[TT][TE];
+        for (int g = 0; g < TE; ++g) wrow[g] = gate_w + (size_t)min(e0 + g, E - 1) * H + lane * 8;   // computed, not stored
+        float acc[TT][TE];
 #pragma unroll
-    for (int q = 0; q < TT; ++q)
+        for (int q = 0; q < TT; ++q)
 #pragma unroll
-        for (int g = 0; g < TE; ++g) acc[q][g] = 0.0f;
-    raw_t xn[TT], wn[TE];
-    auto fetch = [&](int j) {
-        if (lane + j * kWave < nchunk) {
+            for (int g = 0; g < TE; ++g) acc[q][g] = 0.0f;
+        raw_t xn[TT], wn[TE];
+        auto fetch = [&](int j) {
+            if (lane + j * kWave < nchunk) {
 #pragma unroll
-            for (int q = 0; q < TT; ++q) xn[q] = *reinterpret_cast<const raw_t*>(xrow[q] + (size_t)j * (kWave * 8));
+                for (int q = 0; q < TT; ++q) xn[q] = *reinterpret_cast<const raw_t*>(xrow[q] + (size_t)j * (kWave * 8));
 #pragma unroll
-            for (int g = 0; g < TE; ++g) wn[g] = *reinterpret_cast<const raw_t*>(wrow[g] + (size_t)j * (kWave * 8));
+                for (int g = 0; g < TE; ++g) wn[g] = *reinterpret_cast<const raw_t*>(wrow[g] + (size_t)j * (kWave * 8));
+            }
+        };
+        fetch(0);
+        for (int j = 0; j < nstep; ++j) {
+            raw_t xc[TT], wc[TE];
+#pragma unroll
+            for (int q = 0; q < TT; ++q) xc[q] = xn[q];
+#pragma unroll
+            for (int g = 0; g < TE; ++g) wc[g] = wn[g];
+            if (j + 1 < nstep) fetch(j + 1);
+            if (lane + j * kWave < nchunk) {      // partial sum `lane` takes chunk lane + 64 j only if the row has it
+                float xv[TT][8];
+#pragma unroll
+                for (int q = 0; q < TT; ++q) widen8<T>(xc[q], xv[q]);
+#pragma unroll
+                for (int g = 0; g < TE; ++g) {
+                    float wv[8];
+                    widen8<T>(wc[g], wv);
+#pragma unroll
+                    for (int q = 0; q < TT; ++q)
+#pragma unroll
+                        for (int v = 0; v < 8; ++v) acc[q][g] = __builtin_fmaf(xv[q][v], wv[v], acc[q][g]);
+                }
+            }
         }
-    };
-    fetch(0);
-    for (int j = 0; j < nstep; ++j) {
-        raw_t xc[TT], wc[TE];
+        constexpr int EG = 16 / TT;       // experts per fold
+        const int r = fold16_index(lane);
 #pragma unroll
-        for (int q = 0; q < TT; ++q) xc[q] = xn[q];
+        for (int gb = 0; gb < TE; gb += EG) {
+            float red[16];
 #pragma unroll
-        for (int g = 0; g < TE; ++g) wc[g] = wn[g];
-        if (j + 1 < nstep) fetch(j + 1);
-        if (lane + j * kWave < nchunk) {      // partial sum `lane` takes chunk lane + 64 j only if the row has it
-            float xv[TT][8];
+            for (int g = 0; g < EG; ++g)
 #pragma unroll
-            for (int q = 0; q < TT; ++q) widen8<T>(xc[q], xv[q]);
-#pragma unroll
-            for (int g = 0; g < TE; ++g) {
-                float wv[8];
-                widen8<T>(wc[g], wv);
-#pragma unroll
-                for (int q = 0; q < TT; ++q)
-#pragma unroll
-                    for (int v = 0; v < 8; ++v) acc[q][g] = __builtin_fmaf(xv[q][v], wv[v], acc[q][g]);
+                for (int q = 0; q < TT; ++q) red[g * TT + q] = acc[q][gb + g];
+            const float sum = fold16(red, lane);
+            const int e = e0 + gb + r / TT, t = t0 + r % TT;
+            if ((lane & 3) == 0 && e < E && t < S) {
+                const float val = gate_bias ? sum + gate_bias[e] : sum;
+                if (!FUSE || logits) logits[(size_t)t * E + e] = val;
+                if (FUSE) s_log[((wave / WE) * TT + r % TT) * ECOLS + e] = val;     // one expert tile per row: e < ECOLS
             }
         }
     }
-    constexpr int EG = 16 / TT;       // experts per fold
-    const int r = fold16_index(lane);
-#pragma unroll
-    for (int gb = 0; gb < TE; gb += EG) {
-        float red[16];
-#pragma unroll
-        for (int g = 0; g < EG; ++g)
-#pragma unroll
-            for (int q = 0; q < TT; ++q) red[g * TT + q] = acc[q][gb + g];
-        const float sum = fold16(red, lane);
-        const int e = e0 + gb + r / TT, t = t0 + r % TT;
-        if ((lane & 3) == 0 && e < E && t < S) logits[(size_t)t * E + e] = gate_bias ? sum + gate_bias[e] : sum;
+    if constexpr (FUSE) {
+        __syncthreads();
+        for (int q = wave; q < WT * TT; q += WT * WE) {   // this wavefront's share of the workgroup's tokens
+            const int t = blockIdx.x * (WT * TT) + q;
+            if (t < S) topk_one_token<1>(s_log + q * ECOLS, t, E, tk.k, tk.gate_fn, tk.norm, tk.idx, tk.w, lane);
+        }
     }
 }
 
+// Returns through *fused whether the launch also selected (tk non-null and every expert in one workgroup's columns).
 template <typename T, int TT, int TE, int WT, int WE>
-hipError_t launch_gate_tile(const void* x, const void* gate_w, const float* gate_bias, float* logits, int S, int H,
-                            int E, hipStream_t st) {
+hipError_t launch_gate_tile(const void* x, const void* gate_w, const float* gate_bias, float* logits, bool keep_logits,
+                            int S, int H, int E, const GateTopk* tk, bool* fused, hipStream_t st) {
     const dim3 grid((S + WT * TT - 1) / (WT * TT), (E + WE * TE - 1) / (WE * TE));
-    gate_tile_kernel<T, TT, TE, WT, WE><<<grid, WT * WE * 64, 0, st>>>((const T*)x, (const T*)gate_w, gate_bias, logits,
-                                                                      S, H, E);
+    if (tk && grid.y == 1) {
+        gate_tile_kernel<T, TT, TE, WT, WE, true><<<grid, WT * WE * 64, 0, st>>>((const T*)x, (const T*)gate_w, gate_bias,
+                                                                                keep_logits ? logits : nullptr, S, H, E, *tk);
+        *fused = true;
+    } else {
+        gate_tile_kernel<T, TT, TE, WT, WE, false><<<grid, WT * WE * 64, 0, st>>>((const T*)x, (const T*)gate_w, gate_bias,
+                                                                                 logits, S, H, E, GateTopk{});
+    }
     return hipGetLastError();
 }
 
@@ -316,22 +350,21 @@ hipError_t launch_gate_tile(const void* x, const void* gate_w, const float* gate
 // the layer is decode-sized and only more wavefronts bring more loads in flight; a 4 x 1 wavefront arrangement when
 // the experts fit one wavefront's tile.
 template <typename T>
-hipError_t launch_gate_tiled(const void* x, const void* gate_w, const float* gate_bias, float* logits, int S, int H,
-                             int E, int opt_tile, hipStream_t st) {
+hipError_t launch_gate_tiled(const void* x, const void* gate_w, const float* gate_bias, float* logits, bool keep_logits,
+                             int S, int H, int E, int opt_tile, const GateTopk* tk, bool* fused, hipStream_t st) {
     const int64_t pairs = (int64_t)S * E;
     int variant = pairs >= 32768 ? 0 : 1;
     if (opt_tile >= 0 && opt_tile <= 2) variant = opt_tile;
+#define MOE355_GATE_TILE_ARGS x, gate_w, gate_bias, logits, keep_logits, S, H, E, tk, fused, st
     switch (variant) {
         case 0:
-            return E <= 8 ? launch_gate_tile<T, 4, 8, 4, 1>(x, gate_w, gate_bias, logits, S, H, E, st)
-                          : launch_gate_tile<T, 4, 8, 2, 2>(x, gate_w, gate_bias, logits, S, H, E, st);
+            return E <= 8 ? launch_gate_tile<T, 4, 8, 4, 1>(MOE355_GATE_TILE_ARGS) : launch_gate_tile<T, 4, 8, 2, 2>(MOE355_GATE_TILE_ARGS);
         case 1:
-            return E <= 4 ? launch_gate_tile<T, 4, 4, 4, 1>(x, gate_w, gate_bias, logits, S, H, E, st)
-                          : launch_gate_tile<T, 4, 4, 2, 2>(x, gate_w, gate_bias, logits, S, H, E, st);
+            return E <= 4 ? launch_gate_tile<T, 4, 4, 4, 1>(MOE355_GATE_TILE_ARGS) : launch_gate_tile<T, 4, 4, 2, 2>(MOE355_GATE_TILE_ARGS);
         default:
-            return E <= 8 ? launch_gate_tile<T, 2, 8, 4, 1>(x, gate_w, gate_bias, logits, S, H, E, st)
-                          : launch_gate_tile<T, 2, 8, 2, 2>(x, gate_w, gate_bias, logits, S, H, E, st);
+            return E <= 8 ? launch_gate_tile<T, 2, 8, 4, 1>(MOE355_GATE_TILE_ARGS) : launch_gate_tile<T, 2, 8, 2, 2>(MOE355_GATE_TILE_ARGS);
     }
+#undef MOE355_GATE_TILE_ARGS
 }
 
 // ---- third logits kernel: the same sums on the matrix cores (16-bit layers, H a multiple of 512) ----
@@ -350,16 +383,20 @@ hipError_t launch_gate_tiled(const void* x, const void* gate_w, const float* gat
 // then with p + 2 and p + 1 (b) in the lane again -- the pairings of fold16, so the logits are bit-identical.
 typedef float gate_f32x16 __attribute__((ext_vector_type(16)));
 
-template <typename T>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gate_mfma_kernel(const T* __restrict__ x, const T* __restrict__ gate_w,
+// PAIRS wavefront pairs per workgroup, 16 expert columns each.  FUSE: the workgroup's columns cover every expert
+// (grid.y == 1) and the selection follows right behind the sums, as in gate_tile_kernel.
+template <typename T, int PAIRS, bool FUSE>
+__global__ __launch_bounds__(PAIRS * 128) __attribute__((amdgpu_waves_per_eu(2, 2))) void gate_mfma_kernel(const T* __restrict__ x, const T* __restrict__ gate_w,
                                                         const float* __restrict__ gate_bias, float* __restrict__ logits,
-                                                        int S, int H, int E) {
+                                                        int S, int H, int E, GateTopk tk) {
     typedef typename RawChunk<T>::type raw_t;
-    __shared__ float s_odd[2][16][64];          // [pair][4 b + r][lane]: the odd wavefront's sums over its g
+    constexpr int ECOLS = PAIRS * 16;
+    __shared__ float s_odd[PAIRS][16][64];      // [pair][4 b + r][lane]: the odd wavefront's sums over its g
+    __shared__ float s_log[FUSE ? 16 * ECOLS : 1];   // [token of the tile][expert]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int pair = wave >> 1, odd = wave & 1;
     const int b = lane >> 4, i = lane & 15;
-    const int t0 = blockIdx.x * 16, e0 = (blockIdx.y * 2 + pair) * 16;
+    const int t0 = blockIdx.x * 16, e0 = (blockIdx.y * PAIRS + pair) * 16;
     const bool live = e0 < E;                   // an expert tile past the last one: nothing to do, but meet the barrier
     gate_f32x16 acc[8];
 #pragma unroll
@@ -414,31 +451,57 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int v = 0; v < 16; ++v) s_odd[pair][v][lane] = u[v];
     }
     __syncthreads();
-    if (odd || !live) return;
-    const int e = e0 + i;
+    if (!FUSE && (odd || !live)) return;
+    if (!odd && live) {
+        const int e = e0 + i;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        float q[4];
+        for (int r = 0; r < 4; ++r) {
+            float q[4];
 #pragma unroll
-        for (int bb = 0; bb < 4; ++bb) q[bb] = u[4 * bb + r] + s_odd[pair][4 * bb + r][lane];     // ... p + 4
-        const float sum = (q[0] + q[2]) + (q[1] + q[3]);                                           // ... p + 2, p + 1
-        const int t = t0 + 4 * b + r;
-        if (t < S && e < E) logits[(size_t)t * E + e] = gate_bias ? sum + gate_bias[e] : sum;
+            for (int bb = 0; bb < 4; ++bb) q[bb] = u[4 * bb + r] + s_odd[pair][4 * bb + r][lane];     // ... p + 4
+            const float sum = (q[0] + q[2]) + (q[1] + q[3]);                                           // ... p + 2, p + 1
+            const int t = t0 + 4 * b + r;
+            if (t < S && e < E) {
+                const float val = gate_bias ? sum + gate_bias[e] : sum;
+                if (!FUSE || logits) logits[(size_t)t * E + e] = val;
+                if (FUSE) s_log[(4 * b + r) * ECOLS + e] = val;                       // grid.y == 1: e < ECOLS
+            }
+        }
+    }
+    if constexpr (FUSE) {
+        __syncthreads();
+        for (int q = wave; q < 16; q += 2 * PAIRS) {      // this wavefront's share of the tile's tokens
+            const int t = t0 + q;
+            if (t < S) topk_one_token<1>(s_log + q * ECOLS, t, E, tk.k, tk.gate_fn, tk.norm, tk.idx, tk.w, lane);
+        }
     }
 }
 
 // The matrix-core kernel takes 16-bit layers whose rows split into full steps of 512 elements, when the experts fill
-// most of its 16 columns and there are enough 16 x 16 tiles for every SIMD of the chip to get several.
+// most of its 16 columns and there are enough 16 x 16 tiles for every SIMD of the chip to get several.  With at most 64
+// experts one workgroup holds them all (two or four wavefront pairs) and selects as well (*fused).
 template <typename T>
-bool launch_gate_mfma(const void* x, const void* gate_w, const float* gate_bias, float* logits, int S, int H, int E,
-                      int opt_mfma, hipStream_t st, hipError_t* err) {
+bool launch_gate_mfma(const void* x, const void* gate_w, const float* gate_bias, float* logits, bool keep_logits, int S,
+                      int H, int E, int opt_mfma, const GateTopk* tk, bool wide_fusion, bool* fused, hipStream_t st,
+                      hipError_t* err) {
     if (H % 512 != 0) return false;
     const int et = (E + 15) / 16;
     bool use = et * 16 * 3 <= E * 4 && (int64_t)((S + 15) / 16) * et >= 2048;
     if (opt_mfma != MOE_OPT_AUTO) use = opt_mfma != 0;
     if (!use) return false;
-    const dim3 grid((S + 15) / 16, (et + 1) / 2);
-    gate_mfma_kernel<T><<<grid, 256, 0, st>>>((const T*)x, (const T*)gate_w, gate_bias, logits, S, H, E);
+    const unsigned tiles = (unsigned)((S + 15) / 16);
+    if (tk && et <= 2) {
+        gate_mfma_kernel<T, 2, true><<<dim3(tiles, 1), 256, 0, st>>>((const T*)x, (const T*)gate_w, gate_bias,
+                                                                    keep_logits ? logits : nullptr, S, H, E, *tk);
+        *fused = true;
+    } else if (tk && et <= 4 && wide_fusion) {   // on request only: the 512-thread form measured 17 us slower than two launches
+        gate_mfma_kernel<T, 4, true><<<dim3(tiles, 1), 512, 0, st>>>((const T*)x, (const T*)gate_w, gate_bias,
+                                                                    keep_logits ? logits : nullptr, S, H, E, *tk);
+        *fused = true;
+    } else {
+        gate_mfma_kernel<T, 2, false><<<dim3(tiles, (et + 1) / 2), 256, 0, st>>>((const T*)x, (const T*)gate_w, gate_bias,
+                                                                                logits, S, H, E, GateTopk{});
+    }
     *err = hipGetLastError();
     return true;
 }
@@ -451,7 +514,7 @@ __global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ log
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int t = blockIdx.x * 4 + wave;
     if (t >= S) return;
-    topk_one_token<J>(logits, t, E, k, gate_fn, norm, topk_idx, topk_w, lane);
+    topk_one_token<J>(logits + (size_t)t * E, t, E, k, gate_fn, norm, topk_idx, topk_w, lane);
 }
 
 // Router statistics for a load-balancing loss.  Block b, wavefront w takes tokens (4b + w) + 4*gridDim.x*i; a lane
@@ -550,14 +613,17 @@ hipError_t launch_router_stats(const float* logits, const int32_t* topk_idx, int
     return hipGetLastError();
 }
 
-hipError_t launch_gate_logits(const void* x, const void* gate_w, const float* gate_bias, float* logits, int S, int H,
-                              int E, int act_dtype, const moe_options& opt, hipStream_t st) {
+// Logits kernel by shape; *fused (when tk is given) says whether that launch has selected as well.
+static hipError_t launch_gate_logits(const void* x, const void* gate_w, const float* gate_bias, float* logits, bool keep_logits,
+                                     int S, int H, int E, int act_dtype, const moe_options& opt, const GateTopk* tk, bool* fused,
+                                     hipStream_t st) {
     // Many experts on many tokens: the first kernel (token rows in registers, experts streamed) reads least per sum.
     // Everything else -- few experts, or decode-sized batches -- goes to the register-tiled kernel.
     if (act_dtype != MOE_DTYPE_F32) {
         hipError_t e = hipSuccess;
-        const bool taken = act_dtype == MOE_DTYPE_FP16 ? launch_gate_mfma<f16_s>(x, gate_w, gate_bias, logits, S, H, E, opt.gate_mfma, st, &e)
-                                                       : launch_gate_mfma<bf16_s>(x, gate_w, gate_bias, logits, S, H, E, opt.gate_mfma, st, &e);
+        const bool taken = act_dtype == MOE_DTYPE_FP16
+            ? launch_gate_mfma<f16_s>(x, gate_w, gate_bias, logits, keep_logits, S, H, E, opt.gate_mfma, tk, opt.gate_fused_topk == 1, fused, st, &e)
+            : launch_gate_mfma<bf16_s>(x, gate_w, gate_bias, logits, keep_logits, S, H, E, opt.gate_mfma, tk, opt.gate_fused_topk == 1, fused, st, &e);
         if (taken) return e;
     }
     bool rows_in_registers = E >= 32 && (int64_t)S * E >= ((int64_t)1 << 19);
@@ -567,12 +633,12 @@ hipError_t launch_gate_logits(const void* x, const void* gate_w, const float* ga
         if (act_dtype == MOE_DTYPE_FP16) return launch_gate_typed<f16_s>(x, gate_w, gate_bias, logits, S, H, E, st);
         return launch_gate_typed<bf16_s>(x, gate_w, gate_bias, logits, S, H, E, st);
     }
-    if (act_dtype == MOE_DTYPE_F32) return launch_gate_tiled<float>(x, gate_w, gate_bias, logits, S, H, E, opt.gate_tile, st);
-    if (act_dtype == MOE_DTYPE_FP16) return launch_gate_tiled<f16_s>(x, gate_w, gate_bias, logits, S, H, E, opt.gate_tile, st);
-    return launch_gate_tiled<bf16_s>(x, gate_w, gate_bias, logits, S, H, E, opt.gate_tile, st);
+    if (act_dtype == MOE_DTYPE_F32) return launch_gate_tiled<float>(x, gate_w, gate_bias, logits, keep_logits, S, H, E, opt.gate_tile, tk, fused, st);
+    if (act_dtype == MOE_DTYPE_FP16) return launch_gate_tiled<f16_s>(x, gate_w, gate_bias, logits, keep_logits, S, H, E, opt.gate_tile, tk, fused, st);
+    return launch_gate_tiled<bf16_s>(x, gate_w, gate_bias, logits, keep_logits, S, H, E, opt.gate_tile, tk, fused, st);
 }
 
-hipError_t launch_topk(const float* logits, int S, int E, int k, int gate_fn, int norm, int32_t* topk_idx,
+static hipError_t launch_topk(const float* logits, int S, int E, int k, int gate_fn, int norm, int32_t* topk_idx,
                        float* topk_w, hipStream_t st) {
     const unsigned grid = (unsigned)((S + 3) / 4);
     if (E <= 64) topk_kernel<1><<<grid, 256, 0, st>>>(logits, S, E, k, gate_fn, norm, topk_idx, topk_w);
@@ -580,6 +646,20 @@ hipError_t launch_topk(const float* logits, int S, int E, int k, int gate_fn, in
     else if (E <= 256) topk_kernel<4><<<grid, 256, 0, st>>>(logits, S, E, k, gate_fn, norm, topk_idx, topk_w);
     else topk_kernel<kMaxExperts / kWave><<<grid, 256, 0, st>>>(logits, S, E, k, gate_fn, norm, topk_idx, topk_w);
     return hipGetLastError();
+}
+
+// The router: logits, selection, weights.  One launch where the logits kernel of the shape can hold every expert of a
+// token in one workgroup (option gate_fused_topk, on unless 0), else the logits kernel followed by the top-k kernel.
+// `logits` is always valid scratch [S, E]; with keep_logits false it is written only when the two-launch form needs it.
+hipError_t launch_gate(const void* x, const void* gate_w, const float* gate_bias, float* logits, bool keep_logits, int S,
+                       int H, int E, int k, int gate_fn, int norm, int32_t* topk_idx, float* topk_w, int act_dtype,
+                       const moe_options& opt, hipStream_t st) {
+    const GateTopk tk{topk_idx, topk_w, k, gate_fn, norm};
+    bool fused = false;
+    const hipError_t e = launch_gate_logits(x, gate_w, gate_bias, logits, keep_logits, S, H, E, act_dtype, opt,
+                                            opt.gate_fused_topk == 0 ? nullptr : &tk, &fused, st);
+    if (e != hipSuccess || fused) return e;
+    return launch_topk(logits, S, E, k, gate_fn, norm, topk_idx, topk_w, st);
 }
 
 }  // namespace moe355

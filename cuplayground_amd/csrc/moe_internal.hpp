@@ -78,6 +78,12 @@ struct QueueState {
     int32_t ids_phase1;
     int32_t pad[5];
 };
+// State of the combine tasks of the queue kernels, in a cache line of its own: the workgroups that have run out of GEMM
+// tasks poll it, and must not stand in the way of the queue heads that the busy ones pop.
+struct CombineState {
+    int32_t down_done;         // down-projection tiles finished so far (the combine tasks stop when all are)
+    int32_t pad[63];
+};
 
 // Everything the FFN kernels need; passed by value.
 struct FfnArgs {
@@ -117,6 +123,12 @@ struct FfnArgs {
     void* out;                  // [S, H] in the activation type
     int32_t S, k, nnt1;
     int32_t drop;               // tokens may have lost every pair: their output rows are zeroed at kernel entry
+    // Combine as tasks of the queue kernel (null `combined`: not used).  A unit is (token, slice of 256 x 16 bytes of
+    // its row); combined[unit] is set by the workgroup that takes the unit.
+    int32_t* done1;             // per MTile: finished phase-1 column tiles
+    const int32_t* pair_mt;     // [S, k] row block (MTile index) of every (token, rank), -1 when dropped
+    int32_t* combined;          // [slices, S]: 1 once the unit has been taken
+    CombineState* cs;
 };
 constexpr int kMaxQueueWorkgroups = 4096;   // workgroups of a queue kernel that get a slot in wg_clock
 
@@ -135,7 +147,11 @@ struct RouteArgs {
     Segment* seg_queue;
     QueueState* q;
     int32_t* done0;
-    int32_t* arrive;            // [S, nnt1] arrival counters of the fused combine (null: not used), cleared here
+    int32_t* arrive;            // null, or counters of the combine inside the FFN kernels, cleared here: arrive_n of them
+    int32_t arrive_n;
+    int32_t* done1;             // null, or per MTile the finished phase-1 column tiles (combine as queue tasks), cleared here
+    int32_t* pair_mt;           // [A] row block of every pair (-1: dropped)
+    CombineState* cs;           // null, or the state of the combine tasks, cleared here
     int32_t S, k, E, A, nblk;
     int32_t drop;
     int32_t capacity;
@@ -148,18 +164,19 @@ struct RouteArgs {
 };
 
 // ---- launchers (defined next to their kernels) ----
-// gate_kernel / gate_mfma / gate_tile: the handle's options of those names (MOE_OPT_AUTO: chosen from the shape)
-hipError_t launch_gate_logits(const void* x, const void* gate_w, const float* gate_bias, float* logits, int S, int H,
-                              int E, int act_dtype, const moe_options& opt, hipStream_t st);
-hipError_t launch_topk(const float* logits, int S, int E, int k, int gate_fn, int norm, int32_t* topk_idx,
-                       float* topk_w, hipStream_t st);
+// Router: logits, top-k, weights (gate.hip).  opt: the handle's options gate_kernel / gate_mfma / gate_tile /
+// gate_fused_topk (MOE_OPT_AUTO: chosen from the shape).
+hipError_t launch_gate(const void* x, const void* gate_w, const float* gate_bias, float* logits, bool keep_logits, int S,
+                       int H, int E, int k, int gate_fn, int norm, int32_t* topk_idx, float* topk_w, int act_dtype,
+                       const moe_options& opt, hipStream_t st);
 constexpr int kStatsBlocks = 64;   // per-block partials of the router statistics kept in the workspace
 hipError_t launch_router_stats(const float* logits, const int32_t* topk_idx, int S, int E, int k, int gate_fn,
                                double* part_prob, int32_t* part_cnt, float* load, float* mean_prob, float* aux_loss,
                                hipStream_t st);
 hipError_t launch_route(const RouteArgs& a, hipStream_t st);
+// taken: null, or [slices, S] flags of the (token, slice of 256 x 16 bytes) units that are already combined and are skipped
 hipError_t launch_combine(const void* y_rows, const int32_t* pair_row, const float* topk_w, int S, int k, int H,
-                          int act_dtype, void* out, hipStream_t st);
+                          int act_dtype, void* out, const int32_t* taken, hipStream_t st);
 
 // FFN stage.  block_m / block_n are the tile sizes the routing stage must be told about.
 struct FfnPlan {

@@ -61,7 +61,7 @@ __device__ __forceinline__ void route_count_body(const RouteArgs& a, int blk, in
 // The arrival counters of the fused combine start every call at zero.
 __device__ __forceinline__ void clear_arrivals(const RouteArgs& a, int first, int stride) {
     if (!a.arrive) return;
-    const int n = a.S * a.nnt1;
+    const int n = a.arrive_n;
     for (int i = first; i < n; i += stride) a.arrive[i] = 0;
 }
 
@@ -193,6 +193,7 @@ __device__ __forceinline__ void route_scan_body(const RouteArgs& a, ScanShared& 
     if (e == 0) {
         a.q->groups = a.groups;
         for (int g = 0; g < kMaxQueueGroups; ++g) a.q->heads[g] = 0;
+        if (a.cs) a.cs->down_done = 0;
         if (a.task_trace) a.task_trace[0] = 0;
         a.q->ids_queue = total_tasks;
         a.q->ids_phase0 = total_mt * npg0;
@@ -221,6 +222,8 @@ __device__ __forceinline__ void route_scan_body(const RouteArgs& a, ScanShared& 
         }
     }
     for (int i = threadIdx.x; i < a.max_mtiles; i += blockDim.x) a.done0[i] = 0;
+    if (a.done1)
+        for (int i = threadIdx.x; i < a.max_mtiles; i += blockDim.x) a.done1[i] = 0;
 }
 
 __global__ __launch_bounds__(kMaxExperts) void route_scan_kernel(RouteArgs a) {
@@ -239,6 +242,7 @@ __device__ __forceinline__ void route_finalize_pair(const RouteArgs& a, int p) {
     const int row = dropped ? -1 : a.expert_offset[e] + s;
     a.slot[p] = dropped ? -1 : s;
     a.pair_row[p] = row;
+    if (a.pair_mt) a.pair_mt[p] = dropped ? -1 : a.seg_phase0[e].mt0 + s / a.block_m;
     if (!dropped) a.token_indices[row] = p / a.k;
     if (p >= a.expert_offset[a.E]) a.token_indices[p] = -1;   // rows past the last kept one
 }

@@ -44,13 +44,14 @@ __device__ __forceinline__ Cand wave_best(Cand c) {
     return best;
 }
 
+// `row`: the E logits of token t (global memory, or LDS when the logits kernel selects right behind its sums).
 // Lane l keeps the logits of experts l, l+64, ... (J of them; J * 64 >= E) in registers.  Called by all 64 lanes of a
 // wavefront.  J is a template parameter so that layers with up to 64 experts do not walk eight slots per step.
 // The selection is total: a NaN logit ranks as -inf (behind every number, ties to the lower index), so a token row
 // that overflowed still gets k distinct, valid experts; its weights are computed from the logits as they are and
 // come out NaN, which is what reaches the output of that token and of no other.
 template <int J>
-__device__ __forceinline__ void topk_one_token(const float* __restrict__ logits, int t, int E, int k, int gate_fn,
+__device__ __forceinline__ void topk_one_token(const float* __restrict__ row, int t, int E, int k, int gate_fn,
                                                int norm, int32_t* __restrict__ topk_idx, float* __restrict__ topk_w,
                                                int lane) {
     static_assert(J >= 1 && J <= kMaxExperts / kWave, "slots per lane");
@@ -61,7 +62,7 @@ __device__ __forceinline__ void topk_one_token(const float* __restrict__ logits,
         const int e = j * kWave + lane;
         v[j] = 0.0f;
         if (e < E) {
-            v[j] = logits[(size_t)t * E + e];
+            v[j] = row[e];
             avail |= 1u << j;
         }
     }

@@ -23,7 +23,8 @@ import torch
 
 from . import api
 
-PACKED_KEYS = ("gate_w", "gate_bias", "w_up", "w_gate", "w_down", "b_up", "b_gate", "b_down", "s_up", "s_gate", "s_down")
+PACKED_KEYS = ("gate_w", "gate_bias", "w_up", "w_gate", "w_down", "b_up", "b_gate", "b_down", "s_up", "s_gate", "s_down",
+               "prepared")
 
 
 def pack_experts(gate_w: torch.Tensor, up: Sequence[torch.Tensor], down: Sequence[torch.Tensor],
@@ -87,8 +88,22 @@ def quantize_packed(packed: Mapping[str, torch.Tensor]) -> Dict[str, torch.Tenso
     return out
 
 
+def prepare_packed(packed: Mapping[str, torch.Tensor], layer: "api.MoELayer") -> Dict[str, torch.Tensor]:
+    """Adds the kernel-ready operands of `layer`'s plan (`moe_prepare_weights`) to a packed set under the key
+    "prepared" -- today the bf16 copies an e4m3 layer with many rows per expert would otherwise make in every call.
+    They belong to the plan of `layer` (shape, dtype and options); a packed set saved with them serves handles of the
+    same plan.  Returns `packed` unchanged when the plan prepares nothing."""
+    out = dict(packed)
+    out.pop("prepared", None)
+    prepared = layer.prepare_weights(out)
+    if prepared is not None:
+        out["prepared"] = prepared
+    return out
+
+
 def save_packed(path: str, packed: Mapping[str, torch.Tensor], cfg: api.MoEConfig) -> None:
-    """One safetensors file: the tensors under the argument names of `moe_forward`, the knob file in the metadata."""
+    """One safetensors file: the tensors under the argument names of `moe_forward` (the prepared operands included when
+    the set carries them), the knob file in the metadata."""
     from safetensors.torch import save_file
     unknown = set(packed) - set(PACKED_KEYS)
     if unknown:
@@ -110,5 +125,5 @@ def load_packed(path: str, device="cuda"):
     return tensors, api.MoEConfig.from_json(meta["moe355_config"])
 
 
-__all__ = ["pack_experts", "pack_mixtral_block", "mixtral_config", "quantize_packed", "save_packed", "load_packed",
+__all__ = ["pack_experts", "pack_mixtral_block", "mixtral_config", "quantize_packed", "prepare_packed", "save_packed", "load_packed",
            "PACKED_KEYS"]

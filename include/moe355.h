@@ -143,7 +143,10 @@ typedef struct moe_options {
     int32_t fp8_mfma;        /* e4m3 layers on the tile GEMM: 1 = tokens quantised to e4m3 per (row, 128-wide k block) and
                                 the products taken by the fp8 matrix instructions; 0 = bf16 tokens, weights widened.  Not
                                 bit-compatible with 0: see moe_get_kernel_dtype. */
-    int32_t reserved[8];     /* must be MOE_OPT_AUTO */
+    int32_t prepared_weights;/* 1 = every moe_forward on the handle will carry moe_weights.prepared (moe_prepare_weights): the
+                                workspace then holds no copies of the weights and a call without them is refused; 0 / AUTO =
+                                prepared weights are used when given, else made per call in the workspace */
+    int32_t reserved[7];     /* must be MOE_OPT_AUTO */
 } moe_options;
 /* Every field MOE_OPT_AUTO. */
 int moe_options_default(moe_options* opt);
@@ -184,6 +187,7 @@ typedef struct moe_weights {
     const float* s_up;        /* fp8 only */
     const float* s_gate;
     const float* s_down;
+    const void* prepared;     /* NULL, or what moe_prepare_weights wrote for these weights on this handle */
 } moe_weights;
 
 /* Optional device buffers receiving the routing result (any member may be NULL). */
@@ -195,6 +199,19 @@ typedef struct moe_routing_out {
     int32_t* expert_offset;   /* [E]   exclusive scan of expert_count                           */
     int32_t* token_indices;   /* [S*k] token of each packed row, -1 past the last kept row      */
 } moe_routing_out;
+
+/*
+ * Kernel-ready operands, made once.  The reference keeps its operands resident in one arena for the life of a run
+ * (mma.cuh:385-391); here whatever a handle's plan would otherwise derive from the weights in every call is written
+ * once into a buffer of the caller and handed back through moe_weights.prepared: today the bf16 copies of an e4m3
+ * layer's expert weights on the widening plan (moe_get_kernel_dtype; 2 bytes per weight, moe_prepared_bytes says how
+ * many, 0 when the plan prepares nothing -- then moe_prepare_weights does nothing and `prepared` may stay NULL).
+ * The buffer is device memory, 256-byte aligned; its contents belong to (weights, handle plan) and stay valid as long as
+ * both do; the original weights and scales are still passed with every call (the router and any plan change need
+ * them).  Results are bit-identical to the per-call preparation.  Asynchronous on `stream`.
+ */
+int moe_prepared_bytes(const moe_handle* h, size_t* bytes);
+int moe_prepare_weights(moe_handle* h, const moe_weights* w, void* prepared, size_t prepared_bytes, void* stream);
 
 /* Variants of the FFN stage; MOE_FFN_AUTO lets the library choose. */
 enum { MOE_FFN_AUTO = 0, MOE_FFN_TILED = 1 /* one launch per GEMM */, MOE_FFN_PERSISTENT = 2 /* task queue */ };

@@ -87,3 +87,58 @@ def test_plan_widens_from_a_thousand_rows_per_expert():
     rows = 2 * (2048 - 1024) * (256 + 256) * 2
     assert big.workspace_bytes - mid.workspace_bytes >= 3 * 4 * 256 * 256 * 2 + rows
     mid.close(); big.close()
+
+
+@pytest.mark.parametrize("mode", [FFN_TILED, FFN_PERSISTENT], ids=["tiled", "persistent"])
+def test_prepared_weights_change_no_bit_and_save_the_workspace(mode, tmp_path):
+    """moe_prepare_weights writes the bf16 copies once; a forward call that carries them skips the widening launches and
+    must reproduce the per-call result bit for bit.  A handle created with prepared_weights = 1 asks for a workspace
+    without the copies and refuses a call that comes without them.  The prepared form survives a trip through a
+    packed-layer file."""
+    import torch
+    import cuplayground_amd as moe
+    from cuplayground_amd import weights as wts
+    cfg = SHAPES["swiglu"]
+    inp = ob.make_inputs(cfg, seed=41)
+    dev = upload_inputs(cfg, inp)
+    per_call = _forward(cfg, dev, mode, 1)
+
+    layer = moe.MoELayer(product_config(cfg), ffn_mode=mode, options={"fp8_widen": 1, "fp8_mfma": 0, "prepared_weights": 1})
+    assert layer.options["prepared_weights"] == 1
+    assert layer.prepared_bytes == 3 * cfg.E * cfg.H * cfg.I * 2
+    assert per_call["workspace_bytes"] - layer.workspace_bytes >= layer.prepared_bytes
+    with pytest.raises(moe.MoEError) as e:
+        layer.forward(dev["x"], dev)                     # promised prepared weights, none given
+    assert e.value.status == 4
+    packed = wts.prepare_packed(dev_weights(dev), layer)
+    assert packed["prepared"].numel() == layer.prepared_bytes
+    # the prepared operands are exactly the library's own dequantisation of the three matrices: up, down, gate
+    want = torch.cat([moe.dequantize_block128(dev["w_" + n], dev["s_" + n]).reshape(-1) for n in ("up", "down", "gate")])
+    assert torch.equal(packed["prepared"].view(torch.bfloat16), want)
+    path = str(tmp_path / "layer.safetensors")
+    wts.save_packed(path, packed, product_config(cfg))
+    loaded, pc = wts.load_packed(path)
+    assert pc == product_config(cfg) and torch.equal(loaded["prepared"], packed["prepared"])
+    out = torch.full((cfg.S, cfg.H), float("nan"), dtype=layer.act_dtype, device="cuda")
+    for _ in range(2):
+        layer.forward(dev["x"], dict(loaded, x=dev["x"]), out=out)
+    torch.cuda.synchronize()
+    layer.task_counts()
+    assert np.array_equal(from_device(out), per_call["bits"])
+    layer.close()
+
+    # a handle that keeps the copies in its workspace takes prepared weights too; a plan that prepares nothing has none
+    plain = moe.MoELayer(product_config(cfg), ffn_mode=mode, options={"fp8_widen": 1, "fp8_mfma": 0})
+    out2 = plain.forward(dev["x"], dict(loaded, x=dev["x"]))
+    torch.cuda.synchronize()
+    assert np.array_equal(from_device(out2), per_call["bits"])
+    plain.close()
+    tile = moe.MoELayer(product_config(cfg), ffn_mode=mode, options={"fp8_widen": 0, "fp8_mfma": 0})
+    assert tile.prepared_bytes == 0 and tile.prepare_weights(dev) is None
+    with pytest.raises(moe.MoEError):
+        tile.forward(dev["x"], dict(loaded, x=dev["x"]))   # prepared operands of another plan
+    tile.close()
+
+
+def dev_weights(dev):
+    return {k: v for k, v in dev.items() if k != "x"}

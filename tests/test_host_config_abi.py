@@ -175,6 +175,7 @@ def test_null_arguments_are_errors_not_crashes():
     assert L.moe_options_default(None) == 4 and L.moe_options_from_env(None) == 4
     assert L.moe_get_options(None, None) == 4 and L.moe_get_workspace_bytes(None, None) == 4
     assert L.moe_get_stall(None, None) == 4
+    assert L.moe_prepared_bytes(None, None) == 4 and L.moe_prepare_weights(None, None, None, 0, None) == 4
     assert L.moe_destroy(None) == 0
     assert L.moe_forward(None, None, None, None, None, None, 0, None) == 4
     assert L.moe_gemm_bias_act(None, None, None, None, 1, 1, 1, 0, 0, None) == 4

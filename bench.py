@@ -146,6 +146,21 @@ def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False, balanced_
     except Exception as e:        # reported, never fatal: the figures above do not depend on it
         graph_err = "%s: %s" % (type(e).__name__, e)
 
+    # a plan that derives operands from the weights in every call (the bf16 copies of an e4m3 layer on the widening
+    # plan): the same steps once more with those operands made once by moe_prepare_weights and handed in
+    prepared_ms = None
+    if layer.prepared_bytes:
+        ready = dict(dev, prepared=layer.prepare_weights(dev))
+        for _ in range(warmup):
+            layer.forward(dev["x"], ready, out=out)
+        torch.cuda.synchronize()
+        t5 = time.perf_counter()
+        for _ in range(steps):
+            layer.forward(dev["x"], ready, out=out)
+        torch.cuda.synchronize()
+        prepared_ms = (time.perf_counter() - t5) * 1e3 / steps
+        del ready
+
     routing = layer.new_routing()                 # one extra, untimed call fetches the routing result
     layer.forward(dev["x"], dev, out=out, routing=routing)
     torch.cuda.synchronize()
@@ -194,6 +209,7 @@ def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False, balanced_
     res = {
         "workload": w.describe(), "tokens_per_s": c.tokens / (ms_per_step * 1e-3), "ms_per_step": ms_per_step,
         "ms_per_step_with_events": ms_per_step_events, "ms_per_step_graph_replay": graph_ms if graph_err is None else graph_err,
+        "ms_per_step_prepared_weights": prepared_ms,
         "step_ms": stats(step_ms), "steps": steps, "warmup": warmup,
         "tflops": layer_flops / (ms_per_step * 1e-3) / 1e12,
         "stage_ms": {k: round(v, 4) for k, v in stage_mean.items() if k != "calls"},

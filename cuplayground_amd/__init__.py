@@ -16,6 +16,7 @@ from .api import (  # noqa: F401
     load_library,
     measured_peaks,
     quantize_block128,
+    quantize_rows128,
     dequantize_block128,
     transpose,
 )

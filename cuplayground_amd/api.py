@@ -25,7 +25,7 @@ EXPORTS = (
     "moe_config_tokens", "moe_config_capacity", "moe_create", "moe_destroy", "moe_get_arch", "moe_get_plan", "moe_get_kernel_dtype",
     "moe_workspace_bytes", "moe_options_default", "moe_options_from_env", "moe_create_with_options",
     "moe_workspace_bytes_with_options", "moe_get_options", "moe_get_workspace_bytes", "moe_get_stall", "moe_gemm_bias_act_tile",
-    "moe_prepared_bytes", "moe_prepare_weights",
+    "moe_prepared_bytes", "moe_prepare_weights", "moe_quant_rows128",
     "moe_set_ffn_mode", "moe_get_ffn_mode", "moe_forward", "moe_forward_static", "moe_set_spin_limit", "moe_clear_stall", "moe_gate", "moe_router_stats", "moe_route", "moe_gemm_bias_act", "moe_combine",
     "moe_set_stage_timing", "moe_get_stage_ms", "moe_get_stage_samples", "moe_get_task_counts", "moe_get_queue_balance", "moe_task_trace_bytes", "moe_set_task_trace", "moe_get_task_trace", "moe_measure_mfma_tflops",
     "moe_measure_hbm_read_gbs", "moe_quant_block128", "moe_dequant_block128", "moe_backward_scratch_bytes", "moe_transpose", "moe_expert_gemm",
@@ -150,6 +150,7 @@ def load_library():
     L.moe_get_task_trace.argtypes = [vp, vp, vp, C.c_int64, C.POINTER(C.c_int64)]
     L.moe_quant_block128.argtypes = [vp, C.c_int32, C.c_int64, C.c_int64, C.c_int64, vp, vp, vp]
     L.moe_dequant_block128.argtypes = [vp, vp, C.c_int64, C.c_int64, C.c_int64, vp, vp]
+    L.moe_quant_rows128.argtypes = [vp, C.c_int64, C.c_int64, vp, vp, vp]
     L.moe_measure_mfma_tflops.argtypes = [vp, C.c_size_t, vp, C.c_int, C.POINTER(C.c_float)]
     L.moe_measure_hbm_read_gbs.argtypes = [vp, C.c_size_t, vp, vp, C.POINTER(C.c_float)]
     L.moe_backward_scratch_bytes.argtypes = [cfgp, C.POINTER(C.c_size_t)]
@@ -602,6 +603,20 @@ def quantize_block128(w):
         raise ValueError("quantize_block128 takes fp32 or bf16 weights")
     _check(load_library().moe_quant_block128(_ptr(w), dtype, mats, N, K, _ptr(q), _ptr(s), _stream()),
            "moe_quant_block128")
+    return q, s
+
+
+def quantize_rows128(x):
+    """bf16 rows [R, K] on the GPU -> (uint8 e4m3 codes [R, K], fp32 scales [R, K/128]): one scale per row and 128 columns,
+    the activation format of the e4m3 x e4m3 plan (option fp8_mfma)."""
+    import torch
+    if x.dtype != torch.bfloat16 or x.dim() != 2:
+        raise ValueError("quantize_rows128 takes a 2-d bf16 tensor")
+    x = x.contiguous()
+    R, K = x.shape
+    q = torch.empty(R, K, dtype=torch.uint8, device=x.device)
+    s = torch.empty(R, K // 128, dtype=torch.float32, device=x.device)
+    _check(load_library().moe_quant_rows128(_ptr(x), R, K, _ptr(q), _ptr(s), _stream()), "moe_quant_rows128")
     return q, s
 
 

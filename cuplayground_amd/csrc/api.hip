@@ -36,6 +36,7 @@ int fp8_block_n0(int swiglu);
 int fp8_block_n1();
 int ffn_persistent_occupancy_fp8();
 hipError_t launch_ffn_fp8_tile(const FfnArgs&, int max_mtiles, int nnt0, int nnt1, int blocks, hipStream_t);
+hipError_t launch_ffn_fp8_mfma(const FfnArgs&, int S, int64_t A, int max_mtiles, int nnt0, int nnt1, hipStream_t);
 int fp8_tile_block_m();
 int fp8_tile_block_n0(int swiglu);
 int fp8_tile_block_n1();
@@ -70,7 +71,7 @@ struct Derived {
 struct WsLayout {
     size_t logits, topk_idx, topk_w, slot, pair_row, token_indices, expert_count, expert_offset, rank_local,
         block_hist, mtiles, seg0, seg1, segq, qstate, cstate, done0, done1, pair_mt, wg_clock, arrive, stats_prob, stats_cnt, h, y,
-        wide, total;
+        wide, xq, sx, hq, sh, total;
 };
 
 // Storage type of activations (x, biases, h, y, out): the layer's own, except that tf32 -- fp32 storage with
@@ -143,6 +144,12 @@ WsLayout layout(const Derived& d) {
     w.y = take((size_t)d.A * d.H * d.act_bytes);
     // bf16 copies of an e4m3 layer's expert weights (up, down, gate), rewritten by every call of such a plan
     w.wide = take(d.wide_in_workspace ? (size_t)d.wide_mats * d.E * d.I * d.H * 2 : 0);
+    // e4m3 x e4m3 plan: token rows and intermediate rows as e4m3 codes + one fp32 scale per (row, 128 columns)
+    const bool m8 = d.plan.mfma8;
+    w.xq = take(m8 ? (size_t)d.S * d.H : 0);
+    w.sx = take(m8 ? (size_t)d.S * (d.H / 128) * 4 : 0);
+    w.hq = take(m8 ? (size_t)d.A * d.I : 0);
+    w.sh = take(m8 ? (size_t)d.A * (d.I / 128) * 4 : 0);
     w.total = off;
     return w;
 }
@@ -154,12 +161,14 @@ FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E, const moe_o
     p.tile = 0;
     p.kernel_dtype = dtype;
     p.widen = false;
+    p.mfma8 = false;
     const bool sw = act == MOE_ACT_SWIGLU;
     if (dtype == MOE_DTYPE_FP8_E4M3_B128) {
         // With this many rows per expert one more pass over the weights (e4m3 -> bf16 into the workspace) costs less
         // than the e4m3 tile GEMM loses to the bf16 one.
         p.widen = A / (E > 0 ? E : 1) >= kFp8WidenRowsPerExpert;
         if (o.fp8_widen != MOE_OPT_AUTO) p.widen = o.fp8_widen != 0;
+        if (o.fp8_mfma == 1) p.widen = false;             // asked for the e4m3 x e4m3 tile GEMM: the weights stay as stored
         if (p.widen) p.kernel_dtype = dtype = MOE_DTYPE_BF16;
     }
     if (dtype == MOE_DTYPE_F32 || dtype == MOE_DTYPE_TF32) {
@@ -183,6 +192,7 @@ FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E, const moe_o
         // rows for a weight tile to be reused from LDS instead of being fetched again per 16 rows
         p.tile = A / (E > 0 ? E : 1) >= kFp8TileRowsPerExpert ? 1 : 0;
         if (o.fp8_tile != MOE_OPT_AUTO) p.tile = o.fp8_tile;
+        if (o.fp8_mfma == 1) p.tile = 1, p.mfma8 = true;   // tokens quantised per (row, 128 columns), fp8 matrix instructions
         p.block_m = p.tile ? fp8_tile_block_m() : fp8_block_m();
         p.nnt0 = ceil_div(I, p.tile ? fp8_tile_block_n0(sw) : fp8_block_n0(sw));
         p.nnt1 = ceil_div(H, p.tile ? fp8_tile_block_n1() : fp8_block_n1());
@@ -310,6 +320,8 @@ RouteArgs route_args(const moe_handle* h, void* ws) {
 // layers launch once per projection.  Row blocks are estimated on the host as the larger of kept rows / block rows
 // and the experts that can be hit at all (every hit expert owns at least one row block).
 int resolved_ffn_mode(const moe_handle* h) {
+    // the e4m3 x e4m3 plan quantises the intermediate rows between the projections: always one launch per projection
+    if (h->d.plan.mfma8) return MOE_FFN_TILED;
     if (h->ffn_mode != MOE_FFN_AUTO) return h->ffn_mode;
     const Derived& d = h->d;
     int64_t row_blocks = d.A / d.plan.block_m + 1;
@@ -502,6 +514,7 @@ int moe_create_with_options(const moe_config* cfg, const moe_options* opt, moe_h
     // +18 %, decode +0.9 %): the workgroup that completes a token holds a whole compute unit while it gathers k rows
     // at memory latency, where the separate launch does the same gather with the whole chip's occupancy in 8-38 us.
     h->combine_mode = opt->combine == MOE_OPT_AUTO ? 0 : opt->combine;
+    if (d.plan.mfma8) h->combine_mode = 0;                // that plan's kernels leave the combine to its own launch
     h->spin_limit = kDefaultSpinLimit;
     h->task_trace = nullptr;
     h->task_trace_cap = 0;
@@ -526,6 +539,7 @@ int moe_create_with_options(const moe_config* cfg, const moe_options* opt, moe_h
     h->opt.blocks_per_cu = per_cu;
     h->opt.combine = h->combine_mode;
     h->opt.prepared_weights = d.plan.widen && !d.wide_in_workspace ? 1 : 0;
+    h->opt.fp8_mfma = cfg->torch_dtype == MOE_DTYPE_FP8_E4M3_B128 ? (int)d.plan.mfma8 : MOE_OPT_AUTO;
     resolve_static_scratch(dev);
     *out = h;
     return MOE_OK;
@@ -779,6 +793,12 @@ int forward_on(moe_handle* h, const void* x, const moe_weights* w, void* out, co
     fa.pair_mt = ra.pair_mt;
     fa.combined = ra.done1 ? ra.arrive : nullptr;
     fa.cs = ra.cs;
+    if (d.plan.mfma8) {
+        fa.xq = at<uint8_t>(workspace, L.xq);
+        fa.sx = at<float>(workspace, L.sx);
+        fa.hq = at<uint8_t>(workspace, L.hq);
+        fa.sh = at<float>(workspace, L.sh);
+    }
     fa.task_trace = h->task_trace;
     fa.task_trace_cap = h->task_trace_cap;
     fa.pair_row = ra.pair_row;
@@ -805,7 +825,9 @@ int forward_on(moe_handle* h, const void* x, const moe_weights* w, void* out, co
         for (int i = 0; i < d.wide_mats; ++i) *dst[i] = wide + (size_t)i * d.E * d.I * d.H * 2;
         fa.s_up = fa.s_gate = fa.s_down = nullptr;
     }
-    if (kdt == MOE_DTYPE_FP8_E4M3_B128) {
+    if (d.plan.mfma8) {
+        e = launch_ffn_fp8_mfma(fa, d.S, d.A, d.max_mtiles, d.plan.nnt0, d.plan.nnt1, st);
+    } else if (kdt == MOE_DTYPE_FP8_E4M3_B128) {
         e = (d.plan.tile ? launch_ffn_fp8_tile : launch_ffn_fp8)(fa, d.max_mtiles, d.plan.nnt0, d.plan.nnt1,
                                                                  mode == MOE_FFN_PERSISTENT ? h->arch.persistent_blocks : 0, st);
     } else if (mode == MOE_FFN_PERSISTENT) {

@@ -56,6 +56,9 @@ struct TileTask {
     int act;                    // up projection without SwiGLU: the activation of the epilogue (else MOE_ACT_NONE)
     bool paired;                // up projection with SwiGLU: 64 gate + 64 up rows; otherwise 128 rows of one matrix
     bool publish;               // rows are read by other workgroups of the same launch
+    // e4m3 x e4m3 plan: the token operand as e4m3 codes (rows as a_base's: gathered or a_row0 + r) and its scales
+    const uint8_t* aq;          // [*, K]
+    const float* sa;            // [*, K / 128]
 };
 
 // 16 e4m3 bytes -> 2 x 8 bf16.  Every e4m3 value is a bf16 value, so the upper half of its fp32 form is exact.
@@ -252,6 +255,129 @@ __device__ __forceinline__ void tile_mainloop(const TileTask& p, unsigned char* 
     end_slab(std::false_type{});
 }
 
+// ---- the same tile with both operands e4m3: v_mfma_f32_16x16x128_f8f6f4 ----
+//
+// One matrix instruction takes a whole 128-wide k block (32 bytes of each operand per lane), twice the rate of the 16-bit
+// instructions, and nothing is widened: token rows arrive as e4m3 codes with one fp32 scale per (row, k block)
+// (quant_rows128 passes in front of the two projections), weights are fed as stored.  A slab is one k block: 128 bytes
+// per row, both operands global -> LDS directly, the 16-bit tiles' row layout (128-byte rows, 16-byte chunks xor-swizzled
+// by (row >> 1) & 7); a lane's fragment is chunks 2 fk and 2 fk + 1 of its row (which k a lane's bytes stand for inside the
+// instruction does not matter as long as both operands agree: the block's dot product is a sum over all of them).
+// Every MFMA starts from zero; its 16 x 16 partial sums are scaled by (weight block scale) x (token row scale) and added
+// in fp32: y[t, n] = sum over k blocks of s_w[n / 128][kb] * s_a[t][kb] * (dot product of the block's codes).
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+
+template <bool PARTIAL>
+__device__ __forceinline__ void tile_mainloop_mfma8(const TileTask& p, unsigned char* smem, f32x4 (&acc)[PTM][PTN]) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int KB = p.K >> 7;
+
+    // both operands: 8 threads per 128-byte row, four passes of 32 rows; LDS slot (row, c) holds chunk c ^ ((row >> 1) & 7)
+    const int prow = tid >> 3;
+    const int chunk = (tid & 7) ^ ((prow >> 1) & 7);
+    const uint8_t* a_src[4];
+    const uint8_t* b_src[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int r = prow + i * 32;
+        if (r >= p.rows) r = 0;                                   // padding rows re-read row 0; never stored
+        const int64_t src_row = p.gather ? (int64_t)p.gather[r] : p.a_row0 + r;
+        a_src[i] = p.aq + src_row * p.K + chunk * 16;
+        const int j = prow + i * 32;                              // row of the weight tile
+        const uint8_t* base = p.w[0];
+        int col;
+        if (p.paired) {       // wavefront column w owns tile rows [64 w, 64 w + 64): 32 gate rows, then 32 up rows
+            const int w = j >> 6, jj = j & 63;
+            col = p.c0 + w * 32 + (jj & 31);
+            base = (jj >> 5) ? p.w[1] : p.w[0];
+        } else {
+            col = p.c0 + j;
+        }
+        b_src[i] = base + (int64_t)col * p.K + chunk * 16;
+    }
+    const int wrow = __builtin_amdgcn_readfirstlane(prow & ~7);
+    auto issue = [&](int kb) {
+        unsigned char* sa = smem + (kb & 1) * PSTAGE;
+        unsigned char* sb = sa + PBM * PROW;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            __builtin_amdgcn_global_load_lds((gbl_void*)(a_src[i] + kb * 128), (lds_void*)(sa + (wrow + i * 32) * PROW), 16, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            __builtin_amdgcn_global_load_lds((gbl_void*)(b_src[i] + kb * 128), (lds_void*)(sb + (wrow + i * 32) * PROW), 16, 0, 0);
+    };
+
+    const int frow = lane & 15, fk = lane >> 4;
+    const int sw = (frow >> 1) & 7;
+    const int ta = PARTIAL ? min(PTM, max(0, (p.rows - wm * 16 * PTM + 15) >> 4)) : PTM;
+    const int a_off = (wm * 16 * PTM + frow) * PROW;
+    const int b_off = PBM * PROW + (wn * 16 * PTN + frow) * PROW;
+    const int c0 = ((2 * fk) ^ sw) << 4, c1 = ((2 * fk + 1) ^ sw) << 4;
+
+    // the scales of this lane's token rows (one row per 16 x 16 fragment), a k block ahead
+    const float* sa_row[PTM];
+#pragma unroll
+    for (int i = 0; i < PTM; ++i) {
+        int r = wm * 16 * PTM + i * 16 + frow;
+        if (r >= p.rows) r = 0;
+        const int64_t src_row = p.gather ? (int64_t)p.gather[r] : p.a_row0 + r;
+        sa_row[i] = p.sa + src_row * KB;
+    }
+    typedef const __attribute__((address_space(4))) float cfloat;
+    cfloat* sc0 = (cfloat*)(uintptr_t)p.s[0];
+    cfloat* sc1 = (cfloat*)(uintptr_t)p.s[1];
+
+#pragma unroll
+    for (int i = 0; i < PTM; ++i)
+#pragma unroll
+        for (int j = 0; j < PTN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    auto frag = [&](const unsigned char* base) {
+        const u32x4 lo = *reinterpret_cast<const u32x4*>(base + c0), hi = *reinterpret_cast<const u32x4*>(base + c1);
+        return i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+    };
+
+    __syncthreads();                        // the previous task may still be reading the stages
+    issue(0);
+    float san[PTM];
+#pragma unroll
+    for (int i = 0; i < PTM; ++i) san[i] = sa_row[i][0];
+    for (int kb = 0; kb < KB; ++kb) {
+        // slab kb has landed (it was requested a whole slab ago, and nothing younger is outstanding that we could let
+        // fly: wait for all), and every wavefront is done reading the other stage
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        float sac[PTM];
+#pragma unroll
+        for (int i = 0; i < PTM; ++i) sac[i] = san[i];
+        if (kb + 1 < KB) {
+            issue(kb + 1);
+#pragma unroll
+            for (int i = 0; i < PTM; ++i) san[i] = sa_row[i][kb + 1];
+        }
+        const float s0 = sc0[kb], s1 = sc1[kb];
+        const unsigned char* st = smem + (kb & 1) * PSTAGE;
+        i32x8 bf[PTN];
+#pragma unroll
+        for (int j = 0; j < PTN; ++j) bf[j] = frag(st + b_off + j * 16 * PROW);
+#pragma unroll
+        for (int i = 0; i < PTM; ++i) {
+            if (PARTIAL && i >= ta) continue;
+            const i32x8 af = frag(st + a_off + i * 16 * PROW);
+            const float m0 = s0 * sac[i], m1 = s1 * sac[i];
+#pragma unroll
+            for (int j = 0; j < PTN; ++j) {
+                const f32x4 part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], af, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+                const float m = j < PTN / 2 ? m0 : m1;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[i][j][r] = __builtin_fmaf(m, part[r], acc[i][j][r]);
+            }
+        }
+    }
+}
+
 // acc[i][j][r]: token row = 64 wm + 16 i + (lane & 15); weight row inside fragment j = 4 (lane >> 4) + r.
 __device__ __forceinline__ void tile_epilogue(const TileTask& p, f32x4 (&acc)[PTM][PTN]) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -303,6 +429,12 @@ __device__ __forceinline__ void fp8_gemm_tile(const TileTask& p, unsigned char* 
     else tile_mainloop<false>(p, smem, acc);
     tile_epilogue(p, acc);
 }
+__device__ __forceinline__ void fp8_gemm_tile_mfma8(const TileTask& p, unsigned char* smem) {
+    f32x4 acc[PTM][PTN];
+    if (p.rows < PBM) tile_mainloop_mfma8<true>(p, smem, acc);
+    else tile_mainloop_mfma8<false>(p, smem, acc);
+    tile_epilogue(p, acc);
+}
 
 __device__ __forceinline__ TileTask resolve_tile(const FfnArgs& a, const Task& t, bool publish) {
     TileTask p;
@@ -312,6 +444,8 @@ __device__ __forceinline__ TileTask resolve_tile(const FfnArgs& a, const Task& t
     p.phase = t.phase;
     p.rows = t.rows;
     p.act = MOE_ACT_NONE;
+    p.aq = t.phase == 0 ? a.xq : a.hq;
+    p.sa = t.phase == 0 ? a.sx : a.sh;
     p.paired = t.phase == 0 && a.act == MOE_ACT_SWIGLU;
     if (t.phase == 0) {
         p.c0 = t.ntile * (p.paired ? PN0 : PN1);
@@ -392,6 +526,16 @@ __global__ __launch_bounds__(PTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
     queue_clock_stamp(a.wg_clock, 1);
 }
 
+// The e4m3 x e4m3 plan: one launch per projection (the intermediate rows are quantised by a pass of their own between
+// the two, so the projections cannot share a queue).
+__global__ __launch_bounds__(PTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void ffn_tiled_fp8_mfma_kernel(FfnArgs a, int phase) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    Task t;
+    if (!tiled_task(a, phase, blockIdx.x, t)) return;
+    const TileTask p = resolve_tile(a, t, false);
+    fp8_gemm_tile_mfma8(p, smem);
+}
+
 template <class K>
 hipError_t allow_lds(K kernel) {
     return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, PLDS);
@@ -423,6 +567,19 @@ hipError_t launch_ffn_fp8_tile(const FfnArgs& a, int max_mtiles, int nnt0, int n
         ffn_tiled_fp8_tile_kernel<<<tiled_grid(max_mtiles, nnt0, a.groups), PTHREADS, PLDS, st>>>(a, 0);
         ffn_tiled_fp8_tile_kernel<<<tiled_grid(max_mtiles, nnt1, a.groups), PTHREADS, PLDS, st>>>(a, 1);
     }
+    return hipGetLastError();
+}
+
+// x -> e4m3 rows, up projection, h -> e4m3 rows (the kept ones), down projection.
+hipError_t launch_ffn_fp8_mfma(const FfnArgs& a, int S, int64_t A, int max_mtiles, int nnt0, int nnt1, hipStream_t st) {
+    hipError_t e = allow_lds(&ffn_tiled_fp8_mfma_kernel);
+    if (e != hipSuccess) return e;
+    e = launch_quant_rows128(a.x, a.xq, a.sx, S, a.H, nullptr, st);
+    if (e != hipSuccess) return e;
+    ffn_tiled_fp8_mfma_kernel<<<tiled_grid(max_mtiles, nnt0, a.groups), PTHREADS, PLDS, st>>>(a, 0);
+    e = launch_quant_rows128(a.h, a.hq, a.sh, A, a.I, &a.q->kept_rows, st);
+    if (e != hipSuccess) return e;
+    ffn_tiled_fp8_mfma_kernel<<<tiled_grid(max_mtiles, nnt1, a.groups), PTHREADS, PLDS, st>>>(a, 1);
     return hipGetLastError();
 }
 

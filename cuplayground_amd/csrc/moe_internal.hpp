@@ -129,6 +129,12 @@ struct FfnArgs {
     const int32_t* pair_mt;     // [S, k] row block (MTile index) of every (token, rank), -1 when dropped
     int32_t* combined;          // [slices, S]: 1 once the unit has been taken
     CombineState* cs;
+    // e4m3 x e4m3 plan (null xq: not used): the token rows and the intermediate rows as e4m3 codes with one scale per
+    // (row, 128 columns), written by quant_rows128 passes in front of the two projections
+    uint8_t* xq;                // [S, H]
+    float* sx;                  // [S, H / 128]
+    uint8_t* hq;                // [A, I]
+    float* sh;                  // [A, I / 128]
 };
 constexpr int kMaxQueueWorkgroups = 4096;   // workgroups of a queue kernel that get a slot in wg_clock
 
@@ -182,6 +188,7 @@ hipError_t launch_combine(const void* y_rows, const int32_t* pair_row, const flo
 struct FfnPlan {
     int kernel_dtype;   // the dtype whose kernels run: the layer's, or bf16 for an e4m3 layer whose weights are widened
     bool widen;         // e4m3 layer run as a bf16 layer on weights widened into the workspace by every call
+    bool mfma8;         // e4m3 layer on the tile GEMM with both operands e4m3 (tokens quantised per row and 128 columns)
     int tile;        // 16-bit layers: which tile the kernels are instantiated with (ffn_bf16.hip: bf16_tile)
     int block_m;
     int nnt0;        // column tiles of phase 0
@@ -190,6 +197,9 @@ struct FfnPlan {
 FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E, const moe_options& o);
 hipError_t launch_widen_block128(const void* q, const float* scales, void* out, int64_t matrices, int64_t N, int64_t K,
                                  hipStream_t st);
+// bf16 rows -> e4m3 codes + one fp32 scale per (row, 128 columns); limit: null, or a device word with the rows that matter
+hipError_t launch_quant_rows128(const void* x, void* q, float* scales, int64_t rows, int64_t K, const int32_t* limit,
+                                hipStream_t st);
 hipError_t launch_ffn_tiled(const FfnArgs& a, int dtype, const FfnPlan& p, int max_mtiles, hipStream_t st);
 hipError_t launch_ffn_persistent(const FfnArgs& a, int dtype, const FfnPlan& p, int blocks, bool early, hipStream_t st);
 int ffn_persistent_blocks(int dtype, int tile, int compute_units);

@@ -107,7 +107,49 @@ __global__ __launch_bounds__(256) void widen_block128_kernel(const uint8_t* __re
     dst[1] = make_uint4(o[4], o[5], o[6], o[7]);
 }
 
+// Activation rows for the e4m3 x e4m3 products: one fp32 scale per (row, 128 columns), scale = amax / 448 over that piece
+// of the row (1 when it is all zero), q = e4m3(x / scale).  x is bf16 [rows, K], K a multiple of 128.  Sixteen lanes
+// share a piece (8 values each); the maximum travels over xor 8, 4, 2, 1, which stays inside the sixteen.  limit
+// (may be null): a device word holding the number of rows that matter; rows behind it are skipped.
+__global__ __launch_bounds__(256) void quant_rows128_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ q,
+                                                            float* __restrict__ scales, int64_t rows, int64_t K,
+                                                            const int32_t* __restrict__ limit) {
+    const int64_t chunk = (int64_t)blockIdx.x * 256 + threadIdx.x;   // 8 values each
+    const int64_t per_row = K / 8;
+    const int64_t row = chunk / per_row, c8 = chunk - row * per_row;
+    if (row >= rows || (limit && row >= *limit)) return;              // K % 128 == 0: the sixteen lanes of a piece agree
+    const uint4 in = *reinterpret_cast<const uint4*>(x + row * K + c8 * 8);
+    const uint32_t w[4] = {in.x, in.y, in.z, in.w};
+    float v[8];
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        v[2 * i] = __uint_as_float(w[i] << 16);
+        v[2 * i + 1] = __uint_as_float(w[i] & 0xFFFF0000u);
+        amax = fmaxf(amax, fmaxf(fabsf(v[2 * i]), fabsf(v[2 * i + 1])));   // fmaxf passes over a NaN, as the comparison of the restatement does
+    }
+#pragma unroll
+    for (int off = 8; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, kWave));
+    const float s = amax > 0.0f ? amax / 448.0f : 1.0f;
+    if ((c8 & 15) == 0) scales[row * (K / 128) + c8 / 16] = s;
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        lo |= f32_to_e4m3(v[e] / s) << (8 * e);
+        hi |= f32_to_e4m3(v[e + 4] / s) << (8 * e);
+    }
+    *reinterpret_cast<uint2*>(q + row * K + c8 * 8) = uint2{lo, hi};
+}
+
 }  // namespace
+
+hipError_t launch_quant_rows128(const void* x, void* q, float* scales, int64_t rows, int64_t K, const int32_t* limit,
+                                hipStream_t st) {
+    const int64_t chunks = rows * (K / 8);
+    if (chunks <= 0) return hipSuccess;
+    quant_rows128_kernel<<<(unsigned)((chunks + 255) / 256), 256, 0, st>>>((const uint16_t*)x, (uint8_t*)q, scales, rows, K, limit);
+    return hipGetLastError();
+}
 
 hipError_t launch_widen_block128(const void* q, const float* scales, void* out, int64_t matrices, int64_t N, int64_t K,
                                  hipStream_t st) {
@@ -133,6 +175,12 @@ extern "C" int moe_quant_block128(const void* w, int32_t src_dtype, int64_t matr
     else
         quant_block128_kernel<uint16_t><<<grid, 256, 0, st>>>((const uint16_t*)w, (uint8_t*)q, scales, N, K);
     return hipGetLastError() == hipSuccess ? MOE_OK : MOE_ERR_HIP;
+}
+
+extern "C" int moe_quant_rows128(const void* x, int64_t rows, int64_t K, void* q, float* scales, void* stream) {
+    if (!x || !q || !scales || rows < 0 || K < 128 || (K % 128)) return MOE_ERR_BAD_ARGUMENT;
+    if (rows * (K / 8) > (int64_t)0x7FFFFFFF * 256) return MOE_ERR_BAD_ARGUMENT;
+    return launch_quant_rows128(x, q, scales, rows, K, nullptr, (hipStream_t)stream) == hipSuccess ? MOE_OK : MOE_ERR_HIP;
 }
 
 extern "C" int moe_dequant_block128(const void* q, const float* scales, int64_t matrices, int64_t N, int64_t K, void* out,

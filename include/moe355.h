@@ -140,9 +140,12 @@ typedef struct moe_options {
                                 queue segments run as this many partial sums over the intermediate dimension (1 = whole
                                 tiles, 2 or 4).  Changes the order of the fp32 sum of those tiles (within the layer's
                                 tolerance, deterministic); the two-launch mode then splits the same tiles the same way. */
-    int32_t fp8_mfma;        /* e4m3 layers on the tile GEMM: 1 = tokens quantised to e4m3 per (row, 128-wide k block) and
-                                the products taken by the fp8 matrix instructions; 0 = bf16 tokens, weights widened.  Not
-                                bit-compatible with 0: see moe_get_kernel_dtype. */
+    int32_t fp8_mfma;        /* e4m3 layers: 1 = the tile GEMM with both operands e4m3 on the fp8 matrix instructions: token rows and
+                                intermediate rows are quantised to e4m3 with one fp32 scale per (row, 128 columns) by a pass in
+                                front of each projection (moe_quant_rows128), weights are fed as stored; one launch per
+                                projection; overrides fp8_tile and fp8_widen.  0 / AUTO = bf16 activations.  Opt-in because it
+                                changes the arithmetic: results stay within the e4m3 tolerance (3e-2 of the output range) of the
+                                bf16-activation layer but are not its bits. */
     int32_t prepared_weights;/* 1 = every moe_forward on the handle will carry moe_weights.prepared (moe_prepare_weights): the
                                 workspace then holds no copies of the weights and a call without them is refused; 0 / AUTO =
                                 prepared weights are used when given, else made per call in the workspace */
@@ -355,6 +358,13 @@ int moe_measure_hbm_read_gbs(const void* src, size_t bytes, void* scratch, void*
  * `stream`.  No counterpart in the reference, whose dtypes stop at fp16 (aristos_config.schema.json:49-53). */
 int moe_quant_block128(const void* w, int32_t src_dtype, int64_t matrices, int64_t N, int64_t K, void* q,
                        float* scales, void* stream);
+
+/* Activation rows for the e4m3 x e4m3 plan (moe_options::fp8_mfma): x [rows, K] in bf16, K a multiple of 128, becomes
+ * q [rows, K] e4m3 codes plus scales [rows, K / 128] fp32, scale = amax / 448 over that piece of the row (1 when it is all
+ * zero), q = e4m3(x / scale) rounded to nearest even.  moe_forward runs this on the tokens and on the intermediate rows of
+ * such a handle; exported so that the format can be checked and reused.  Asynchronous on `stream`.  No counterpart in the
+ * reference (same reason). */
+int moe_quant_rows128(const void* x, int64_t rows, int64_t K, void* q, float* scales, void* stream);
 
 /* The inverse: out[matrices,N,K] (bf16) = e4m3(q) * scale of its block, rounded to nearest even once.  moe_forward
  * runs this on an e4m3 layer's weights, into its workspace, when the experts see enough rows for the bf16 tile GEMM

@@ -68,6 +68,8 @@ def lib():
         L.orc_f16_to_f32.argtypes = [C.c_uint16]; L.orc_f16_to_f32.restype = f32
         L.orc_quant_block128.argtypes = [vp, i64, i64, vp, vp]
         L.orc_dequant_block128.argtypes = [vp, vp, i64, i64, vp]
+        L.orc_quant_rows128.argtypes = [vp, i64, i64, vp, vp]
+        L.orc_dequant_rows128.argtypes = [vp, vp, i64, i64, vp]
         L.orc_capacity.argtypes = [C.c_double, i64, i64, i64, C.POINTER(i64)]
         L.orc_gate_logits.argtypes = [vp, vp, vp, i32, i32, i32, i32, vp]
         L.orc_topk.argtypes = [vp, i32, i32, i32, i32, i32, vp, vp]
@@ -86,7 +88,7 @@ def lib():
         L.orc_num_threads.restype = C.c_int
         for fn in ("orc_philox4x32_10", "orc_fill_normal", "orc_fill_uniform", "orc_round_bf16", "orc_widen_bf16",
                    "orc_round_f16", "orc_widen_f16",
-                   "orc_quant_block128", "orc_dequant_block128", "orc_gate_logits", "orc_topk", "orc_route",
+                   "orc_quant_block128", "orc_dequant_block128", "orc_quant_rows128", "orc_dequant_rows128", "orc_gate_logits", "orc_topk", "orc_route",
                    "orc_gemm_bias_act", "orc_expert_gemm", "orc_expert_wgrad", "orc_act_backward", "orc_bias_grad",
                    "orc_combine_backward", "orc_ffn_rows", "orc_combine", "orc_forward", "orc_forward_tokens"):
             getattr(L, fn).restype = None
@@ -231,6 +233,24 @@ def dequant_block128(q, s):
     for i in range(qf.shape[0]):
         lib().orc_dequant_block128(_p(qf[i]), _p(sf[i]), N, K, _p(wf[i]))
     return w
+
+
+def quant_rows128(x):
+    """x: float32 [R, K] -> (uint8 [R, K], float32 [R, ceil(K/128)]): e4m3 codes with one scale per row and 128 columns."""
+    x = _c(x, np.float32)
+    R, K = x.shape
+    q = np.empty((R, K), np.uint8)
+    s = np.empty((R, (K + 127) // 128), np.float32)
+    lib().orc_quant_rows128(_p(x), R, K, _p(q), _p(s))
+    return q, s
+
+
+def dequant_rows128(q, s):
+    q = _c(q, np.uint8); s = _c(s, np.float32)
+    R, K = q.shape
+    x = np.empty((R, K), np.float32)
+    lib().orc_dequant_rows128(_p(q), _p(s), R, K, _p(x))
+    return x
 
 
 def zipf_gate_bias(E, seed, s=1.1):

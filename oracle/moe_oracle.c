@@ -197,6 +197,35 @@ void orc_dequant_block128(const uint8_t* q, const float* scales, int64_t N, int6
         for (int64_t k = 0; k < K; ++k) w[n * K + k] = orc_e4m3_to_f32(q[n * K + k]) * scales[(n / 128) * kb + k / 128];
 }
 
+/* Activation rows for the products of two e4m3 operands (build-defined, like the weight format above): one fp32 scale
+ * per row and 128-wide block of columns, scale = amax/448 over that piece of the row (1 when it is all zero),
+ * q = e4m3(x / scale).  x is [R,K] in fp32 (the widened bf16 activations), scales is [R, ceil(K/128)] row-major.
+ * A NaN in a piece makes its amax comparison false everywhere, so the scale comes from the other elements and the NaN
+ * becomes the e4m3 NaN code. */
+void orc_quant_rows128(const float* x, int64_t R, int64_t K, uint8_t* q, float* scales) {
+    const int64_t kb = (K + 127) / 128;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < R; ++r) {
+        for (int64_t bj = 0; bj < kb; ++bj) {
+            const int64_t k1 = (bj * 128 + 128 < K) ? bj * 128 + 128 : K;
+            float amax = 0.0f;
+            for (int64_t k = bj * 128; k < k1; ++k) {
+                float a = fabsf(x[r * K + k]);
+                if (a > amax) amax = a;
+            }
+            float s = amax > 0.0f ? amax / 448.0f : 1.0f;
+            scales[r * kb + bj] = s;
+            for (int64_t k = bj * 128; k < k1; ++k) q[r * K + k] = orc_f32_to_e4m3(x[r * K + k] / s);
+        }
+    }
+}
+void orc_dequant_rows128(const uint8_t* q, const float* scales, int64_t R, int64_t K, float* x) {
+    const int64_t kb = (K + 127) / 128;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < R; ++r)
+        for (int64_t k = 0; k < K; ++k) x[r * K + k] = orc_e4m3_to_f32(q[r * K + k]) * scales[r * kb + k / 128];
+}
+
 int orc_num_threads(void) {
 #ifdef _OPENMP
     return omp_get_max_threads();

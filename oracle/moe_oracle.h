@@ -85,6 +85,9 @@ void orc_round_bf16(const float* src, uint16_t* dst, int64_t n);
 void orc_widen_bf16(const uint16_t* src, float* dst, int64_t n);
 void orc_quant_block128(const float* w, int64_t N, int64_t K, uint8_t* q, float* scales);
 void orc_dequant_block128(const uint8_t* q, const float* scales, int64_t N, int64_t K, float* w);
+/* the same per (row, 128 columns): the activation operand of a product of two e4m3 matrices */
+void orc_quant_rows128(const float* x, int64_t R, int64_t K, uint8_t* q, float* scales);
+void orc_dequant_rows128(const uint8_t* q, const float* scales, int64_t R, int64_t K, float* x);
 
 /* ---- the path ---- */
 int orc_capacity(double capacity_factor, int64_t S, int64_t k, int64_t E, int64_t* out);

@@ -122,6 +122,49 @@ def test_block128_quantisation():
     assert np.array_equal(np.abs(d).reshape(2, 2, 128, 3, 128).max(axis=(2, 4)) > 0, s != 1.0)
 
 
+def test_rows128_quantisation():
+    """The activation operand of the e4m3 x e4m3 products: one scale per (row, 128 columns).  Pinned by the scale's
+    definition computed independently, by torch's own e4m3 cast of x / scale, by every code point, by the error bound of
+    a 3-bit significand, and by the independence of rows and column blocks."""
+    rng = np.random.default_rng(3)
+    x = (rng.standard_normal((7, 300)) * np.exp(rng.uniform(-6, 6, (7, 1)))).astype(np.float32)     # ragged last block (44)
+    x[2, 128:256] = 0.0                                                                               # an all-zero piece
+    q, s = ob.quant_rows128(x)
+    assert q.shape == (7, 300) and s.shape == (7, 3)
+    for r in range(7):
+        for j in range(3):
+            piece = x[r, j * 128:(j + 1) * 128]
+            amax = np.abs(piece).max()
+            want_s = np.float32(amax) / np.float32(448.0) if amax > 0 else np.float32(1.0)
+            assert s[r, j] == want_s
+            want_q = torch.from_numpy((piece / want_s).astype(np.float32)).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+            assert np.array_equal(q[r, j * 128:(j + 1) * 128], want_q), (r, j)
+    assert not q[2, 128:256].any() and s[2, 1] == 1.0
+    d = ob.dequant_rows128(q, s)
+    scale = np.repeat(s, 128, axis=1)[:, :300]
+    assert (np.abs(d - x) <= np.maximum(np.abs(x) * 2.0 ** -4, scale * 2.0 ** -10) * (1 + 1e-6)).all()
+    # every finite code point: a piece that holds 448 has scale 1, so its values come back as their own codes
+    codes = np.array([c for c in range(256) if c & 0x7F != 0x7F], np.uint8)
+    vals = torch.from_numpy(codes).view(torch.float8_e4m3fn).float().numpy()
+    row = np.zeros((1, 256), np.float32)
+    row[0, :codes.size] = vals
+    q1, s1 = ob.quant_rows128(row)
+    assert s1[0, 0] == 1.0 and s1[0, 1] == 1.0
+    keep = vals != 0                                   # -0.0 and +0.0 may share a code
+    assert np.array_equal(q1[0, :codes.size][keep], codes[keep])
+    # a power-of-two multiple of the row scales exactly: same codes, scale times that power
+    q2, s2 = ob.quant_rows128(row * np.float32(2.0 ** -5))
+    assert np.array_equal(q2, q1) and s2[0, 0] == np.float32(2.0 ** -5)
+    # rows and column blocks do not see each other
+    y = x.copy()
+    y[4, 130] = 1e6
+    q3, s3 = ob.quant_rows128(y)
+    same = np.ones((7, 300), bool)
+    same[4, 128:256] = False
+    assert np.array_equal(q3[same], q[same]) and s3[4, 1] == np.float32(1e6) / np.float32(448.0)
+    assert q3[4, 130] == 0x7E and np.array_equal(np.delete(s3, 1, axis=1), np.delete(s, 1, axis=1))
+
+
 def test_capacity_formula():
     assert ob.BASELINE["C1"].capacity == 16
     assert ob.BASELINE["C2"].capacity == 640

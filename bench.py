@@ -467,7 +467,7 @@ def main():
                     help="target CPU time of the baseline sample of each --extra workload (0 = skip)")
     ap.add_argument("--option", action="append", default=[], metavar="FIELD=VALUE",
                     help="a tuning option of the handle by its moe_options field name (repeatable), e.g. --option "
-                         "combine=0 --option tail_split=1; applies to every workload measured; without any, handles are "
+                         "combine=0 --option tail_round=0; applies to every workload measured; without any, handles are "
                          "created by moe_create (library defaults, MOE355_* environment variables honoured)")
     ap.add_argument("--seed", type=int, default=42)
     ap.add_argument("--balanced-routing", action="store_true",

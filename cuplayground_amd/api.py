@@ -49,7 +49,7 @@ class _CConfig(C.Structure):
 
 OPTION_FIELDS = ("tile16", "block_rows", "f32_tile", "fp8_tile", "fp8_widen", "queue_groups", "queue_lag", "queue_early",
                  "row_chunk", "blocks_per_cu", "combine", "gate_kernel", "gate_mfma", "gate_tile", "gate_fused_topk",
-                 "grouped_tile", "tail_split", "fp8_mfma", "prepared_weights")
+                 "grouped_tile", "tail_round", "fp8_mfma", "prepared_weights")
 OPT_AUTO = -1
 COMBINE_SEPARATE, COMBINE_ARRIVALS, COMBINE_QUEUE = 0, 1, 2
 

@@ -130,7 +130,7 @@ WsLayout layout(const Derived& d) {
     w.mtiles = take((size_t)d.max_mtiles * sizeof(MTile));
     w.seg0 = take((size_t)d.E * sizeof(Segment));
     w.seg1 = take((size_t)d.E * sizeof(Segment));
-    w.segq = take((size_t)2 * d.E * sizeof(Segment));
+    w.segq = take((size_t)(2 * d.E + 1) * sizeof(Segment));   // one more: round_tail cuts a segment in two
     w.qstate = take(sizeof(QueueState));
     w.cstate = take(sizeof(CombineState));
     w.done0 = take((size_t)d.max_mtiles * 4);
@@ -313,6 +313,7 @@ RouteArgs route_args(const moe_handle* h, void* ws) {
     a.max_mtiles = d.max_mtiles;
     a.lag = h->queue_lag;
     a.groups = h->queue_groups;
+    a.tail_workgroups = h->opt.tail_round == 0 ? 0 : h->arch.persistent_blocks;
     return a;
 }
 
@@ -370,7 +371,7 @@ const OptField kOptFields[] = {
     {"gate_tile", &moe_options::gate_tile, 0, 2, false},
     {"gate_fused_topk", &moe_options::gate_fused_topk, 0, 1, false},
     {"grouped_tile", &moe_options::grouped_tile, 0, 2, false},
-    {"tail_split", &moe_options::tail_split, 1, 4, true},
+    {"tail_round", &moe_options::tail_round, 0, 1, false},
     {"fp8_mfma", &moe_options::fp8_mfma, 0, 1, false},
     {"prepared_weights", &moe_options::prepared_weights, 0, 1, false},
 };

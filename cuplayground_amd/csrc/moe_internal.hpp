@@ -5,6 +5,7 @@
 #include <stdint.h>
 
 #include "../../include/moe355.h"
+#include "queue_order.hpp"
 
 namespace moe355 {
 
@@ -23,25 +24,6 @@ struct MTile {
     int32_t row0;
     int32_t rows;
     int32_t pad;
-};
-
-// A run of consecutive task ids that share (phase, expert).
-//
-// The queue exists once per queue group (one group per XCD when the kernels ask for it, else a single group), and
-// every group sees the same id space: in a segment, group g owns the column tiles c with (c + rot) % groups == g,
-// i.e. c = (g - rot) mod groups + groups * j for j < ceil(nnt / groups), and id - begin = j * nmt + mtile_local
-// (row blocks fastest, so neighbouring ids share the weight tile).  An id whose c falls behind nnt is a hole:
-// popped and skipped.  rot = expert * nnt mod groups continues the round robin over the experts, so groups stay
-// balanced when nnt is not a multiple of the group count.
-struct Segment {
-    int32_t begin;    // first task id (in the id space of one group)
-    int32_t phase;    // 0 = up(/gate) projection + activation, 1 = down projection
-    int32_t expert;
-    int32_t mt0;      // index of the expert's first MTile
-    int32_t nmt;      // row blocks of the expert
-    int32_t nnt;      // column tiles of this phase
-    int32_t rot;      // rotation of the column-tile round robin over the groups
-    int32_t pad1;
 };
 
 // Words at the start of the queue-state block of the workspace (carved out of the workspace in api.hip).
@@ -166,6 +148,7 @@ struct RouteArgs {
     int32_t max_mtiles;
     int32_t lag;                // experts of phase-0 work queued between an expert's two phases
     int32_t groups;             // queue groups: 1, or one per XCD
+    int32_t tail_workgroups;    // 0, or the workgroups of the queue kernel: the tail of the queue is rounded to them (route.hip: round_tail)
     int64_t* task_trace;        // null, or the FFN stage's trace buffer: its record count starts every call at zero
 };
 

@@ -14,6 +14,7 @@
 //   3. finalize: slot = prefix + local rank; dropped when slot >= capacity; packed row = offset + slot.
 // Every step is integer arithmetic with a fixed order, so results do not depend on scheduling.
 #include "moe_internal.hpp"
+#include "queue_order.hpp"
 
 namespace moe355 {
 namespace {
@@ -101,14 +102,6 @@ __device__ __forceinline__ int block_exclusive_scan(int v, int* s_wave, int* tot
     return base + inc - v;
 }
 
-// Queue order with lag L: phase-0 segments of experts 0..L-1, then (phase-0 of e, phase-1 of e-L) for
-// e = L..E-1, then the phase-1 segments of the last L experts.
-__device__ __forceinline__ void queue_slot(int s, int E, int L, int* phase, int* ex) {
-    if (s < L) { *phase = 0; *ex = s; }
-    else if (s < 2 * E - L) { const int r = s - L; *phase = r & 1; *ex = (r & 1) ? (r >> 1) : L + (r >> 1); }
-    else { *phase = 1; *ex = E - L + (s - (2 * E - L)); }
-}
-
 // One workgroup of kMaxExperts threads: thread e owns expert e.
 struct ScanShared {
     int wave[kMaxExperts / kWave];
@@ -190,6 +183,14 @@ __device__ __forceinline__ void route_scan_body(const RouteArgs& a, ScanShared& 
             write_segment(a.seg_queue + sidx, begin + (j ? size[0] : 0), ph[j], ex[j], s_mt0[ex[j]], s_nmt[ex[j]],
                           ph[j] ? a.nnt1 : a.nnt0, a.groups);
     }
+    int nseg_final = nseg;
+    if (a.tail_workgroups > 0) {
+        __syncthreads();                                  // the segment table is complete
+        if (e == 0) {
+            const TailParams tp{a.E, a.lag, a.nnt0, a.nnt1, a.groups, a.tail_workgroups};
+            nseg_final = round_tail(a.seg_queue, nseg, tp, &total_tasks);
+        }
+    }
     if (e == 0) {
         a.q->groups = a.groups;
         for (int g = 0; g < kMaxQueueGroups; ++g) a.q->heads[g] = 0;
@@ -204,7 +205,7 @@ __device__ __forceinline__ void route_scan_body(const RouteArgs& a, ScanShared& 
         a.q->num_mtiles = total_mt;
         a.q->kept_rows = total_rows;
         a.q->stall = 0;
-        a.q->nseg = nseg;
+        a.q->nseg = nseg_final;
         a.expert_offset[a.E] = total_rows;
     }
     if (e < a.E) {

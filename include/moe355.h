@@ -136,10 +136,9 @@ typedef struct moe_options {
     int32_t gate_fused_topk; /* 1 = top-k inside the logits kernel where one exists for the shape (no logits round trip
                                 through memory unless the caller asks for them), 0 = always a launch of its own */
     int32_t grouped_tile;    /* moe_expert_gemm on a 16-bit handle: 0 = 128x128, 1 = 256x256, 2 = 128x256 */
-    int32_t tail_split;      /* 16-bit layers on the 256x256 tile, task-queue mode: the down-projection tiles of the last
-                                queue segments run as this many partial sums over the intermediate dimension (1 = whole
-                                tiles, 2 or 4).  Changes the order of the fp32 sum of those tiles (within the layer's
-                                tolerance, deterministic); the two-launch mode then splits the same tiles the same way. */
+    int32_t tail_round;      /* task-queue mode: 1 (and AUTO) = the last up-projection segment of the queue is placed so that the
+                                down-projection tasks behind it fill whole rounds of the resident workgroups (a permutation
+                                of whole row blocks inside the queue: results and tables do not change), 0 = plain order */
     int32_t fp8_mfma;        /* e4m3 layers: 1 = the tile GEMM with both operands e4m3 on the fp8 matrix instructions: token rows and
                                 intermediate rows are quantised to e4m3 with one fp32 scale per (row, 128 columns) by a pass in
                                 front of each projection (moe_quant_rows128), weights are fed as stored; one launch per

@@ -40,7 +40,7 @@ def _cases(n=36, seed=2024):
         knobs["fp8_widen"] = i // 10 % 2      # ... or the bf16 tiles on weights widened in the workspace
         knobs["fp8_mfma"] = 0                 # bf16 tokens: the arithmetic the oracle's layer restates
         knobs["gate_fused_topk"] = i // 3 % 2 # top-k inside the logits kernel or as a launch of its own
-        knobs["tail_split"] = (1, 2, 4)[i // 4 % 3]   # down-projection tiles of the last queue segments as partial sums
+        knobs["tail_round"] = i // 4 % 2      # the last up-projection segment moved so that the tail fills whole rounds
         out.append(pytest.param(cfg, knobs, int(rng.integers(1, 3)), bool(rng.integers(0, 2)), id="case%02d" % i))
     return out
 

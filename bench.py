@@ -300,21 +300,28 @@ def task_trace_summary(layer, dev, out):
     layer.disable_task_trace()
     dur = rec["end_us"] - rec["start_us"]
     full = int(rec["rows"].max())
+    # a task that computed one of P partial sums of its tile (option tail_split) carries 1 + 4 * part + 16 * P in `phase`
+    parts = rec["phase"] >> 4
+    phase = rec["phase"] & 3
     groups = []
     for ph in (0, 1):
-        for lo, hi, label in ((full, full, "full"), (full // 2 + 1, full - 1, "more than half"), (1, full // 2, "at most half")):
-            m = (rec["phase"] == ph) & (rec["rows"] >= lo) & (rec["rows"] <= hi)
-            if m.any():
-                groups.append({"phase": ph, "rows": label, "tasks": int(m.sum()), "mean_us": round(float(dur[m].mean()), 2),
-                               "median_us": round(float(np.median(dur[m])), 2), "min_us": round(float(dur[m].min()), 2),
-                               "max_us": round(float(dur[m].max()), 2)})
+        for np_ in sorted(set(parts[phase == ph].tolist())):
+            for lo, hi, label in ((full, full, "full"), (full // 2 + 1, full - 1, "more than half"), (1, full // 2, "at most half")):
+                m = (phase == ph) & (parts == np_) & (rec["rows"] >= lo) & (rec["rows"] <= hi)
+                if m.any():
+                    g = {"phase": ph, "rows": label, "tasks": int(m.sum()), "mean_us": round(float(dur[m].mean()), 2),
+                         "median_us": round(float(np.median(dur[m])), 2), "min_us": round(float(dur[m].min()), 2),
+                         "max_us": round(float(dur[m].max()), 2)}
+                    if np_:
+                        g["partial_sums_per_tile"] = int(np_)
+                    groups.append(g)
     gaps = {0: [], 1: []}
     busy, idle_after, per_wg = [], [], []
     end = float(rec["end_us"].max())
     for w in np.unique(rec["workgroup"]):
         r = np.sort(rec[rec["workgroup"] == w], order="start_us")
         for a, b in zip(r[:-1], r[1:]):
-            gaps[int(b["phase"])].append(float(b["start_us"] - a["end_us"]))
+            gaps[int(b["phase"]) & 3].append(float(b["start_us"] - a["end_us"]))
         busy.append(float((r["end_us"] - r["start_us"]).sum()))
         idle_after.append(end - float(r["end_us"][-1]))
         per_wg.append(len(r))

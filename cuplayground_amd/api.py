@@ -49,13 +49,13 @@ class _CConfig(C.Structure):
 
 OPTION_FIELDS = ("tile16", "block_rows", "f32_tile", "fp8_tile", "fp8_widen", "queue_groups", "queue_lag", "queue_early",
                  "row_chunk", "blocks_per_cu", "combine", "gate_kernel", "gate_mfma", "gate_tile", "gate_fused_topk",
-                 "grouped_tile", "tail_round", "fp8_mfma", "prepared_weights")
+                 "grouped_tile", "tail_round", "fp8_mfma", "prepared_weights", "tail_split")
 OPT_AUTO = -1
 COMBINE_SEPARATE, COMBINE_ARRIVALS, COMBINE_QUEUE = 0, 1, 2
 
 
 class _COptions(C.Structure):
-    _fields_ = [(n, C.c_int32) for n in OPTION_FIELDS] + [("reserved", C.c_int32 * 7)]
+    _fields_ = [(n, C.c_int32) for n in OPTION_FIELDS] + [("reserved", C.c_int32 * 6)]
 
 
 def make_options(options: dict | None = None, from_env: bool = False) -> _COptions:
@@ -392,7 +392,8 @@ class MoELayer:
 
     def task_trace(self):
         """Records of the last forward's queue kernel as a numpy structured array (phase, expert, row_block, col_tile,
-        rows, workgroup, start_us, end_us); synchronises the current stream."""
+        rows, workgroup, start_us, end_us); synchronises the current stream.  A task that computed one of P partial sums of
+        its tile (option tail_split) carries 1 + 4 * part + 16 * P in `phase`."""
         import numpy as np
         dt = np.dtype([("phase", "i4"), ("expert", "i4"), ("row_block", "i4"), ("col_tile", "i4"), ("rows", "i4"),
                        ("workgroup", "i4"), ("start_us", "f4"), ("end_us", "f4")])

@@ -53,6 +53,7 @@ int ffn_persistent_occupancy_f32_tile();
 namespace {
 
 constexpr size_t kAlign = 256;
+constexpr int kSplitWorkgroups = 256;   // resident workgroups the partial-sum tail is sized for (one per compute unit of a whole MI355X)
 size_t align_up(size_t v) { return (v + kAlign - 1) / kAlign * kAlign; }
 int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
 
@@ -71,7 +72,7 @@ struct Derived {
 struct WsLayout {
     size_t logits, topk_idx, topk_w, slot, pair_row, token_indices, expert_count, expert_offset, rank_local,
         block_hist, mtiles, seg0, seg1, segq, qstate, cstate, done0, done1, pair_mt, wg_clock, arrive, stats_prob, stats_cnt, h, y,
-        wide, xq, sx, hq, sh, total;
+        wide, xq, sx, hq, sh, split_cnt, split_part, total;
 };
 
 // Storage type of activations (x, biases, h, y, out): the layer's own, except that tf32 -- fp32 storage with
@@ -129,8 +130,8 @@ WsLayout layout(const Derived& d) {
     w.block_hist = take((size_t)d.nblk * d.E * 4);
     w.mtiles = take((size_t)d.max_mtiles * sizeof(MTile));
     w.seg0 = take((size_t)d.E * sizeof(Segment));
-    w.seg1 = take((size_t)d.E * sizeof(Segment));
-    w.segq = take((size_t)(2 * d.E + 1) * sizeof(Segment));   // one more: round_tail cuts a segment in two
+    w.seg1 = take((size_t)(d.E + 1) * sizeof(Segment));       // one more: split_tail cuts a segment in two
+    w.segq = take((size_t)(2 * d.E + 1) * sizeof(Segment));   // one more: round_tail or split_tail cuts a segment in two
     w.qstate = take(sizeof(QueueState));
     w.cstate = take(sizeof(CombineState));
     w.done0 = take((size_t)d.max_mtiles * 4);
@@ -150,6 +151,10 @@ WsLayout layout(const Derived& d) {
     w.sx = take(m8 ? (size_t)d.S * (d.H / 128) * 4 : 0);
     w.hq = take(m8 ? (size_t)d.A * d.I : 0);
     w.sh = take(m8 ? (size_t)d.A * (d.I / 128) * 4 : 0);
+    // down-projection tiles computed as partial sums: a counter and ksplit fp32 copies of the tile for each
+    const size_t split_tiles = d.plan.ksplit > 1 ? (size_t)d.plan.tail_blocks * d.plan.nnt1 : 0;
+    w.split_cnt = take(split_tiles * 4);
+    w.split_part = take(split_tiles * d.plan.ksplit * ((size_t)d.plan.block_m * bf16_block_n1(d.plan.tile)) * 4);
     w.total = off;
     return w;
 }
@@ -162,6 +167,8 @@ FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E, const moe_o
     p.kernel_dtype = dtype;
     p.widen = false;
     p.mfma8 = false;
+    p.ksplit = 1;
+    p.tail_blocks = 0;
     const bool sw = act == MOE_ACT_SWIGLU;
     if (dtype == MOE_DTYPE_FP8_E4M3_B128) {
         // With this many rows per expert one more pass over the weights (e4m3 -> bf16 into the workspace) costs less
@@ -201,6 +208,16 @@ FfnPlan ffn_plan(int dtype, int act, int H, int I, int64_t A, int E, const moe_o
         p.block_m = bf16_block_m(p.tile);
         p.nnt0 = sw ? ceil_div(I, bf16_block_n0(p.tile) / 2) : ceil_div(I, bf16_block_n0(p.tile));
         p.nnt1 = ceil_div(H, bf16_block_n1(p.tile));
+        // Partial sums for the down-projection tiles of the last row blocks: F tasks of a 1/F of the contraction
+        // dimension each (the hand-ordered slab loop takes multiples of 128).  How many row blocks: the workgroups reach
+        // the short tasks spread over the length of a long one, F short ones; F / 2 rounds of short tasks absorb that
+        // spread on average, one more round is the tail proper.  Sized for kSplitWorkgroups resident workgroups whatever
+        // the device has (the workspace size must not depend on the device).
+        const int F = o.tail_split == 2 || o.tail_split == 4 ? o.tail_split : 1;
+        if (F > 1 && p.tile != 0 && I % (128 * F) == 0 && o.combine <= 0 && o.queue_early != 1) {
+            p.ksplit = F;
+            p.tail_blocks = ceil_div((int64_t)(F / 2 + 1) * kSplitWorkgroups, (int64_t)p.nnt1 * F);
+        }
     }
     return p;
 }
@@ -314,6 +331,11 @@ RouteArgs route_args(const moe_handle* h, void* ws) {
     a.lag = h->queue_lag;
     a.groups = h->queue_groups;
     a.tail_workgroups = h->opt.tail_round == 0 ? 0 : h->arch.persistent_blocks;
+    if (d.plan.ksplit > 1) {
+        a.tail_split = d.plan.ksplit;
+        a.tail_blocks = d.plan.tail_blocks;
+        a.split_cnt = at<int32_t>(ws, w.split_cnt);
+    }
     return a;
 }
 
@@ -374,6 +396,7 @@ const OptField kOptFields[] = {
     {"tail_round", &moe_options::tail_round, 0, 1, false},
     {"fp8_mfma", &moe_options::fp8_mfma, 0, 1, false},
     {"prepared_weights", &moe_options::prepared_weights, 0, 1, false},
+    {"tail_split", &moe_options::tail_split, 1, 4, true},
 };
 bool opt_in_domain(const OptField& f, int v) {
     if (v == MOE_OPT_AUTO) return true;
@@ -541,6 +564,7 @@ int moe_create_with_options(const moe_config* cfg, const moe_options* opt, moe_h
     h->opt.combine = h->combine_mode;
     h->opt.prepared_weights = d.plan.widen && !d.wide_in_workspace ? 1 : 0;
     h->opt.fp8_mfma = cfg->torch_dtype == MOE_DTYPE_FP8_E4M3_B128 ? (int)d.plan.mfma8 : MOE_OPT_AUTO;
+    h->opt.tail_split = tile16 ? d.plan.ksplit : MOE_OPT_AUTO;
     resolve_static_scratch(dev);
     *out = h;
     return MOE_OK;
@@ -794,6 +818,11 @@ int forward_on(moe_handle* h, const void* x, const moe_weights* w, void* out, co
     fa.pair_mt = ra.pair_mt;
     fa.combined = ra.done1 ? ra.arrive : nullptr;
     fa.cs = ra.cs;
+    if (d.plan.ksplit > 1) {
+        fa.split_cnt = ra.split_cnt;
+        fa.split_part = at<float>(workspace, L.split_part);
+        fa.split_extra_blocks = (d.plan.ksplit - 1) * d.plan.tail_blocks;
+    }
     if (d.plan.mfma8) {
         fa.xq = at<uint8_t>(workspace, L.xq);
         fa.sx = at<float>(workspace, L.sx);

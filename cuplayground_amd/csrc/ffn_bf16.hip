@@ -83,6 +83,11 @@ struct TaskPtrs {
     bool swiglu;
     bool publish;                // the rows will be read by other workgroups of the same launch
     uint32_t a_extent, b_extent; // bytes of the token operand (from a_base) and of one weight matrix (from b0 / b1)
+    // A task that is one of `kparts` partial sums of its tile over the contraction dimension (null part: a whole tile):
+    float* part;                 // the tile's partial-sum buffers, kparts x (block rows x block columns) fp32
+    int32_t* part_cnt;           // parts of the tile stored so far
+    int kparts, kpart;
+    bool poison;                 // such a task whose rows never became ready: its part is NaN
 };
 
 // silu for a bf16 result: hardware exp2 and reciprocal (about 1 ulp each in fp32, far below the bf16 rounding of
@@ -366,19 +371,36 @@ __device__ __forceinline__ void epilogue(const TaskPtrs& p, f32x4 (&acc)[T::TM][
 // padded by 16 bytes, which puts the 8-byte writes of 32 neighbouring lanes on distinct banks.  The bias values of
 // this lane's columns are loaded once (or are -0.0f, the neutral element of the addition), so the element loop has
 // no branch.
+// A store of more than 8 bytes reads its data registers over the cycles behind its issue, and an instruction that
+// writes one of them must keep two wait states' distance.  The compiler sees to that for the stores it emits, not for one
+// inside an asm statement -- it may well put the next value into the same registers right behind it -- so the statement
+// brings the wait states along.
+#define MOE_STORE16_AGENT "global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1"
 __device__ __forceinline__ void store16(uint16_t* p, u32x4 v, bool publish) {
-    if (publish) asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");   // agent scope, as publish8
+    if (publish) asm volatile(MOE_STORE16_AGENT ::"v"(p), "v"(v) : "memory");   // agent scope, as publish8
     else *reinterpret_cast<u32x4*>(p) = v;
 }
 
 struct NoHook {
     __device__ __forceinline__ void operator()(int) const {}
 };
+// The epilogue of a tile that was computed as KP partial sums (partial_tile_arrive): `base` is this lane's place in the
+// partial-sum buffers of the tile (two parts: in the other part's buffer; four parts: in the buffer of part 0).
+struct WholeTile {
+    static constexpr int KP = 1;
+};
+template <int KP_>
+struct SummedTile {
+    static constexpr int KP = KP_;
+    const float* base;
+};
 
 // `between(i)` runs in front of row group i (i = 0..7): the queue kernel issues the next task's first loads there, a
 // few at a time, so that they leave the compute unit under the epilogue's arithmetic instead of in front of it.
-template <class T, int MODE, class Hook>
-__device__ __forceinline__ void epilogue_full_n_impl(const TaskPtrs& p, unsigned char* smem, f32x4 (&acc)[8][T::TN], const Hook& between) {
+template <class T, int MODE, class Hook, class Parts = WholeTile>
+__device__ __forceinline__ void epilogue_full_n_impl(const TaskPtrs& p, unsigned char* smem, f32x4 (&acc)[8][T::TN], const Hook& between,
+                                                     const Parts& parts = Parts()) {
+    static_assert(Parts::KP == 1 || MODE == 0, "partial sums: the down projection only");
 
     static_assert(T::HAND, "four wavefronts of 128 x 128 or 128 x 64");
     constexpr int NJ = MODE == 3 ? T::TN / 2 : T::TN;   // groups of 16 output columns per wavefront
@@ -425,6 +447,36 @@ __device__ __forceinline__ void epilogue_full_n_impl(const TaskPtrs& p, unsigned
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         between(i);
+        // Partial sums: the row group's sums of the other parts come back from memory (written through by their tasks,
+        // read past this XCD's L2) and are added here -- two parts: own registers + the other part, which is the same
+        // in either order; four parts: all four as stored, in the order of the parts, whichever of them runs this.
+        f32x4 whole[Parts::KP == 1 ? 1 : NJ];
+        if constexpr (Parts::KP == 2) {
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+                asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(whole[j]) : "v"(parts.base + (i * NJ + j) * 256) : "memory");
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) asm volatile("s_waitcnt vmcnt(0)" : "+v"(whole[j])::"memory");
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) whole[j] = acc[i][j] + whole[j];
+        } else if constexpr (Parts::KP == 4) {
+            constexpr size_t kPartFloats = (size_t)T::BM * T::BN;
+#pragma unroll
+            for (int j0 = 0; j0 < NJ; j0 += 4) {
+                f32x4 v[4][4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v[k][j]) : "v"(parts.base + k * kPartFloats + (i * NJ + j0 + j) * 256) : "memory");
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) asm volatile("s_waitcnt vmcnt(0)" : "+v"(v[k][j])::"memory");
+#pragma unroll
+                for (int j = 0; j < 4; ++j) whole[j0 + j] = ((v[0][j] + v[1][j]) + v[2][j]) + v[3][j];
+            }
+        }
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
             float v[4];
@@ -434,7 +486,9 @@ __device__ __forceinline__ void epilogue_full_n_impl(const TaskPtrs& p, unsigned
                     const float g = acc[i][j][r] + b1[j][r], u = acc[i][j + NJ][r] + b0[j][r];
                     v[r] = silu_fast(g) * u;
                 } else {
-                    const float u = acc[i][j][r] + b0[j][r];
+                    float sum;
+                    if constexpr (Parts::KP == 1) sum = acc[i][j][r]; else sum = whole[j][r];
+                    const float u = sum + b0[j][r];
                     v[r] = MODE == 2 ? gelu_fast(u) : (u < relu_floor ? relu_floor : u);
                 }
             }
@@ -768,6 +822,63 @@ __device__ __forceinline__ bool ring_slabs(int rows, const RingLoads& L, unsigne
     return true;
 }
 
+// A tile computed as kparts partial sums over the contraction dimension, one task each (the down-projection tiles at the
+// end of the task queue: the tasks every workgroup ends its launch with, made short).  Every part stores its fp32
+// accumulators (written through: the parts run on any compute unit of the chip), then adds one to the tile's counter;
+// the part that finds all the others there runs the epilogue, which adds the parts up in an order that does not depend
+// on which part that is (epilogue_full_n_impl), so the result depends on kparts only, never on the schedule.  Returns
+// true in that workgroup; every wavefront of the workgroup calls it, `active` false for one whose rows are all padding (it
+// keeps the barriers company).
+// The buffer has the accumulator layout: [part][wavefront][register group i * TN + j][lane], 16 bytes each; tile_lane is
+// this lane's place in part 0.
+template <class T>
+__device__ __forceinline__ bool partial_tile_arrive(const TaskPtrs& p, unsigned char* smem, f32x4 (&acc)[8][T::TN], bool active,
+                                                    float* tile_lane) {
+    constexpr int TN = T::TN;
+    constexpr size_t kPartFloats = (size_t)T::BM * T::BN;
+    static_assert((size_t)T::THREADS / 64 * 8 * TN * 64 * 4 == kPartFloats, "the accumulators of the workgroup are the tile");
+    if (active) {
+        float* mine = tile_lane + (size_t)p.kpart * kPartFloats;
+        const float fill = __int_as_float(0x7FC00000);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                // (a part whose rows never became ready stores NaN: that is what the tile then holds)
+                const f32x4 v = p.poison ? f32x4{fill, fill, fill, fill} : acc[i][j];
+                asm volatile(MOE_STORE16_AGENT ::"v"(mine + (i * TN + j) * 256), "v"(v) : "memory");
+            }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // this wavefront's part has reached memory
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    int* s_before = reinterpret_cast<int*>(smem + T::NS * T::STAGE_BYTES);    // the staging area is idle until the epilogue
+    __syncthreads();
+    if (threadIdx.x == 0) *s_before = __hip_atomic_fetch_add(p.part_cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    const int before = __builtin_amdgcn_readfirstlane(*s_before);
+    __syncthreads();                                      // the word may be overwritten from here on
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    return before == p.kparts - 1;
+}
+
+// A task that is a part of a tile, behind its slab loop.
+template <class T>
+__device__ __forceinline__ void partial_tile_finish(const TaskPtrs& p, unsigned char* smem, f32x4 (&acc)[8][T::TN], bool active) {
+    constexpr size_t kPartFloats = (size_t)T::BM * T::BN;
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    const int lane = tid & 63, wave = tid >> 6;
+    float* tile_lane = p.part + ((size_t)wave * 8 * T::TN * 64 + lane) * 4;
+    if (!partial_tile_arrive<T>(p, smem, acc, active, tile_lane) || !active) return;
+    if (p.kparts == 2) {
+        const SummedTile<2> parts{tile_lane + (size_t)(1 - p.kpart) * kPartFloats};
+        epilogue_full_n_impl<T, 0>(p, smem, acc, NoHook(), parts);
+    } else {
+        const SummedTile<4> parts{tile_lane};
+        epilogue_full_n_impl<T, 0>(p, smem, acc, NoHook(), parts);
+    }
+}
+
 // One task from start to end: the form the two-launch and the plain-GEMM kernels use.
 template <class T>
 __device__ __forceinline__ void gemm_tile_ring(const TaskPtrs& p, unsigned char* smem) {
@@ -776,6 +887,18 @@ __device__ __forceinline__ void gemm_tile_ring(const TaskPtrs& p, unsigned char*
     ring_first_loads<T>(L, smem);
     f32x4 acc[8][T::TN];
     if (ring_slabs<T>(p.rows, L, smem, acc)) epilogue_full_n<T>(p, smem, acc);
+}
+// The same for a task that is a part of a tile (TaskPtrs::part).  A copy of its own, slab loop included: with both ends
+// behind one loop the compiler reads all accumulators in front of the branch between them and spills what does not fit,
+// which costs the whole tiles -- nearly all of them -- 4 to 13 % of their time.
+template <class T>
+__device__ __forceinline__ void gemm_tile_ring_part(const TaskPtrs& p, unsigned char* smem) {
+    const RingLoads L = ring_prepare<T>(p);
+    __syncthreads();
+    ring_first_loads<T>(L, smem);
+    f32x4 acc[8][T::TN];
+    const bool active = ring_slabs<T>(p.rows, L, smem, acc);
+    partial_tile_finish<T>(p, smem, acc, active);
 }
 
 template <class T, bool PARTIAL>
@@ -840,6 +963,25 @@ __device__ __forceinline__ TaskPtrs resolve(const FfnArgs& a, const Task& t, boo
     p.rows = t.rows;
     p.a_extent = t.phase == 0 ? a.x_bytes : a.h_bytes;
     p.b_extent = a.w_bytes;
+    p.part = nullptr;
+    p.part_cnt = nullptr;
+    p.kparts = 1;
+    p.kpart = 0;
+    p.poison = false;
+    if (t.phase == 1 && t.kparts > 1) {       // one of kparts partial sums: this part's share of the intermediate dimension
+        const int Kp = a.I / t.kparts, k0 = t.kpart * Kp;
+        p.K = Kp;
+        p.a_base += k0;
+        p.b0 += k0;
+        p.a_extent -= (uint32_t)k0 * 2;       // the descriptors start where the operands now start
+        p.b_extent -= (uint32_t)k0 * 2;
+        const int tile = (t.mtile - a.q->split_mt0) * a.nnt1 + t.ntile;
+        p.part = a.split_part + (size_t)tile * t.kparts * ((size_t)T::BM * T::BN);
+        p.part_cnt = a.split_cnt + tile;
+        p.kparts = t.kparts;
+        p.kpart = t.kpart;
+        p.poison = t.poison;
+    }
     return p;
 }
 
@@ -873,14 +1015,27 @@ using MediumPlanH = Plan<Tile128x256H, Tile128x256H>;
 using SmallPlanH = Plan<Tile<128, 128, 2, 2, 2, true>, Tile<128, 128, 2, 2, 2, true>>;
 
 // One task of a plan: the plan's tile, or its small-row-block tile when the block has few enough rows.
-template <class P>
+// SPLIT: the task may be a part of a tile (kernels of their own: the code for it costs the others 1-2 % in short tasks).
+template <class P, bool SPLIT = false>
 __device__ __forceinline__ void plan_tile(const FfnArgs& a, const Task& t, bool publish, unsigned char* smem) {
     static_assert(std::is_same<typename P::T0, typename P::T1>::value, "one tile for both projections: one inlined copy");
     const TaskPtrs p = resolve<typename P::T0>(a, t, publish);
     if constexpr (P::MIXED) {
         static_assert(P::TS::BN == P::T0::BN && P::TS::LDS_BYTES <= P::LDS_BYTES, "same columns per task");
         if (t.rows <= P::TS::BM) {
+            if constexpr (SPLIT && P::TS::HAND) {
+                if (p.part) {
+                    gemm_tile_ring_part<typename P::TS>(p, smem);
+                    return;
+                }
+            }
             gemm_tile<typename P::TS>(p, smem);
+            return;
+        }
+    }
+    if constexpr (SPLIT && P::T0::HAND) {
+        if (p.part) {
+            gemm_tile_ring_part<typename P::T0>(p, smem);
             return;
         }
     }
@@ -888,7 +1043,7 @@ __device__ __forceinline__ void plan_tile(const FfnArgs& a, const Task& t, bool 
 }
 
 // One launch per phase; workgroup b runs task b of that phase.
-template <class P>
+template <class P, bool SPLIT = false>
 __global__ __launch_bounds__(P::THREADS) void ffn_tiled_kernel(FfnArgs a, int phase) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ int s_list[1 + P::T0::BM];
@@ -896,7 +1051,7 @@ __global__ __launch_bounds__(P::THREADS) void ffn_tiled_kernel(FfnArgs a, int ph
     if (phase == 0) zero_unrouted_rows(a, 2);
     Task t;
     if (!tiled_task(a, phase, blockIdx.x, t)) return;
-    plan_tile<P>(a, t, phase == 1 && a.arrive, smem);       // rows another workgroup may combine go out write-through
+    plan_tile<P, SPLIT>(a, t, phase == 1 && a.arrive, smem);   // rows another workgroup may combine go out write-through
     if (phase == 1 && a.arrive) combine_arrivals<ET>(combine_args(a), t.row0, t.rows, t.ntile, t.ntile * P::T1::BN, P::T1::BN, s_list);
 }
 
@@ -911,7 +1066,7 @@ __device__ __forceinline__ const FfnArgs& kernel_args_again() {
 }
 
 // Persistent workgroups popping (expert, tile) tasks from the queue of their XCD (protocol: ffn_common.hpp).
-template <class P>
+template <class P, bool SPLIT = false>
 __global__ __launch_bounds__(P::THREADS) void ffn_persistent_kernel(FfnArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ int s_task, s_ok;
@@ -929,14 +1084,19 @@ __global__ __launch_bounds__(P::THREADS) void ffn_persistent_kernel(FfnArgs a) {
     while (next_task(a, cur, &s_task, ids, nseg, nnt0, t)) {   // uniform exit: every wavefront leaves together
         if (t.phase == 1 && !wait_phase0_done(a.done0, t.mtile, nnt0, a.spin_limit, a.q, a.host_stall, &s_ok)) {
             // the rows never became ready: NaN instead of a result, and a tile of no rows (it loads, computes and
-            // stores nothing of its own), so that the loop keeps its one shape
-            poison_tile((uint16_t*)a.y + (int64_t)t.row0 * a.H, t.rows, a.H, t.ntile * P::T1::BN, P::T1::BN, 2);
-            t.rows = 0;
+            // stores nothing of its own), so that the loop keeps its one shape; a part of a tile keeps its shape too (the
+            // parts must agree on it) and hands on NaN in place of its sums
+            if (t.kparts > 1) {
+                t.poison = true;
+            } else {
+                poison_tile((uint16_t*)a.y + (int64_t)t.row0 * a.H, t.rows, a.H, t.ntile * P::T1::BN, P::T1::BN, 2);
+                t.rows = 0;
+            }
         }
         const long long started = trace_clock(kernel_args_again().task_trace);
-        plan_tile<P>(a, t, t.phase == 0 || publish_y(a), smem);
+        plan_tile<P, SPLIT>(a, t, t.phase == 0 || publish_y(a), smem);
         if (kernel_args_again().task_trace)
-            trace_task(kernel_args_again().task_trace, kernel_args_again().task_trace_cap, t.phase, t.expert, t.mtile, t.ntile, t.rows, started);
+            trace_task(kernel_args_again().task_trace, kernel_args_again().task_trace_cap, t.phase | (t.kparts > 1 ? (t.kpart << 2) | (t.kparts << 4) : 0), t.expert, t.mtile, t.ntile, t.rows, started);
         if (t.phase == 0) signal_phase0_done(a.done0, t.mtile);
         else                 // the row count from the table: a tile whose wait expired runs with none, and still arrives
             after_down_tile<ET>(kernel_args_again(), t.row0, a.mtiles[t.mtile].rows, t.mtile, t.ntile, t.ntile * P::T1::BN, P::T1::BN, s_list);
@@ -989,6 +1149,7 @@ __global__ __launch_bounds__(P::THREADS) void ffn_persistent_ring_kernel(FfnArgs
     auto as_task = [&]() {
         Task q;
         q.phase = ph; q.expert = ex; q.mtile = mt; q.ntile = nt; q.row0 = row0; q.rows = rows; q.nnt0 = nnt0; q.valid = true;
+        q.kparts = 1; q.kpart = 0; q.poison = false;     // (the host never asks for this loop and partial sums together)
         return q;
     };
     RingLoads L;
@@ -1107,6 +1268,7 @@ __global__ __launch_bounds__(T::THREADS) void gemm_dense_kernel(const uint16_t* 
     p.publish = false;
     p.a_extent = (uint32_t)((int64_t)M * K * 2);
     p.b_extent = (uint32_t)((int64_t)N * K * 2);
+    p.part = nullptr; p.part_cnt = nullptr; p.kparts = 1; p.kpart = 0; p.poison = false;
     gemm_tile<T>(p, smem);
 }
 
@@ -1153,6 +1315,7 @@ __global__ __launch_bounds__(T::THREADS) void grouped_gemm_kernel(const uint16_t
     p.publish = false;
     p.a_extent = a_bytes;
     p.b_extent = (uint32_t)((int64_t)N * K * 2);
+    p.part = nullptr; p.part_cnt = nullptr; p.kparts = 1; p.kpart = 0; p.poison = false;
     gemm_tile<T>(p, smem);
 }
 
@@ -1197,6 +1360,7 @@ __global__ __launch_bounds__(T::THREADS) void wgrad_kernel(const uint16_t* dyT, 
     p.publish = false;
     p.a_extent = dy_bytes - (uint32_t)p0 * 2;
     p.b_extent = a_bytes - (uint32_t)p0 * 2;
+    p.part = nullptr; p.part_cnt = nullptr; p.kparts = 1; p.kpart = 0; p.poison = false;
     gemm_tile<T>(p, smem);
 }
 
@@ -1211,6 +1375,14 @@ hipError_t launch_tiled(const FfnArgs& a, int max_mtiles, int nnt0, int nnt1, hi
     hipError_t e = allow_lds(&ffn_tiled_kernel<P>, P::LDS_BYTES);
     if (e != hipSuccess) return e;
     ffn_tiled_kernel<P><<<tiled_grid(max_mtiles, nnt0, a.groups), P::THREADS, P::LDS_BYTES, st>>>(a, 0);
+    if constexpr (P::T0::HAND) {
+        if (a.split_cnt) {      // row blocks whose tiles run as partial sums count once per part
+            e = allow_lds(&ffn_tiled_kernel<P, true>, P::LDS_BYTES);
+            if (e != hipSuccess) return e;
+            ffn_tiled_kernel<P, true><<<tiled_grid(max_mtiles + a.split_extra_blocks, nnt1, a.groups), P::THREADS, P::LDS_BYTES, st>>>(a, 1);
+            return hipGetLastError();
+        }
+    }
     ffn_tiled_kernel<P><<<tiled_grid(max_mtiles, nnt1, a.groups), P::THREADS, P::LDS_BYTES, st>>>(a, 1);
     return hipGetLastError();
 }
@@ -1224,6 +1396,14 @@ hipError_t launch_persistent(const FfnArgs& a, int blocks, bool early, hipStream
             hipError_t e = allow_lds(&ffn_persistent_ring_kernel<P>, P::LDS_BYTES);
             if (e != hipSuccess) return e;
             ffn_persistent_ring_kernel<P><<<blocks, P::THREADS, P::LDS_BYTES, st>>>(a);
+            return hipGetLastError();
+        }
+    }
+    if constexpr (P::T0::HAND) {
+        if (a.split_cnt) {
+            hipError_t e = allow_lds(&ffn_persistent_kernel<P, true>, P::LDS_BYTES);
+            if (e != hipSuccess) return e;
+            ffn_persistent_kernel<P, true><<<blocks, P::THREADS, P::LDS_BYTES, st>>>(a);
             return hipGetLastError();
         }
     }

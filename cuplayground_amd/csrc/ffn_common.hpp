@@ -25,44 +25,26 @@ struct Task {
     int row0;      // first packed row
     int rows;      // valid rows in the block
     int nnt0;      // phase-0 column tiles per row block (the dependency target)
+    int kparts;    // 1, or F: the task is one of F partial sums of its tile over the contraction dimension ...
+    int kpart;     // ... this one
+    bool poison;   // such a task whose rows never became ready (its part is stored as NaN)
     bool valid;    // false: a hole of this group's id space, nothing to do
 };
 
-// Finds the segment holding id `id` of queue group `group` (segments are sorted by begin, possibly empty) and
-// decodes it.  All arguments are wavefront-uniform, so the loads are scalar.
-//
-// Order inside a segment (ids of one group): row blocks fastest -- consecutive ids, popped by workgroups that run side by
-// side, share one column tile's weights.  With row_chunk R > 0 the expert's row blocks are taken R at a time: all
-// column tiles of the first R row blocks, then of the next R, ...; the workgroups of an XCD then hold fewer row blocks
-// and more column tiles at a time (for kernels whose token rows cost more L2 space than their weight rows).
+// The task behind id `id` of queue group `group` (queue_order.hpp: decode_id), with its rows from the MTile table.  All
+// arguments are wavefront-uniform, so the loads are scalar.
 __device__ __forceinline__ Task decode_task(const Segment* __restrict__ segs, int nseg, const MTile* __restrict__ mtiles,
                                             int id, int group, int groups, int nnt0, int row_chunk = 0) {
-    int lo = 0, hi = nseg - 1;
-    while (lo < hi) {   // last segment with begin <= id
-        const int mid = (lo + hi + 1) >> 1;
-        if (segs[mid].begin <= id) lo = mid; else hi = mid - 1;
-    }
-    const Segment s = segs[lo];
-    const int local = id - s.begin;
+    const TaskId d = decode_id(segs, nseg, id, group, groups, row_chunk);
     Task t;
-    t.phase = s.phase;
-    t.expert = s.expert;
-    int j, mb;
-    if (row_chunk > 0 && row_chunk < s.nmt) {
-        const int per_chunk = row_chunk * ((s.nnt + groups - 1) / groups);   // ids of a full chunk
-        const int c = local / per_chunk, rem = local - c * per_chunk;
-        const int rc = min(row_chunk, s.nmt - c * row_chunk);               // the last chunk may be shorter
-        j = rem / rc;
-        mb = c * row_chunk + (rem - j * rc);
-    } else {
-        j = local / s.nmt;
-        mb = local - j * s.nmt;
-    }
-    int first = group - s.rot;
-    if (first < 0) first += groups;
-    t.ntile = first + groups * j;
-    t.valid = t.ntile < s.nnt;
-    t.mtile = s.mt0 + mb;
+    t.phase = d.phase;
+    t.expert = d.expert;
+    t.mtile = d.mtile;
+    t.ntile = d.ntile;
+    t.kparts = d.kparts;
+    t.kpart = d.kpart;
+    t.poison = false;
+    t.valid = d.valid;
     const MTile m = mtiles[t.mtile];
     t.row0 = m.row0;
     t.rows = m.rows;
@@ -140,7 +122,7 @@ __device__ __forceinline__ bool next_task(const FfnArgs& a, QueueCursor& c, int*
 __device__ __forceinline__ bool tiled_task(const FfnArgs& a, int phase, int b, Task& t) {
     const int group = b % a.groups, id = b / a.groups;
     if (id >= (phase ? a.q->ids_phase1 : a.q->ids_phase0)) return false;
-    t = decode_task(phase ? a.seg_phase1 : a.seg_phase0, a.E, a.mtiles, id, group, a.groups, a.seg_phase0[0].nnt, a.row_chunk);
+    t = decode_task(phase ? a.seg_phase1 : a.seg_phase0, phase ? a.q->nseg_phase1 : a.E, a.mtiles, id, group, a.groups, a.seg_phase0[0].nnt, a.row_chunk);
     return t.valid;
 }
 

@@ -58,7 +58,9 @@ struct QueueState {
     int32_t ids_queue;     // ids per group in the merged queue (holes included)
     int32_t ids_phase0;    // ids per group in the phase-0 table / the phase-1 table (tiled mode)
     int32_t ids_phase1;
-    int32_t pad[5];
+    int32_t split_mt0;     // first row block whose down-projection tiles run as partial sums (num_mtiles: none)
+    int32_t nseg_phase1;   // segments of the phase-1 table (the experts, plus one when a run was cut at split_mt0)
+    int32_t pad[3];
 };
 // State of the combine tasks of the queue kernels, in a cache line of its own: the workgroups that have run out of GEMM
 // tasks poll it, and must not stand in the way of the queue heads that the busy ones pop.
@@ -84,7 +86,7 @@ struct FfnArgs {
     void* y;                    // [A,H] expert outputs, activation dtype
     const MTile* mtiles;
     const Segment* seg_phase0;  // E segments, task ids local to phase 0
-    const Segment* seg_phase1;  // E segments, task ids local to phase 1
+    const Segment* seg_phase1;  // QueueState::nseg_phase1 segments, task ids local to phase 1
     const Segment* seg_queue;   // 2E segments in queue order
     QueueState* q;
     int32_t* done0;             // per MTile: finished phase-0 column tiles
@@ -111,6 +113,10 @@ struct FfnArgs {
     const int32_t* pair_mt;     // [S, k] row block (MTile index) of every (token, rank), -1 when dropped
     int32_t* combined;          // [slices, S]: 1 once the unit has been taken
     CombineState* cs;
+    // Down-projection tiles of the queue's tail as partial sums over the contraction dimension (null split_cnt: not used)
+    int32_t* split_cnt;         // [tiles]: parts of the tile that have been stored
+    float* split_part;          // [tiles][parts][block rows x block columns] fp32, in the accumulator layout of the tile
+    int32_t split_extra_blocks; // (parts - 1) x the most row blocks that can run so: what the down projection's id space grows by
     // e4m3 x e4m3 plan (null xq: not used): the token rows and the intermediate rows as e4m3 codes with one scale per
     // (row, 128 columns), written by quant_rows128 passes in front of the two projections
     uint8_t* xq;                // [S, H]
@@ -149,6 +155,9 @@ struct RouteArgs {
     int32_t lag;                // experts of phase-0 work queued between an expert's two phases
     int32_t groups;             // queue groups: 1, or one per XCD
     int32_t tail_workgroups;    // 0, or the workgroups of the queue kernel: the tail of the queue is rounded to them (route.hip: round_tail)
+    int32_t tail_split;         // 0 / 1: whole tiles everywhere; F: the down-projection tiles of the last row blocks run as F partial sums
+    int32_t tail_blocks;        // ... how many row blocks (what the partial-sum buffers were sized for)
+    int32_t* split_cnt;         // [tail_blocks * nnt1] arrival counters of those tiles, cleared here
     int64_t* task_trace;        // null, or the FFN stage's trace buffer: its record count starts every call at zero
 };
 
@@ -171,6 +180,8 @@ hipError_t launch_combine(const void* y_rows, const int32_t* pair_row, const flo
 struct FfnPlan {
     int kernel_dtype;   // the dtype whose kernels run: the layer's, or bf16 for an e4m3 layer whose weights are widened
     bool widen;         // e4m3 layer run as a bf16 layer on weights widened into the workspace by every call
+    int ksplit;         // 16-bit layers on the hand-ordered tiles: parts a down-projection tile of the last row blocks is summed in (1: whole tiles)
+    int tail_blocks;    // ... and how many row blocks those are
     bool mfma8;         // e4m3 layer on the tile GEMM with both operands e4m3 (tokens quantised per row and 128 columns)
     int tile;        // 16-bit layers: which tile the kernels are instantiated with (ffn_bf16.hip: bf16_tile)
     int block_m;

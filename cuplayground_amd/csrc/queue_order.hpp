@@ -29,8 +29,64 @@ struct Segment {
     int32_t nmt;      // row blocks of the run
     int32_t nnt;      // column tiles of this phase
     int32_t rot;      // rotation of the column-tile round robin over the groups
-    int32_t pad1;
+    int32_t split;    // 0 or 1: whole tiles; F > 1 (down projection only): every tile of the run is F tasks, each a partial
+                      // sum over a 1/F of the contraction dimension -- ids then run (j * nmt + mtile_local) * F + part
 };
+
+// What a task id of one queue group stands for.
+struct TaskId {
+    int32_t phase, expert;
+    int32_t mtile;    // index into the MTile table
+    int32_t ntile;    // column tile of this phase
+    int32_t kparts;   // 1, or F: the task is one of F partial sums of its tile over the contraction dimension ...
+    int32_t kpart;    // ... this one
+    bool valid;       // false: a hole of this group's id space, nothing to do
+};
+
+// Finds the segment holding id `id` of queue group `group` (segments are sorted by begin, possibly empty; 0 <= id < the
+// table's total) and decodes it.
+//
+// Order inside a segment (ids of one group): row blocks fastest -- consecutive ids, popped by workgroups that run side by
+// side, share one column tile's weights.  With row_chunk R > 0 the run's row blocks are taken R at a time: all
+// column tiles of the first R row blocks, then of the next R, ...; the workgroups of an XCD then hold fewer row blocks
+// and more column tiles at a time (for kernels whose token rows cost more L2 space than their weight rows).  In a run
+// of partial sums the parts of a tile are consecutive ids: they run side by side and meet again soon.
+MOE_HD inline TaskId decode_id(const Segment* __restrict__ segs, int nseg, int id, int group, int groups, int row_chunk) {
+    int lo = 0, hi = nseg - 1;
+    while (lo < hi) {   // last segment with begin <= id
+        const int mid = (lo + hi + 1) >> 1;
+        if (segs[mid].begin <= id) lo = mid; else hi = mid - 1;
+    }
+    const Segment s = segs[lo];
+    int local = id - s.begin;
+    TaskId t;
+    t.phase = s.phase;
+    t.expert = s.expert;
+    t.kparts = s.split > 1 ? s.split : 1;
+    t.kpart = 0;
+    if (t.kparts > 1) {
+        t.kpart = local % t.kparts;
+        local /= t.kparts;
+    }
+    int j, mb;
+    if (row_chunk > 0 && row_chunk < s.nmt) {
+        const int per_chunk = row_chunk * ((s.nnt + groups - 1) / groups);   // ids of a full chunk
+        const int c = local / per_chunk, rem = local - c * per_chunk;
+        const int left = s.nmt - c * row_chunk;
+        const int rc = row_chunk < left ? row_chunk : left;                  // the last chunk may be shorter
+        j = rem / rc;
+        mb = c * row_chunk + (rem - j * rc);
+    } else {
+        j = local / s.nmt;
+        mb = local - j * s.nmt;
+    }
+    int first = group - s.rot;
+    if (first < 0) first += groups;
+    t.ntile = first + groups * j;
+    t.valid = t.ntile < s.nnt;
+    t.mtile = s.mt0 + mb;
+    return t;
+}
 
 struct TailParams {
     int32_t E, lag, nnt0, nnt1, groups, tail_workgroups;
@@ -98,10 +154,46 @@ MOE_HD inline int round_tail(Segment* q, int nseg, const TailParams& a, int* tot
     int begin = q[p - 1].begin;
     for (int i = p - 1; i <= nseg; ++i) {
         q[i].begin = begin;
-        begin += q[i].nmt * (q[i].phase ? npg1 : npg0);
+        begin += q[i].nmt * (q[i].phase ? npg1 : npg0) * (q[i].split > 1 ? q[i].split : 1);
     }
     *total_ids = begin;
     return nseg + 1;
+}
+
+// The down-projection tiles of the last row blocks as partial sums.
+//
+// Row blocks [split_mt0, ...) -- the end of the last experts' runs, hence the end of the queue -- have each of their
+// down-projection tiles computed as F tasks over a 1/F of the contraction dimension each (Segment::split): the tasks a
+// workgroup ends its launch with are then a 1/F as long, and so is the time the others idle behind the last of them.
+// Segments of phase 1 that lie wholly in that range are marked, one that straddles its start is cut in two (an
+// expert's row blocks are consecutive and the experts' runs follow each other, so at most one does), and every begin
+// is recomputed.  The order of the tasks does not change, so in every queue a row block's up-projection tasks still
+// precede its down-projection tasks.  Takes the merged queue or the table of phase 1 alone.
+// Run by one thread behind the segment table's barrier (q has room for nseg + 1 segments).  Returns the new segment count.
+MOE_HD inline int split_tail(Segment* q, int nseg, int split_mt0, int F, int npg0, int npg1, int* total_ids) {
+    if (F > 1) {
+        int cut = -1;
+        for (int i = 0; i < nseg; ++i)
+            if (q[i].phase == 1 && q[i].mt0 < split_mt0 && q[i].mt0 + q[i].nmt > split_mt0) cut = i;
+        if (cut >= 0) {
+            for (int i = nseg; i > cut + 1; --i) q[i] = q[i - 1];
+            const int keep = split_mt0 - q[cut].mt0;
+            q[cut + 1] = q[cut];
+            q[cut + 1].mt0 = split_mt0;
+            q[cut + 1].nmt = q[cut].nmt - keep;
+            q[cut].nmt = keep;
+            ++nseg;
+        }
+        for (int i = 0; i < nseg; ++i)
+            if (q[i].phase == 1 && q[i].nmt > 0 && q[i].mt0 >= split_mt0) q[i].split = F;
+    }
+    int begin = 0;
+    for (int i = 0; i < nseg; ++i) {
+        q[i].begin = begin;
+        begin += q[i].nmt * (q[i].phase ? npg1 : npg0) * (q[i].split > 1 ? q[i].split : 1);
+    }
+    *total_ids = begin;
+    return nseg;
 }
 
 }  // namespace moe355

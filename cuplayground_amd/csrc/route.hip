@@ -75,7 +75,7 @@ __global__ __launch_bounds__(kRouteBlock) void route_count_kernel(RouteArgs a) {
 __device__ __forceinline__ void write_segment(Segment* s, int begin, int phase, int expert, int mt0, int nmt, int nnt,
                                               int groups) {
     s->begin = begin; s->phase = phase; s->expert = expert; s->mt0 = mt0; s->nmt = nmt; s->nnt = nnt;
-    s->rot = (int)(((int64_t)expert * nnt) % groups); s->pad1 = 0;
+    s->rot = (int)(((int64_t)expert * nnt) % groups); s->split = 0;
 }
 
 // Exclusive prefix sum of one int per thread over a workgroup of kMaxExperts threads (wave shuffles, then the
@@ -109,6 +109,11 @@ struct ScanShared {
     int mt0[kMaxExperts];
     int part[kMaxExperts];
     int total[kMaxExperts];
+    // the segment tables while one thread rearranges them (split_tail): in LDS, where its dependent accesses cost cycles,
+    // not memory round trips
+    Segment segq[2 * kMaxExperts + 1];
+    Segment seg1[kMaxExperts + 1];
+    int nseg_out[2], ids_out[2];
 };
 __device__ __forceinline__ void route_scan_body(const RouteArgs& a, ScanShared& sh) {
     int* s_wave = sh.wave;
@@ -183,8 +188,34 @@ __device__ __forceinline__ void route_scan_body(const RouteArgs& a, ScanShared& 
             write_segment(a.seg_queue + sidx, begin + (j ? size[0] : 0), ph[j], ex[j], s_mt0[ex[j]], s_nmt[ex[j]],
                           ph[j] ? a.nnt1 : a.nnt0, a.groups);
     }
-    int nseg_final = nseg;
-    if (a.tail_workgroups > 0) {
+    if (e < a.E) {
+        a.expert_count[e] = kept;
+        a.expert_offset[e] = off;
+        write_segment(a.seg_phase0 + e, mt0 * npg0, 0, e, mt0, nmt, a.nnt0, a.groups);
+        write_segment(a.seg_phase1 + e, mt0 * npg1, 1, e, mt0, nmt, a.nnt1, a.groups);
+    }
+    // Down-projection tiles of the last tail_blocks row blocks as tail_split partial sums each (queue_order.hpp:
+    // split_tail); a tail of short tasks needs no rounding.
+    const int F = a.tail_split > 1 ? a.tail_split : 1;
+    const int split_mt0 = F > 1 ? max(total_mt - a.tail_blocks, 0) : total_mt;
+    int nseg_final = nseg, nseg_phase1 = a.E, ids_phase1 = total_mt * npg1;
+    if (F > 1) {
+        __syncthreads();                                  // the segment tables are complete
+        for (int i = threadIdx.x; i < nseg; i += blockDim.x) sh.segq[i] = a.seg_queue[i];
+        for (int i = threadIdx.x; i < a.E; i += blockDim.x) sh.seg1[i] = a.seg_phase1[i];
+        __syncthreads();
+        if (e == 0) {
+            sh.nseg_out[0] = split_tail(sh.segq, nseg, split_mt0, F, npg0, npg1, &sh.ids_out[0]);
+            sh.nseg_out[1] = split_tail(sh.seg1, a.E, split_mt0, F, npg0, npg1, &sh.ids_out[1]);
+        }
+        __syncthreads();
+        nseg_final = sh.nseg_out[0];
+        nseg_phase1 = sh.nseg_out[1];
+        total_tasks = sh.ids_out[0];
+        ids_phase1 = sh.ids_out[1];
+        for (int i = threadIdx.x; i < nseg_final; i += blockDim.x) a.seg_queue[i] = sh.segq[i];
+        for (int i = threadIdx.x; i < nseg_phase1; i += blockDim.x) a.seg_phase1[i] = sh.seg1[i];
+    } else if (a.tail_workgroups > 0) {
         __syncthreads();                                  // the segment table is complete
         if (e == 0) {
             const TailParams tp{a.E, a.lag, a.nnt0, a.nnt1, a.groups, a.tail_workgroups};
@@ -198,7 +229,9 @@ __device__ __forceinline__ void route_scan_body(const RouteArgs& a, ScanShared& 
         if (a.task_trace) a.task_trace[0] = 0;
         a.q->ids_queue = total_tasks;
         a.q->ids_phase0 = total_mt * npg0;
-        a.q->ids_phase1 = total_mt * npg1;
+        a.q->ids_phase1 = ids_phase1;
+        a.q->nseg_phase1 = nseg_phase1;
+        a.q->split_mt0 = split_mt0;
         a.q->total_tasks = total_mt * (a.nnt0 + a.nnt1);
         a.q->tasks_phase0 = total_mt * a.nnt0;
         a.q->tasks_phase1 = total_mt * a.nnt1;
@@ -208,11 +241,7 @@ __device__ __forceinline__ void route_scan_body(const RouteArgs& a, ScanShared& 
         a.q->nseg = nseg_final;
         a.expert_offset[a.E] = total_rows;
     }
-    if (e < a.E) {
-        a.expert_count[e] = kept;
-        a.expert_offset[e] = off;
-        write_segment(a.seg_phase0 + e, mt0 * npg0, 0, e, mt0, nmt, a.nnt0, a.groups);
-        write_segment(a.seg_phase1 + e, mt0 * npg1, 1, e, mt0, nmt, a.nnt1, a.groups);
+    if (e < a.E) {          // (behind the tail's one-thread section: the other threads get on with this meanwhile)
         for (int i = 0; i < nmt; ++i) {
             MTile t;
             t.expert = e;
@@ -225,6 +254,8 @@ __device__ __forceinline__ void route_scan_body(const RouteArgs& a, ScanShared& 
     for (int i = threadIdx.x; i < a.max_mtiles; i += blockDim.x) a.done0[i] = 0;
     if (a.done1)
         for (int i = threadIdx.x; i < a.max_mtiles; i += blockDim.x) a.done1[i] = 0;
+    if (a.split_cnt)
+        for (int i = threadIdx.x; i < a.tail_blocks * a.nnt1; i += blockDim.x) a.split_cnt[i] = 0;
 }
 
 __global__ __launch_bounds__(kMaxExperts) void route_scan_kernel(RouteArgs a) {

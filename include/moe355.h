@@ -148,7 +148,14 @@ typedef struct moe_options {
     int32_t prepared_weights;/* 1 = every moe_forward on the handle will carry moe_weights.prepared (moe_prepare_weights): the
                                 workspace then holds no copies of the weights and a call without them is refused; 0 / AUTO =
                                 prepared weights are used when given, else made per call in the workspace */
-    int32_t reserved[7];     /* must be MOE_OPT_AUTO */
+    int32_t tail_split;      /* 16-bit layers on the 256-column tiles (tile16 1, 2, 3): 2 or 4 = every down-projection tile of the last
+                                row blocks -- the tasks the launch ends with -- is computed as that many tasks, each a partial sum
+                                over its share of the intermediate dimension, kept in fp32 in the workspace and added up in a
+                                fixed order by the task that finishes last: the launch's tail gets shorter tasks, the sums
+                                of those tiles are associated differently (same tolerance, other bits; the same in both
+                                ffn modes).  1 / AUTO = whole tiles.  Ignored where the intermediate size is not a multiple of
+                                128 x parts, with combine != 0 and with queue_early. */
+    int32_t reserved[6];     /* must be MOE_OPT_AUTO */
 } moe_options;
 /* Every field MOE_OPT_AUTO. */
 int moe_options_default(moe_options* opt);
@@ -313,7 +320,8 @@ int moe_get_queue_balance(moe_handle* h, const void* workspace, void* stream, in
  * and one atomic per task.  Counterpart in the reference: the clock stamps its kernels print (mma.cuh:51-57,162-169;
  * scheduling.cuh:261-263). */
 typedef struct moe_task_record {
-    int32_t phase;      /* 0: up(/gate) projection + activation, 1: down projection */
+    int32_t phase;      /* 0: up(/gate) projection + activation, 1: down projection; a task that computed one of P partial
+                           sums of its tile (option tail_split) has 1 + 4 * part + 16 * P here */
     int32_t expert;
     int32_t row_block;  /* index into the layer's row-block table (expert-major) */
     int32_t col_tile;

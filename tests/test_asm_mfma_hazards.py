@@ -239,3 +239,20 @@ def test_fp8_tile_weight_bytes_are_not_touched_in_flight():
                     raise AssertionError("no wait for " + y)
                 checked += 1
         assert checked >= 4, (name, checked)       # two loads per slab, two slabs per loop iteration
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
+def test_asm_stores_keep_their_data_registers():
+    """A store of more than 8 bytes reads its data registers over the cycles behind its issue; whoever writes one of
+    them must keep two wait states' distance.  The compiler pads the stores it emits itself but does not look inside an
+    asm statement -- and it does reuse the data registers right away (the partial-sum stores of the queue kernel came
+    out as store v[0:3]; v_accvgpr_read v0 and lost a dword in a quarter of the lanes).  So every 16-byte store that
+    comes from an asm statement must bring its wait states along."""
+    text = _assembly()
+    stores = 0
+    lines = [l.strip() for l in text.split("\n")]
+    for k, l in enumerate(lines):
+        if l.startswith(";;#ASMSTART") and k + 1 < len(lines) and lines[k + 1].startswith(("global_store_dwordx3", "global_store_dwordx4")):
+            stores += 1
+            assert lines[k + 2].startswith("s_nop 1"), "asm store without wait states: %s / %s" % (lines[k + 1], lines[k + 2])
+    assert stores > 100      # the published rows of the hand-ordered tiles and the partial sums

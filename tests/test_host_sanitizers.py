@@ -34,7 +34,8 @@ def test_config_loader_is_clean_under_asan_and_ubsan(tmp_path):
 def test_queue_order_keeps_every_dependency_under_asan_and_ubsan(tmp_path):
     """csrc/queue_order.hpp is the code the routing kernel builds its merged task queue with; the same functions run here
     on the host for 20000 random layers: every row block's up-projection run stands in front of its down-projection run,
-    the id space has no gaps, and a rounded tail fills whole rounds of the workgroups."""
+    the id space has no gaps, a rounded tail fills whole rounds of the workgroups, and with the last row blocks' tiles cut into
+    partial sums every id of every queue decodes to each (row block, column tile, part) exactly once."""
     exe = str(tmp_path / "queue_order")
     cmd = ["g++", "-std=c++17", "-O1", "-g", "-fno-omit-frame-pointer", "-fsanitize=address,undefined",
            "-fno-sanitize-recover=all", "-static-libasan", "-I", os.path.join(ROOT, "cuplayground_amd", "csrc"), "-o", exe,
@@ -45,4 +46,4 @@ def test_queue_order_keeps_every_dependency_under_asan_and_ubsan(tmp_path):
     env.pop("LD_PRELOAD", None)
     r = subprocess.run([exe], capture_output=True, text=True, env=env, timeout=300)
     assert r.returncode == 0, (r.stdout + r.stderr)[-4000:]
-    assert " 0 failed checks" in r.stdout and "with a rounded tail" in r.stdout
+    assert " 0 failed checks" in r.stdout and "with a rounded tail" in r.stdout and "with partial sums decoded id by id" in r.stdout

@@ -37,24 +37,28 @@ FP8_SOURCES = ("ffn_fp8.hip", "ffn_common.hpp", "route.hip")
 FP8_TILE_SOURCES = ("ffn_fp8_tile.hip", "ffn_common.hpp", "route.hip")
 WIDEN_SOURCES = BF16_SOURCES + ("quant.hip",)
 F32_TILE_SOURCES = ("ffn_f32_tile.hip", "ffn_common.hpp", "route.hip")
+FP8_MFMA_SOURCES = FP8_TILE_SOURCES + ("quant.hip",)
 MEASURED_TRAFFIC = {
-    "mixtral": {"bytes": 19.48e9, "sources": BF16_SOURCES, "kernel_digest": "2192860045c2",
+    "mixtral": {"bytes": 18.25e9, "sources": BF16_SOURCES, "kernel_digest": "87bf3a72935d",
                 "profile": "profiles/ffn_persistent_kernel_bf16_mixtral_c3_hbm_traffic.txt"},
-    "mid": {"bytes": 0.808e9, "sources": BF16_SOURCES, "kernel_digest": "2192860045c2",
+    "mid": {"bytes": 0.807e9, "sources": BF16_SOURCES, "kernel_digest": "87bf3a72935d",
             "profile": "profiles/ffn_persistent_kernel_bf16_mid_c2_hbm_traffic.txt"},
-    "finegrained": {"bytes": 3.35e9, "sources": BF16_SOURCES, "kernel_digest": "2192860045c2",
+    "finegrained": {"bytes": 3.349e9, "sources": BF16_SOURCES, "kernel_digest": "87bf3a72935d",
                     "profile": "profiles/ffn_persistent_kernel_bf16_finegrained_c4_hbm_traffic.txt"},
-    "decode_fp8": {"bytes": 9.884e9, "sources": FP8_SOURCES, "kernel_digest": "f8fa608ab58a",
+    "decode_fp8": {"bytes": 9.909e9, "sources": FP8_SOURCES, "kernel_digest": "47ddccc0e23f",
                    "profile": "profiles/ffn_persistent_fp8_kernel_decode_c5_hbm_traffic.txt"},
     # a single-expert fp32 layer runs as two launches (one per projection); the figure is their sum
-    "reference_default": {"bytes": 1.084e9, "sources": F32_TILE_SOURCES, "kernel_digest": "9dde156ff4df", "ffn_mode": 1,
+    "reference_default": {"bytes": 0.919e9, "sources": F32_TILE_SOURCES, "kernel_digest": "3e84a4ffa895", "ffn_mode": 1,
                           "profile": "profiles/ffn_tiled_f32_tile_kernel_reference_default_hbm_traffic.txt"},
     # the widening pass and the bf16 queue kernel together (what the layer's FFN stage launches by default) ...
-    "prefill_fp8": {"bytes": 24.82e9, "sources": WIDEN_SOURCES, "kernel_digest": "b11cdfccc263",
+    "prefill_fp8": {"bytes": 22.96e9, "sources": WIDEN_SOURCES, "kernel_digest": "af9c27a45a60",
                     "profile": "profiles/widen_plus_ffn_persistent_kernel_prefill_fp8_hbm_traffic.txt"},
-    # ... and the e4m3 tile GEMM on the same layer (MOE355_FP8_WIDEN=0)
-    "prefill_fp8/e4m3_tile": {"bytes": 26.98e9, "sources": FP8_TILE_SOURCES, "kernel_digest": "8f1a6919616f",
+    # ... the e4m3 tile GEMM on the same layer (option fp8_widen = 0) ...
+    "prefill_fp8/e4m3_tile": {"bytes": 26.70e9, "sources": FP8_TILE_SOURCES, "kernel_digest": "3dfd4df82d0e",
                               "profile": "profiles/ffn_persistent_fp8_tile_kernel_prefill_fp8_hbm_traffic.txt"},
+    # ... and the e4m3 x e4m3 plan (option fp8_mfma = 1): two quantising passes and two GEMM launches
+    "prefill_fp8/e4m3_mfma": {"bytes": 14.11e9, "sources": FP8_MFMA_SOURCES, "kernel_digest": "6f0a4dcd7bde", "ffn_mode": 1,
+                              "profile": "profiles/ffn_tiled_fp8_mfma_kernel_prefill_fp8_hbm_traffic.txt"},
 }
 
 
@@ -196,7 +200,10 @@ def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False, balanced_
     roof["kernel_ms"] = ffn["mean"]
     roof["kernel_ms_median"] = ffn["median"]
     roof["kernel_ms_min"] = ffn["min"]
-    t = MEASURED_TRAFFIC.get(name + ("/e4m3_tile" if fp8 and w.bound == "mfma" and not widened else ""))
+    plan = ""
+    if fp8 and w.bound == "mfma" and not widened:
+        plan = "/e4m3_mfma" if layer.options.get("fp8_mfma") == 1 else "/e4m3_tile"
+    t = MEASURED_TRAFFIC.get(name + plan)
     digest = kernel_digest(t["sources"]) if t else None
     same_schedule = t is not None and t.get("ffn_mode", 2) == layer.ffn_mode
     if same_schedule and t["kernel_digest"] == digest:
@@ -304,7 +311,7 @@ def task_trace_summary(layer, dev, out):
     parts = rec["phase"] >> 4
     phase = rec["phase"] & 3
     groups = []
-    for ph in (0, 1):
+    for ph in sorted(set(phase.tolist())):          # 0 up, 1 down projection; 2: a combine sweep of an idle workgroup (option combine = 2)
         for np_ in sorted(set(parts[phase == ph].tolist())):
             for lo, hi, label in ((full, full, "full"), (full // 2 + 1, full - 1, "more than half"), (1, full // 2, "at most half")):
                 m = (phase == ph) & (parts == np_) & (rec["rows"] >= lo) & (rec["rows"] <= hi)
@@ -315,7 +322,7 @@ def task_trace_summary(layer, dev, out):
                     if np_:
                         g["partial_sums_per_tile"] = int(np_)
                     groups.append(g)
-    gaps = {0: [], 1: []}
+    gaps = {0: [], 1: [], 2: [], 3: []}
     busy, idle_after, per_wg = [], [], []
     end = float(rec["end_us"].max())
     for w in np.unique(rec["workgroup"]):

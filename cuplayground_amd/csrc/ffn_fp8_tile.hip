@@ -261,8 +261,10 @@ __device__ __forceinline__ void tile_mainloop(const TileTask& p, unsigned char* 
 // instructions, and nothing is widened: token rows arrive as e4m3 codes with one fp32 scale per (row, k block)
 // (quant_rows128 passes in front of the two projections), weights are fed as stored.  A slab is one k block: 128 bytes
 // per row, both operands global -> LDS directly, the 16-bit tiles' row layout (128-byte rows, 16-byte chunks xor-swizzled
-// by (row >> 1) & 7); a lane's fragment is chunks 2 fk and 2 fk + 1 of its row (which k a lane's bytes stand for inside the
-// instruction does not matter as long as both operands agree: the block's dot product is a sum over all of them).
+// by (row >> 1) & 7); a lane's fragment is chunks fk and 4 + fk of its row -- the two chunks the 16-bit tiles read, a
+// pattern without LDS bank conflicts; with chunks 2 fk and 2 fk + 1 every second cycle of the reads was one (which k a
+// lane's bytes stand for inside the instruction does not matter as long as both operands agree: the block's dot product
+// is a sum over all of them).
 // Every MFMA starts from zero; its 16 x 16 partial sums are scaled by (weight block scale) x (token row scale) and added
 // in fp32: y[t, n] = sum over k blocks of s_w[n / 128][kb] * s_a[t][kb] * (dot product of the block's codes).
 typedef int i32x8 __attribute__((ext_vector_type(8)));
@@ -313,7 +315,7 @@ __device__ __forceinline__ void tile_mainloop_mfma8(const TileTask& p, unsigned 
     const int ta = PARTIAL ? min(PTM, max(0, (p.rows - wm * 16 * PTM + 15) >> 4)) : PTM;
     const int a_off = (wm * 16 * PTM + frow) * PROW;
     const int b_off = PBM * PROW + (wn * 16 * PTN + frow) * PROW;
-    const int c0 = ((2 * fk) ^ sw) << 4, c1 = ((2 * fk + 1) ^ sw) << 4;
+    const int c0 = (fk ^ sw) << 4, c1 = ((4 + fk) ^ sw) << 4;
 
     // the scales of this lane's token rows (one row per 16 x 16 fragment), a k block ahead
     const float* sa_row[PTM];

@@ -321,7 +321,9 @@ int moe_get_queue_balance(moe_handle* h, const void* workspace, void* stream, in
  * scheduling.cuh:261-263). */
 typedef struct moe_task_record {
     int32_t phase;      /* 0: up(/gate) projection + activation, 1: down projection; a task that computed one of P partial
-                           sums of its tile (option tail_split) has 1 + 4 * part + 16 * P here */
+                           sums of its tile (option tail_split) has 1 + 4 * part + 16 * P here; 2: a combine sweep of
+                           an idle workgroup (option combine = 2): expert = column slice, row_block = chunk of tokens,
+                           col_tile = rows = (slice, token) units it combined */
     int32_t expert;
     int32_t row_block;  /* index into the layer's row-block table (expert-major) */
     int32_t col_tile;

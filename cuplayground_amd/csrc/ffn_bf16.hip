@@ -1106,7 +1106,7 @@ __global__ __launch_bounds__(P::THREADS) void ffn_persistent_kernel(FfnArgs a) {
 }
 
 // The same queue for the 256 x 256 tile, with the start of the next task moved under the end of the current one
-// (opt-in: MOE355_QUEUE_EARLY=1).
+// (opt-in: option queue_early = 1).
 //
 // Between two tiles a workgroup pops (an atomic round trip and two barriers), decodes, computes its row offsets (eight
 // gathered token indices per thread), issues the first 32 loads and waits for slab 0.  Here the next id is reserved
@@ -1439,7 +1439,7 @@ static bool large_tile_ok(int64_t pairs, int H, int I, bool swiglu) {
 
 // Tile of a layer: 0 = 128 x 128, 1 = 256 x 256, 2 = 128 x 256, 3 = 256 x 256 with the 128 x 256 tile for the row
 // blocks of at most 128 rows.  1 where its conditions hold and the layer has enough rows, else 0; 2 and 3 are tuning
-// knobs (MOE355_TILE).
+// knobs (option tile16).
 //
 // Measured (FFN stage, one box, alternating runs): the 128 x 256 tile reaches 93 % of the 256 x 256 tile's rate on a
 // plain 4096 x 8192 x 4096 GEMM, but as the tile of a whole layer it loses everywhere (Mixtral shape 5.48 against

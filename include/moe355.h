@@ -178,7 +178,7 @@ int moe_get_arch(const moe_handle* h, moe_arch* out);
  * Task totals follow the reference's bound tilesM*tilesNx + tilesM*tilesN (scheduling.cuh:212-222) per expert. */
 int moe_get_plan(const moe_handle* h, int32_t* block_rows, int32_t* col_tiles_up, int32_t* col_tiles_down);
 /* The dtype whose FFN kernels the handle runs: cfg.torch_dtype, except MOE_DTYPE_BF16 for an e4m3 layer whose experts
- * see so many rows (768 on average; MOE355_FP8_WIDEN = 0 / 1 overrides) that every moe_forward first widens the weights
+ * see so many rows (768 on average; option fp8_widen = 0 / 1 overrides) that every moe_forward first widens the weights
  * to bf16 in the workspace (moe_dequant_block128; moe_workspace_bytes then includes 2 bytes per weight) and runs
  * the bf16 tiles on them.  The reference fixes its element types at compile time (processor/tiling.cuh:97-159). */
 int moe_get_kernel_dtype(const moe_handle* h, int32_t* dtype);

@@ -107,7 +107,7 @@ static void split_and_check(const Layer& L, int F, int tail_blocks, int row_chun
         int total_ids = -1;
         const int nseg = split_tail(q.data(), n0, split_mt0, F, npg0, npg1, &total_ids);
         CHECK(nseg == n0 || nseg == n0 + 1, "nseg %d", nseg);
-        int expect = 0, pos0_last = -1;
+        int expect = 0;
         std::vector<int> pos0(total_mt, -1), pos1(total_mt, -1);
         for (int i = 0; i < nseg; ++i) {
             const Segment& s = q[i];
@@ -125,9 +125,7 @@ static void split_and_check(const Layer& L, int F, int tail_blocks, int row_chun
                 CHECK(pos[b] == -1, "row block %d covered twice in phase %d", b, s.phase);
                 pos[b] = i;
             }
-            if (s.phase == 0) pos0_last = i;
         }
-        (void)pos0_last;
         CHECK(expect == total_ids, "ids %d / %d", expect, total_ids);
         for (int b = 0; b < total_mt; ++b) {
             CHECK(pos1[b] >= 0, "row block %d has no down projection", b);

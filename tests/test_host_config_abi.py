@@ -155,7 +155,7 @@ def test_options_default_env_and_domains(monkeypatch):
     assert cfg.workspace_bytes() == wide                   # no options argument: MOE355_FP8_WIDEN=1 from the environment
     monkeypatch.delenv("MOE355_FP8_WIDEN")
     assert cfg.workspace_bytes() == ws({})[1] == plain     # 128 rows per expert: below the widening threshold
-    for bad in ({"tile16": 4}, {"queue_groups": 3}, {"block_rows": 200}, {"combine": 3}, {"tail_round": 2},
+    for bad in ({"tile16": 4}, {"queue_groups": 3}, {"block_rows": 200}, {"combine": 3}, {"tail_round": 2}, {"tail_split": 3}, {"tail_split": 0},
                 {"blocks_per_cu": 0}, {"fp8_tile": -2}):
         assert ws(bad)[0] == 4, bad
     r = api.make_options()

@@ -93,8 +93,16 @@ __device__ __forceinline__ void tile_mainloop(const TileTask& p, unsigned char* 
         const int64_t src_row = p.gather ? (int64_t)p.gather[r] : p.a_row0 + r;
         a_src[i] = p.a_base + src_row * p.K + chunk * 8;
     }
-    // weight rows: 4 threads per row, 16 e4m3 bytes each = two bf16 chunks of the LDS row
-    const int brow = tid >> 2, bc = tid & 3;
+    // weight rows: 4 threads per row, 16 e4m3 bytes each = two bf16 chunks of the LDS row.  Which lanes take which rows
+    // decides the bank conflicts of the 16-byte LDS writes: the LDS serves such a write eight consecutive lanes at a time,
+    // 128 bytes a cycle, so the eight must differ in their 16-byte position modulo 128 bytes -- the row does not matter,
+    // rows are 128 bytes apart.  Four lanes of a row write chunks {0, 2, 4, 6} ^ swizzle (then {1, 3, 5, 7} ^ swizzle);
+    // the other four lanes of the pass must therefore sit in a row whose swizzle differs in its lowest bit: rows r and
+    // r + 2.  (With lanes 4..7 in row r + 1, which has the swizzle of row r, every such write took twice its cycles:
+    // a conflict in every fourth LDS cycle of the kernel, measured with two-lane and whole-wavefront probes under
+    // SQ_LDS_BANK_CONFLICT.)
+    const int t = tid >> 2;
+    const int brow = (t & ~3) | ((t & 1) << 1) | ((t >> 1) & 1), bc = tid & 3;
     const uint8_t* b_src[PRB];
     int b_dst[PRB][2];
 #pragma unroll

@@ -279,6 +279,17 @@ def measure_backward(layer, cfg, dev, routing, steps, warmup):
         res[name] = {"ms": round(ms, 4), "tflops": round(flops / (ms * 1e-3) / 1e12, 1),
                      "frac": round(flops / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)}
     res["flops_per_op"] = flops
+    # the activation's derivative: a pass of its own over dH (reads dH, U [, G]; writes dU [, dG]) against the same
+    # arithmetic in the epilogue of the down projection's data gradient (dH never reaches memory)
+    gated = c.hidden_act == moe.api.ACT_SWIGLU
+    urows = hrows
+    grows = hrows.clone() if gated else None
+    du = torch.zeros(A, I, dtype=dt, device="cuda")
+    dg = torch.zeros(A, I, dtype=dt, device="cuda") if gated else None
+    res["act_backward_ms"] = round(timed(lambda: layer.act_backward(out_i, urows, grows, du=du, dg=dg)), 4)
+    if layer.fused_act_backward:
+        res["dgrad_down_act_fused_ms"] = round(timed(
+            lambda: layer.expert_gemm_act_backward(dy, w_down_t, urows, grows, cnt, off, du=du, dg=dg)), 4)
     return res
 
 

@@ -29,7 +29,7 @@ EXPORTS = (
     "moe_set_ffn_mode", "moe_get_ffn_mode", "moe_forward", "moe_forward_static", "moe_set_spin_limit", "moe_clear_stall", "moe_gate", "moe_router_stats", "moe_route", "moe_gemm_bias_act", "moe_combine",
     "moe_set_stage_timing", "moe_get_stage_ms", "moe_get_stage_samples", "moe_get_task_counts", "moe_get_queue_balance", "moe_task_trace_bytes", "moe_set_task_trace", "moe_get_task_trace", "moe_measure_mfma_tflops",
     "moe_measure_hbm_read_gbs", "moe_quant_block128", "moe_dequant_block128", "moe_backward_scratch_bytes", "moe_transpose", "moe_expert_gemm",
-    "moe_expert_wgrad", "moe_act_backward", "moe_bias_grad", "moe_combine_backward", "moe_last_hip_error", "moe_status_string",
+    "moe_expert_gemm_act_backward", "moe_expert_gemm_act_backward_supported", "moe_expert_wgrad", "moe_act_backward", "moe_bias_grad", "moe_combine_backward", "moe_last_hip_error", "moe_status_string",
     "moe_version",
 )
 
@@ -157,6 +157,8 @@ def load_library():
     L.moe_transpose.argtypes = [vp, vp, i64, i64, i64, i32, vp]
     L.moe_expert_gemm.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, vp, C.c_size_t, vp]
     L.moe_expert_wgrad.argtypes = [vp, vp, vp, vp, vp, i32, i32, vp, vp, C.c_size_t, vp]
+    L.moe_expert_gemm_act_backward.argtypes = [vp, vp, vp, vp, vp, vp, vp, i32, i32, vp, vp, vp, C.c_size_t, vp]
+    L.moe_expert_gemm_act_backward_supported.argtypes = [vp, C.POINTER(C.c_int32)]
     L.moe_act_backward.argtypes = [vp, vp, vp, vp, i64, vp, vp, vp]
     L.moe_bias_grad.argtypes = [vp, vp, vp, vp, i32, vp, vp]
     L.moe_combine_backward.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp]
@@ -527,6 +529,29 @@ class MoELayer:
                "moe_expert_gemm")
         return out
 
+    @property
+    def fused_act_backward(self) -> bool:
+        """Whether expert_gemm_act_backward exists for this layer (16-bit, shape fit for the hand-ordered tiles)."""
+        v = C.c_int32(0)
+        _check(self.L.moe_expert_gemm_act_backward_supported(self._h, C.byref(v)))
+        return bool(v.value)
+
+    def expert_gemm_act_backward(self, dy_rows, w_down_t, u_rows, g_rows, expert_count, expert_offset, du=None, dg=None):
+        """(du_rows, dg_rows) = (dy_rows . w_down_t[e(r)]^T) * act'(u_rows, g_rows): the data gradient of the down
+        projection and the activation's derivative in one kernel; w_down_t [E, I, H]; dg_rows is None unless SwiGLU.
+        Rows of no expert are not written (zeros in the buffers made here)."""
+        import torch
+        N, K = w_down_t.shape[1], w_down_t.shape[2]
+        if du is None:
+            du = torch.zeros(dy_rows.shape[0], N, dtype=dy_rows.dtype, device=dy_rows.device)
+        if dg is None and g_rows is not None:
+            dg = torch.zeros_like(du)
+        sc = self.backward_scratch()
+        _check(self.L.moe_expert_gemm_act_backward(self._h, _ptr(dy_rows), _ptr(w_down_t), _ptr(u_rows), _ptr(g_rows),
+                                                   _ptr(expert_count), _ptr(expert_offset), N, K, _ptr(du), _ptr(dg),
+                                                   _ptr(sc), sc.numel(), _stream()), "moe_expert_gemm_act_backward")
+        return du, dg
+
     def expert_wgrad(self, dy_rows, a_rows, expert_count, expert_offset, out=None):
         """dw[e] [N,K] = sum over expert e's rows of dy_rows[r,:N]^T a_rows[r,:K]."""
         import torch
@@ -538,11 +563,13 @@ class MoELayer:
                                        N, K, _ptr(out), _ptr(sc), sc.numel(), _stream()), "moe_expert_wgrad")
         return out
 
-    def act_backward(self, dh_rows, u_rows, g_rows=None):
+    def act_backward(self, dh_rows, u_rows, g_rows=None, du=None, dg=None):
         """(du_rows, dg_rows) for the layer's activation; dg_rows is None unless the layer is SwiGLU."""
         import torch
-        du = torch.empty_like(dh_rows)
-        dg = torch.empty_like(dh_rows) if g_rows is not None else None
+        if du is None:
+            du = torch.empty_like(dh_rows)
+        if dg is None and g_rows is not None:
+            dg = torch.empty_like(dh_rows)
         _check(self.L.moe_act_backward(self._h, _ptr(dh_rows), _ptr(u_rows), _ptr(g_rows), dh_rows.shape[0], _ptr(du),
                                        _ptr(dg), _stream()), "moe_act_backward")
         return du, dg

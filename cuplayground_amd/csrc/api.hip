@@ -1129,6 +1129,29 @@ int moe_expert_gemm(moe_handle* h, const void* a_rows, const void* w, const void
     return e == hipSuccess ? MOE_OK : hip_fail(h, e);
 }
 
+int moe_expert_gemm_act_backward(moe_handle* h, const void* dy_rows, const void* w, const void* u_rows, const void* g_rows,
+                                 const int32_t* expert_count, const int32_t* expert_offset, int32_t N, int32_t K,
+                                 void* du_rows, void* dg_rows, void* scratch, size_t scratch_bytes, void* stream) {
+    if (!h || !dy_rows || !w || !u_rows || !expert_count || !expert_offset || !du_rows) return MOE_ERR_BAD_ARGUMENT;
+    const bool gated = h->cfg.hidden_act == MOE_ACT_SWIGLU;
+    if (gated != (g_rows != nullptr) || gated != (dg_rows != nullptr)) return MOE_ERR_BAD_ARGUMENT;
+    const int rc = check_backward_call(h, N, K, scratch, scratch_bytes);
+    if (rc) return rc;
+    if (N != h->d.I || K != h->d.H) return MOE_ERR_BAD_ARGUMENT;      // the data gradient of the down projection: [rows, H] -> [rows, I]
+    if (expert_gemm_dact_tile(h->d.A, h->d.E, N, K, h->d.act_dtype, h->opt) == 0) return MOE_ERR_UNSUPPORTED;
+    const hipError_t e = launch_expert_gemm_dact(dy_rows, w, u_rows, g_rows, expert_count, expert_offset, h->d.A, h->d.E, N, K,
+                                                 h->cfg.hidden_act, h->d.act_dtype, h->opt, du_rows, dg_rows, scratch,
+                                                 (hipStream_t)stream);
+    return e == hipSuccess ? MOE_OK : hip_fail(h, e);
+}
+
+int moe_expert_gemm_act_backward_supported(const moe_handle* h, int32_t* supported) {
+    if (!h || !supported) return MOE_ERR_BAD_ARGUMENT;
+    *supported = h->cfg.torch_dtype != MOE_DTYPE_FP8_E4M3_B128 &&
+                 expert_gemm_dact_tile(h->d.A, h->d.E, h->d.I, h->d.H, h->d.act_dtype, h->opt) != 0;
+    return MOE_OK;
+}
+
 int moe_expert_wgrad(moe_handle* h, const void* dy_rows, const void* a_rows, const int32_t* expert_count,
                      const int32_t* expert_offset, int32_t N, int32_t K, void* dw, void* scratch, size_t scratch_bytes,
                      void* stream) {

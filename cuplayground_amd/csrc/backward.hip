@@ -10,7 +10,10 @@
 //     expert is then one tile GEMM over its window.
 #include <algorithm>
 
+#include <type_traits>
+
 #include "moe_internal.hpp"
+#include "act_deriv.hpp"
 
 namespace moe355 {
 
@@ -21,6 +24,9 @@ hipError_t launch_grouped_gemm_16(const void* a_rows, const void* w, const void*
 hipError_t launch_wgrad_16(const void* dyT, const void* aT, void* dw, const int32_t* poff, int E, int N, int K,
                            int64_t ld, bool f16, hipStream_t st);
 
+hipError_t launch_grouped_gemm_deriv_16(const void* a_rows, const void* w, const void* u, const void* g, void* du, void* dg,
+                                        const MTile* mtiles, const int32_t* num_mtiles, const int32_t* count, int max_mtiles,
+                                        int tile, int64_t A, int N, int K, int hidden_act, bool f16, hipStream_t st);
 hipError_t launch_grouped_gemm_f32(const void* a_rows, const void* w, const void* bias, void* out, const MTile* mtiles,
                                    const int32_t* num_mtiles, int max_mtiles, int N, int K, int act, hipStream_t st);
 hipError_t launch_wgrad_f32(const void* dyT, const void* aT, void* dw, const int32_t* poff, int E, int N, int K, int64_t ld,
@@ -228,24 +234,72 @@ template <> __device__ __forceinline__ uint16_t st16<f16_s>(float v) { return __
 template <> __device__ __forceinline__ float st16<f32_s>(float v) { return v; }
 
 // du = dh * act'(u); SwiGLU (h = silu(g) u): du = dh silu(g), dg = dh u s (1 + g (1 - s)), s = sigmoid(g).
+// fp32 layers use the library functions; 16-bit layers the forms of act_deriv.hpp, which the fused data gradient's
+// epilogue inlines as well (same bits on both paths).
+template <class T16>
+__device__ __forceinline__ void act_backward_one(float d, float uv, float gv, int act, float& a, float& b) {
+    constexpr bool kF32 = std::is_same<T16, f32_s>::value;
+    b = 0.0f;
+    if (act == MOE_ACT_SWIGLU) {
+        if constexpr (kF32) {
+            const float sg = 1.0f / (1.0f + expf(-gv));
+            a = d * (gv * sg);
+            b = d * uv * (sg * (1.0f + gv * (1.0f - sg)));
+        } else {
+            dswiglu16(d, uv, gv, a, b);
+        }
+    } else if (act == MOE_ACT_GELU) {
+        if constexpr (kF32) {
+            const float cdf = 0.5f * (1.0f + erff(uv * 0.70710678118654752440f));
+            const float pdf = 0.39894228040143267794f * expf(-0.5f * uv * uv);
+            a = d * (cdf + uv * pdf);
+        } else {
+            a = dgelu16(d, uv);
+        }
+    } else {
+        a = drelu16(d, uv);
+    }
+}
+
+// 16 bytes of every operand per thread and step (8 or 4 elements): the pass is a stream over five arrays at most and
+// has nothing else to wait for.  n is a multiple of the intermediate size, which is a multiple of 64; all pointers
+// 16-byte aligned (the launcher checks both).
 template <class T16, class RAW = typename RawOf<T16>::type>
 __global__ __launch_bounds__(256) void act_backward_kernel(const RAW* __restrict__ dh, const RAW* __restrict__ u,
                                                            const RAW* __restrict__ g, size_t n, int act,
                                                            RAW* __restrict__ du, RAW* __restrict__ dg) {
-    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
-        const float d = ld16<T16>(dh, i), uv = ld16<T16>(u, i);
-        if (act == MOE_ACT_SWIGLU) {
-            const float gv = ld16<T16>(g, i);
-            const float sg = 1.0f / (1.0f + expf(-gv));
-            du[i] = st16<T16>(d * (gv * sg));
-            dg[i] = st16<T16>(d * uv * (sg * (1.0f + gv * (1.0f - sg))));
-        } else if (act == MOE_ACT_GELU) {
-            const float cdf = 0.5f * (1.0f + erff(uv * 0.70710678118654752440f));
-            const float pdf = 0.39894228040143267794f * expf(-0.5f * uv * uv);
-            du[i] = st16<T16>(d * (cdf + uv * pdf));
-        } else {
-            du[i] = st16<T16>(uv > 0.0f ? d : 0.0f);
+    constexpr int VEC = 16 / (int)sizeof(RAW);
+    union Pack { uint4 q; RAW e[VEC]; };
+    const size_t nv = n / VEC, id = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const bool gated = act == MOE_ACT_SWIGLU;
+    for (size_t i = id; i < nv; i += (size_t)gridDim.x * 256) {
+        Pack d, uu, gg, oa, ob;
+        d.q = reinterpret_cast<const uint4*>(dh)[i];
+        uu.q = reinterpret_cast<const uint4*>(u)[i];
+        gg.q = gated ? reinterpret_cast<const uint4*>(g)[i] : uint4{0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+            float a, b;
+            act_backward_one<T16>(ld16<T16>(d.e, k), ld16<T16>(uu.e, k), ld16<T16>(gg.e, k), act, a, b);
+            oa.e[k] = st16<T16>(a);
+            ob.e[k] = st16<T16>(b);
         }
+        reinterpret_cast<uint4*>(du)[i] = oa.q;
+        if (gated) reinterpret_cast<uint4*>(dg)[i] = ob.q;
+    }
+}
+
+// The same one element at a time, for operands that are not 16-byte aligned.
+template <class T16, class RAW = typename RawOf<T16>::type>
+__global__ __launch_bounds__(256) void act_backward_unaligned_kernel(const RAW* __restrict__ dh, const RAW* __restrict__ u,
+                                                                     const RAW* __restrict__ g, size_t n, int act,
+                                                                     RAW* __restrict__ du, RAW* __restrict__ dg) {
+    const bool gated = act == MOE_ACT_SWIGLU;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+        float a, b;
+        act_backward_one<T16>(ld16<T16>(dh, i), ld16<T16>(u, i), gated ? ld16<T16>(g, i) : 0.0f, act, a, b);
+        du[i] = st16<T16>(a);
+        if (gated) dg[i] = st16<T16>(b);
     }
 }
 
@@ -367,6 +421,42 @@ hipError_t launch_expert_gemm(const void* a_rows, const void* w, const void* bia
                                   dtype == MOE_DTYPE_FP16, st);
 }
 
+// The tile the fused data gradient (product + activation derivative) would run on: 1 or 2 (the hand-ordered tiles), or 0
+// when the shape or the options leave only the 128 x 128 tile, which has no such epilogue.
+int expert_gemm_dact_tile(int64_t A, int E, int N, int K, int dtype, const moe_options& opt) {
+    if (dtype != MOE_DTYPE_BF16 && dtype != MOE_DTYPE_FP16) return 0;
+    int tile = grouped_gemm_takes_large_tile(A, E, N, K) ? 1 : 0;
+    const int64_t lim = (int64_t)1 << 32;
+    const bool hand_ok = N % 256 == 0 && K % 128 == 0 && A * K * 2 < lim && (int64_t)N * K * 2 < lim;
+    if (opt.grouped_tile != MOE_OPT_AUTO) {
+        const int v = opt.grouped_tile;
+        if ((v == 1 || v == 2) && hand_ok) tile = v;
+        if (v == 0) tile = 0;
+    } else if (tile == 0 && hand_ok) {
+        tile = 2;      // few rows per expert: the 128-row hand-ordered tile rather than no fusion at all
+    }
+    return tile;
+}
+
+// du_rows = (dy_rows . w[e(r)]^T) * act'(u_rows) (and dg_rows for SwiGLU): launch_expert_gemm with act NONE and
+// launch_act_backward in one kernel; the product is rounded to the storage type before the derivative, as the two-call
+// chain does when it stores dh, so both give the same bits.  16-bit layers on the hand-ordered tiles only.
+hipError_t launch_expert_gemm_dact(const void* dy_rows, const void* w, const void* u_rows, const void* g_rows,
+                                   const int32_t* count, const int32_t* offset, int64_t A, int E, int N, int K, int hidden_act,
+                                   int dtype, const moe_options& opt, void* du_rows, void* dg_rows, void* scratch,
+                                   hipStream_t st) {
+    const int tile = expert_gemm_dact_tile(A, E, N, K, dtype, opt);
+    if (tile == 0) return hipErrorNotSupported;
+    const ScratchTables t = scratch_tables(scratch, A, E);
+    const int block_m = tile == 1 ? 256 : 128;
+    const int max_mtiles = (int)(A / block_m + E);
+    backward_tables_kernel<<<1, kMaxExperts, 0, st>>>(count, offset, E, block_m, t.mtiles, t.num_mtiles, nullptr);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    return launch_grouped_gemm_deriv_16(dy_rows, w, u_rows, g_rows, du_rows, dg_rows, t.mtiles, t.num_mtiles, count, max_mtiles,
+                                        tile, A, N, K, hidden_act, dtype == MOE_DTYPE_FP16, st);
+}
+
 // dw[e] [N,K] = dy_e^T . a_e; scratch holds the window offsets and the two transposed operands.
 hipError_t launch_expert_wgrad(const void* dy_rows, const void* a_rows, const int32_t* count, const int32_t* offset,
                                int64_t A, int E, int N, int K, int dtype, const moe_options& opt, void* dw, void* scratch,
@@ -394,13 +484,26 @@ hipError_t launch_expert_wgrad(const void* dy_rows, const void* a_rows, const in
     return launch_wgrad_16(dyT, aT, dw, t.poff, E, N, K, ld, dtype == MOE_DTYPE_FP16, st);
 }
 
+template <class T16, class RAW>
+static void launch_act_backward_t(const void* dh, const void* u, const void* g, int64_t n, int act, void* du, void* dg,
+                                  hipStream_t st) {
+    constexpr int VEC = 16 / (int)sizeof(RAW);
+    const uintptr_t bits = (uintptr_t)dh | (uintptr_t)u | (uintptr_t)g | (uintptr_t)du | (uintptr_t)dg;
+    if (bits % 16 == 0 && n % VEC == 0) {
+        const int grid = (int)std::min<int64_t>((n / VEC + 255) / 256, 65536);
+        act_backward_kernel<T16><<<grid, 256, 0, st>>>((const RAW*)dh, (const RAW*)u, (const RAW*)g, (size_t)n, act, (RAW*)du, (RAW*)dg);
+    } else {
+        const int grid = (int)std::min<int64_t>((n + 255) / 256, 65536);
+        act_backward_unaligned_kernel<T16><<<grid, 256, 0, st>>>((const RAW*)dh, (const RAW*)u, (const RAW*)g, (size_t)n, act, (RAW*)du, (RAW*)dg);
+    }
+}
+
 hipError_t launch_act_backward(const void* dh, const void* u, const void* g, int64_t n, int act, int dtype, void* du,
                                void* dg, hipStream_t st) {
     if (n <= 0) return hipSuccess;
-    const int grid = (int)std::min<int64_t>((n + 255) / 256, 65536);
-    if (dtype == MOE_DTYPE_F32) act_backward_kernel<f32_s><<<grid, 256, 0, st>>>((const float*)dh, (const float*)u, (const float*)g, (size_t)n, act, (float*)du, (float*)dg);
-    else if (dtype == MOE_DTYPE_FP16) act_backward_kernel<f16_s><<<grid, 256, 0, st>>>((const uint16_t*)dh, (const uint16_t*)u, (const uint16_t*)g, (size_t)n, act, (uint16_t*)du, (uint16_t*)dg);
-    else act_backward_kernel<bf16_s><<<grid, 256, 0, st>>>((const uint16_t*)dh, (const uint16_t*)u, (const uint16_t*)g, (size_t)n, act, (uint16_t*)du, (uint16_t*)dg);
+    if (dtype == MOE_DTYPE_F32) launch_act_backward_t<f32_s, float>(dh, u, g, n, act, du, dg, st);
+    else if (dtype == MOE_DTYPE_FP16) launch_act_backward_t<f16_s, uint16_t>(dh, u, g, n, act, du, dg, st);
+    else launch_act_backward_t<bf16_s, uint16_t>(dh, u, g, n, act, du, dg, st);
     return hipGetLastError();
 }
 

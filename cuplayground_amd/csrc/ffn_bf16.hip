@@ -20,6 +20,7 @@
 #include <type_traits>
 
 #include "ffn_common.hpp"
+#include "act_deriv.hpp"
 
 namespace moe355 {
 namespace {
@@ -88,6 +89,13 @@ struct TaskPtrs {
     int32_t* part_cnt;           // parts of the tile stored so far
     int kparts, kpart;
     bool poison;                 // such a task whose rows never became ready: its part is NaN
+    // The data gradient of the down projection with the activation's derivative in its epilogue (grouped kernel only;
+    // deriv 0: an ordinary task): the tile's sums are dh, and what is stored is dh * act'(u) (and, for SwiGLU, the gate's
+    // share beside it) from the saved projections u (and g), which have the output's shape.
+    int deriv;                   // 0, or 1 + the layer's hidden_act
+    const uint16_t* aux0;        // u rows, first row of the block
+    const uint16_t* aux1;        // g rows (SwiGLU), else null
+    uint16_t* c1_base;           // dg rows (SwiGLU), else null
 };
 
 // silu for a bf16 result: hardware exp2 and reciprocal (about 1 ulp each in fp32, far below the bf16 rounding of
@@ -397,10 +405,14 @@ struct SummedTile {
 
 // `between(i)` runs in front of row group i (i = 0..7): the queue kernel issues the next task's first loads there, a
 // few at a time, so that they leave the compute unit under the epilogue's arithmetic instead of in front of it.
-template <class T, int MODE, class Hook, class Parts = WholeTile>
+// DERIV: what leaves the staging area is not stored as it is (dh, rounded to 16 bits as a stored data gradient would be)
+// but multiplied by the activation's derivative at the saved projections (TaskPtrs::deriv): a row segment's 8 values
+// meet the 8 values of u (and g) of the same rows and columns, loaded at the top of the row group.
+template <class T, int MODE, class Hook, class Parts = WholeTile, bool DERIV = false>
 __device__ __forceinline__ void epilogue_full_n_impl(const TaskPtrs& p, unsigned char* smem, f32x4 (&acc)[8][T::TN], const Hook& between,
                                                      const Parts& parts = Parts()) {
     static_assert(Parts::KP == 1 || MODE == 0, "partial sums: the down projection only");
+    static_assert(!DERIV || (MODE == 0 && Parts::KP == 1), "the derivative follows a plain product");
 
     static_assert(T::HAND, "four wavefronts of 128 x 128 or 128 x 64");
     constexpr int NJ = MODE == 3 ? T::TN / 2 : T::TN;   // groups of 16 output columns per wavefront
@@ -447,6 +459,20 @@ __device__ __forceinline__ void epilogue_full_n_impl(const TaskPtrs& p, unsigned
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         between(i);
+        // (DERIV) the saved projections of this row group's rows: requested here, used behind the staging round trip
+        u32x4 uu[DERIV ? NQ : 1], gg[DERIV ? NQ : 1];
+        if constexpr (DERIV) {
+            const int64_t group = (int64_t)(wm * 128 + i * 16) * p.N;
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) {
+                uu[q] = gg[q] = u32x4{0u, 0u, 0u, 0u};
+                if (i * 16 + q * ROWS_PER_PASS < rows_left) {
+                    const int64_t at = group + (int64_t)(q * ROWS_PER_PASS) * p.N + lane_off;
+                    uu[q] = *reinterpret_cast<const u32x4*>(p.aux0 + at);
+                    if (p.deriv == 1 + MOE_ACT_SWIGLU) gg[q] = *reinterpret_cast<const u32x4*>(p.aux1 + at);
+                }
+            }
+        }
         // Partial sums: the row group's sums of the other parts come back from memory (written through by their tasks,
         // read past this XCD's L2) and are added here -- two parts: own registers + the other part, which is the same
         // in either order; four parts: all four as stored, in the order of the parts, whichever of them runs this.
@@ -499,6 +525,38 @@ __device__ __forceinline__ void epilogue_full_n_impl(const TaskPtrs& p, unsigned
 #pragma unroll
         for (int q = 0; q < NQ; ++q) v[q] = *reinterpret_cast<const u32x4*>(rd + q * ROWS_PER_PASS * PITCH);
         uint16_t* rows0 = p.c_base + (int64_t)(wm * 128 + i * 16) * p.N;   // uniform
+        if constexpr (DERIV) {
+            const int64_t group = (int64_t)(wm * 128 + i * 16) * p.N;
+            const bool gated = p.deriv == 1 + MOE_ACT_SWIGLU;
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) {
+                if (i * 16 + q * ROWS_PER_PASS >= rows_left) continue;
+                const int64_t at = group + (int64_t)(q * ROWS_PER_PASS) * p.N + lane_off;
+                u32x4 o0, o1 = {0u, 0u, 0u, 0u};
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    const float d0 = widen1<T>((uint16_t)(v[q][w] & 0xFFFFu)), d1 = widen1<T>((uint16_t)(v[q][w] >> 16));
+                    const float u0 = widen1<T>((uint16_t)(uu[q][w] & 0xFFFFu)), u1 = widen1<T>((uint16_t)(uu[q][w] >> 16));
+                    float a0, a1, b0v = 0.0f, b1v = 0.0f;
+                    if (gated) {
+                        const float g0 = widen1<T>((uint16_t)(gg[q][w] & 0xFFFFu)), g1 = widen1<T>((uint16_t)(gg[q][w] >> 16));
+                        dswiglu16(d0, u0, g0, a0, b0v);
+                        dswiglu16(d1, u1, g1, a1, b1v);
+                    } else if (p.deriv == 1 + MOE_ACT_GELU) {
+                        a0 = dgelu16(d0, u0);
+                        a1 = dgelu16(d1, u1);
+                    } else {
+                        a0 = drelu16(d0, u0);
+                        a1 = drelu16(d1, u1);
+                    }
+                    o0[w] = pack2<T>(a0, a1);
+                    o1[w] = pack2<T>(b0v, b1v);
+                }
+                store16(p.c_base + at, o0, false);
+                if (gated) store16(p.c1_base + at, o1, false);
+            }
+            continue;
+        }
         if (publish) {
 #pragma unroll
             for (int q = 0; q < NQ; ++q)
@@ -888,6 +946,15 @@ __device__ __forceinline__ void gemm_tile_ring(const TaskPtrs& p, unsigned char*
     f32x4 acc[8][T::TN];
     if (ring_slabs<T>(p.rows, L, smem, acc)) epilogue_full_n<T>(p, smem, acc);
 }
+// The same with the activation's derivative behind the product (TaskPtrs::deriv; the grouped kernel of the backward pass).
+template <class T>
+__device__ __forceinline__ void gemm_tile_ring_deriv(const TaskPtrs& p, unsigned char* smem) {
+    const RingLoads L = ring_prepare<T>(p);
+    __syncthreads();
+    ring_first_loads<T>(L, smem);
+    f32x4 acc[8][T::TN];
+    if (ring_slabs<T>(p.rows, L, smem, acc)) epilogue_full_n_impl<T, 0, NoHook, WholeTile, true>(p, smem, acc, NoHook());
+}
 // The same for a task that is a part of a tile (TaskPtrs::part).  A copy of its own, slab loop included: with both ends
 // behind one loop the compiler reads all accumulators in front of the branch between them and spills what does not fit,
 // which costs the whole tiles -- nearly all of them -- 4 to 13 % of their time.
@@ -968,6 +1035,10 @@ __device__ __forceinline__ TaskPtrs resolve(const FfnArgs& a, const Task& t, boo
     p.kparts = 1;
     p.kpart = 0;
     p.poison = false;
+    p.deriv = 0;
+    p.aux0 = nullptr;
+    p.aux1 = nullptr;
+    p.c1_base = nullptr;
     if (t.phase == 1 && t.kparts > 1) {       // one of kparts partial sums: this part's share of the intermediate dimension
         const int Kp = a.I / t.kparts, k0 = t.kpart * Kp;
         p.K = Kp;
@@ -1269,6 +1340,7 @@ __global__ __launch_bounds__(T::THREADS) void gemm_dense_kernel(const uint16_t* 
     p.a_extent = (uint32_t)((int64_t)M * K * 2);
     p.b_extent = (uint32_t)((int64_t)N * K * 2);
     p.part = nullptr; p.part_cnt = nullptr; p.kparts = 1; p.kpart = 0; p.poison = false;
+    p.deriv = 0; p.aux0 = nullptr; p.aux1 = nullptr; p.c1_base = nullptr;
     gemm_tile<T>(p, smem);
 }
 
@@ -1316,8 +1388,56 @@ __global__ __launch_bounds__(T::THREADS) void grouped_gemm_kernel(const uint16_t
     p.a_extent = a_bytes;
     p.b_extent = (uint32_t)((int64_t)N * K * 2);
     p.part = nullptr; p.part_cnt = nullptr; p.kparts = 1; p.kpart = 0; p.poison = false;
+    p.deriv = 0; p.aux0 = nullptr; p.aux1 = nullptr; p.c1_base = nullptr;
     gemm_tile<T>(p, smem);
 }
+
+// The grouped product with the activation's derivative in its epilogue (gemm_tile_ring_deriv): the data gradient of the
+// down projection that hands on dU (and dG) instead of dH.  Same grid, same order of the tiles as grouped_gemm_kernel.
+template <class T>
+__global__ __launch_bounds__(T::THREADS) void grouped_gemm_deriv_kernel(const uint16_t* a_rows, const uint16_t* w,
+                                                                        const uint16_t* u_rows, const uint16_t* g_rows,
+                                                                        uint16_t* du_rows, uint16_t* dg_rows,
+                                                                        const MTile* mtiles, const int32_t* num_mtiles,
+                                                                        const int32_t* count, int N, int K, int hidden_act,
+                                                                        uint32_t a_bytes) {
+    static_assert(T::HAND, "the derivative lives in the epilogue of the hand-ordered tiles");
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int ncol = (N + T::BN - 1) / T::BN;
+    const int id = blockIdx.x;
+    if (id >= *num_mtiles * ncol) return;
+    const MTile probe = mtiles[id / ncol];
+    const int first = probe.pad, blocks = (max(count[probe.expert], 0) + T::BM - 1) / T::BM;
+    const int local = id - ncol * first, ctile = local / blocks;
+    const MTile m = mtiles[first + (local - ctile * blocks)];
+    TaskPtrs p;
+    p.a_base = a_rows;
+    p.gather = nullptr;
+    p.a_row0 = m.row0;
+    p.a_ld = K;
+    p.b0 = w + (int64_t)m.expert * N * K;
+    p.b1 = nullptr;
+    p.b_ld = K;
+    p.bias0 = nullptr;
+    p.bias1 = nullptr;
+    p.c_base = du_rows + (int64_t)m.row0 * N;
+    p.N = N;
+    p.K = K;
+    p.rows = m.rows;
+    p.n0 = ctile * T::BN;
+    p.act = MOE_ACT_NONE;
+    p.swiglu = false;
+    p.publish = false;
+    p.a_extent = a_bytes;
+    p.b_extent = (uint32_t)((int64_t)N * K * 2);
+    p.part = nullptr; p.part_cnt = nullptr; p.kparts = 1; p.kpart = 0; p.poison = false;
+    p.deriv = 1 + hidden_act;
+    p.aux0 = u_rows + (int64_t)m.row0 * N;
+    p.aux1 = g_rows ? g_rows + (int64_t)m.row0 * N : nullptr;
+    p.c1_base = dg_rows ? dg_rows + (int64_t)m.row0 * N : nullptr;
+    gemm_tile_ring_deriv<T>(p, smem);
+}
+
 
 // Weight gradient of one projection: dw[e] [N, K] = dy_e^T . a_e, the sum running over the rows of expert e.  Both
 // operands arrive transposed and padded: dyT [N, ld] and aT [K, ld] hold expert e's rows in columns
@@ -1361,6 +1481,7 @@ __global__ __launch_bounds__(T::THREADS) void wgrad_kernel(const uint16_t* dyT, 
     p.a_extent = dy_bytes - (uint32_t)p0 * 2;
     p.b_extent = a_bytes - (uint32_t)p0 * 2;
     p.part = nullptr; p.part_cnt = nullptr; p.kparts = 1; p.kpart = 0; p.poison = false;
+    p.deriv = 0; p.aux0 = nullptr; p.aux1 = nullptr; p.c1_base = nullptr;
     gemm_tile<T>(p, smem);
 }
 
@@ -1560,6 +1681,33 @@ hipError_t launch_grouped_gemm_16(const void* a_rows, const void* w, const void*
                    : launch_grouped<LargePlan::T0>(a_rows, w, bias, out, mtiles, num_mtiles, count, max_mtiles, A, N, K, act, st);
     return f16 ? launch_grouped<SmallPlanH::T0>(a_rows, w, bias, out, mtiles, num_mtiles, count, max_mtiles, A, N, K, act, st)
                : launch_grouped<SmallPlan::T0>(a_rows, w, bias, out, mtiles, num_mtiles, count, max_mtiles, A, N, K, act, st);
+}
+
+template <class T>
+static hipError_t launch_grouped_deriv(const void* a_rows, const void* w, const void* u, const void* g, void* du, void* dg,
+                                       const MTile* mtiles, const int32_t* num_mtiles, const int32_t* count, int max_mtiles,
+                                       int64_t A, int N, int K, int hidden_act, hipStream_t st) {
+    hipError_t e = allow_lds(&grouped_gemm_deriv_kernel<T>, T::LDS_BYTES);
+    if (e != hipSuccess) return e;
+    const int64_t blocks = (int64_t)max_mtiles * ((N + T::BN - 1) / T::BN);
+    if (blocks > INT32_MAX) return hipErrorInvalidValue;
+    grouped_gemm_deriv_kernel<T><<<(unsigned)blocks, T::THREADS, T::LDS_BYTES, st>>>(
+        (const uint16_t*)a_rows, (const uint16_t*)w, (const uint16_t*)u, (const uint16_t*)g, (uint16_t*)du, (uint16_t*)dg, mtiles,
+        num_mtiles, count, N, K, hidden_act, (uint32_t)(A * K * 2));
+    return hipGetLastError();
+}
+
+// tile: 1 (256 x 256) or 2 (128 x 256): the hand-ordered tiles only.
+hipError_t launch_grouped_gemm_deriv_16(const void* a_rows, const void* w, const void* u, const void* g, void* du, void* dg,
+                                        const MTile* mtiles, const int32_t* num_mtiles, const int32_t* count, int max_mtiles,
+                                        int tile, int64_t A, int N, int K, int hidden_act, bool f16, hipStream_t st) {
+    if (tile == 2)
+        return f16 ? launch_grouped_deriv<Tile128x256H>(a_rows, w, u, g, du, dg, mtiles, num_mtiles, count, max_mtiles, A, N, K, hidden_act, st)
+                   : launch_grouped_deriv<Tile128x256>(a_rows, w, u, g, du, dg, mtiles, num_mtiles, count, max_mtiles, A, N, K, hidden_act, st);
+    if (tile == 1)
+        return f16 ? launch_grouped_deriv<LargePlanH::T0>(a_rows, w, u, g, du, dg, mtiles, num_mtiles, count, max_mtiles, A, N, K, hidden_act, st)
+                   : launch_grouped_deriv<LargePlan::T0>(a_rows, w, u, g, du, dg, mtiles, num_mtiles, count, max_mtiles, A, N, K, hidden_act, st);
+    return hipErrorInvalidValue;
 }
 
 template <class T>

@@ -202,6 +202,11 @@ int ffn_persistent_blocks(int dtype, int tile, int compute_units);
 size_t backward_scratch_bytes(int64_t A, int E, int H, int I, int elem_bytes);
 hipError_t launch_transpose(const void* src, void* dst, int64_t batch, int64_t rows, int64_t cols, int elem_bytes,
                             hipStream_t st);
+int expert_gemm_dact_tile(int64_t A, int E, int N, int K, int dtype, const moe_options& opt);
+hipError_t launch_expert_gemm_dact(const void* dy_rows, const void* w, const void* u_rows, const void* g_rows,
+                                   const int32_t* count, const int32_t* offset, int64_t A, int E, int N, int K, int hidden_act,
+                                   int dtype, const moe_options& opt, void* du_rows, void* dg_rows, void* scratch,
+                                   hipStream_t st);
 hipError_t launch_expert_gemm(const void* a_rows, const void* w, const void* bias, const int32_t* count,
                               const int32_t* offset, int64_t A, int E, int N, int K, int act, int dtype,
                               const moe_options& opt, void* out_rows, void* scratch, hipStream_t st);

@@ -5,8 +5,11 @@ Here it has a consumer: `MoE355Train` runs the expert projections through `moe_e
 from `moe_expert_gemm` on the transposed weight (data gradient) and `moe_expert_wgrad` (weight gradient).  Routing
 decisions (top-k indices, slots, capacity drops) come from the library's router and are not differentiated; the gate
 weights that scale the expert outputs are recomputed in torch from the same logits formula, so the router's weight
-matrix and the tokens receive gradients through them.  Activation, gather and the weighted combine are elementwise /
-indexing work left to torch's autograd.  There is no CPU path: every tensor lives on the GPU.
+matrix and the tokens receive gradients through them.  The activation and the down projection are one autograd node
+(`_ActDown`): its backward is `moe_expert_gemm_act_backward` -- the data gradient of the down projection with the
+activation's derivative in the product's epilogue -- where the layer has it, else `moe_expert_gemm` followed by
+`moe_act_backward`.  Gather and the weighted combine are indexing work left to torch's autograd.  There is no CPU path:
+every tensor lives on the GPU.
 """
 from __future__ import annotations
 
@@ -40,6 +43,43 @@ class _ExpertLinear(torch.autograd.Function):
 
 def expert_linear(a_rows, w, layer: api.MoELayer, expert_count, expert_offset):
     return _ExpertLinear.apply(a_rows, w, layer, expert_count, expert_offset)
+
+
+class _ActDown(torch.autograd.Function):
+    """(u rows, g rows or None) -> act(u, g) . w_down[e(r)]^T over packed expert-major rows."""
+
+    @staticmethod
+    def forward(ctx, u, g, w, layer, count, offset):
+        act = layer.cfg.hidden_act
+        if act == api.ACT_SWIGLU:
+            h = torch.nn.functional.silu(g.float()) * u.float()
+        elif act == api.ACT_GELU:
+            h = torch.nn.functional.gelu(u.float())
+        else:
+            h = torch.relu(u.float())
+        h = h.to(u.dtype)
+        ctx.save_for_backward(u, g, h, w, count, offset)
+        ctx.layer = layer
+        return layer.expert_gemm(h, w, None, count, offset, api.ACT_NONE)
+
+    @staticmethod
+    def backward(ctx, dy):
+        u, g, h, w, count, offset = ctx.saved_tensors
+        layer = ctx.layer
+        dy = dy.contiguous()
+        w_t = api.transpose(w)                                                                     # [E, I, H]
+        if layer.fused_act_backward:
+            du, dg = layer.expert_gemm_act_backward(dy, w_t, u, g, count, offset)
+        else:
+            dh = layer.expert_gemm(dy, w_t, None, count, offset, api.ACT_NONE)                     # dH = dY . W_down
+            du, dg = layer.act_backward(dh, u, g)
+        dw = layer.expert_wgrad(dy, h, count, offset) if ctx.needs_input_grad[2] else None
+        return du, dg, dw, None, None, None
+
+
+def act_down(u_rows, g_rows, w_down, layer: api.MoELayer, expert_count, expert_offset):
+    return _ActDown.apply(u_rows.contiguous(), None if g_rows is None else g_rows.contiguous(), w_down, layer,
+                          expert_count, expert_offset)
 
 
 class MoE355Train(torch.nn.Module):
@@ -82,13 +122,8 @@ class MoE355Train(torch.nn.Module):
         tok = r["token_indices"].clamp(min=0).long()      # rows past the last kept one gather token 0 and are never used
         x_rows = x.index_select(0, tok)
         up = expert_linear(x_rows, self.w_up, self.layer, count, offset)
-        if c.hidden_act == api.ACT_SWIGLU:
-            h = torch.nn.functional.silu(expert_linear(x_rows, self.w_gate, self.layer, count, offset).float()) * up.float()
-        elif c.hidden_act == api.ACT_GELU:
-            h = torch.nn.functional.gelu(up.float())
-        else:
-            h = torch.relu(up.float())
-        y = expert_linear(h.to(x.dtype), self.w_down, self.layer, count, offset)
+        gate = expert_linear(x_rows, self.w_gate, self.layer, count, offset) if c.hidden_act == api.ACT_SWIGLU else None
+        y = act_down(up, gate, self.w_down, self.layer, count, offset)
         w = self.gate_weights(x, idx)
         rows = r["pair_row"]
         kept = (rows >= 0).unsqueeze(-1)

@@ -406,6 +406,20 @@ int moe_expert_gemm(moe_handle* h, const void* a_rows, const void* w, const void
 int moe_expert_wgrad(moe_handle* h, const void* dy_rows, const void* a_rows, const int32_t* expert_count,
                      const int32_t* expert_offset, int32_t N, int32_t K, void* dw, void* scratch, size_t scratch_bytes,
                      void* stream);
+/* The data gradient of the down projection with the activation's derivative in its epilogue -- the "fuse what is
+ * elementwise" of a backward chain (is_training, aristos_config.schema.json:20-23, names the mode; the reference has no
+ * backward code): du_rows = (dy_rows . w[e(r)]^T) * act'(u_rows) and, for SwiGLU, dg_rows beside it, i.e.
+ * moe_expert_gemm(dy_rows, w = transpose(w_down), no bias, MOE_ACT_NONE) followed by moe_act_backward, in one kernel and
+ * without dh ever reaching memory.  N = intermediate_size, K = hidden_size; the activation is the layer's hidden_act;
+ * u_rows / g_rows / du_rows / dg_rows are [rows, N] (g_rows and dg_rows exactly when the layer is SwiGLU).  The product
+ * is rounded to the storage type before the derivative, as the two calls do when they store dh, so both give the same
+ * bits.  Exists for bf16 and fp16 layers whose shape meets the hand-ordered tiles' conditions (N % 256 == 0,
+ * K % 128 == 0, operands below 4 GiB; option grouped_tile = 0 switches it off): moe_expert_gemm_act_backward_supported
+ * tells, and the call returns MOE_ERR_UNSUPPORTED otherwise -- the two calls remain the general path. */
+int moe_expert_gemm_act_backward_supported(const moe_handle* h, int32_t* supported);
+int moe_expert_gemm_act_backward(moe_handle* h, const void* dy_rows, const void* w, const void* u_rows, const void* g_rows,
+                                 const int32_t* expert_count, const int32_t* expert_offset, int32_t N, int32_t K,
+                                 void* du_rows, void* dg_rows, void* scratch, size_t scratch_bytes, void* stream);
 /* The elementwise and reduction steps between those products (same layers; fp32 arithmetic, one rounding on store):
  * moe_act_backward: for the first `rows` packed rows of width I, du = dh * act'(u) for hidden_act ReLU (1 where u > 0)
  *   and GELU (Phi(u) + u phi(u)); for SwiGLU, where h = silu(g) * u, du = dh * silu(g) and dg = dh * u * s * (1 + g (1 - s))

@@ -215,6 +215,48 @@ def test_activation_backward_vs_oracle(moe, act, dtype):
 
 
 @pytest.mark.parametrize("dtype", [ob.BF16, ob.F16, ob.F32])
+@pytest.mark.parametrize("act", [ob.ACT_GELU, ob.ACT_SWIGLU])
+def test_activation_backward_does_not_depend_on_alignment(moe, act, dtype):
+    """16 bytes per operand and thread where every pointer allows it, one element at a time where not: the same bits
+    either way, and nothing written in front of the first element or past the last."""
+    import torch
+    cfg = ob.Cfg(S=300, H=128, I=320, E=4, k=2, dtype=dtype, act=act, drop=0)
+    layer = moe.MoELayer(product_config(cfg))
+    kind = KIND[dtype]
+    rng = np.random.default_rng(77 + act)
+    rows = cfg.S * cfg.k - 7
+    n = rows * cfg.I
+    sw = act == ob.ACT_SWIGLU
+    host = {name: ob.from_f32(rng.standard_normal(n).astype(np.float32) * 2, dtype) for name in ("dh", "u", "g")}
+
+    def run(shift):
+        """Operands and results `shift` elements into their buffers; a guard value behind each result."""
+        dev = {}
+        for name, v in host.items():
+            buf = torch.zeros(n + 16, dtype=layer.act_dtype, device="cuda")
+            buf[shift:shift + n] = to_device(v, kind)
+            dev[name] = buf[shift:shift + n].view(rows, cfg.I)
+        outs = [torch.full((n + 16,), 7.0, dtype=layer.act_dtype, device="cuda") for _ in range(2)]
+        du, dg = (o[shift:shift + n].view(rows, cfg.I) for o in outs)
+        layer.act_backward(dev["dh"], dev["u"], dev["g"] if sw else None, du=du, dg=dg if sw else None)
+        torch.cuda.synchronize()
+        for o in outs[:2 if sw else 1]:
+            assert (o[:shift] == 7.0).all() and (o[shift + n:] == 7.0).all()
+        return from_device(du.contiguous()), from_device(dg.contiguous()) if sw else None
+
+    du0, dg0 = run(0)
+    du1, dg1 = run(1)
+    assert np.array_equal(du0, du1)
+    want_du, want_dg = ob.act_backward(host["dh"].reshape(rows, -1), host["u"].reshape(rows, -1),
+                                       host["g"].reshape(rows, -1) if sw else None, dtype, act)
+    assert max_rel_err(ob.to_f32(du0, dtype), ob.to_f32(want_du, dtype)) <= OUT_TOL[dtype]
+    if sw:
+        assert np.array_equal(dg0, dg1)
+        assert max_rel_err(ob.to_f32(dg0, dtype), ob.to_f32(want_dg, dtype)) <= OUT_TOL[dtype]
+    layer.close()
+
+
+@pytest.mark.parametrize("dtype", [ob.BF16, ob.F16, ob.F32])
 def test_bias_gradient_is_bit_exact(moe, dtype):
     """One thread per column adds the rows in ascending order, as the oracle does: the same fp32 sums, bit for bit."""
     S, H, I, E, k, cf, skew = CASES[1]
@@ -250,3 +292,84 @@ def test_combine_backward_vs_oracle(moe, dtype):
         assert (from_device(dy) != want_dy).mean() < 1e-3
     assert np.abs(from_device(dw) - want_dw).max() <= 1e-5 * max(np.abs(want_dw).max(), 1.0)
     assert not from_device(dw)[r["pair_row"] < 0].any()
+
+
+FUSED_CASES = [  # S, H, I, E, k, capacity factor, router skew, option grouped_tile (None: the library's choice)
+    (2048, 512, 1024, 4, 2, 1.25, 0.0, None),    # 256-row blocks
+    (2048, 512, 1024, 4, 2, 1.25, 0.3, 2),       # the same rows on 128-row blocks
+    (512, 128, 256, 4, 1, 2.0, 0.7, None),       # few rows per expert, ragged last blocks, an expert that may stay empty
+    (700, 256, 512, 3, 2, 1.0, 0.0, 1),          # 256-row blocks forced on few rows
+]
+
+
+@pytest.mark.parametrize("dtype", [ob.BF16, ob.F16])
+@pytest.mark.parametrize("act", [ob.ACT_RELU, ob.ACT_GELU, ob.ACT_SWIGLU])
+@pytest.mark.parametrize("case", FUSED_CASES)
+def test_fused_activation_backward_is_the_two_call_chain(moe, case, act, dtype):
+    """moe_expert_gemm_act_backward against moe_expert_gemm (no activation) followed by moe_act_backward: the product is
+    rounded to the storage type before the derivative in both, and both inline the same derivative, so the kept rows
+    agree bit for bit; against the oracle's chain within the layer's tolerance."""
+    S, H, I, E, k, cf, skew, tile = case
+    cfg, rng, count, offset = routed_case(S, H, I, E, k, dtype, seed=5 + act, cf=cf, skew=skew)
+    cfg = cfg.scaled(act=act)
+    kind = KIND[dtype]
+    layer = moe.MoELayer(product_config(cfg), options={} if tile is None else {"grouped_tile": tile})
+    assert layer.fused_act_backward
+    R = S * k
+    kept = int(count.sum())
+    assert 0 < kept <= R
+    dy, _, w_t, _ = operands(rng, R, E, I, H, dtype)              # dy [R, H] is the product's left operand; w_t [E, I, H]
+    u = ob.from_f32(rng.standard_normal((R, I)).astype(np.float32) * 2, dtype)
+    sw = act == ob.ACT_SWIGLU
+    g = ob.from_f32(rng.standard_normal((R, I)).astype(np.float32) * 2, dtype) if sw else None
+    d = {n: to_device(v, kind) for n, v in (("dy", dy), ("w", w_t), ("u", u))}
+    dg_in = to_device(g, kind) if sw else None
+    cnt, off = to_device(count, "i32"), to_device(offset, "i32")
+    du, dg = layer.expert_gemm_act_backward(d["dy"], d["w"], d["u"], dg_in, cnt, off)
+    dh = layer.expert_gemm(d["dy"], d["w"], None, cnt, off, ob.ACT_NONE)
+    du2, dg2 = layer.act_backward(dh[:kept], d["u"][:kept], dg_in[:kept] if sw else None)
+    assert np.array_equal(from_device(du)[:kept], from_device(du2))
+    assert not from_device(du)[kept:].any()                       # rows of no expert are not written
+    want_dh = ob.expert_gemm(dy, w_t, None, count, offset, dtype, ob.ACT_NONE)
+    want_du, want_dg = ob.act_backward(want_dh[:kept], u[:kept], g[:kept] if sw else None, dtype, act)
+    assert max_rel_err(ob.to_f32(from_device(du), dtype)[:kept], ob.to_f32(want_du, dtype)) <= OUT_TOL[dtype]
+    if sw:
+        assert np.array_equal(from_device(dg)[:kept], from_device(dg2))
+        assert not from_device(dg)[kept:].any()
+        assert max_rel_err(ob.to_f32(from_device(dg), dtype)[:kept], ob.to_f32(want_dg, dtype)) <= OUT_TOL[dtype]
+    else:
+        assert dg is None and dg2 is None
+    layer.close()
+
+
+def test_fused_activation_backward_says_where_it_does_not_exist(moe):
+    import torch
+    base = ob.Cfg(S=256, H=128, I=256, E=4, k=1, dtype=ob.BF16, act=ob.ACT_SWIGLU, drop=0)
+    cases = [
+        (base, {}, True),
+        (base, {"grouped_tile": 0}, False),                       # the 128 x 128 tile has no such epilogue
+        (base.scaled(I=384), {}, False),                          # 384 columns are no multiple of the tile's 256
+        (base.scaled(H=192), {}, False),                          # the slab loop takes 128 elements of the sum at a time
+        (base.scaled(dtype=ob.F32), {}, False),
+    ]
+    for cfg, opts, want in cases:
+        layer = moe.MoELayer(product_config(cfg), options=opts)
+        assert layer.fused_act_backward == want, (cfg.H, cfg.I, cfg.dtype, opts)
+        if not want:
+            dt = layer.act_dtype
+            z = lambda *s: torch.zeros(*s, dtype=dt, device="cuda")
+            cnt = torch.zeros(cfg.E, dtype=torch.int32, device="cuda")
+            with pytest.raises(moe.MoEError) as e:
+                layer.expert_gemm_act_backward(z(cfg.S, cfg.H), z(cfg.E, cfg.I, cfg.H), z(cfg.S, cfg.I), z(cfg.S, cfg.I), cnt, cnt)
+            assert e.value.status == 2
+        layer.close()
+    layer = moe.MoELayer(product_config(base))
+    z = lambda *s: torch.zeros(*s, dtype=torch.bfloat16, device="cuda")
+    cnt = torch.zeros(base.E, dtype=torch.int32, device="cuda")
+    with pytest.raises(moe.MoEError) as e:                        # a SwiGLU layer needs the gate's rows
+        layer.expert_gemm_act_backward(z(256, 128), z(4, 256, 128), z(256, 256), None, cnt, cnt)
+    assert e.value.status == 4
+    with pytest.raises(moe.MoEError) as e:                        # (N, K) = (128, 256) is the up projection's gradient
+        layer.expert_gemm_act_backward(z(256, 256), z(4, 128, 256), z(256, 128), z(256, 128), cnt, cnt)
+    assert e.value.status == 4
+    layer.close()

@@ -20,17 +20,21 @@ def rel(a, b):
     return float((a - b).abs().max() / b.abs().max().clamp(min=1e-30))
 
 
-@pytest.mark.parametrize("act,dtype,drop", [(2, 2, 0), (1, 2, 1), (0, 3, 0), (2, 3, 1), (0, 0, 0), (2, 0, 1), (1, 1, 0)])
-def test_trainable_layer_matches_torch_autograd(moe, act, dtype, drop):
+@pytest.mark.parametrize("act,dtype,drop,inter", [(2, 2, 0, 384), (1, 2, 1, 512), (0, 3, 0, 512), (2, 3, 1, 384), (0, 0, 0, 512),
+                                                  (2, 0, 1, 384), (1, 1, 0, 512), (2, 2, 1, 512), (2, 3, 0, 512)])
+def test_trainable_layer_matches_torch_autograd(moe, act, dtype, drop, inter):
     import torch
     from cuplayground_amd import training, torch_op
     cfg = moe.MoEConfig(capacity_factor=1.0, drop_tokens=drop, expert_top_k=2, hidden_act=act, hidden_size=256,
-                        intermediate_size=384 if act == 2 else 512, micro_batch=1, num_experts=6, sequence_len=700,
+                        intermediate_size=inter, micro_batch=1, num_experts=6, sequence_len=700,
                         torch_dtype=dtype, gate_fn=0, norm_topk_prob=1, is_training=1)
     m = training.MoE355Train(cfg, init_std=0.05, seed=3)
     g = torch.Generator(device="cuda").manual_seed(1)
     x = torch.randn(cfg.tokens, cfg.hidden_size, generator=g, device="cuda").to(m.layer.act_dtype).requires_grad_(True)
     dout = torch.randn(cfg.tokens, cfg.hidden_size, generator=g, device="cuda").to(m.layer.act_dtype)
+    # the activation's derivative rides in the epilogue of the down projection's data gradient where the layer has
+    # that kernel (16-bit, 256 | intermediate size), else the two building blocks run one after the other
+    assert m.layer.fused_act_backward == (dtype in (2, 3) and inter % 256 == 0)
     out = m(x)
     out.backward(dout)
 

@@ -143,8 +143,9 @@ typedef struct moe_options {
                                 intermediate rows are quantised to e4m3 with one fp32 scale per (row, 128 columns) by a pass in
                                 front of each projection (moe_quant_rows128), weights are fed as stored; one launch per
                                 projection; overrides fp8_tile and fp8_widen.  0 / AUTO = bf16 activations.  Opt-in because it
-                                changes the arithmetic: results stay within the e4m3 tolerance (3e-2 of the output range) of the
-                                bf16-activation layer but are not its bits. */
+                                changes the arithmetic: e4m3 activations keep 3 mantissa bits, and results stand 2.4e-2 to
+                                4.2e-2 of the output range away from the bf16-activation layer -- past the 3e-2 that the
+                                other e4m3 plans keep. */
     int32_t prepared_weights;/* 1 = every moe_forward on the handle will carry moe_weights.prepared (moe_prepare_weights): the
                                 workspace then holds no copies of the weights and a call without them is refused; 0 / AUTO =
                                 prepared weights are used when given, else made per call in the workspace */

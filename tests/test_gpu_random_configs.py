@@ -1,12 +1,13 @@
 """Seeded random layer shapes crossed with the tuning knobs (tile, FFN mode, queue count, early start of the next
 task, combine inside the FFN kernels, task order inside a queue segment, e4m3 streamer or tile): every combination must match the CPU oracle -- routing bit for bit, output
 within the dtype's bound -- because no knob is allowed to change what is computed (tail_split alone re-associates a sum,
-within the same bound)."""
+within the same bound).  Where the layer has the fused data gradient of the down projection, it is checked against
+the two calls it replaces on the same routing."""
 import numpy as np
 import pytest
 
 from oracle import binding as ob
-from helpers import OUT_TOL, from_device, max_rel_err, product_config, upload_inputs
+from helpers import OUT_TOL, from_device, max_rel_err, product_config, to_device, upload_inputs
 from test_gpu_layer import check_routing
 
 pytestmark = pytest.mark.gpu
@@ -75,4 +76,28 @@ def test_random_shape_and_knobs_vs_oracle(cfg, knobs, mode, with_bias):
     assert max_rel_err(o, ref) <= OUT_TOL[cfg.dtype], (knobs, mode)
     dead = (want["slot"] < 0).all(axis=1)
     assert not o[dead].any()
+    if cfg.dtype in (ob.BF16, ob.F16) and layer.fused_act_backward:
+        _fused_backward_is_the_chain(moe, layer, cfg, dev, routing, got)
     layer.close()
+
+
+def _fused_backward_is_the_chain(moe, layer, cfg, dev, routing, got):
+    """On the routing the layer just produced: the data gradient of the down projection with the activation's derivative
+    in its epilogue against the two calls it replaces, bit for bit on the kept rows."""
+    import torch
+    kind = "bf16" if cfg.dtype == ob.BF16 else "f16"
+    rng = np.random.default_rng(cfg.S + cfg.I)
+    R, kept = cfg.S * cfg.k, int(got["expert_count"].sum())
+    rand = lambda cols, scale: to_device(ob.from_f32(rng.standard_normal((R, cols)).astype(np.float32) * scale, cfg.dtype), kind)
+    dy, u = rand(cfg.H, 1.0), rand(cfg.I, 2.0)
+    g = rand(cfg.I, 2.0) if cfg.act == ob.ACT_SWIGLU else None
+    cnt, off = routing["expert_count"], routing["expert_offset"]
+    w_t = moe.transpose(dev["w_down"])
+    du, dg = layer.expert_gemm_act_backward(dy, w_t, u, g, cnt, off)
+    dh = layer.expert_gemm(dy, w_t, None, cnt, off, ob.ACT_NONE)
+    du2, dg2 = layer.act_backward(dh[:kept], u[:kept], None if g is None else g[:kept])
+    torch.cuda.synchronize()
+    assert np.array_equal(from_device(du)[:kept], from_device(du2))
+    assert not from_device(du)[kept:].any()
+    if g is not None:
+        assert np.array_equal(from_device(dg)[:kept], from_device(dg2))

@@ -26,6 +26,7 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
 PEAK_F32_TFLOPS = 157.3
+PEAK_FP8_TFLOPS = 5000.0      # MI355X dense fp8 MFMA: what bounds a layer whose both GEMM operands are e4m3 (option fp8_mfma)
 PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
 
 # Bytes per FFN-kernel launch that crossed the L2 <-> memory-fabric boundary, from two rocprofv3 --pmc runs of this
@@ -39,25 +40,25 @@ WIDEN_SOURCES = BF16_SOURCES + ("quant.hip",)
 F32_TILE_SOURCES = ("ffn_f32_tile.hip", "ffn_common.hpp", "route.hip")
 FP8_MFMA_SOURCES = FP8_TILE_SOURCES + ("quant.hip",)
 MEASURED_TRAFFIC = {
-    "mixtral": {"bytes": 18.25e9, "sources": BF16_SOURCES, "kernel_digest": "3c477f620de7",
+    "mixtral": {"bytes": 18.13e9, "sources": BF16_SOURCES, "kernel_digest": "3c477f620de7",
                 "profile": "profiles/ffn_persistent_kernel_bf16_mixtral_c3_hbm_traffic.txt"},
-    "mid": {"bytes": 0.8072e9, "sources": BF16_SOURCES, "kernel_digest": "3c477f620de7",
+    "mid": {"bytes": 0.8081e9, "sources": BF16_SOURCES, "kernel_digest": "3c477f620de7",
             "profile": "profiles/ffn_persistent_kernel_bf16_mid_c2_hbm_traffic.txt"},
-    "finegrained": {"bytes": 3.350e9, "sources": BF16_SOURCES, "kernel_digest": "3c477f620de7",
+    "finegrained": {"bytes": 3.336e9, "sources": BF16_SOURCES, "kernel_digest": "3c477f620de7",
                     "profile": "profiles/ffn_persistent_kernel_bf16_finegrained_c4_hbm_traffic.txt"},
-    "decode_fp8": {"bytes": 9.907e9, "sources": FP8_SOURCES, "kernel_digest": "47ddccc0e23f",
+    "decode_fp8": {"bytes": 9.909e9, "sources": FP8_SOURCES, "kernel_digest": "47ddccc0e23f",
                    "profile": "profiles/ffn_persistent_fp8_kernel_decode_c5_hbm_traffic.txt"},
     # a single-expert fp32 layer runs as two launches (one per projection); the figure is their sum
-    "reference_default": {"bytes": 0.9181e9, "sources": F32_TILE_SOURCES, "kernel_digest": "3e84a4ffa895", "ffn_mode": 1,
+    "reference_default": {"bytes": 0.9158e9, "sources": F32_TILE_SOURCES, "kernel_digest": "3e84a4ffa895", "ffn_mode": 1,
                           "profile": "profiles/ffn_tiled_f32_tile_kernel_reference_default_hbm_traffic.txt"},
     # the widening pass and the bf16 queue kernel together (what the layer's FFN stage launches by default) ...
-    "prefill_fp8": {"bytes": 22.96e9, "sources": WIDEN_SOURCES, "kernel_digest": "967a29900dec",
+    "prefill_fp8": {"bytes": 23.05e9, "sources": WIDEN_SOURCES, "kernel_digest": "967a29900dec",
                     "profile": "profiles/widen_plus_ffn_persistent_kernel_prefill_fp8_hbm_traffic.txt"},
     # ... the e4m3 tile GEMM on the same layer (option fp8_widen = 0) ...
-    "prefill_fp8/e4m3_tile": {"bytes": 26.39e9, "sources": FP8_TILE_SOURCES, "kernel_digest": "ed8b975c9d71",
+    "prefill_fp8/e4m3_tile": {"bytes": 26.29e9, "sources": FP8_TILE_SOURCES, "kernel_digest": "5197e02dde8f",
                               "profile": "profiles/ffn_persistent_fp8_tile_kernel_prefill_fp8_hbm_traffic.txt"},
     # ... and the e4m3 x e4m3 plan (option fp8_mfma = 1): two quantising passes and two GEMM launches
-    "prefill_fp8/e4m3_mfma": {"bytes": 14.08e9, "sources": FP8_MFMA_SOURCES, "kernel_digest": "c53e91f1af02", "ffn_mode": 1,
+    "prefill_fp8/e4m3_mfma": {"bytes": 14.60e9, "sources": FP8_MFMA_SOURCES, "kernel_digest": "7f390a4e2f33", "ffn_mode": 1,
                               "profile": "profiles/ffn_tiled_fp8_mfma_kernel_prefill_fp8_hbm_traffic.txt"},
 }
 
@@ -188,9 +189,12 @@ def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False, balanced_
                 # the whole step held against the same bytes: what a caller of moe_forward sees
                 "layer_frac": nbytes / (ms_per_step * 1e-3) / 1e9 / PEAK_HBM_GBS}
     else:
+        e4m3_mfma = fp8 and layer.options.get("fp8_mfma") == 1
         roof = {"bound": "mfma", "achieved": flops / (ffn["mean"] * 1e-3) / 1e12,
-                "peak": PEAK_F32_TFLOPS if c.torch_dtype == api.DTYPE_F32 else PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                "kernel": (("ffn_persistent_fp8_tile_kernel" if queue else "ffn_tiled_fp8_tile_kernel x2")
+                "peak": PEAK_F32_TFLOPS if c.torch_dtype == api.DTYPE_F32 else (PEAK_FP8_TFLOPS if e4m3_mfma else PEAK_BF16_TFLOPS),
+                "unit": "TFLOP/s",
+                "kernel": "quant_rows128_kernel x2 + ffn_tiled_fp8_mfma_kernel x2" if e4m3_mfma else
+                          (("ffn_persistent_fp8_tile_kernel" if queue else "ffn_tiled_fp8_tile_kernel x2")
                            if fp8 and not widened else
                            ("widen_block128_kernel x%d + " % (3 if c.hidden_act == api.ACT_SWIGLU else 2) if widened else "") +
                            ("ffn_persistent%s_kernel" if queue else "ffn_tiled%s_kernel x2") % f32_kind),
@@ -532,8 +536,9 @@ def main():
     peaks = moe.measured_peaks()
     roof = res["roofline"]
     # for the MFMA bound: the issue-only rate on random operands (the power limit lowers the clock on real data)
-    roof["measured_peak"] = peaks["hbm_read_gbs"] if roof["bound"] == "hbm" else peaks["mfma_bf16_tflops_random_operands"]
-    roof["frac_of_measured_peak"] = roof["achieved"] / roof["measured_peak"]
+    if roof["bound"] == "hbm" or roof["peak"] == PEAK_BF16_TFLOPS:
+        roof["measured_peak"] = peaks["hbm_read_gbs"] if roof["bound"] == "hbm" else peaks["mfma_bf16_tflops_random_operands"]
+        roof["frac_of_measured_peak"] = roof["achieved"] / roof["measured_peak"]
 
     trace = None
     if args.task_trace and layer.ffn_mode == 2:

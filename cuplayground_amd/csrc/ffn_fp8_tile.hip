@@ -39,6 +39,7 @@ constexpr int PBK = 64;           // k per slab
 constexpr int PROW = 128;         // bytes per LDS row (64 bf16)
 constexpr int PSTAGE = (PBM + PBN) * PROW;
 constexpr int PLDS = 2 * PSTAGE;
+constexpr int PLDS_M8 = PLDS + 2 * PBM * 4;       // e4m3 x e4m3 loop: behind the two stages, the token rows' scales of either slab
 constexpr int PTHREADS = 256;
 constexpr int PTM = 4, PTN = 4;   // 16 x 16 fragments per wavefront: tokens, weight rows
 constexpr int PRA = PBM * 8 / PTHREADS;        // 16-byte token loads per thread per slab
@@ -307,6 +308,19 @@ __device__ __forceinline__ void tile_mainloop_mfma8(const TileTask& p, unsigned 
         b_src[i] = base + (int64_t)col * p.K + chunk * 16;
     }
     const int wrow = __builtin_amdgcn_readfirstlane(prow & ~7);
+    // The scales of the slab's token rows travel like the slab, global -> LDS, one float per row (wavefronts 0 and 1: a row
+    // per lane).  As register loads they sat between the slab's requests in the memory counter, and the wait the compiler
+    // puts in front of their use waited for the next slab's requests as well: no request was in flight during a slab's
+    // MFMAs (MFMA pipes busy 24 % of the time).
+    float* const ssc = reinterpret_cast<float*>(smem + 2 * PSTAGE);        // [stage][PBM]
+    const float* sc_src = nullptr;
+    if (wave < 2) {
+        int r = tid;
+        if (r >= p.rows) r = 0;
+        const int64_t src_row = p.gather ? (int64_t)p.gather[r] : p.a_row0 + r;
+        sc_src = p.sa + src_row * KB;
+    }
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     auto issue = [&](int kb) {
         unsigned char* sa = smem + (kb & 1) * PSTAGE;
         unsigned char* sb = sa + PBM * PROW;
@@ -316,6 +330,8 @@ __device__ __forceinline__ void tile_mainloop_mfma8(const TileTask& p, unsigned 
 #pragma unroll
         for (int i = 0; i < 4; ++i)
             __builtin_amdgcn_global_load_lds((gbl_void*)(b_src[i] + kb * 128), (lds_void*)(sb + (wrow + i * 32) * PROW), 16, 0, 0);
+        if (wave_u < 2)
+            __builtin_amdgcn_global_load_lds((gbl_void*)(sc_src + kb), (lds_void*)(ssc + (kb & 1) * PBM + wave_u * 64), 4, 0, 0);
     };
 
     const int frow = lane & 15, fk = lane >> 4;
@@ -325,15 +341,7 @@ __device__ __forceinline__ void tile_mainloop_mfma8(const TileTask& p, unsigned 
     const int b_off = PBM * PROW + (wn * 16 * PTN + frow) * PROW;
     const int c0 = (fk ^ sw) << 4, c1 = ((4 + fk) ^ sw) << 4;
 
-    // the scales of this lane's token rows (one row per 16 x 16 fragment), a k block ahead
-    const float* sa_row[PTM];
-#pragma unroll
-    for (int i = 0; i < PTM; ++i) {
-        int r = wm * 16 * PTM + i * 16 + frow;
-        if (r >= p.rows) r = 0;
-        const int64_t src_row = p.gather ? (int64_t)p.gather[r] : p.a_row0 + r;
-        sa_row[i] = p.sa + src_row * KB;
-    }
+    const int sc_off = wm * 16 * PTM + frow;          // this lane's token rows (one per 16 x 16 fragment) in a stage's scales
     typedef const __attribute__((address_space(4))) float cfloat;
     cfloat* sc0 = (cfloat*)(uintptr_t)p.s[0];
     cfloat* sc1 = (cfloat*)(uintptr_t)p.s[1];
@@ -350,23 +358,16 @@ __device__ __forceinline__ void tile_mainloop_mfma8(const TileTask& p, unsigned 
 
     __syncthreads();                        // the previous task may still be reading the stages
     issue(0);
-    float san[PTM];
-#pragma unroll
-    for (int i = 0; i < PTM; ++i) san[i] = sa_row[i][0];
     for (int kb = 0; kb < KB; ++kb) {
         // slab kb has landed (it was requested a whole slab ago, and nothing younger is outstanding that we could let
         // fly: wait for all), and every wavefront is done reading the other stage
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
+        if (kb + 1 < KB) issue(kb + 1);
         float sac[PTM];
 #pragma unroll
-        for (int i = 0; i < PTM; ++i) sac[i] = san[i];
-        if (kb + 1 < KB) {
-            issue(kb + 1);
-#pragma unroll
-            for (int i = 0; i < PTM; ++i) san[i] = sa_row[i][kb + 1];
-        }
+        for (int i = 0; i < PTM; ++i) sac[i] = ssc[(kb & 1) * PBM + sc_off + i * 16];
         const float s0 = sc0[kb], s1 = sc1[kb];
         const unsigned char* st = smem + (kb & 1) * PSTAGE;
         i32x8 bf[PTN];
@@ -582,14 +583,15 @@ hipError_t launch_ffn_fp8_tile(const FfnArgs& a, int max_mtiles, int nnt0, int n
 
 // x -> e4m3 rows, up projection, h -> e4m3 rows (the kept ones), down projection.
 hipError_t launch_ffn_fp8_mfma(const FfnArgs& a, int S, int64_t A, int max_mtiles, int nnt0, int nnt1, hipStream_t st) {
-    hipError_t e = allow_lds(&ffn_tiled_fp8_mfma_kernel);
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&ffn_tiled_fp8_mfma_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, PLDS_M8);
     if (e != hipSuccess) return e;
     e = launch_quant_rows128(a.x, a.xq, a.sx, S, a.H, nullptr, st);
     if (e != hipSuccess) return e;
-    ffn_tiled_fp8_mfma_kernel<<<tiled_grid(max_mtiles, nnt0, a.groups), PTHREADS, PLDS, st>>>(a, 0);
+    ffn_tiled_fp8_mfma_kernel<<<tiled_grid(max_mtiles, nnt0, a.groups), PTHREADS, PLDS_M8, st>>>(a, 0);
     e = launch_quant_rows128(a.h, a.hq, a.sh, A, a.I, &a.q->kept_rows, st);
     if (e != hipSuccess) return e;
-    ffn_tiled_fp8_mfma_kernel<<<tiled_grid(max_mtiles, nnt1, a.groups), PTHREADS, PLDS, st>>>(a, 1);
+    ffn_tiled_fp8_mfma_kernel<<<tiled_grid(max_mtiles, nnt1, a.groups), PTHREADS, PLDS_M8, st>>>(a, 1);
     return hipGetLastError();
 }
 

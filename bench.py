@@ -78,7 +78,8 @@ def stats(samples):
             "min": round(min(samples), 5), "n": len(samples)}
 
 
-def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False, balanced_routing=False, options=None):
+def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False, balanced_routing=False, options=None,
+            other_plans=False):
     """Runs one workload; returns (result dict, layer, device operands, output tensor, routing tensors)."""
     import torch
     import cuplayground_amd as moe
@@ -166,6 +167,21 @@ def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False, balanced_
         prepared_ms = (time.perf_counter() - t5) * 1e3 / steps
         del ready
 
+    # the same steps with e4m3 activations on the fp8 matrix instruction (option fp8_mfma: other arithmetic, opt-in;
+    # reported beside the default plan of a prefill-sized e4m3 layer, never in its place)
+    fp8_mfma_ms = None
+    if other_plans and c.torch_dtype == api.DTYPE_FP8 and w.bound == "mfma" and (options or {}).get("fp8_mfma") is None:
+        alt = moe.MoELayer(c, ffn_mode=ffn_mode, options=dict(options or {}, fp8_mfma=1))
+        for _ in range(warmup):
+            alt.forward(dev["x"], dev, out=out)
+        torch.cuda.synchronize()
+        t6 = time.perf_counter()
+        for _ in range(steps):
+            alt.forward(dev["x"], dev, out=out)
+        torch.cuda.synchronize()
+        fp8_mfma_ms = (time.perf_counter() - t6) * 1e3 / steps
+        alt.close()
+
     routing = layer.new_routing()                 # one extra, untimed call fetches the routing result
     layer.forward(dev["x"], dev, out=out, routing=routing)
     torch.cuda.synchronize()
@@ -221,6 +237,7 @@ def measure(name, steps, warmup, seed, ffn_mode, calibrate_copy=False, balanced_
         "workload": w.describe(), "tokens_per_s": c.tokens / (ms_per_step * 1e-3), "ms_per_step": ms_per_step,
         "ms_per_step_with_events": ms_per_step_events, "ms_per_step_graph_replay": graph_ms if graph_err is None else graph_err,
         "ms_per_step_prepared_weights": prepared_ms,
+        "ms_per_step_fp8_mfma": fp8_mfma_ms,
         "step_ms": stats(step_ms), "steps": steps, "warmup": warmup,
         "tflops": layer_flops / (ms_per_step * 1e-3) / 1e12,
         "stage_ms": {k: round(v, 4) for k, v in stage_mean.items() if k != "calls"},
@@ -559,7 +576,8 @@ def main():
         if name not in wl.WORKLOADS:
             print("bench.py: unknown workload %r in --extra" % name, file=sys.stderr)
             sys.exit(2)
-        r, l2, d2, o2, rt2 = measure(name, args.extra_steps, args.warmup, args.seed, args.ffn_mode, options=options)
+        r, l2, d2, o2, rt2 = measure(name, args.extra_steps, args.warmup, args.seed, args.ffn_mode, options=options,
+                                     other_plans=True)
         if args.extra_cpu_seconds > 0:      # every workload has its CPU baseline beside it, on a smaller sample
             r["cpu_baseline"], r["cpu_baseline_oracle"], r["parity"] = cpu_leg(name, d2, o2, rt2, args.extra_cpu_seconds,
                                                                                 args.seed)
